@@ -1,0 +1,128 @@
+/*
+ * q4_linear.h -- C ABI of libq4linear.so: int4 weight-only quantized linear layer
+ * (GPTQ and AWQ checkpoint layouts) for AMD MI355X (gfx950).
+ *
+ * The library is stateless: every buffer is owned by the caller (PyTorch tensors on
+ * the Python side), nothing is allocated on the device, every call is asynchronous
+ * on the HIP stream it is given and can be recorded into a HIP graph.  Functions
+ * return 0 on success or a negative Q4_ERR_* code; q4_last_error() then describes
+ * the failure (thread-local).  No C++ exception crosses this boundary.
+ *
+ * Tensor conventions (K = in-features, N = out-features, G = number of groups):
+ *   GPTQ (layout 0): qweight int32 [K/8, N]  nibble j of word [r, n] = q[8r+j, n]
+ *                    qzeros  int32 [G, N/8]  nibble j of word [g, c] = zstored[g, 8c+j]
+ *                    effective zero = (zstored + 1) & 15
+ *   AWQ  (layout 1): qweight int32 [K, N/8]  nibble p of word [k, c] = q[k, 8c+ORDER[p]]
+ *                    qzeros  int32 [G, N/8]  same column order, used as stored
+ *                    ORDER = {0, 2, 4, 6, 1, 3, 5, 7}
+ *   scales fp16 [G, N] (always fp16, also for bf16 activations)
+ *   g_idx  int32 [K] or NULL: group of row k (GPTQ act-order); NULL -> k / groupsize
+ *   W[k, n] = round_to_dtype( float(scales[g(k), n]) * (q[k, n] - zero[g(k), n]) )
+ *   y[m, n] = sum_k x[m, k] * W[k, n]  accumulated in fp32 (+ bias[n]), cast to dtype
+ *   x [M, K], y [M, N], bias [N] (nullable) row-major contiguous in `dtype`.
+ */
+#ifndef Q4_LINEAR_H
+#define Q4_LINEAR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define Q4_LAYOUT_GPTQ 0
+#define Q4_LAYOUT_AWQ 1
+
+#define Q4_DTYPE_F16 0
+#define Q4_DTYPE_BF16 1
+
+#define Q4_OK 0
+#define Q4_ERR_INVALID_ARGUMENT (-1) /* null pointer, bad enum, bad shape */
+#define Q4_ERR_UNSUPPORTED (-2)      /* a shape the kernels do not cover */
+#define Q4_ERR_WORKSPACE (-3)        /* workspace missing or too small */
+#define Q4_ERR_LAUNCH (-4)           /* HIP reported a launch error */
+
+/* Which kernel q4_linear picks; also accepted by q4_linear_ex to force one. */
+#define Q4_PATH_AUTO 0
+#define Q4_PATH_GEMV 1    /* split-K dequant GEMV, decode (small M) */
+#define Q4_PATH_GEMM 2    /* dequant-to-LDS + MFMA GEMM, prefill (large M) */
+#define Q4_PATH_GENERIC 3 /* shape-agnostic kernel for unaligned K / N */
+
+/* Problem description shared by every entry point. */
+typedef struct q4_weight {
+  const uint32_t* qweight; /* packed nibbles, see layout above */
+  const uint32_t* qzeros;  /* packed zero points [G, N/8] */
+  const void* scales;      /* fp16 [G, N] */
+  const int32_t* g_idx;    /* int32 [K] or NULL */
+  int32_t K;               /* in-features, multiple of 8 */
+  int32_t N;               /* out-features, multiple of 8 */
+  int32_t groupsize;       /* rows per group when g_idx is NULL (K for "one group") */
+  int32_t num_groups;      /* G: rows of scales / qzeros */
+  int32_t layout;          /* Q4_LAYOUT_* */
+} q4_weight;
+
+/*
+ * Materialise the dense dequantized weight W [K, N] in `dtype` (bit-exact with the
+ * reference's dequantize step).  Replaces exllamav2 reconstruct_gptq_kernel
+ * (server/exllamav2_kernels/exllamav2_kernels/cuda/q_matrix.cu:182-299, pybind
+ * `reconstruct` path of ext.cpp) and exllama v1 reconstruct_kernel
+ * (server/exllama_kernels/exllama_kernels/cuda_func/q4_matrix.cu:166-220); used by the
+ * parity tests and by callers that want a dense copy.
+ */
+int q4_dequant(const q4_weight* w, void* w_out, int dtype, void* stream);
+
+/*
+ * y = x @ W (+ bias).  The forward of the quantized linear layer; picks the decode or
+ * the prefill kernel from M.  Replaces `gemm_half_q_half` (server/exllamav2_kernels/
+ * exllamav2_kernels/ext.cpp:100-131 -> cuda/q_gemm.cu:116-191), `q4_matmul`
+ * (server/exllama_kernels/exllama_kernels/exllama_ext.cpp:168-213), the Triton
+ * `matmul248` launcher (server/text_generation_server/layers/gptq/triton.py:204-241)
+ * and `awq_inference_engine.gemm_forward_cuda` (call site
+ * server/text_generation_server/layers/awq/quantize/cuda.py:45-47).
+ *
+ * workspace: device buffer of at least q4_workspace_bytes(M, K, N) bytes whose first
+ * Q4_WORKSPACE_COUNTER_BYTES bytes were zero before the first call that used it; the
+ * kernels leave them zero again.  Calls that share a workspace must be ordered on
+ * one stream.
+ */
+int q4_linear(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+              void* workspace, size_t workspace_bytes, void* stream);
+
+/* Same as q4_linear with the kernel path forced (Q4_PATH_*); for tests and benchmarks. */
+int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                 void* workspace, size_t workspace_bytes, int path, void* stream);
+
+/*
+ * Decode kernel with an explicit work decomposition, for tuning sweeps: `wcol` waves
+ * across columns and `wk` waves across K per workgroup (wcol * wk <= 8), `splits`
+ * workgroups across K.  K must be a multiple of 128 * wk * splits and N of 64 * wcol.
+ * Plays the role of exllama's `set_tuning_params`
+ * (server/exllama_kernels/exllama_kernels/exllama_ext.cpp:78-100) without global state.
+ */
+int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                  void* workspace, size_t workspace_bytes, int wcol, int wk, int splits,
+                  void* stream);
+
+/*
+ * Bytes of workspace q4_linear needs for an [M, K] x [K, N] problem (split-K partial
+ * sums + ticket counters).  Replaces the scratch sizing of
+ * server/text_generation_server/layers/gptq/exllamav2.py:233-240
+ * (temp_dq_size / temp_fwd_size / scratch_space_fixed).
+ */
+#define Q4_WORKSPACE_COUNTER_BYTES 16384
+size_t q4_workspace_bytes(int M, int K, int N);
+
+/* The Q4_PATH_* value q4_linear would take for this problem (negative on bad arguments). */
+int q4_select_path(const q4_weight* w, int M, int dtype);
+
+/* Message for the last failing call on this thread ("" if none). */
+const char* q4_last_error(void);
+
+/* ABI version; bumped when a signature changes. */
+int q4_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* Q4_LINEAR_H */

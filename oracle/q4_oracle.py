@@ -1,0 +1,299 @@
+"""CPU oracle for the int4 weight-only quantized linear layer (GPTQ / AWQ).
+
+THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only tests/, __graft_entry__.smoke()
+and bench.py's cpu_baseline leg may import it, and only as the checker.  The product
+path (the HIP kernels behind the C-ABI library) never routes through this file.
+
+It restates, in NumPy, the arithmetic the reference performs on this path.  Each
+function cites the reference file:line it follows (paths relative to the reference
+checkout root).
+
+Pinning status (what proves each function right, other than itself):
+  unpack_rows / unpack_cols / pack_rows / pack_cols
+        pinned: literal known-answer words (0x76543210 etc.), round trips through an
+        independent restatement of the reference's writer (QuantLinear.pack), pure
+        Python element-wise brute force on tiny shapes.
+  gptq_zero_points (+1 rule)
+        pinned: the reference writer stores z-1 (triton.py:326) so writer->reader round
+        trip recovers W only with the +1; literal 0x77777777 -> 8.
+  awq_unpack_cols / awq_pack_cols / fast_awq_to_gptq
+        pinned: ORDER/REVERSE are mutual inverses, literal words, and the equivalence
+        dequant_awq(q, z, s) == dequant_gptq(*fast_awq_to_gptq(q, z), s) bit for bit.
+  dequant_gptq / dequant_awq
+        pinned: closed-form cases (constant nibbles), writer round trip, g_idx
+        permutation invariance, trivial g_idx == no g_idx, IEEE single-rounding check
+        against float64.
+  matmul_fp32 / linear_forward
+        pinned: float64 matmul, linearity, identity/one-hot activations that read
+        single weight rows back.
+  awq_inference_engine.gemm_forward_cuda (third-party, huggingface/llm-awq @ bd1dc2d5,
+  not in the reference tree): parity unpinned by any runnable reference test; covered
+  through the in-tree equivalence fast_awq_to_gptq (awq/conversion_utils.py:83-97).
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+# server/text_generation_server/layers/awq/conversion_utils.py:5-6
+AWQ_PACK_ORDER = [0, 2, 4, 6, 1, 3, 5, 7]
+REVERSE_AWQ_PACK_ORDER = [0, 4, 1, 5, 2, 6, 3, 7]
+
+_SHIFTS = np.arange(0, 32, 4, dtype=np.uint32)
+
+
+def _as_u32(a: np.ndarray) -> np.ndarray:
+    a = np.asarray(a)
+    if a.dtype == np.int32:
+        return a.view(np.uint32)
+    if a.dtype == np.uint32:
+        return a
+    raise TypeError(f"packed tensors must be int32/uint32, got {a.dtype}")
+
+
+# --------------------------------------------------------------------------- unpack / pack
+
+
+def unpack_rows(qmatrix: np.ndarray) -> np.ndarray:
+    """[R, C] packed words -> [8R, C] nibbles; nibble j of word [r, c] is element [8r+j, c].
+
+    Follows layers/gptq/triton.py:160-169,191 (shifter = (k % 8) * 4 on qweight rows) and
+    layers/awq/conversion_utils.py:52-55 (direction="row").
+    """
+    q = _as_u32(qmatrix)
+    out = (q[:, None, :] >> _SHIFTS[None, :, None]) & np.uint32(0xF)
+    return out.reshape(q.shape[0] * 8, q.shape[1]).astype(np.uint8)
+
+
+def unpack_cols(qmatrix: np.ndarray) -> np.ndarray:
+    """[R, C] packed words -> [R, 8C] nibbles; nibble j of word [r, c] is element [r, 8c+j].
+
+    Follows layers/gptq/triton.py:167,170,184 (zeros_shifter = (n % 8) * 4),
+    exllamav2_kernels/cuda/matrix_view.cuh:85-119 and conversion_utils.py:47-50.
+    """
+    q = _as_u32(qmatrix)
+    out = (q[:, :, None] >> _SHIFTS[None, None, :]) & np.uint32(0xF)
+    return out.reshape(q.shape[0], q.shape[1] * 8).astype(np.uint8)
+
+
+def pack_rows(imatrix: np.ndarray) -> np.ndarray:
+    """Inverse of unpack_rows (conversion_utils.py:26-28; writer triton.py:316-324)."""
+    i = (np.asarray(imatrix).astype(np.int64) & 0xF).astype(np.uint32)
+    assert i.shape[0] % 8 == 0
+    i = i.reshape(i.shape[0] // 8, 8, i.shape[1])
+    q = np.bitwise_or.reduce(i << _SHIFTS[None, :, None], axis=1)
+    return q.astype(np.uint32).view(np.int32)
+
+
+def pack_cols(imatrix: np.ndarray) -> np.ndarray:
+    """Inverse of unpack_cols (conversion_utils.py:22-24; writer triton.py:332-343)."""
+    i = (np.asarray(imatrix).astype(np.int64) & 0xF).astype(np.uint32)
+    assert i.shape[1] % 8 == 0
+    i = i.reshape(i.shape[0], i.shape[1] // 8, 8)
+    q = np.bitwise_or.reduce(i << _SHIFTS[None, None, :], axis=2)
+    return q.astype(np.uint32).view(np.int32)
+
+
+def awq_unpack_cols(qmatrix: np.ndarray) -> np.ndarray:
+    """AWQ GEMM layout -> logical [R, 8C] nibbles.
+
+    Position p of word [r, c] holds logical column 8c + AWQ_PACK_ORDER[p]
+    (conversion_utils.py:83-92: unpack by columns then reorder with REVERSE_AWQ_PACK_ORDER).
+    """
+    raw = unpack_cols(qmatrix)
+    r = raw.reshape(raw.shape[0], -1, 8)[:, :, REVERSE_AWQ_PACK_ORDER]
+    return r.reshape(raw.shape)
+
+
+def awq_pack_cols(imatrix: np.ndarray) -> np.ndarray:
+    """Logical [R, 8C] nibbles -> AWQ GEMM layout words (inverse of awq_unpack_cols)."""
+    i = np.asarray(imatrix)
+    r = i.reshape(i.shape[0], -1, 8)[:, :, AWQ_PACK_ORDER].reshape(i.shape)
+    return pack_cols(r)
+
+
+def fast_awq_to_gptq(qweight: np.ndarray, qzeros: np.ndarray):
+    """AWQ (qweight [K, N/8], qzeros [G, N/8]) -> GPTQ (qweight [K/8, N], qzeros [G, N/8]).
+
+    Follows conversion_utils.py:83-97: un-interleave, subtract 1 from the zero points
+    (masked to 4 bits by pack), repack weights by rows and zeros by columns.
+    """
+    izeros = awq_unpack_cols(qzeros).astype(np.int16) - 1
+    iweights = awq_unpack_cols(qweight)
+    return pack_rows(iweights), pack_cols(izeros)
+
+
+# --------------------------------------------------------------------------- dequant
+
+
+def gptq_zero_points(qzeros: np.ndarray) -> np.ndarray:
+    """[G, N/8] words -> effective zero points [G, N] = (stored + 1) & 0xF.
+
+    Follows triton.py:184-185, exllamav2 q_gemm_kernel_gptq.cuh:155-158,
+    exllama q4_matmul.cu:89 and gaudi hpu.py:58-69 (all apply the same +1).
+    """
+    return ((unpack_cols(qzeros).astype(np.int16) + 1) & 0xF).astype(np.uint8)
+
+
+def group_index(K: int, groupsize: int, g_idx: np.ndarray | None) -> np.ndarray:
+    """Group of every input row: g_idx[k] if given, else k // groupsize (triton.py:174-182)."""
+    if g_idx is not None:
+        g = np.asarray(g_idx).astype(np.int64)
+        assert g.shape == (K,)
+        return g
+    if groupsize == -1:
+        groupsize = K
+    return np.arange(K, dtype=np.int64) // groupsize
+
+
+def f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
+    """float32 -> bfloat16 bit patterns (uint16), round to nearest even, NaN kept quiet."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    rounded = (u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)
+    nan = np.isnan(a)
+    rounded = np.where(nan, (u >> np.uint32(16)) | np.uint32(0x40), rounded)
+    return rounded.astype(np.uint16)
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def _scale_diff(scales: np.ndarray, q: np.ndarray, z: np.ndarray, g: np.ndarray, dtype: str):
+    """W[k, n] = round_dtype(float(s[g(k), n]) * float(q[k, n] - z[g(k), n])).
+
+    The product of an 11-bit significand and an integer of magnitude <= 15 is exact in
+    float32, so rounding it once to fp16 equals the reference's single fp16 multiply
+    (triton.py:192; q_matrix.cu:282-293; q4_matrix.cu:194-202).  For bf16 the same exact
+    product is rounded once to bf16 (extension; the reference is fp16-only here).
+    """
+    s = np.asarray(scales)
+    assert s.dtype == np.float16, "scales are fp16 on this path (gptq/__init__.py:29-31)"
+    diff = q.astype(np.int16) - z[g].astype(np.int16)
+    prod = s[g].astype(np.float32) * diff.astype(np.float32)
+    if dtype == "f16":
+        return prod.astype(np.float16)
+    if dtype == "bf16":
+        return f32_to_bf16_bits(prod)
+    raise ValueError(dtype)
+
+
+def dequant_gptq(qweight, qzeros, scales, g_idx=None, groupsize=128, dtype="f16"):
+    """Dense W [K, N] (np.float16, or uint16 bf16 bit patterns) from GPTQ tensors.
+
+    Follows triton.py:139-192 (layout + arithmetic) and gaudi hpu.py:58-78.
+    """
+    q = unpack_rows(qweight)
+    z = gptq_zero_points(qzeros)
+    K, N = q.shape
+    assert z.shape[1] == N and scales.shape == z.shape, (q.shape, z.shape, scales.shape)
+    g = group_index(K, groupsize, g_idx)
+    assert g.min() >= 0 and g.max() < z.shape[0]
+    return _scale_diff(scales, q, z, g, dtype)
+
+
+def dequant_awq(qweight, qzeros, scales, groupsize=128, dtype="f16"):
+    """Dense W [K, N] from AWQ GEMM-layout tensors; zero points are used as stored.
+
+    Follows awq/conversion_utils.py:35-97 (layout) and gaudi awq/quantize/hpu.py:22-72
+    (W = s * (q - z), no +1).
+    """
+    q = awq_unpack_cols(qweight)
+    z = awq_unpack_cols(qzeros)
+    K, N = q.shape
+    assert z.shape[1] == N and scales.shape == z.shape, (q.shape, z.shape, scales.shape)
+    g = group_index(K, groupsize, None)
+    assert g.max() < z.shape[0]
+    return _scale_diff(scales, q, z, g, dtype)
+
+
+# --------------------------------------------------------------------------- matmul / forward
+
+
+def to_f32(a: np.ndarray, dtype: str) -> np.ndarray:
+    if dtype == "f16":
+        assert a.dtype == np.float16
+        return a.astype(np.float32)
+    if dtype == "bf16":
+        assert a.dtype == np.uint16
+        return bf16_bits_to_f32(a)
+    raise ValueError(dtype)
+
+
+def matmul_fp32(x_f32: np.ndarray, w_f32: np.ndarray) -> np.ndarray:
+    """y = x @ W with float32 accumulation (the fp32-accumulated reference of the parity bar)."""
+    return np.matmul(x_f32.astype(np.float32), w_f32.astype(np.float32))
+
+
+def linear_forward(x, w, bias=None, dtype="f16"):
+    """Reference forward contract (triton.py:351-363; awq/quantize/cuda.py:43-49).
+
+    x: [..., K] in `dtype`; w: dense dequantized [K, N] in `dtype`.  Returns
+    (y_f32 [..., N] before the output cast, y_cast in `dtype`).  The bias is added after
+    the matmul result has been cast to the activation dtype, as the reference does
+    (`out + self.bias` on an fp16 tensor).
+    """
+    K, N = w.shape
+    lead = x.shape[:-1]
+    x2 = to_f32(x.reshape(-1, K), dtype)
+    y = matmul_fp32(x2, to_f32(w, dtype))
+    if dtype == "f16":
+        yc = y.astype(np.float16)
+        if bias is not None:
+            yc = (yc.astype(np.float32) + bias.astype(np.float32)).astype(np.float16)
+            y = y + bias.astype(np.float32)
+    else:
+        yc = f32_to_bf16_bits(y)
+        if bias is not None:
+            yc = f32_to_bf16_bits(bf16_bits_to_f32(yc) + bf16_bits_to_f32(bias))
+            y = y + bf16_bits_to_f32(bias)
+    return y.reshape(lead + (N,)), yc.reshape(lead + (N,))
+
+
+# --------------------------------------------------------------------------- synthetic inputs
+
+
+def make_gptq(K, N, groupsize=128, seed=0, sym=True, act_order=False):
+    """Seeded synthetic GPTQ tensors of the benchmark's shape.
+
+    nibbles uniform 0..15 packed 8 per int32 along K; scales fp16 uniform [1e-3, 2e-2];
+    sym -> stored zero nibble 7 (effective 8, the value the reference writer emits for
+    symmetric quantisation, triton.py:326-343), else uniform 0..15; act_order ->
+    g_idx[perm[i]] = i // groupsize for a random permutation (every group has exactly
+    `groupsize` rows).
+    """
+    rng = np.random.default_rng(seed)
+    gs = K if groupsize == -1 else groupsize
+    G = (K + gs - 1) // gs
+    q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    qweight = pack_rows(q)
+    if sym:
+        zs = np.full((G, N), 7, dtype=np.uint8)
+    else:
+        zs = rng.integers(0, 16, size=(G, N), dtype=np.uint8)
+    qzeros = pack_cols(zs)
+    scales = rng.uniform(1e-3, 2e-2, size=(G, N)).astype(np.float16)
+    g_idx = None
+    if act_order:
+        perm = rng.permutation(K)
+        g_idx = np.empty(K, dtype=np.int32)
+        g_idx[perm] = (np.arange(K) // gs).astype(np.int32)
+    return qweight, qzeros, scales, g_idx
+
+
+def make_awq(K, N, groupsize=128, seed=0):
+    """Seeded synthetic AWQ GEMM-layout tensors: nibbles and zero points uniform 0..15."""
+    rng = np.random.default_rng(seed)
+    gs = K if groupsize == -1 else groupsize
+    G = K // gs
+    q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(G, N), dtype=np.uint8)
+    scales = rng.uniform(1e-3, 2e-2, size=(G, N)).astype(np.float16)
+    return awq_pack_cols(q), awq_pack_cols(z), scales
+
+
+def make_x(M, K, seed=0, dtype="f16"):
+    """Activations ~ N(0, 1) in the given dtype (fp16 array, or bf16 bit patterns)."""
+    rng = np.random.default_rng(seed + 7919)
+    x = rng.standard_normal((M, K), dtype=np.float32)
+    return x.astype(np.float16) if dtype == "f16" else f32_to_bf16_bits(x)

@@ -1,0 +1,108 @@
+"""GPU parity of y = x @ dequant(W): every kernel path against the oracle.
+
+Bar (BASELINE.json north_star): max|y - ref| / max|ref| <= 2e-3 against an
+fp32-accumulated reference built from the bit-exact dequantized weights.  The fp16/bf16
+output rounding itself is up to 2^-11 / 2^-8 relative, so the comparison target is the
+oracle's output rounded to the activation dtype; the fp32 value is checked too.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from tests.util import max_rel_err, to_dev, to_f32
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-3       # north_star tolerance, fp16
+TOL_BF16 = 8e-3  # bf16 output rounding alone is 2^-8 = 3.9e-3 per element
+
+
+def _run(pkg, oracle, gpu, K, N, gs, M, dtype="f16", layout="gptq", sym=True, act=False, bias=False, path=0, cfg=None, seed=0):
+    bf = dtype == "bf16"
+    if layout == "gptq":
+        qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=seed, sym=sym, act_order=act)
+        w = oracle.dequant_gptq(qw, qz, sc, gi, gs, dtype)
+        lay = 0
+    else:
+        qw, qz, sc = oracle.make_awq(K, N, gs, seed=seed)
+        gi = None
+        w = oracle.dequant_awq(qw, qz, sc, gs, dtype)
+        lay = 1
+    x = oracle.make_x(M, K, seed=seed, dtype=dtype)
+    b = None
+    if bias:
+        rng = np.random.default_rng(seed + 1)
+        bf32 = rng.standard_normal(N).astype(np.float32)
+        b = bf32.astype(np.float16) if not bf else oracle.f32_to_bf16_bits(bf32)
+    y32, ycast = oracle.linear_forward(x, w, b, dtype)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), gs, lay)
+    xt = to_dev(x, gpu, bf16=bf)
+    bt = to_dev(b, gpu, bf16=bf)
+    got = pkg.ops.linear(pk, xt, bt, path=path, gemv_config=cfg)
+    torch.cuda.synchronize()
+    assert got.shape == (M, N)
+    assert got.dtype == (torch.bfloat16 if bf else torch.float16)
+    g = to_f32(got)
+    assert np.isfinite(g).all()
+    err = max_rel_err(g, y32)
+    assert err <= (TOL_BF16 if bf else TOL), f"max rel err {err:.3e}"
+    return g, y32
+
+
+GEMV_SHAPES = [(4096, 4096), (4096, 6144), (4096, 28672), (14336, 4096)]
+
+
+def test_cfg1_gptq_m16(pkg, oracle, gpu):
+    """BASELINE configs[0]: K=N=4096, groupsize 128, sym, M=16."""
+    _run(pkg, oracle, gpu, 4096, 4096, 128, 16, seed=1)
+
+
+@pytest.mark.parametrize("K,N", GEMV_SHAPES)
+@pytest.mark.parametrize("M", [1, 2, 4, 8, 16])
+def test_gemv_llama3_8b(pkg, oracle, gpu, K, N, M):
+    pk_path = 1  # force the decode kernel
+    _run(pkg, oracle, gpu, K, N, 128, M, path=pk_path, seed=K // 64 + N // 64 + M)
+
+
+@pytest.mark.parametrize("M", [1, 3, 5, 7, 11, 13, 16])
+def test_gemv_ragged_m_asym_bias(pkg, oracle, gpu, M):
+    _run(pkg, oracle, gpu, 1024, 512, 128, M, sym=False, bias=True, path=1, seed=M)
+
+
+@pytest.mark.parametrize("gs", [32, 64, 128, 256, 512, -1])
+def test_gemv_groupsizes(pkg, oracle, gpu, gs):
+    _run(pkg, oracle, gpu, 1024, 256, gs, 3, sym=False, path=1, seed=gs + 100)
+
+
+@pytest.mark.parametrize("cfg", [(1, 1, 1), (1, 1, 8), (2, 1, 4), (4, 1, 2), (1, 4, 2), (2, 2, 2), (4, 2, 1), (1, 8, 1), (2, 4, 1), (4, 1, 16)])
+@pytest.mark.parametrize("M", [1, 6, 16])
+def test_gemv_decompositions(pkg, oracle, gpu, cfg, M):
+    if M * (2048 // cfg[2] * 2 + 16) > 65536:
+        # the activation slab of this decomposition does not fit 64 KB of LDS: the library
+        # must refuse it with a clear error instead of launching
+        with pytest.raises(pkg._lib.Q4Error, match="LDS"):
+            _run(pkg, oracle, gpu, 2048, 1024, 128, M, sym=False, cfg=cfg, seed=1)
+        return
+    _run(pkg, oracle, gpu, 2048, 1024, 128, M, sym=False, bias=(M == 6), cfg=cfg, seed=sum(cfg) + M)
+
+
+def test_gemv_bf16(pkg, oracle, gpu):
+    _run(pkg, oracle, gpu, 4096, 4096, 128, 8, dtype="bf16", sym=False, path=1, seed=9)
+
+
+def test_gemv_deterministic_and_tickets_reset(pkg, oracle, gpu):
+    """Split-K combines partials in a fixed order: repeated calls are bit-identical, and
+    the ticket counters return to zero so the same workspace serves the next call."""
+    a, _ = _run(pkg, oracle, gpu, 4096, 4096, 128, 4, path=1, seed=3)
+    b, _ = _run(pkg, oracle, gpu, 4096, 4096, 128, 4, path=1, seed=3)
+    assert np.array_equal(a, b)
+    for ws in pkg.ops._workspaces.values():
+        assert int(ws[: pkg._lib.WORKSPACE_COUNTER_BYTES].sum().item()) == 0
+
+
+@pytest.mark.parametrize("layout,act", [("gptq", True), ("awq", False), ("gptq", False)])
+@pytest.mark.parametrize("M", [1, 5, 33])
+def test_generic_path(pkg, oracle, gpu, layout, act, M):
+    _run(pkg, oracle, gpu, 1000 if layout == "gptq" and not act else 1024, 264, 40 if (layout == "gptq" and not act) else 128, M,
+         layout=layout, sym=False, act=act, bias=True, path=3, seed=M + 50)

@@ -1,0 +1,157 @@
+// C ABI of libq4linear.so: argument validation, path selection, error reporting.
+// Nothing here allocates device memory or synchronises; every launch goes to the
+// caller's stream.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "q4_common.cuh"
+
+namespace {
+thread_local char g_error[512] = "";
+}
+
+namespace q4host {
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+}  // namespace q4host
+
+using namespace q4host;
+
+static int validate_weight(const q4_weight* w, const char* who) {
+  if (w == nullptr) {
+    set_error("%s: null q4_weight", who);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (w->layout != Q4_LAYOUT_GPTQ && w->layout != Q4_LAYOUT_AWQ) {
+    set_error("%s: unknown layout %d", who, w->layout);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (w->K < 0 || w->N < 0 || w->K % 8 != 0 || w->N % 8 != 0) {
+    set_error("%s: K=%d and N=%d must be non-negative multiples of 8", who, w->K, w->N);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (w->K == 0 || w->N == 0) return Q4_OK;
+  if (w->qweight == nullptr || w->qzeros == nullptr || w->scales == nullptr) {
+    set_error("%s: null qweight/qzeros/scales", who);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (w->groupsize < 1 || w->num_groups < 1) {
+    set_error("%s: groupsize=%d num_groups=%d must be positive", who, w->groupsize, w->num_groups);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (w->g_idx == nullptr && (long)w->num_groups * w->groupsize < w->K) {
+    set_error("%s: %d groups of %d rows do not cover K=%d", who, w->num_groups, w->groupsize, w->K);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (w->layout == Q4_LAYOUT_AWQ && w->g_idx != nullptr) {
+    set_error("%s: g_idx is not defined for the AWQ layout", who);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  return Q4_OK;
+}
+
+static int validate_dtype(int dtype, const char* who) {
+  if (dtype != Q4_DTYPE_F16 && dtype != Q4_DTYPE_BF16) {
+    set_error("%s: unknown dtype %d", who, dtype);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  return Q4_OK;
+}
+
+extern "C" {
+
+int q4_abi_version(void) { return 1; }
+
+const char* q4_last_error(void) { return g_error; }
+
+int q4_dequant(const q4_weight* w, void* w_out, int dtype, void* stream) {
+  int rc = validate_weight(w, "q4_dequant");
+  if (rc == Q4_OK) rc = validate_dtype(dtype, "q4_dequant");
+  if (rc != Q4_OK) return rc;
+  if (w->K == 0 || w->N == 0) return Q4_OK;
+  if (w_out == nullptr) {
+    set_error("q4_dequant: null output");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  return launch_dequant(w, w_out, dtype, (hipStream_t)stream);
+}
+
+int q4_select_path(const q4_weight* w, int M, int dtype) {
+  if (validate_weight(w, "q4_select_path") != Q4_OK) return Q4_ERR_INVALID_ARGUMENT;
+  if (M <= 16 && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
+  if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;
+  return Q4_PATH_GENERIC;
+}
+
+size_t q4_workspace_bytes(int M, int K, int N) {
+  if (M < 1 || K < 1 || N < 1) return Q4_WORKSPACE_COUNTER_BYTES;
+  const int rows = M < 16 ? M : 16;
+  q4_weight w = {};
+  w.K = K;
+  w.N = N;
+  w.layout = Q4_LAYOUT_GPTQ;
+  w.groupsize = 128;
+  w.num_groups = (K + 127) / 128;
+  int splits = 1;
+  if (K % 128 == 0 && N % 64 == 0) {
+    for (int m = 1; m <= rows; ++m) {
+      const int s = gemv_pick_config(&w, m).splits;
+      if (s > splits) splits = s;
+    }
+  }
+  return (size_t)Q4_WORKSPACE_COUNTER_BYTES + (size_t)splits * rows * N * sizeof(float);
+}
+
+int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                 void* workspace, size_t workspace_bytes, int path, void* stream) {
+  int rc = validate_weight(w, "q4_linear");
+  if (rc == Q4_OK) rc = validate_dtype(dtype, "q4_linear");
+  if (rc != Q4_OK) return rc;
+  if (M < 0) {
+    set_error("q4_linear: negative M=%d", M);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M == 0 || w->N == 0) return Q4_OK;
+  if (y == nullptr || (x == nullptr && w->K > 0)) {
+    set_error("q4_linear: null x or y");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (path == Q4_PATH_AUTO) path = q4_select_path(w, M, dtype);
+  switch (path) {
+    case Q4_PATH_GEMV:
+      return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, nullptr,
+                         (hipStream_t)stream);
+    case Q4_PATH_GEMM:
+      return launch_gemm(w, x, bias, y, M, dtype, (hipStream_t)stream);
+    case Q4_PATH_GENERIC:
+      return launch_generic(w, x, bias, y, M, dtype, (hipStream_t)stream);
+    default:
+      set_error("q4_linear: unknown path %d", path);
+      return Q4_ERR_INVALID_ARGUMENT;
+  }
+}
+
+int q4_linear(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+              void* workspace, size_t workspace_bytes, void* stream) {
+  return q4_linear_ex(w, x, bias, y, M, dtype, workspace, workspace_bytes, Q4_PATH_AUTO, stream);
+}
+
+int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                  void* workspace, size_t workspace_bytes, int wcol, int wk, int splits,
+                  void* stream) {
+  int rc = validate_weight(w, "q4_gemv_tuned");
+  if (rc == Q4_OK) rc = validate_dtype(dtype, "q4_gemv_tuned");
+  if (rc != Q4_OK) return rc;
+  if (M < 1 || x == nullptr || y == nullptr) {
+    set_error("q4_gemv_tuned: bad M=%d or null x/y", M);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  GemvConfig cfg{wcol, wk, splits};
+  return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, &cfg, (hipStream_t)stream);
+}
+
+}  // extern "C"

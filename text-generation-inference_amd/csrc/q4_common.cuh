@@ -1,0 +1,137 @@
+// Shared device helpers for the int4 weight-only linear kernels (gfx950 / CDNA4 only).
+//
+// Nibble -> half conversion uses the exponent-splice identity: for 0 <= q <= 15 the
+// fp16 bit pattern 0x6400 | q is exactly 1024 + q, and 0x6400 | (q << 4) is exactly
+// 1024 + 16 q.  One 32-bit AND+OR therefore converts two nibbles that sit 16 bits apart
+// (nibbles j and j+4 of a packed word) into a half2 with no integer->float conversion.
+// The pairing (j, j+4) is kept all the way into the MFMA operand; the activation tile
+// is permuted to the same order instead of repacking the weights.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "q4_linear.h"
+
+namespace q4 {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+// Logical column held at nibble position p of an AWQ word is 8c + kAwqOrder[p]
+// (server/text_generation_server/layers/awq/conversion_utils.py:5).
+__device__ __forceinline__ int awq_order(int p) { return ((p & 3) << 1) | (p >> 2); }
+// Nibble position that holds logical column 8c + i (conversion_utils.py:6).
+__device__ __forceinline__ int awq_position(int i) { return ((i & 1) << 2) | (i >> 1); }
+
+__device__ __forceinline__ uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
+__device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+
+// (stored + 1) & 15 on eight packed nibbles at once (GPTQ zero-point rule,
+// server/text_generation_server/layers/gptq/triton.py:184-185).
+__device__ __forceinline__ uint32_t gptq_zero_plus_one(uint32_t z) {
+  return ((z & 0x77777777u) + 0x11111111u) ^ (z & 0x88888888u);
+}
+
+// float -> bf16 bits, round to nearest even (inputs here are finite).
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
+  return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+
+// One dequantized weight in the reference's arithmetic: round_once(s * (q - z)).
+// (q - z) is an exact small integer; in fp16 the single multiply rounds once
+// (triton.py:192, q_matrix.cu:282-293); in bf16 the exact fp32 product is rounded once.
+template <int DTYPE>
+__device__ __forceinline__ uint16_t dequant_one(half_t s, int q, int z) {
+  if constexpr (DTYPE == Q4_DTYPE_F16) {
+    half_t w = (half_t)(float)(q - z) * s;
+    return __builtin_bit_cast(uint16_t, w);
+  } else {
+    return f32_to_bf16_rne((float)s * (float)(q - z));
+  }
+}
+
+template <int DTYPE>
+__device__ __forceinline__ float load_act(const void* p, size_t idx) {
+  if constexpr (DTYPE == Q4_DTYPE_F16) {
+    return (float)((const half_t*)p)[idx];
+  } else {
+    return bf16_bits_to_f32(((const uint16_t*)p)[idx]);
+  }
+}
+
+template <int DTYPE>
+__device__ __forceinline__ uint16_t store_act(float v) {
+  if constexpr (DTYPE == Q4_DTYPE_F16) {
+    half_t h = (half_t)v;
+    return __builtin_bit_cast(uint16_t, h);
+  } else {
+    return f32_to_bf16_rne(v);
+  }
+}
+
+// Output rounding used by every kernel: the fp32 sum is cast to the activation dtype,
+// then the bias is added in that dtype's arithmetic (fp32 add, rounded once), matching
+// `out + self.bias` on a half tensor (triton.py:362).
+template <int DTYPE>
+__device__ __forceinline__ uint16_t finish_output(float acc, const void* bias, int n) {
+  uint16_t y = store_act<DTYPE>(acc);
+  if (bias != nullptr) {
+    float yb;
+    if constexpr (DTYPE == Q4_DTYPE_F16) {
+      yb = (float)__builtin_bit_cast(half_t, y) + (float)((const half_t*)bias)[n];
+    } else {
+      yb = bf16_bits_to_f32(y) + bf16_bits_to_f32(((const uint16_t*)bias)[n]);
+    }
+    y = store_act<DTYPE>(yb);
+  }
+  return y;
+}
+
+// Kernel-side view of q4_weight plus the activation-side pointers.
+struct Problem {
+  const uint32_t* __restrict__ qweight;
+  const uint32_t* __restrict__ qzeros;
+  const half_t* __restrict__ scales;
+  const int32_t* __restrict__ g_idx;
+  const void* __restrict__ x;
+  const void* __restrict__ bias;
+  void* __restrict__ y;
+  int M, K, N, groupsize, num_groups;
+};
+
+}  // namespace q4
+
+// Host-side launchers implemented by the kernel translation units.
+namespace q4host {
+void set_error(const char* fmt, ...);
+int launch_dequant(const q4_weight* w, void* w_out, int dtype, hipStream_t stream);
+int launch_generic(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                   hipStream_t stream);
+struct GemvConfig {
+  int wcol;    // waves across columns in a workgroup (64 columns each)
+  int wk;      // waves across K in a workgroup
+  int splits;  // workgroups across K (cross-workgroup reduction through the workspace)
+};
+bool gemv_supported(const q4_weight* w, int M, int dtype);
+GemvConfig gemv_pick_config(const q4_weight* w, int M);
+int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                void* workspace, size_t workspace_bytes, const GemvConfig* cfg, hipStream_t stream);
+bool gemm_supported(const q4_weight* w, int M, int dtype);
+int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                hipStream_t stream);
+}  // namespace q4host

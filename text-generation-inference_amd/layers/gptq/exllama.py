@@ -1,0 +1,78 @@
+"""ExllamaQuantLinear: the handle-free equivalent of the reference's exllama modules.
+
+Mirrors the constructor `(weight: GPTQWeight, bias)` and forward of
+server/text_generation_server/layers/gptq/exllamav2.py:178-231 and
+gptq/exllama.py:66-134.  The reference needs a Warmup hook (`set_device`,
+`create_exllama_buffers`, server.py:103-116) to allocate a dequant scratch buffer and to
+repack qweight in place; nothing of that exists here (the kernels read the checkpoint
+layout and never materialise W), so both hooks are kept as no-ops for call
+compatibility.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from ... import ops
+from ..._lib import LAYOUT_GPTQ
+from .quant_linear import is_trivial_g_idx
+
+DEVICE = None
+
+
+def set_device(device):
+    """Kept for call compatibility (exllamav2.py:154-156); the library holds no device state."""
+    global DEVICE
+    DEVICE = device
+
+
+def create_exllama_buffers(max_total_tokens: int):
+    """No scratch buffers to create: W is never materialised (exllamav2.py:159-175)."""
+    return None
+
+
+class ExllamaQuantLinear(nn.Module):
+    QUANT_TYPE = "q4-mi355x"
+
+    def __init__(self, weight, bias):
+        super().__init__()
+        if weight.bits != 4:
+            raise ValueError(
+                f"The int4 kernels support only bits=4, requested bits={weight.bits}. "
+                "Something is wrong in the model initialization."
+            )
+        self.q_tensors = weight
+        self.infeatures = weight.qweight.shape[0] // weight.bits * 32
+        self.outfeatures = weight.qweight.shape[1]
+        self.device = weight.device
+        self.bias = bias if bias is not None else None
+        g_idx = weight.g_idx
+        # act-order only if g_idx is a real permutation (exllamav2.py:106, exllama.py:81-92)
+        if g_idx is not None and (
+            bool((g_idx == 0).all()) or is_trivial_g_idx(g_idx, weight.groupsize)
+        ):
+            g_idx = None
+        self.act_order = g_idx is not None
+        groupsize = weight.groupsize
+        if g_idx is None and weight.scales.shape[0] == 1:
+            groupsize = self.infeatures
+        self._packed = ops.make_packed(
+            weight.qweight, weight.qzeros, weight.scales, g_idx, groupsize, LAYOUT_GPTQ
+        )
+
+    def post_init(self, temp_dq=None):
+        """The reference builds its device matrix here (exllamav2.py:215-224); nothing to do."""
+        return None
+
+    @torch.no_grad()
+    def forward(self, x, force_cuda=False):
+        out_shape = x.shape[:-1] + (self.outfeatures,)
+        x2 = x.reshape(-1, x.shape[-1])
+        if x2.dtype not in (torch.float16, torch.bfloat16):
+            raise TypeError(f"x must be float16 (or bfloat16), got {x2.dtype}")  # ext.cpp:110
+        out = ops.linear(self._packed, x2, self.bias)
+        return out.reshape(out_shape)
+
+    def dequantize(self, dtype: torch.dtype = torch.float16) -> torch.Tensor:
+        return ops.dequantize(self._packed, dtype)

@@ -1,0 +1,94 @@
+"""QuantLinear: the GPTQ linear module with the reference's constructor and forward.
+
+Mirrors server/text_generation_server/layers/gptq/triton.py:252-292,351-363: same
+positional constructor, same attributes (qweight, qzeros, scales, g_idx, bias, bits,
+maxq, groupsize, infeatures, outfeatures), same `new()` factory, same forward contract
+(any leading dims, reshape to [-1, K], bias added after, reshape back).  The matmul is
+the HIP library's q4_linear instead of the Triton kernel.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from ... import ops
+from ..._lib import LAYOUT_GPTQ
+
+
+def is_trivial_g_idx(g_idx: torch.Tensor, groupsize: int) -> bool:
+    """True when g_idx is the sequential map k -> k // groupsize (no activation order).
+
+    The same test the reference's exllama wrappers run at construction
+    (gptq/exllama.py:81-92: all zeros, or equal to [i // groupsize]); it runs once per
+    layer at load time, so the device->host sync it implies is outside the forward path.
+    """
+    K = g_idx.numel()
+    if K == 0:
+        return True
+    gs = K if groupsize == -1 else int(groupsize)
+    expect = torch.arange(K, device=g_idx.device, dtype=torch.int64) // gs
+    return bool(torch.equal(g_idx.to(torch.int64), expect))
+
+
+class QuantLinear(nn.Module):
+    def __init__(self, qweight, qzeros, scales, g_idx, bias, bits, groupsize):
+        super().__init__()
+        self.register_buffer("qweight", qweight)
+        self.register_buffer("qzeros", qzeros)
+        self.register_buffer("scales", scales)
+        self.register_buffer("g_idx", g_idx)
+        if bias is not None:
+            self.register_buffer("bias", bias)
+        else:
+            self.bias = None
+        if bits not in [4]:
+            raise NotImplementedError("Only 4 bits are supported.")
+        self.bits = int(bits)
+        self.maxq = 2**self.bits - 1
+        self.groupsize = int(groupsize)
+
+        self.outfeatures = qweight.shape[1]
+        self.infeatures = qweight.shape[0] * 32 // self.bits
+        self._packed: Optional[ops.PackedWeight] = None
+
+    @classmethod
+    def new(cls, bits, groupsize, infeatures, outfeatures, bias):
+        """Zero-filled layer of the given geometry (triton.py:272-292)."""
+        if bits not in [4]:
+            raise NotImplementedError("Only 4 bits are supported.")
+        gs = infeatures if groupsize == -1 else groupsize
+        groups = math.ceil(infeatures / gs)
+        qweight = torch.zeros((infeatures // 32 * bits, outfeatures), dtype=torch.int32)
+        qzeros = torch.zeros((groups, outfeatures // 32 * bits), dtype=torch.int32)
+        scales = torch.zeros((groups, outfeatures), dtype=torch.float16)
+        g_idx = (torch.arange(infeatures, dtype=torch.int64) // gs).to(torch.int32)
+        bias_t = torch.zeros((outfeatures,), dtype=torch.float16) if bias else None
+        return cls(qweight, qzeros, scales, g_idx, bias_t, bits, groupsize)
+
+    def packed(self) -> ops.PackedWeight:
+        """Validated kernel view of the buffers, rebuilt if they moved (e.g. `.to(device)`)."""
+        pk = self._packed
+        if pk is None or pk.qweight.data_ptr() != self.qweight.data_ptr():
+            g_idx = self.g_idx
+            if g_idx is not None and is_trivial_g_idx(g_idx, self.groupsize):
+                g_idx = None  # sequential groups: the kernels index by k // groupsize
+            pk = ops.make_packed(self.qweight, self.qzeros, self.scales, g_idx, self.groupsize, LAYOUT_GPTQ)
+            self._packed = pk
+        return pk
+
+    @torch.no_grad()
+    def forward(self, x):
+        out_shape = x.shape[:-1] + (self.outfeatures,)
+        x2 = x.reshape(-1, x.shape[-1])
+        if x2.dtype not in (torch.float16, torch.bfloat16):
+            x2 = x2.to(torch.float16)  # the reference computes this path in fp16 (triton.py:246)
+        out = ops.linear(self.packed(), x2, self.bias)
+        return out.reshape(out_shape)
+
+    def dequantize(self, dtype: torch.dtype = torch.float16) -> torch.Tensor:
+        """Dense [K, N] weight, bit-exact with the reference's dequantize step."""
+        return ops.dequantize(self.packed(), dtype)

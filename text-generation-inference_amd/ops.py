@@ -1,0 +1,204 @@
+"""Tensor-level wrappers over the C ABI: pointers, shapes, stream and workspace.
+
+PyTorch is used for device memory and streams only; all arithmetic happens in the HIP
+kernels of libq4linear.so.  CPU tensors are rejected: there is no host fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import (
+    DTYPE_BF16,
+    DTYPE_F16,
+    LAYOUT_AWQ,
+    LAYOUT_GPTQ,
+    PATH_AUTO,
+    Q4Weight,
+)
+
+_DTYPES = {torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}
+
+# (device index, stream handle) -> zero-initialised workspace tensor (uint8)
+_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def _require_cuda(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"{name} is on {t.device}: the int4 linear kernels run on the GPU only "
+            "(no CPU fallback exists in this package)"
+        )
+
+
+@dataclass
+class PackedWeight:
+    """Validated view of one quantized weight, ready to be passed through the C ABI."""
+
+    qweight: torch.Tensor
+    qzeros: torch.Tensor
+    scales: torch.Tensor
+    g_idx: Optional[torch.Tensor]
+    K: int
+    N: int
+    groupsize: int
+    num_groups: int
+    layout: int
+
+    def struct(self) -> Q4Weight:
+        return Q4Weight(
+            self.qweight.data_ptr(),
+            self.qzeros.data_ptr(),
+            self.scales.data_ptr(),
+            self.g_idx.data_ptr() if self.g_idx is not None else None,
+            self.K,
+            self.N,
+            self.groupsize,
+            self.num_groups,
+            self.layout,
+        )
+
+
+def make_packed(qweight, qzeros, scales, g_idx, groupsize: int, layout: int) -> PackedWeight:
+    """Check dtypes/shapes the way the reference's extension does before building a matrix.
+
+    Mirrors the TORCH_CHECKs of server/exllamav2_kernels/exllamav2_kernels/ext.cpp:60-70
+    (qweight.size(1) == qzeros.size(1) * 8 == scales.size(1), int32 packed tensors).
+    """
+    for name, t in (("qweight", qweight), ("qzeros", qzeros)):
+        if t.dtype != torch.int32:
+            raise TypeError(f"{name} must be int32, got {t.dtype}")
+    if scales.dtype != torch.float16:
+        raise TypeError(f"scales must be float16, got {scales.dtype}")
+    if qweight.dim() != 2 or qzeros.dim() != 2 or scales.dim() != 2:
+        raise ValueError("qweight, qzeros and scales must be 2-D")
+    if layout == LAYOUT_GPTQ:
+        K, N = qweight.shape[0] * 8, qweight.shape[1]
+    else:
+        K, N = qweight.shape[0], qweight.shape[1] * 8
+    G = scales.shape[0]
+    if scales.shape[1] != N or tuple(qzeros.shape) != (G, N // 8) or N % 8 != 0:
+        raise ValueError(
+            f"inconsistent shapes: qweight {tuple(qweight.shape)} qzeros {tuple(qzeros.shape)} "
+            f"scales {tuple(scales.shape)}"
+        )
+    groupsize = int(groupsize)
+    if groupsize == -1:
+        groupsize = K
+    if groupsize < 1:
+        raise ValueError(f"bad groupsize {groupsize}")
+    if g_idx is not None:
+        if layout == LAYOUT_AWQ:
+            raise ValueError("g_idx is not defined for the AWQ layout")
+        if g_idx.dtype != torch.int32:
+            g_idx = g_idx.to(torch.int32)
+        if g_idx.numel() != K:
+            raise ValueError(f"g_idx has {g_idx.numel()} entries, expected {K}")
+        g_idx = g_idx.contiguous()
+    elif G * groupsize < K:
+        raise ValueError(f"{G} groups of {groupsize} rows do not cover K={K}")
+    dev = qweight.device
+    for name, t in (("qzeros", qzeros), ("scales", scales), ("g_idx", g_idx)):
+        if t is not None and t.device != dev:
+            raise ValueError(f"{name} is on {t.device}, qweight on {dev}")
+    return PackedWeight(
+        qweight.contiguous(), qzeros.contiguous(), scales.contiguous(), g_idx, K, N, groupsize, G, layout
+    )
+
+
+def _stream_handle(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def reserve_workspace(device: torch.device, nbytes: int, stream: Optional[int] = None) -> torch.Tensor:
+    """Return this (device, stream)'s workspace, growing it to at least `nbytes`.
+
+    The first bytes hold the split-K ticket counters: they must start at zero and the
+    kernels leave them at zero, so a grown buffer is freshly zeroed and the old one dropped.
+    """
+    if stream is None:
+        stream = _stream_handle(device)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(int(nbytes), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def workspace_bytes(M: int, K: int, N: int) -> int:
+    return int(_lib.load().q4_workspace_bytes(int(M), int(K), int(N)))
+
+
+def dequantize(w: PackedWeight, dtype: torch.dtype = torch.float16) -> torch.Tensor:
+    """Dense W [K, N] in `dtype`, produced by the HIP dequant kernel."""
+    _require_cuda(w.qweight, "qweight")
+    if dtype not in _DTYPES:
+        raise TypeError(f"dequantize supports float16/bfloat16, got {dtype}")
+    out = torch.empty((w.K, w.N), dtype=dtype, device=w.qweight.device)
+    with torch.cuda.device(w.qweight.device):
+        st = w.struct()
+        _lib.check(
+            _lib.load().q4_dequant(ctypes.byref(st), out.data_ptr(), _DTYPES[dtype], _stream_handle(out.device))
+        )
+    return out
+
+
+def linear(
+    w: PackedWeight,
+    x: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    path: int = PATH_AUTO,
+    gemv_config: Optional[tuple[int, int, int]] = None,
+) -> torch.Tensor:
+    """y[M, N] = x[M, K] @ dequant(W) (+ bias) on the current stream of x's device."""
+    _require_cuda(x, "x")
+    _require_cuda(w.qweight, "qweight")
+    if x.device != w.qweight.device:
+        raise RuntimeError(f"x is on {x.device}, weights on {w.qweight.device}")
+    if x.dtype not in _DTYPES:
+        raise TypeError(f"x must be float16 or bfloat16, got {x.dtype}")
+    if x.dim() != 2 or x.shape[1] != w.K:
+        raise ValueError(f"x must be [M, {w.K}], got {tuple(x.shape)}")
+    x = x.contiguous()
+    M = x.shape[0]
+    y = torch.empty((M, w.N), dtype=x.dtype, device=x.device)
+    if M == 0 or w.N == 0:
+        return y
+    fused_bias = bias is not None and bias.dtype == x.dtype and bias.is_cuda and bias.numel() == w.N
+    bias_ptr = bias.contiguous().data_ptr() if fused_bias else None
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        stream = _stream_handle(x.device)
+        ws = reserve_workspace(x.device, workspace_bytes(min(M, 16), w.K, w.N), stream)
+        st = w.struct()
+        if gemv_config is not None:
+            wcol, wk, splits = gemv_config
+            need = _lib.WORKSPACE_COUNTER_BYTES + splits * M * w.N * 4
+            if ws.numel() < need:
+                ws = reserve_workspace(x.device, need, stream)
+            rc = lib.q4_gemv_tuned(
+                ctypes.byref(st), x.data_ptr(), bias_ptr, y.data_ptr(), M, _DTYPES[x.dtype],
+                ws.data_ptr(), ws.numel(), wcol, wk, splits, stream,
+            )
+        else:
+            rc = lib.q4_linear_ex(
+                ctypes.byref(st), x.data_ptr(), bias_ptr, y.data_ptr(), M, _DTYPES[x.dtype],
+                ws.data_ptr(), ws.numel(), path, stream,
+            )
+        _lib.check(rc)
+    if bias is not None and not fused_bias:
+        y = y + bias
+    return y
+
+
+def select_path(w: PackedWeight, M: int, dtype: torch.dtype = torch.float16) -> str:
+    st = w.struct()
+    rc = _lib.load().q4_select_path(ctypes.byref(st), int(M), _DTYPES[dtype])
+    _lib.check(rc)
+    return _lib.PATH_NAMES[rc]
