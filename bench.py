@@ -1,0 +1,280 @@
+#!/usr/bin/env python3
+"""Benchmark of the int4 weight-only linear hot path on one MI355X.
+
+Workload (BASELINE.json configs[1]): GPTQ int4 decode GEMV, M=1, fp16, groupsize 128,
+symmetric zeros, over the four Llama-3-8B projections (qkv 4096x6144, o 4096x4096,
+gate_up 4096x28672, down 14336x4096).  One *step* = those four projections once, i.e.
+the quantized-linear work of one decoder layer for one token.  Weights rotate over R
+distinct copies (R * 113 MB >= 512 MB) so that every step streams from HBM and not from
+the 256 MB Infinity Cache.  Inputs are resident in HBM before the timed region.
+
+`value` = algorithmic bytes of all timed steps / wall time of the timed region (GB/s).
+`roofline` = the decode kernel against the 8 TB/s HBM peak, from per-launch durations
+measured with HIP events on the launch stream inside this script.
+`gemm` (when the prefill kernel is built) = M=2048 TFLOP/s on the same shapes.
+`cpu_baseline` = the NumPy oracle (dequantize then fp32 matmul) on the host cores.
+
+Prints exactly one JSON line on stdout.
+"""
+
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E peak
+MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16/bf16 MFMA peak
+
+SHAPES = [  # name, K, N
+    ("qkv_proj", 4096, 6144),
+    ("o_proj", 4096, 4096),
+    ("gate_up_proj", 4096, 28672),
+    ("down_proj", 14336, 4096),
+]
+GROUPSIZE = 128
+
+
+def gemv_bytes(M, K, N, gs=GROUPSIZE, g_idx=False):
+    """Algorithmic bytes of one call: packed weights + scales + zeros (+ g_idx) + x + y."""
+    G = K // gs
+    return K * N // 2 + G * N * 2 + G * N // 2 + (4 * K if g_idx else 0) + 2 * M * (K + N)
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--m", type=int, default=1, help="activation rows of the decode workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM leg")
+    ap.add_argument("--gemm-m", type=int, default=2048)
+    ap.add_argument("--copies", type=int, default=0, help="weight copies to rotate over (0 = auto)")
+    return ap.parse_args()
+
+
+def make_weights(pkg, torch, device, K, N, seed):
+    """Synthetic GPTQ tensors generated on the device (same distribution as the oracle's
+    make_gptq: uniform nibbles, stored zero 7, scales uniform [1e-3, 2e-2])."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    qweight = torch.randint(-(2**31), 2**31 - 1, (K // 8, N), dtype=torch.int64, device=device, generator=g).to(torch.int32)
+    G = K // GROUPSIZE
+    qzeros = torch.full((G, N // 8), 0x77777777, dtype=torch.int32, device=device)
+    scales = (torch.rand((G, N), device=device, generator=g) * (2e-2 - 1e-3) + 1e-3).to(torch.float16)
+    return pkg.ops.make_packed(qweight, qzeros, scales, None, GROUPSIZE, 0)
+
+
+def time_kernel_launches(torch, fn_list, reps):
+    """Average duration of single launches, each bracketed by its own pair of HIP events
+    recorded on the launch stream (the current torch stream)."""
+    durs = []
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+    for i in range(reps):
+        fn = fn_list[i % len(fn_list)]
+        starts[i].record()
+        fn()
+        stops[i].record()
+    torch.cuda.synchronize()
+    for i in range(reps):
+        durs.append(starts[i].elapsed_time(stops[i]) * 1e-3)
+    return durs
+
+
+def cpu_baseline(M):
+    """Oracle (dequantize -> fp32 matmul) on the host, one call per projection."""
+    import numpy as np
+    from oracle import q4_oracle as o
+
+    total_bytes = 0
+    total_t = 0.0
+    detail = {}
+    for name, K, N in SHAPES:
+        qw, qz, sc, _ = o.make_gptq(K, N, GROUPSIZE, seed=1)
+        x = o.make_x(M, K, seed=1)
+        t0 = time.perf_counter()
+        w = o.dequant_gptq(qw, qz, sc, None, GROUPSIZE, "f16")
+        t1 = time.perf_counter()
+        o.linear_forward(x, w, None, "f16")
+        t2 = time.perf_counter()
+        detail[name] = {"dequant_ms": round((t1 - t0) * 1e3, 1), "matmul_ms": round((t2 - t1) * 1e3, 1)}
+        total_bytes += gemv_bytes(M, K, N)
+        total_t += t2 - t0
+        del w
+    return {
+        "value": round(total_bytes / total_t / 1e9, 4),
+        "unit": "GB/s",
+        "cores": os.cpu_count(),
+        "kind": "port",
+        "sample": f"one step (4 Llama-3-8B projections, M={M}) of the NumPy oracle: dequantize then fp32 matmul; "
+                  f"{total_t:.1f} s total",
+        "ms_per_step": round(total_t * 1e3, 1),
+        "detail": detail,
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
+              "(no collectives or sharding are part of the hot path)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    pkg = importlib.import_module("text-generation-inference_amd")
+    lib = pkg._lib.load()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    M = args.m
+    step_weight_bytes = sum(gemv_bytes(0, K, N) for _, K, N in SHAPES)
+    step_bytes = sum(gemv_bytes(M, K, N) for _, K, N in SHAPES)
+    copies = args.copies or max(2, -(-512 * 1024 * 1024 // step_weight_bytes) + 1)
+
+    weights = [[make_weights(pkg, torch, dev, K, N, seed=17 * c + i) for i, (_, K, N) in enumerate(SHAPES)]
+               for c in range(copies)]
+    xs = [torch.randn((M, K), device=dev, dtype=torch.float16) for _, K, N in SHAPES]
+    ys = [torch.empty((M, N), device=dev, dtype=torch.float16) for _, K, N in SHAPES]
+    for _, K, N in SHAPES:
+        pkg.ops.reserve_workspace(dev, pkg.ops.workspace_bytes(M, K, N))
+
+    def step(c):
+        for i in range(len(SHAPES)):
+            pkg.ops.linear(weights[c % copies][i], xs[i], None, out=ys[i])
+
+    # ---- whole-job throughput: W warmup steps, then exactly K steps in one HIP graph
+    for c in range(args.warmup):
+        step(c)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for _, K, N in SHAPES:
+            pkg.ops.reserve_workspace(dev, pkg.ops.workspace_bytes(M, K, N))
+        step(0)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for c in range(args.steps):
+                step(c)
+    torch.cuda.synchronize()
+    graph.replay()  # untimed replay: instantiation and first-launch costs
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    total_s = e0.elapsed_time(e1) * 1e-3
+    ms_per_step = total_s / args.steps * 1e3
+    value = step_bytes * args.steps / total_s / 1e9
+
+    # ---- per-kernel durations (decode kernel), one event pair per launch, weights rotating
+    per_shape = {}
+    all_durs = []
+    all_bytes = 0
+    reps = max(200, copies * 8)
+    for i, (name, K, N) in enumerate(SHAPES):
+        fns = [(lambda c=c, i=i: pkg.ops.linear(weights[c][i], xs[i], None, out=ys[i])) for c in range(copies)]
+        time_kernel_launches(torch, fns, copies)  # warm
+        d = time_kernel_launches(torch, fns, reps)
+        d.sort()
+        med = d[len(d) // 2]
+        avg = sum(d) / len(d)
+        b = gemv_bytes(M, K, N)
+        hot = time_kernel_launches(torch, fns[:1], reps)
+        hot_avg = sum(hot) / len(hot)
+        per_shape[name] = {
+            "K": K, "N": N, "bytes": b,
+            "us_avg": round(avg * 1e6, 2), "us_median": round(med * 1e6, 2),
+            "GBps": round(b / avg / 1e9, 1), "frac_of_hbm_peak": round(b / avg / 1e9 / HBM_PEAK_GBS, 4),
+            "cache_hot_us": round(hot_avg * 1e6, 2), "cache_hot_GBps": round(b / hot_avg / 1e9, 1),
+            "path": pkg.ops.select_path(weights[0][i], M),
+        }
+        all_durs.append(avg)
+        all_bytes += b
+    achieved = all_bytes / sum(all_durs) / 1e9
+    roofline = {
+        "bound": "hbm",
+        "kernel": "q4::gemv_gptq_kernel",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "bytes_per_launch": all_bytes // len(SHAPES),
+        "us_per_launch": round(sum(all_durs) / len(SHAPES) * 1e6, 2),
+    }
+
+    out = {
+        "metric": "int4 GEMV HBM GB/s (M=1) + GEMM TFLOP/s (M=2048), Llama-3-8B shapes, % roofline",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"GPTQ int4 decode GEMV M={M}, Llama-3-8B projections (qkv/o/gate_up/down), fp16, "
+                        f"groupsize 128, sym; one step = the four projections once",
+            "weight_copies_rotated": copies,
+            "bytes_per_step": step_bytes,
+            "timing": "one HIP graph of all timed steps, bracketed by HIP events + synchronize",
+        },
+        "roofline": roofline,
+        "per_shape": per_shape,
+    }
+
+    # ---- prefill GEMM leg (M=2048) when the kernel is available
+    if not args.no_gemm:
+        gm = {}
+        Mg = args.gemm_m
+        tot_f = 0.0
+        tot_t = 0.0
+        for i, (name, K, N) in enumerate(SHAPES):
+            if pkg.ops.select_path(weights[0][i], Mg) != "gemm":
+                continue
+            xg = torch.randn((Mg, K), device=dev, dtype=torch.float16)
+            yg = torch.empty((Mg, N), device=dev, dtype=torch.float16)
+            fns = [(lambda c=c, i=i: pkg.ops.linear(weights[c][i], xg, None, out=yg)) for c in range(copies)]
+            time_kernel_launches(torch, fns, 3)
+            d = time_kernel_launches(torch, fns, 20)
+            avg = sum(d) / len(d)
+            fl = 2.0 * Mg * N * K
+            gm[name] = {"us_avg": round(avg * 1e6, 1), "TFLOPs": round(fl / avg / 1e12, 1),
+                        "frac_of_mfma_peak": round(fl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)}
+            tot_f += fl
+            tot_t += avg
+            del xg, yg
+        if gm:
+            out["gemm"] = {
+                "M": Mg, "per_shape": gm,
+                "roofline": {"bound": "mfma", "kernel": "q4::gemm_kernel", "achieved": round(tot_f / tot_t / 1e12, 1),
+                             "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                             "frac": round(tot_f / tot_t / 1e12 / MFMA_PEAK_TFLOPS, 4), "traffic": None},
+            }
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(M)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

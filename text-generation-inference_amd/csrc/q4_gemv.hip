@@ -29,6 +29,7 @@ namespace q4 {
 
 constexpr int kChunkSteps = 4;              // 32-row MFMA steps per software-pipelined chunk
 constexpr int kChunkRows = 32 * kChunkSteps;  // 128 K rows
+constexpr int kPrefetch = 4;                  // chunks of weight loads in flight per wave
 
 struct GemvParams {
   Problem p;
@@ -38,19 +39,30 @@ struct GemvParams {
   int slab_stride;  // bytes between activation rows in LDS
 };
 
-__device__ __forceinline__ uint32_t nib_lo(uint32_t w) { return (w & 0x000F000Fu) | 0x64006400u; }
-__device__ __forceinline__ uint32_t nib_hi(uint32_t w) { return (w & 0x00F000F0u) | 0x64006400u; }
+// Constants of the nibble splice, hidden from constant folding (empty asm, no instruction
+// is emitted): as literals the compiler must split (w & mask) | magic into v_and + v_or
+// because a three-operand VALU instruction cannot carry a literal; as register operands it
+// selects the fused v_and_or_b32.  The asm must stay empty: an instruction inside inline
+// asm is invisible to the MFMA hazard recognizer.
+struct SpliceConsts {
+  uint32_t mask_lo, mask_hi, magic;
+};
+__device__ __forceinline__ SpliceConsts splice_consts() {
+  SpliceConsts k{0x000F000Fu, 0x00F000F0u, 0x64006400u};
+  asm volatile("" : "+s"(k.mask_lo), "+s"(k.mask_hi), "+v"(k.magic));
+  return k;
+}
 
 // Eight exact (q - z) values of one packed word, as four half2 in K order [0,4,1,5,2,6,3,7].
 // czlo = half2(-(1024 + z)), czhi = half2(-(64 + z)).
 __device__ __forceinline__ void unpack_word_f16(uint32_t w, half2_t czlo, half2_t czhi,
-                                                half2_t out[4]) {
+                                                const SpliceConsts& k, half2_t out[4]) {
   const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
   const uint32_t w8 = w >> 8;
-  out[0] = as_half2(nib_lo(w)) + czlo;
-  out[1] = as_half2(nib_hi(w)) * sixteenth + czhi;
-  out[2] = as_half2(nib_lo(w8)) + czlo;
-  out[3] = as_half2(nib_hi(w8)) * sixteenth + czhi;
+  out[0] = as_half2((w & k.mask_lo) | k.magic) + czlo;
+  out[1] = as_half2((w & k.mask_hi) | k.magic) * sixteenth + czhi;
+  out[2] = as_half2((w8 & k.mask_lo) | k.magic) + czlo;
+  out[3] = as_half2((w8 & k.mask_hi) | k.magic) * sixteenth + czhi;
 }
 
 __device__ __forceinline__ uint32_t pack_bf16_pair(half2_t h) {
@@ -88,7 +100,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   const Problem& p = gp.p;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps tile/K-range math scalar
   const int wc = wave % gp.wcol;
   const int wkk = wave / gp.wcol;
   const int j = lane & 15;
@@ -109,41 +121,73 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   const int N = p.N;
   constexpr int GPC = kChunkSteps / GSTEPS;  // groups per chunk
 
-  // ---- issue the first chunk of weight loads before anything else
-  const uint4_t* qw = (const uint4_t*)(p.qweight + (size_t)(kw0 / 8 + kq) * N + nl);
-  const size_t step_stride = (size_t)N;  // uint4 units between consecutive 32-row steps
-  uint4_t wq[kChunkSteps], wq_next[kChunkSteps];
+  // ---- activation slab [M][KR] -> LDS, each 8-block in K order 0,4,1,5,2,6,3,7.  The
+  // global loads are issued before the weight loads: memory returns in issue order, so the
+  // slab (L2 hits) must not queue behind the HBM stream it is needed to consume.
+  constexpr int kSlabLoads = 2;  // 16-byte activation loads per thread kept in flight
+  const int kb_per_row = KR >> 3;
+  const int slab_items = p.M * kb_per_row;
+  const uint16_t* xs = (const uint16_t*)p.x;
+  uint4_t xv[kSlabLoads];
 #pragma unroll
-  for (int s = 0; s < kChunkSteps; ++s) wq[s] = __builtin_nontemporal_load(qw + s * step_stride);
-
-  const int zshift = (nl & 4) * 4;
-  auto load_group = [&](int k, uint2_t& sc, uint32_t& zw) {
-    int g = k / p.groupsize;
-    g = min(g, p.num_groups - 1);
-    sc = *(const uint2_t*)(p.scales + (size_t)g * N + nl);
-    zw = p.qzeros[(size_t)g * (N >> 3) + (nl >> 3)];
-  };
-  uint2_t sc[GPC], sc_next[GPC];
-  uint32_t zw[GPC], zw_next[GPC];
-#pragma unroll
-  for (int g = 0; g < GPC; ++g) load_group(kw0 + g * GSTEPS * 32, sc[g], zw[g]);
-
-  // ---- stage the activation slab [M][KR] into LDS, each 8-block in order 0,4,1,5,2,6,3,7
-  {
-    const int kb_per_row = KR >> 3;
-    const int total = p.M * kb_per_row;
-    const uint16_t* xs = (const uint16_t*)p.x;
-    for (int idx = tid; idx < total; idx += nthreads) {
+  for (int u = 0; u < kSlabLoads; ++u) {
+    const int idx = tid + u * nthreads;
+    if (idx < slab_items) {
       const int m = idx / kb_per_row;
       const int kb = idx - m * kb_per_row;
-      const uint4_t v = *(const uint4_t*)(xs + (size_t)m * p.K + kwg0 + kb * 8);
-      uint4_t o;
-      o.x = (v.x & 0xFFFFu) | (v.z << 16);
-      o.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
-      o.z = (v.y & 0xFFFFu) | (v.w << 16);
-      o.w = (v.y >> 16) | (v.w & 0xFFFF0000u);
-      *(uint4_t*)(smem + (size_t)m * gp.slab_stride + kb * 16) = o;
+      xv[u] = *(const uint4_t*)(xs + (size_t)m * p.K + kwg0 + kb * 8);
     }
+  }
+  auto store_slab = [&](int idx, uint4_t v) {
+    const int m = idx / kb_per_row;
+    const int kb = idx - m * kb_per_row;
+    uint4_t o;
+    o.x = (v.x & 0xFFFFu) | (v.z << 16);
+    o.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
+    o.z = (v.y & 0xFFFFu) | (v.w << 16);
+    o.w = (v.y >> 16) | (v.w & 0xFFFF0000u);
+    *(uint4_t*)(smem + (size_t)m * gp.slab_stride + kb * 16) = o;
+  };
+
+  // ---- issue the first kPrefetch chunks of weight loads before anything else
+  // Addresses are a wave-uniform 64-bit base (scalar registers, advanced per step) plus a
+  // per-lane 32-bit byte offset, so the loads use the scalar-base addressing mode and the
+  // VALU does no address arithmetic in the loop.
+  const char* wbase = (const char*)(p.qweight + (size_t)(kw0 / 8) * N);
+  const uint32_t w_lane = ((uint32_t)kq * (uint32_t)N + (uint32_t)nl) * 4u;
+  const size_t step_bytes = (size_t)N * 16;  // four packed rows
+  const uint32_t s_lane = (uint32_t)nl * 2u;
+  const uint32_t z_lane = (uint32_t)(nl >> 3) * 4u;
+  const int zshift = (nl & 4) * 4;
+  uint4_t wq[kPrefetch][kChunkSteps];
+  uint2_t sc[kPrefetch][GPC];
+  uint32_t zw[kPrefetch][GPC];
+  auto load_chunk = [&](int c, uint4_t (&w)[kChunkSteps], uint2_t (&s)[GPC], uint32_t (&z)[GPC]) {
+#pragma unroll
+    for (int st = 0; st < kChunkSteps; ++st)
+      w[st] = __builtin_nontemporal_load(
+          (const uint4_t*)(wbase + (size_t)(c * kChunkSteps + st) * step_bytes + w_lane));
+#pragma unroll
+    for (int g = 0; g < GPC; ++g) {
+      int gi = (kw0 + c * kChunkRows + g * GSTEPS * 32) / p.groupsize;
+      gi = min(gi, p.num_groups - 1);
+      s[g] = *(const uint2_t*)((const char*)p.scales + (size_t)gi * N * 2 + s_lane);
+      z[g] = *(const uint32_t*)((const char*)p.qzeros + (size_t)gi * (N >> 3) * 4 + z_lane);
+    }
+  };
+#pragma unroll
+  for (int b = 0; b < kPrefetch; ++b)
+    if (b < nchunks) load_chunk(b, wq[b], sc[b], zw[b]);
+
+#pragma unroll
+  for (int u = 0; u < kSlabLoads; ++u) {
+    const int idx = tid + u * nthreads;
+    if (idx < slab_items) store_slab(idx, xv[u]);
+  }
+  for (int idx = tid + kSlabLoads * nthreads; idx < slab_items; idx += nthreads) {
+    const int m = idx / kb_per_row;
+    const int kb = idx - m * kb_per_row;
+    store_slab(idx, *(const uint4_t*)(xs + (size_t)m * p.K + kwg0 + kb * 8));
   }
   __syncthreads();
 
@@ -154,59 +198,48 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   float4_t tot[4] = {zero4, zero4, zero4, zero4};
   float4_t acc[4] = {zero4, zero4, zero4, zero4};
   half2_t czlo[4], czhi[4];
+  const SpliceConsts splice = splice_consts();
 
-  for (int c = 0; c < nchunks; ++c) {
+  auto process_chunk = [&](int c, const uint4_t (&w)[kChunkSteps], const uint2_t (&s)[GPC],
+                           const uint32_t (&z)[GPC]) {
     const int kc = kw0 + c * kChunkRows;
-    if (c + 1 < nchunks) {
-#pragma unroll
-      for (int s = 0; s < kChunkSteps; ++s)
-        wq_next[s] = __builtin_nontemporal_load(qw + (size_t)((c + 1) * kChunkSteps + s) * step_stride);
-#pragma unroll
-      for (int g = 0; g < GPC; ++g) load_group(kc + kChunkRows + g * GSTEPS * 32, sc_next[g], zw_next[g]);
-    }
-    bool group_start, group_end;
-    if constexpr (STATIC128) {
-      group_start = true;
-      group_end = true;
-    } else if constexpr (GSTEPS == kChunkSteps) {
+    bool group_start = true, group_end = true;
+    if constexpr (!STATIC128 && GSTEPS == kChunkSteps) {
       group_start = (c == 0) || (kc % p.groupsize == 0);
       group_end = (c == nchunks - 1) || ((kc + kChunkRows) % p.groupsize == 0);
-    } else {
-      group_start = true;
-      group_end = true;
     }
 #pragma unroll
-    for (int s = 0; s < kChunkSteps; ++s) {
-      const int gi = s / GSTEPS;
-      const bool first = (s % GSTEPS) == 0;
-      const bool last = (s % GSTEPS) == GSTEPS - 1;
-      if (first && (GSTEPS != kChunkSteps || group_start || STATIC128)) {
+    for (int st = 0; st < kChunkSteps; ++st) {
+      const int gi = st / GSTEPS;
+      const bool first = (st % GSTEPS) == 0;
+      const bool last = (st % GSTEPS) == GSTEPS - 1;
+      constexpr bool kStaticGroups = STATIC128 || GSTEPS != kChunkSteps;
+      if (first && (kStaticGroups || group_start)) {
         // zero-point constants of the group: z = (stored + 1) & 15 per column
-        const uint32_t z4 = gptq_zero_plus_one(zw[gi]) >> zshift;
+        const uint32_t z4 = gptq_zero_plus_one(z[gi]) >> zshift;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          const uint32_t z = (z4 >> (4 * t)) & 0xFu;
-          czlo[t] = as_half2(0xE400E400u | z | (z << 16));        // -(1024 + z)
-          czhi[t] = as_half2(0xD400D400u | (z << 4) | (z << 20));  // -(64 + z)
+          const uint32_t zz = (z4 >> (4 * t)) & 0xFu;
+          czlo[t] = as_half2(0xE400E400u | zz | (zz << 16));        // -(1024 + z)
+          czhi[t] = as_half2(0xD400D400u | (zz << 4) | (zz << 20));  // -(64 + z)
         }
       }
       uint4_t a = {0u, 0u, 0u, 0u};
-      if (row_live) a = *(const uint4_t*)(a_base + (size_t)(c * kChunkRows + s * 32) * 2);
-      const uint32_t words[4] = {wq[s].x, wq[s].y, wq[s].z, wq[s].w};
-      const bool fresh = first && (STATIC128 || GSTEPS != kChunkSteps);
+      if (row_live) a = *(const uint4_t*)(a_base + (size_t)(c * kChunkRows + st * 32) * 2);
+      const uint32_t words[4] = {w[st].x, w[st].y, w[st].z, w[st].w};
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         half2_t b[4];
-        unpack_word_f16(words[t], czlo[t], czhi[t], b);
-        if (fresh) {
+        unpack_word_f16(words[t], czlo[t], czhi[t], splice, b);
+        if (first && kStaticGroups) {
           acc[t] = mfma16<DTYPE>(a, b, zero4);
         } else {
           if (first && group_start) acc[t] = zero4;
           acc[t] = mfma16<DTYPE>(a, b, acc[t]);
         }
       }
-      if (last && (GSTEPS != kChunkSteps || group_end || STATIC128)) {
-        const half2_t s01 = as_half2(sc[gi].x), s23 = as_half2(sc[gi].y);
+      if (last && (kStaticGroups || group_end)) {
+        const half2_t s01 = as_half2(s[gi].x), s23 = as_half2(s[gi].y);
         const float sf[4] = {(float)s01.x, (float)s01.y, (float)s23.x, (float)s23.y};
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -215,12 +248,17 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
         }
       }
     }
+  };
+
+  // ring of kPrefetch chunk buffers: consume slot b, then refill it with chunk c + kPrefetch
+  for (int c0 = 0; c0 < nchunks; c0 += kPrefetch) {
 #pragma unroll
-    for (int s = 0; s < kChunkSteps; ++s) wq[s] = wq_next[s];
-#pragma unroll
-    for (int g = 0; g < GPC; ++g) {
-      sc[g] = sc_next[g];
-      zw[g] = zw_next[g];
+    for (int b = 0; b < kPrefetch; ++b) {
+      const int c = c0 + b;
+      if (c < nchunks) {
+        process_chunk(c, wq[b], sc[b], zw[b]);
+        if (c + kPrefetch < nchunks) load_chunk(c + kPrefetch, wq[b], sc[b], zw[b]);
+      }
     }
   }
 
@@ -267,45 +305,53 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
     return;
   }
 
-  // ---- cross-workgroup split-K: write the partial, take a ticket, last one reduces
+  // ---- cross-workgroup split-K: write the partial, take a ticket, last one reduces.
+  // Partials and the ticket move with agent-scope relaxed atomics (coherent loads/stores
+  // that bypass the per-XCD L2 state) instead of release/acquire fences: a fence here
+  // would write back and invalidate the whole L2 once per workgroup, which costs more
+  // than the kernel itself.  Ordering comes from waiting for the stores to be
+  // acknowledged (vmcnt(0)) before the workgroup barrier that precedes the ticket.
   if (wkk == 0) {
 #pragma unroll
     for (int r = 0; r < RMAX; ++r) {
       const int m = 4 * kq + r;
       if (m < p.M) {
-        float4_t v = {tot[0][r], tot[1][r], tot[2][r], tot[3][r]};
-        *(float4_t*)(gp.partials + ((size_t)split * p.M + m) * N + nl) = v;
+        float* dst = gp.partials + ((size_t)split * p.M + m) * N + nl;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          __hip_atomic_store(dst + t, tot[t][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
   }
-  __threadfence();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   __shared__ uint32_t ticket_s;
   if (tid == 0) {
-    ticket_s = __hip_atomic_fetch_add(gp.tickets + tile, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    ticket_s = __hip_atomic_fetch_add(gp.tickets + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
   if (ticket_s != (uint32_t)(gp.splits - 1)) return;
-  __threadfence();
   {
-    const int quads = tile_cols >> 2;
-    const int items = p.M * quads;
+    const int items = p.M * tile_cols;
     const int nbase = tile * tile_cols;
     for (int idx = tid; idx < items; idx += nthreads) {
-      const int m = idx / quads;
-      const int n = nbase + (idx - m * quads) * 4;
-      float4_t sum = zero4;
-      for (int s = 0; s < gp.splits; ++s) {
-        const float4_t v = *(const float4_t*)(gp.partials + ((size_t)s * p.M + m) * N + n);
-        sum += v;
-      }
-      uint16_t o[4];
+      const int m = idx / tile_cols;
+      const int n = nbase + (idx - m * tile_cols);
+      const float* src = gp.partials + (size_t)m * N + n;
+      const size_t sstride = (size_t)p.M * N;
+      float sum = 0.f;
+      int sp = 0;
+      for (; sp + 8 <= gp.splits; sp += 8) {
+        float v[8];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) o[t] = finish_output<DTYPE>(sum[t], p.bias, n + t);
-      uint2_t packed;
-      packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
-      packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
-      *(uint2_t*)(y + (size_t)m * N + n) = packed;
+        for (int u = 0; u < 8; ++u)
+          v[u] = __hip_atomic_load(src + (size_t)(sp + u) * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += v[u];
+      }
+      for (; sp < gp.splits; ++sp)
+        sum += __hip_atomic_load(src + (size_t)sp * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      y[(size_t)m * N + n] = finish_output<DTYPE>(sum, p.bias, n);
     }
     if (tid == 0) __hip_atomic_store(gp.tickets + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
@@ -331,24 +377,26 @@ bool gemv_supported(const q4_weight* w, int M, int dtype) {
 }
 
 GemvConfig gemv_pick_config(const q4_weight* w, int M) {
-  // Enough workgroups to cover 256 CUs several times over, each wave streaming at least
-  // one 128-row chunk, with the activation slab (M rows x K/splits) inside 60 KB of LDS.
+  // Measured on MI355X (Llama-3-8B shapes, M=1): 64-column tiles with 4 waves along K per
+  // workgroup and about two workgroups per CU (512 in flight) is the best point; wider
+  // workgroups start too slowly and more splits lengthen the reduction tail.  The
+  // activation slab (M rows x K/splits) must fit 60 KB of LDS.
   GemvConfig c;
   const int chunks = w->K / 128;
-  c.wcol = (w->N % 256 == 0) ? 4 : (w->N % 128 == 0 ? 2 : 1);
-  c.wk = 1;
-  const int ntiles = w->N / (64 * c.wcol);
-  const int target_wgs = M <= 4 ? 1024 : 512;  // partial-sum traffic grows with M
-  int want = (target_wgs + ntiles - 1) / ntiles;
-  if (want > 32) want = 32;
+  c.wcol = 1;
+  c.wk = chunks % 4 == 0 ? 4 : (chunks % 2 == 0 ? 2 : 1);
+  const int per_wg = chunks / c.wk;  // chunks left to distribute over splits x per-wave work
+  const int ntiles = w->N / 64;
+  const int target_wgs = M <= 4 ? 512 : 384;  // partial-sum traffic grows with M
+  int want = (target_wgs + ntiles / 2) / ntiles;
   if (want < 1) want = 1;
   const long lds_budget = 60000 - 16L * M;
   int min_splits = (int)(((long)M * w->K * 2 + lds_budget - 1) / lds_budget);
   if (min_splits < 1) min_splits = 1;
-  int best = chunks;  // always legal: one chunk per workgroup
+  int best = per_wg;  // always legal: one chunk per wave
   long best_cost = -1;
-  for (int d = 1; d <= chunks; ++d) {
-    if (chunks % d != 0 || d < min_splits) continue;
+  for (int d = 1; d <= per_wg; ++d) {
+    if (per_wg % d != 0 || d < min_splits) continue;
     const long cost = d > want ? (long)d * 1000 / want : (long)want * 1000 / d;
     if (best_cost < 0 || cost < best_cost) {
       best_cost = cost;

@@ -155,8 +155,14 @@ def linear(
     bias: Optional[torch.Tensor] = None,
     path: int = PATH_AUTO,
     gemv_config: Optional[tuple[int, int, int]] = None,
+    out: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
-    """y[M, N] = x[M, K] @ dequant(W) (+ bias) on the current stream of x's device."""
+    """y[M, N] = x[M, K] @ dequant(W) (+ bias) on the current stream of x's device.
+
+    `out`, if given, must be a contiguous [M, N] tensor of x's dtype on x's device; it is
+    written in place (no allocation happens in the call, which keeps it graph-capturable
+    with a pre-reserved workspace).
+    """
     _require_cuda(x, "x")
     _require_cuda(w.qweight, "qweight")
     if x.device != w.qweight.device:
@@ -167,7 +173,12 @@ def linear(
         raise ValueError(f"x must be [M, {w.K}], got {tuple(x.shape)}")
     x = x.contiguous()
     M = x.shape[0]
-    y = torch.empty((M, w.N), dtype=x.dtype, device=x.device)
+    if out is not None:
+        if tuple(out.shape) != (M, w.N) or out.dtype != x.dtype or out.device != x.device or not out.is_contiguous():
+            raise ValueError(f"out must be a contiguous [{M}, {w.N}] {x.dtype} tensor on {x.device}")
+        y = out
+    else:
+        y = torch.empty((M, w.N), dtype=x.dtype, device=x.device)
     if M == 0 or w.N == 0:
         return y
     fused_bias = bias is not None and bias.dtype == x.dtype and bias.is_cuda and bias.numel() == w.N
@@ -193,7 +204,10 @@ def linear(
             )
         _lib.check(rc)
     if bias is not None and not fused_bias:
-        y = y + bias
+        if out is not None:
+            y.add_(bias)
+        else:
+            y = y + bias
     return y
 
 
