@@ -106,3 +106,55 @@ def test_gemv_deterministic_and_tickets_reset(pkg, oracle, gpu):
 def test_generic_path(pkg, oracle, gpu, layout, act, M):
     _run(pkg, oracle, gpu, 1000 if layout == "gptq" and not act else 1024, 264, 40 if (layout == "gptq" and not act) else 128, M,
          layout=layout, sym=False, act=act, bias=True, path=3, seed=M + 50)
+
+
+# --------------------------------------------------------------------------- prefill GEMM
+
+
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 6144), (14336, 4096)])
+@pytest.mark.parametrize("M", [512, 2048])
+def test_gemm_llama3_8b_fp16(pkg, oracle, gpu, K, N, M):
+    _run(pkg, oracle, gpu, K, N, 128, M, path=2, seed=K // 128 + N // 128 + M)
+
+
+def test_gemm_gate_up_bf16(pkg, oracle, gpu):
+    """cfg3: bf16 activations, widest projection."""
+    _run(pkg, oracle, gpu, 4096, 28672, 128, 512, dtype="bf16", path=2, seed=77)
+
+
+@pytest.mark.parametrize("M", [17, 64, 100, 129, 300])
+def test_gemm_ragged_m_asym_bias(pkg, oracle, gpu, M):
+    _run(pkg, oracle, gpu, 1024, 512, 128, M, sym=False, bias=True, path=2, seed=M)
+
+
+@pytest.mark.parametrize("gs", [32, 64, 128, 256, -1])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gemm_groupsizes(pkg, oracle, gpu, gs, dtype):
+    _run(pkg, oracle, gpu, 1024, 256, gs, 96, dtype=dtype, sym=False, path=2, seed=gs + 200)
+
+
+def test_gemm_bit_exact_weights_through_identity(pkg, oracle, gpu):
+    """x = identity rows: y[m, :] must be W[m, :] exactly (fp16 W is what the MFMA sees, and
+    a one-hot fp32 accumulation adds nothing), so the in-register unpack of the GEMM kernel is
+    pinned bit for bit against the oracle's dequantized matrix."""
+    K, N, gs = 512, 256, 128
+    qw, qz, sc, _ = oracle.make_gptq(K, N, gs, seed=11, sym=False)
+    w = oracle.dequant_gptq(qw, qz, sc, None, gs, "f16")
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, gs, 0)
+    eye = torch.eye(K, dtype=torch.float16, device=gpu)
+    got = pkg.ops.linear(pk, eye, None, path=2)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), w.view(np.uint16))
+
+
+def test_auto_dispatch(pkg, oracle, gpu):
+    """q4_linear picks decode for M <= 16 and the MFMA GEMM above, generic for odd shapes."""
+    qw, qz, sc, _ = oracle.make_gptq(1024, 512, 128, seed=3)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
+    assert pkg.ops.select_path(pk, 1) == "gemv"
+    assert pkg.ops.select_path(pk, 16) == "gemv"
+    assert pkg.ops.select_path(pk, 17) == "gemm"
+    assert pkg.ops.select_path(pk, 2048) == "gemm"
+    qw, qz, sc, _ = oracle.make_gptq(1000, 264, 40, seed=3)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 40, 0)
+    assert pkg.ops.select_path(pk, 1) == "generic"
+    assert pkg.ops.select_path(pk, 2048) == "generic"

@@ -1,10 +1,364 @@
-// Prefill path placeholder translation unit: filled in by the MFMA GEMM kernel.
+// Prefill path: y[M, N] = x @ dequant(W) for large M on the MFMA units (gfx950).
+//
+// MFMA-bound: 2*M*N*K flops against 0.5 B/weight of HBM traffic.  Tiling (wave64):
+//   * a workgroup of 4 waves owns a BM x 256 output tile; wave w owns columns
+//     n0 + 64 w .. + 63 for all BM rows (4 waves side by side along N);
+//   * the B operand never touches LDS: a packed GPTQ word holds 8 consecutive K values of
+//     one column, which is exactly what lane (column j, K block kq) of a
+//     v_mfma_f32_32x32x16 supplies.  Each lane loads two adjacent words (columns
+//     nw + 2j, nw + 2j + 1) of packed row K/8 + kq with one 64-bit load (256 contiguous
+//     bytes per half-wave), unpacks them in registers to the reference's fp16 weight
+//     round_once(s * (q - z)) -- bit-identical to the dense dequantized matrix -- and feeds
+//     BM/32 MFMAs with each fragment.  Because the waves split N, no weight is unpacked
+//     twice inside a workgroup;
+//   * the A operand (activations) is staged through LDS, double buffered, in 16-byte
+//     units [row][K block] whose 8 values are stored in the order [0,4,1,5,2,6,3,7] that
+//     the nibble splice produces (see q4_common.cuh), so weights are never repacked;
+//     the row stride is padded to 9 units, which makes the 128-bit fragment reads
+//     conflict free;
+//   * packed weights are prefetched two K tiles (128 rows) ahead in registers, activations
+//     one tile ahead; fp32 accumulators live in VGPRs (BM = 128: 128 of them, two
+//     workgroups per CU so one wave's unpacking overlaps the other's MFMAs).
+#include <type_traits>
+
 #include "q4_common.cuh"
 
-namespace q4host {
-bool gemm_supported(const q4_weight*, int, int) { return false; }
-int launch_gemm(const q4_weight*, const void*, const void*, void*, int, int, hipStream_t) {
-  set_error("q4_linear(gemm): not built");
-  return Q4_ERR_UNSUPPORTED;
+namespace q4 {
+
+constexpr int kBK = 64;            // K rows per tile
+constexpr int kKSteps = kBK / 16;  // MFMA K steps per tile
+constexpr int kAUnitsPerRow = kBK / 8 + 1;  // 16-byte units per LDS row, padded
+constexpr int kBN = 256;           // columns per workgroup (4 waves x 64)
+
+struct GemmParams {
+  Problem p;
+};
+
+struct SpliceK {
+  uint32_t mask_lo, mask_hi, magic;
+};
+__device__ __forceinline__ SpliceK gemm_splice_consts() {
+  // Hidden from constant folding so that (w & mask) | magic selects v_and_or_b32 (a
+  // three-operand VALU op cannot carry literals).  The asm is empty on purpose.
+  SpliceK k{0x000F000Fu, 0x00F000F0u, 0x64006400u};
+  asm volatile("" : "+s"(k.mask_lo), "+s"(k.mask_hi), "+v"(k.magic));
+  return k;
 }
+
+// Per-column constants of one quantisation group.
+struct ColConsts {
+  half2_t czlo, czhi;  // -(1024 + z), -(64 + z), both halves equal
+  half2_t s2;          // (s, s)
+  float sf;            // float(s), bf16 path
+};
+
+__device__ __forceinline__ ColConsts make_col_consts(uint32_t z, half_t s) {
+  ColConsts c;
+  c.czlo = as_half2(0xE400E400u | z | (z << 16));
+  c.czhi = as_half2(0xD400D400u | (z << 4) | (z << 20));
+  c.s2 = half2_t{s, s};
+  c.sf = (float)s;
+  return c;
+}
+
+// One packed word -> MFMA B fragment (8 weights of one column, K order 0,4,1,5,2,6,3,7).
+template <int DTYPE>
+__device__ __forceinline__ uint4_t dequant_word(uint32_t w, const ColConsts& c, const SpliceK& k) {
+  const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+  const uint32_t w8 = w >> 8;
+  half2_t d[4];  // exact (q - z)
+  d[0] = as_half2((w & k.mask_lo) | k.magic) + c.czlo;
+  d[1] = as_half2((w & k.mask_hi) | k.magic) * sixteenth + c.czhi;
+  d[2] = as_half2((w8 & k.mask_lo) | k.magic) + c.czlo;
+  d[3] = as_half2((w8 & k.mask_hi) | k.magic) * sixteenth + c.czhi;
+  uint4_t out;
+  if constexpr (DTYPE == Q4_DTYPE_F16) {
+    // one fp16 multiply per weight: the reference's rounding
+    out.x = as_u32(d[0] * c.s2);
+    out.y = as_u32(d[1] * c.s2);
+    out.z = as_u32(d[2] * c.s2);
+    out.w = as_u32(d[3] * c.s2);
+  } else {
+    // bf16: exact fp32 product, rounded once
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float lo = (float)d[i].x * c.sf;
+      const float hi = (float)d[i].y * c.sf;
+      o[i] = (uint32_t)f32_to_bf16_rne(lo) | ((uint32_t)f32_to_bf16_rne(hi) << 16);
+    }
+    out.x = o[0]; out.y = o[1]; out.z = o[2]; out.w = o[3];
+  }
+  return out;
+}
+
+template <int DTYPE>
+__device__ __forceinline__ float16_t mfma32(const uint4_t a, const uint4_t b, float16_t c) {
+  if constexpr (DTYPE == Q4_DTYPE_F16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a),
+                                                  __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+}
+
+// BM: rows per workgroup (128 or 256).  GPT: quantisation groups per K tile (1 or 2).
+template <int DTYPE, int BM, int GPT>
+__global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(GemmParams gp) {
+  constexpr int MT = BM / 32;                      // MFMA row tiles per wave
+  constexpr int A_LOADS = BM * (kBK / 8) / 256;    // 16-byte activation loads per thread per tile
+  constexpr int A_TILE_BYTES = BM * kAUnitsPerRow * 16;
+  extern __shared__ __align__(16) unsigned char smem[];  // two activation tiles
+  const Problem& p = gp.p;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int j = lane & 31;
+  const int kq = lane >> 5;
+  const int N = p.N, K = p.K, M = p.M;
+
+  // XCD-aware tile order: consecutive workgroup ids go to different XCDs, so a group of 8
+  // consecutive ids shares nothing; ids that land on one XCD (id % 8 equal) walk the M
+  // tiles of one column block first and re-use its packed weights from that XCD's L2.
+  const int tiles_m = (M + BM - 1) / BM;
+  const int tiles_n = N / kBN;
+  int bid = blockIdx.x;
+  {
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    const int xcd = bid & 7;
+    const int local = bid >> 3;
+    const int lin = xcd * per_xcd + local;
+    bid = lin < total && (total % 8 == 0) ? lin : bid;
+  }
+  const int tm = bid % tiles_m;
+  const int tn = bid / tiles_m;
+  const int m0 = tm * BM;
+  const int n0 = tn * kBN;
+  const int nw = n0 + wave * 64;   // first column of this wave
+  const int ncol = nw + 2 * j;     // first of this lane's two columns
+
+  const SpliceK splice = gemm_splice_consts();
+  const int KT = K / kBK;
+
+  // ---- packed-weight stream: words [K/8 + kq][ncol, ncol+1], two K tiles ahead
+  const char* wbase = (const char*)p.qweight;
+  const uint32_t w_lane = ((uint32_t)kq * (uint32_t)N + (uint32_t)ncol) * 4u;
+  const size_t kstep_bytes = (size_t)N * 8;  // two packed rows per MFMA K step
+  uint2_t bq[2][kKSteps];
+  auto load_b = [&](int kt, uint2_t (&dst)[kKSteps]) {
+#pragma unroll
+    for (int s = 0; s < kKSteps; ++s)
+      dst[s] = __builtin_nontemporal_load(
+          (const uint2_t*)(wbase + (size_t)(kt * kKSteps + s) * kstep_bytes + w_lane));
+  };
+
+  // ---- group constants for this lane's two columns
+  ColConsts cc[GPT][2];
+  uint32_t sraw[GPT], zraw[GPT];
+  const int zshift = (ncol & 7) * 4;
+  auto load_group_raw = [&](int kt) {
+#pragma unroll
+    for (int g = 0; g < GPT; ++g) {
+      int gi = (kt * kBK + g * (kBK / GPT)) / p.groupsize;
+      gi = min(gi, p.num_groups - 1);
+      sraw[g] = *(const uint32_t*)(p.scales + (size_t)gi * N + ncol);
+      zraw[g] = p.qzeros[(size_t)gi * (N >> 3) + (ncol >> 3)];
+    }
+  };
+  auto make_group = [&]() {
+#pragma unroll
+    for (int g = 0; g < GPT; ++g) {
+      const uint32_t z2 = gptq_zero_plus_one(zraw[g]) >> zshift;
+      const half2_t s01 = as_half2(sraw[g]);
+      cc[g][0] = make_col_consts(z2 & 0xFu, s01.x);
+      cc[g][1] = make_col_consts((z2 >> 4) & 0xFu, s01.y);
+    }
+  };
+  // A tile covers one group, or GPT groups when groupsize < kBK.
+  auto group_changes = [&](int kt) { return GPT > 1 || (kt * kBK) % p.groupsize == 0; };
+
+  // ---- activation tile: global -> registers -> (permuted) LDS
+  const uint16_t* xs = (const uint16_t*)p.x;
+  uint4_t areg[A_LOADS];
+  auto load_a = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int u = tid + 256 * i;
+      const int m = u >> 3, kb = u & 7;
+      uint4_t v = {0u, 0u, 0u, 0u};
+      if (m0 + m < M) v = *(const uint4_t*)(xs + (size_t)(m0 + m) * K + kt * kBK + kb * 8);
+      areg[i] = v;
+    }
+  };
+  auto store_a = [&](int buf) {
+    unsigned char* base = smem + buf * A_TILE_BYTES;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int u = tid + 256 * i;
+      const int m = u >> 3, kb = u & 7;
+      const uint4_t v = areg[i];
+      uint4_t o;
+      o.x = (v.x & 0xFFFFu) | (v.z << 16);
+      o.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
+      o.z = (v.y & 0xFFFFu) | (v.w << 16);
+      o.w = (v.y >> 16) | (v.w & 0xFFFF0000u);
+      *(uint4_t*)(base + (m * kAUnitsPerRow + kb) * 16) = o;
+    }
+  };
+
+  float16_t acc[MT][2];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mt][f][r] = 0.f;
+
+  // ---- prologue
+  load_a(0);
+  load_b(0, bq[0]);
+  if (KT > 1) load_b(1, bq[1]);
+  load_group_raw(0);
+  store_a(0);
+  if (KT > 1) load_a(1);
+  __syncthreads();
+
+  const int a_lane_off = (j * kAUnitsPerRow + kq) * 16;
+
+  // One K tile.  `cur` (LDS buffer and weight-register set) is a compile-time constant so
+  // that the register arrays are indexed statically; the loop below is unrolled by two.
+  auto tile_step = [&](int kt, auto cur_c) {
+    constexpr int cur = decltype(cur_c)::value;
+    if (group_changes(kt)) {
+      make_group();  // raw values were loaded during the previous tile
+    }
+    if (kt + 1 < KT && group_changes(kt + 1)) load_group_raw(kt + 1);
+    const unsigned char* abase = smem + cur * A_TILE_BYTES + a_lane_off;
+#pragma unroll
+    for (int s = 0; s < kKSteps; ++s) {
+      const int g = GPT == 1 ? 0 : (s * 16) / (kBK / GPT);
+      const uint2_t words = bq[cur][s];
+      const uint4_t b0 = dequant_word<DTYPE>(words.x, cc[g][0], splice);
+      const uint4_t b1 = dequant_word<DTYPE>(words.y, cc[g][1], splice);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const uint4_t a = *(const uint4_t*)(abase + (mt * 32 * kAUnitsPerRow + 2 * s) * 16);
+        acc[mt][0] = mfma32<DTYPE>(a, b0, acc[mt][0]);
+        acc[mt][1] = mfma32<DTYPE>(a, b1, acc[mt][1]);
+      }
+    }
+    if (kt + 1 < KT) store_a(cur ^ 1);  // tile kt+1 is in areg
+    if (kt + 2 < KT) {
+      load_a(kt + 2);
+      load_b(kt + 2, bq[cur]);
+    }
+    __syncthreads();
+  };
+  for (int kt = 0; kt < KT; kt += 2) {
+    tile_step(kt, std::integral_constant<int, 0>{});
+    if (kt + 1 < KT) tile_step(kt + 1, std::integral_constant<int, 1>{});
+  }
+
+  // ---- epilogue: C layout of the 32x32 MFMA: register r of lane (j, kq) is row
+  // 8*(r/4) + 4*kq + r%4, column j.  Fragments 0/1 are adjacent columns -> one 32-bit store.
+  uint16_t* y = (uint16_t*)p.y;
+  float bias_f[2] = {0.f, 0.f};
+  const bool has_bias = p.bias != nullptr;
+  if (has_bias) {
+    bias_f[0] = load_act<DTYPE>(p.bias, ncol);
+    bias_f[1] = load_act<DTYPE>(p.bias, ncol + 1);
+  }
+  // The sum is rounded to the activation dtype first and the bias added in that dtype
+  // (one more rounding), like `out + bias` on a half tensor.
+  auto finish = [&](float v, float b) -> uint32_t {
+    uint16_t o = store_act<DTYPE>(v);
+    if (has_bias) {
+      float ob;
+      if constexpr (DTYPE == Q4_DTYPE_F16) ob = (float)__builtin_bit_cast(half_t, o);
+      else ob = bf16_bits_to_f32(o);
+      o = store_act<DTYPE>(ob + b);
+    }
+    return o;
+  };
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
+      if (m < M) {
+        const uint32_t lo = finish(acc[mt][0][r], bias_f[0]);
+        const uint32_t hi = finish(acc[mt][1][r], bias_f[1]);
+        *(uint32_t*)(y + (size_t)m * N + ncol) = lo | (hi << 16);
+      }
+    }
+  }
+}
+
+}  // namespace q4
+
+namespace q4host {
+
+using q4::GemmParams;
+using q4::Problem;
+
+bool gemm_supported(const q4_weight* w, int M, int dtype) {
+  (void)dtype;
+  if (w->layout != Q4_LAYOUT_GPTQ || w->g_idx != nullptr) return false;
+  if (M < 1) return false;
+  if (w->K % q4::kBK != 0 || w->N % q4::kBN != 0) return false;
+  const int gs = w->groupsize;
+  if (!(gs == 32 || (gs >= 64 && gs % 64 == 0))) return false;
+  if ((long)w->num_groups * gs < w->K) return false;
+  return true;
+}
+
+template <int DTYPE, int BM>
+static void launch_bm(const GemmParams& gp, int gs, dim3 grid, size_t smem, hipStream_t stream) {
+  using namespace q4;
+  if (gs == 32) {
+    auto k = gemm_gptq_kernel<DTYPE, BM, 2>;
+    if (smem > 64 * 1024)
+      (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL(k, grid, dim3(256), smem, stream, gp);
+  } else {
+    auto k = gemm_gptq_kernel<DTYPE, BM, 1>;
+    if (smem > 64 * 1024)
+      (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL(k, grid, dim3(256), smem, stream, gp);
+  }
+}
+
+int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                hipStream_t stream) {
+  using namespace q4;
+  if (!gemm_supported(w, M, dtype)) {
+    set_error("q4_linear(gemm): unsupported problem (layout=%d g_idx=%p M=%d K=%d N=%d groupsize=%d)",
+              w->layout, (const void*)w->g_idx, M, w->K, w->N, w->groupsize);
+    return Q4_ERR_UNSUPPORTED;
+  }
+  GemmParams gp;
+  gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, nullptr, x, bias, y,
+                 M,          w->K,      w->N,                     w->groupsize, w->num_groups};
+  constexpr int BM = 128;
+  const int tiles_m = (M + BM - 1) / BM;
+  const int tiles_n = w->N / kBN;
+  const long total = (long)tiles_m * tiles_n;
+  if (total > 0x7fffffffL) {
+    set_error("q4_linear(gemm): grid too large");
+    return Q4_ERR_UNSUPPORTED;
+  }
+  const size_t smem = 2 * (size_t)BM * kAUnitsPerRow * 16;
+  dim3 grid((unsigned)total);
+  if (dtype == Q4_DTYPE_F16) launch_bm<Q4_DTYPE_F16, BM>(gp, w->groupsize, grid, smem, stream);
+  else launch_bm<Q4_DTYPE_BF16, BM>(gp, w->groupsize, grid, smem, stream);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    set_error("q4_linear(gemm): launch failed: %s", hipGetErrorString(err));
+    return Q4_ERR_LAUNCH;
+  }
+  return Q4_OK;
+}
+
 }  // namespace q4host
