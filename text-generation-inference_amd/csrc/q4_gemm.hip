@@ -150,12 +150,12 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
   auto load_b = [&](int kt, uint2_t (&dst)[kKSteps]) {
 #pragma unroll
     for (int s = 0; s < kKSteps; ++s)
-      dst[s] = __builtin_nontemporal_load(
-          (const uint2_t*)(wbase + (size_t)(kt * kKSteps + s) * kstep_bytes + w_lane));
+      dst[s] = *(const uint2_t*)(wbase + (size_t)(kt * kKSteps + s) * kstep_bytes + w_lane);
   };
 
-  // ---- group constants for this lane's two columns
-  ColConsts cc[GPT][2];
+  // ---- group constants for this lane's two columns.  They are rebuilt for every tile
+  // from two tiny (cached) loads, which keeps the steady-state loop free of branches.
+  ColConsts cc[GPT][2], cc_next[GPT][2];
   uint32_t sraw[GPT], zraw[GPT];
   const int zshift = (ncol & 7) * 4;
   auto load_group_raw = [&](int kt) {
@@ -167,17 +167,15 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
       zraw[g] = p.qzeros[(size_t)gi * (N >> 3) + (ncol >> 3)];
     }
   };
-  auto make_group = [&]() {
+  auto make_group = [&](ColConsts (&dst)[GPT][2]) {
 #pragma unroll
     for (int g = 0; g < GPT; ++g) {
       const uint32_t z2 = gptq_zero_plus_one(zraw[g]) >> zshift;
       const half2_t s01 = as_half2(sraw[g]);
-      cc[g][0] = make_col_consts(z2 & 0xFu, s01.x);
-      cc[g][1] = make_col_consts((z2 >> 4) & 0xFu, s01.y);
+      dst[g][0] = make_col_consts(z2 & 0xFu, s01.x);
+      dst[g][1] = make_col_consts((z2 >> 4) & 0xFu, s01.y);
     }
   };
-  // A tile covers one group, or GPT groups when groupsize < kBK.
-  auto group_changes = [&](int kt) { return GPT > 1 || (kt * kBK) % p.groupsize == 0; };
 
   // ---- activation tile: global -> registers -> (permuted) LDS
   const uint16_t* xs = (const uint16_t*)p.x;
@@ -187,9 +185,9 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
     for (int i = 0; i < A_LOADS; ++i) {
       const int u = tid + 256 * i;
       const int m = u >> 3, kb = u & 7;
-      uint4_t v = {0u, 0u, 0u, 0u};
-      if (m0 + m < M) v = *(const uint4_t*)(xs + (size_t)(m0 + m) * K + kt * kBK + kb * 8);
-      areg[i] = v;
+      // rows past M re-read the last row: their results are never stored
+      const int row = min(m0 + m, M - 1);
+      areg[i] = *(const uint4_t*)(xs + (size_t)row * K + kt * kBK + kb * 8);
     }
   };
   auto store_a = [&](int buf) {
@@ -216,49 +214,101 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mt][f][r] = 0.f;
 
-  // ---- prologue
+  const int a_lane_off = (j * kAUnitsPerRow + kq) * 16;
+  uint4_t afrag[2][MT];  // A fragments of the current / next MFMA K step
+  uint4_t bfrag[2][2];   // unpacked B fragments of the current / next step
+  auto read_a = [&](int buf, int s, uint4_t (&dst)[MT]) {
+    const unsigned char* abase = smem + buf * A_TILE_BYTES + a_lane_off;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      dst[mt] = *(const uint4_t*)(abase + (mt * 32 * kAUnitsPerRow + 2 * s) * 16);
+  };
+  auto group_of_step = [](int s) { return GPT == 1 ? 0 : (s * 16) / (kBK / GPT); };
+
+  // ---- prologue: tile 0 staged, tile 1 in flight, first fragments ready
+  const int last_tile = KT - 1;
   load_a(0);
   load_b(0, bq[0]);
-  if (KT > 1) load_b(1, bq[1]);
+  load_b(min(1, last_tile), bq[1]);
   load_group_raw(0);
   store_a(0);
-  if (KT > 1) load_a(1);
+  load_a(min(1, last_tile));
+  make_group(cc);
   __syncthreads();
+  read_a(0, 0, afrag[0]);
+  bfrag[0][0] = dequant_word<DTYPE>(bq[0][0].x, cc[0][0], splice);
+  bfrag[0][1] = dequant_word<DTYPE>(bq[0][0].y, cc[0][1], splice);
 
-  const int a_lane_off = (j * kAUnitsPerRow + kq) * 16;
-
-  // One K tile.  `cur` (LDS buffer and weight-register set) is a compile-time constant so
-  // that the register arrays are indexed statically; the loop below is unrolled by two.
+  // One K tile, software pipelined: while the MFMAs of step s run, the VALU unpacks the
+  // weights of step s+1 and the LDS returns its A fragments; the global loads of tile
+  // kt+2 and the LDS writes of tile kt+1 are spread over the steps.  Tile indices past the
+  // end are clamped (the last tile is fetched again and ignored) so the body has no
+  // branches and the scheduler sees one region per step.  `cur` selects the LDS buffer and
+  // the weight-register set at compile time; the loop is unrolled by two.
   auto tile_step = [&](int kt, auto cur_c) {
     constexpr int cur = decltype(cur_c)::value;
-    if (group_changes(kt)) {
-      make_group();  // raw values were loaded during the previous tile
-    }
-    if (kt + 1 < KT && group_changes(kt + 1)) load_group_raw(kt + 1);
-    const unsigned char* abase = smem + cur * A_TILE_BYTES + a_lane_off;
+    const int kt1 = min(kt + 1, last_tile);
+    const int kt2 = min(kt + 2, last_tile);
 #pragma unroll
     for (int s = 0; s < kKSteps; ++s) {
-      const int g = GPT == 1 ? 0 : (s * 16) / (kBK / GPT);
-      const uint2_t words = bq[cur][s];
-      const uint4_t b0 = dequant_word<DTYPE>(words.x, cc[g][0], splice);
-      const uint4_t b1 = dequant_word<DTYPE>(words.y, cc[g][1], splice);
+      const int sb = s & 1;
+      // (1) LDS reads of the next step's A fragments go first so that they get the early
+      // LDS slots of this step.  The last step reads the first fragments of tile kt+1 from
+      // the other buffer, which the barrier below (between steps 2 and 3) has published.
+      if (s + 1 < kKSteps) read_a(cur, s + 1, afrag[sb ^ 1]);
+      else read_a(cur ^ 1, 0, afrag[sb ^ 1]);
+      // (2) unpack the next step's weights
+      if (s + 1 < kKSteps) {
+        const int g = group_of_step(s + 1);
+        bfrag[sb ^ 1][0] = dequant_word<DTYPE>(bq[cur][s + 1].x, cc[g][0], splice);
+        bfrag[sb ^ 1][1] = dequant_word<DTYPE>(bq[cur][s + 1].y, cc[g][1], splice);
+      } else {
+        bfrag[sb ^ 1][0] = dequant_word<DTYPE>(bq[cur ^ 1][0].x, cc_next[0][0], splice);
+        bfrag[sb ^ 1][1] = dequant_word<DTYPE>(bq[cur ^ 1][0].y, cc_next[0][1], splice);
+      }
+      // (3) side work of this step
+      if (s == 0) {
+        store_a(cur ^ 1);       // tile kt+1 (held in areg) -> the other LDS buffer
+        load_group_raw(kt1);    // scales / zero points the next tile starts with
+      }
+      if (s == 1) load_a(kt2);
+      if (s == 2) make_group(cc_next);
+      // (4) the MFMAs of this step
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        const uint4_t a = *(const uint4_t*)(abase + (mt * 32 * kAUnitsPerRow + 2 * s) * 16);
-        acc[mt][0] = mfma32<DTYPE>(a, b0, acc[mt][0]);
-        acc[mt][1] = mfma32<DTYPE>(a, b1, acc[mt][1]);
+        acc[mt][0] = mfma32<DTYPE>(afrag[sb][mt], bfrag[sb][0], acc[mt][0]);
+        acc[mt][1] = mfma32<DTYPE>(afrag[sb][mt], bfrag[sb][1], acc[mt][1]);
+      }
+      if (s == kKSteps - 1) load_b(kt2, bq[cur]);
+      // interleave: after every MFMA a few VALU ops, one LDS op and one global load
+#pragma unroll
+      for (int i = 0; i < 2 * MT; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+        __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+      if (s == kKSteps - 2) {
+        // One barrier per tile.  Here every wave has finished reading this tile's buffer
+        // (the step-3 fragments were read above) and has written its share of the next
+        // tile into the other buffer (step 0), so after the barrier the other buffer may
+        // be read (step 3) and this one overwritten (step 0 of the next tile).
+        __syncthreads();
       }
     }
-    if (kt + 1 < KT) store_a(cur ^ 1);  // tile kt+1 is in areg
-    if (kt + 2 < KT) {
-      load_a(kt + 2);
-      load_b(kt + 2, bq[cur]);
+#pragma unroll
+    for (int g = 0; g < GPT; ++g) {
+      cc[g][0] = cc_next[g][0];
+      cc[g][1] = cc_next[g][1];
     }
-    __syncthreads();
   };
-  for (int kt = 0; kt < KT; kt += 2) {
-    tile_step(kt, std::integral_constant<int, 0>{});
-    if (kt + 1 < KT) tile_step(kt + 1, std::integral_constant<int, 1>{});
+  {
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+      tile_step(kt, std::integral_constant<int, 0>{});
+      tile_step(kt + 1, std::integral_constant<int, 1>{});
+    }
+    if (kt < KT) tile_step(kt, std::integral_constant<int, 0>{});
   }
 
   // ---- epilogue: C layout of the 32x32 MFMA: register r of lane (j, kq) is row
