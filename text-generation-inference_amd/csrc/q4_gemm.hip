@@ -391,18 +391,26 @@ int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, in
   GemmParams gp;
   gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, nullptr, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
-  constexpr int BM = 128;
-  const int tiles_m = (M + BM - 1) / BM;
   const int tiles_n = w->N / kBN;
+  // 256-row tiles halve the unpacking work per flop (and run at a higher clock for it) but
+  // need one wave per SIMD and a grid of at least two rounds over the 256 CUs; otherwise
+  // 128-row tiles with two workgroups per CU.
+  const int bm = ((long)((M + 255) / 256) * tiles_n >= 512) ? 256 : 128;
+  const int tiles_m = (M + bm - 1) / bm;
   const long total = (long)tiles_m * tiles_n;
   if (total > 0x7fffffffL) {
     set_error("q4_linear(gemm): grid too large");
     return Q4_ERR_UNSUPPORTED;
   }
-  const size_t smem = 2 * (size_t)BM * kAUnitsPerRow * 16;
+  const size_t smem = 2 * (size_t)bm * kAUnitsPerRow * 16;
   dim3 grid((unsigned)total);
-  if (dtype == Q4_DTYPE_F16) launch_bm<Q4_DTYPE_F16, BM>(gp, w->groupsize, grid, smem, stream);
-  else launch_bm<Q4_DTYPE_BF16, BM>(gp, w->groupsize, grid, smem, stream);
+  if (bm == 256) {
+    if (dtype == Q4_DTYPE_F16) launch_bm<Q4_DTYPE_F16, 256>(gp, w->groupsize, grid, smem, stream);
+    else launch_bm<Q4_DTYPE_BF16, 256>(gp, w->groupsize, grid, smem, stream);
+  } else {
+    if (dtype == Q4_DTYPE_F16) launch_bm<Q4_DTYPE_F16, 128>(gp, w->groupsize, grid, smem, stream);
+    else launch_bm<Q4_DTYPE_BF16, 128>(gp, w->groupsize, grid, smem, stream);
+  }
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {
     set_error("q4_linear(gemm): launch failed: %s", hipGetErrorString(err));
