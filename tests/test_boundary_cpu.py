@@ -1,0 +1,217 @@
+"""CPU-side checks of the drop-in boundary: the C ABI exports what the header declares,
+argument validation works without a GPU, and the Python modules keep the reference's
+constructor/attribute/error contract.  No kernel is launched here."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = ROOT / "include" / "q4_linear.h"
+
+
+def declared_functions():
+    text = HEADER.read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(q4_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_functions_are_exported_and_bound(pkg):
+    lib = pkg._lib.load()
+    names = declared_functions()
+    assert {"q4_dequant", "q4_linear", "q4_linear_ex", "q4_gemv_tuned", "q4_workspace_bytes",
+            "q4_select_path", "q4_last_error", "q4_abi_version"} <= set(names)
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in q4_linear.h but not exported"
+        assert name in pkg._lib.SIGNATURES, f"{name} has no ctypes signature"
+    assert sorted(pkg._lib.SIGNATURES) == names
+    assert lib.q4_abi_version() == 1
+
+
+def test_header_constants_match_binding(pkg):
+    text = HEADER.read_text()
+    consts = dict(re.findall(r"#define\s+(Q4_[A-Z_0-9]+)\s+\(?(-?\d+)\)?", text))
+    L = pkg._lib
+    assert int(consts["Q4_LAYOUT_GPTQ"]) == L.LAYOUT_GPTQ and int(consts["Q4_LAYOUT_AWQ"]) == L.LAYOUT_AWQ
+    assert int(consts["Q4_DTYPE_F16"]) == L.DTYPE_F16 and int(consts["Q4_DTYPE_BF16"]) == L.DTYPE_BF16
+    assert int(consts["Q4_PATH_GEMV"]) == L.PATH_GEMV and int(consts["Q4_PATH_GEMM"]) == L.PATH_GEMM
+    assert int(consts["Q4_PATH_GENERIC"]) == L.PATH_GENERIC
+    assert int(consts["Q4_WORKSPACE_COUNTER_BYTES"]) == L.WORKSPACE_COUNTER_BYTES
+    assert int(consts["Q4_ERR_INVALID_ARGUMENT"]) == L.ERR_INVALID_ARGUMENT
+    assert int(consts["Q4_ERR_UNSUPPORTED"]) == L.ERR_UNSUPPORTED
+    assert int(consts["Q4_ERR_WORKSPACE"]) == L.ERR_WORKSPACE
+
+
+def _weight(pkg, K, N, gs, layout=0, g_idx=False):
+    """A q4_weight with fake non-null pointers: only used on paths that never dereference."""
+    G = max(1, K // gs) if gs > 0 else 1
+    return pkg._lib.Q4Weight(0x1000, 0x2000, 0x3000, 0x4000 if g_idx else None, K, N, gs, G, layout)
+
+
+def test_argument_validation_without_gpu(pkg):
+    lib = pkg._lib.load()
+    L = pkg._lib
+    assert lib.q4_dequant(None, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    assert b"null q4_weight" in lib.q4_last_error()
+    w = _weight(pkg, 4096, 4100, 128)  # N not a multiple of 8
+    assert lib.q4_linear(ctypes.byref(w), 0x10, None, 0x20, 1, 0, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    assert b"multiples of 8" in lib.q4_last_error()
+    w = _weight(pkg, 4096, 4096, 128, layout=7)
+    assert lib.q4_linear(ctypes.byref(w), 0x10, None, 0x20, 1, 0, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    w = _weight(pkg, 4096, 4096, 128)
+    assert lib.q4_linear(ctypes.byref(w), 0x10, None, 0x20, 1, 9, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    assert b"dtype" in lib.q4_last_error()
+    assert lib.q4_linear(ctypes.byref(w), 0x10, None, 0x20, -1, 0, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    # groups must cover K when there is no g_idx
+    w = pkg._lib.Q4Weight(0x1000, 0x2000, 0x3000, None, 4096, 4096, 128, 8, 0)
+    assert lib.q4_linear(ctypes.byref(w), 0x10, None, 0x20, 1, 0, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    assert b"do not cover" in lib.q4_last_error()
+    # AWQ has no act-order
+    w = _weight(pkg, 4096, 4096, 128, layout=1, g_idx=True)
+    assert lib.q4_linear(ctypes.byref(w), 0x10, None, 0x20, 1, 0, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    # decode path without the workspace it needs is refused before any launch
+    w = _weight(pkg, 4096, 4096, 128)
+    assert lib.q4_linear_ex(ctypes.byref(w), 0x10, None, 0x20, 1, 0, None, 0, L.PATH_GEMV, None) == L.ERR_WORKSPACE
+    assert b"workspace" in lib.q4_last_error()
+    # empty problems succeed without touching anything
+    w = _weight(pkg, 4096, 0, 128)
+    assert lib.q4_linear(ctypes.byref(w), None, None, None, 4, 0, None, 0, None) == 0
+    w = _weight(pkg, 4096, 4096, 128)
+    assert lib.q4_linear(ctypes.byref(w), None, None, None, 0, 0, None, 0, None) == 0
+
+
+def test_path_selection_and_workspace(pkg):
+    lib = pkg._lib.load()
+    L = pkg._lib
+    w = _weight(pkg, 4096, 4096, 128)
+    for M, want in [(1, L.PATH_GEMV), (16, L.PATH_GEMV), (17, L.PATH_GEMM), (2048, L.PATH_GEMM)]:
+        assert lib.q4_select_path(ctypes.byref(w), M, 0) == want
+    odd = _weight(pkg, 4104, 4104, 8)
+    assert lib.q4_select_path(ctypes.byref(odd), 1, 0) == L.PATH_GENERIC
+    assert lib.q4_select_path(ctypes.byref(odd), 512, 0) == L.PATH_GENERIC
+    for M, K, N in [(1, 4096, 4096), (16, 4096, 28672), (16, 14336, 4096), (4, 8192, 10240)]:
+        nbytes = lib.q4_workspace_bytes(M, K, N)
+        assert nbytes >= L.WORKSPACE_COUNTER_BYTES + M * N * 4
+        assert nbytes <= L.WORKSPACE_COUNTER_BYTES + 64 * 16 * N * 4
+    assert lib.q4_workspace_bytes(0, 0, 0) == L.WORKSPACE_COUNTER_BYTES
+
+
+def _cpu_gptq_tensors(oracle, K=256, N=64, gs=128, **kw):
+    qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=0, **kw)
+    t = lambda a: None if a is None else torch.from_numpy(a)
+    return t(qw), t(qz), t(sc), t(gi)
+
+
+def test_gptq_weight_contract(pkg, oracle):
+    qw, qz, sc, _ = _cpu_gptq_tensors(oracle)
+    w = pkg.GPTQWeight(qw, qz, sc.float(), None, 4, 128, use_awq_kernel=False, use_exllama=False)
+    assert w.scales.dtype == torch.float16        # fp32 scales are narrowed (gptq/__init__.py:29-31)
+    assert w.device == qw.device
+    lin = pkg.get_linear(w, None)
+    assert type(lin).__name__ == "QuantLinear"
+    assert (lin.infeatures, lin.outfeatures, lin.bits, lin.maxq, lin.groupsize) == (256, 64, 4, 15, 128)
+    assert lin.bias is None
+    ex = pkg.get_linear(pkg.GPTQWeight(qw, qz, sc, None, 4, 128, False, True), torch.zeros(64, dtype=torch.float16))
+    assert type(ex).__name__ == "ExllamaQuantLinear" and ex.infeatures == 256 and ex.outfeatures == 64
+    assert ex.act_order is False
+    with pytest.raises(NotImplementedError):
+        pkg.get_linear(torch.zeros(2, 2), None)
+
+
+def test_bits_other_than_four_are_rejected(pkg, oracle):
+    qw, qz, sc, _ = _cpu_gptq_tensors(oracle)
+    with pytest.raises(NotImplementedError, match="4 bits"):
+        pkg.QuantLinear(qw, qz, sc, None, None, 8, 128)
+    with pytest.raises(NotImplementedError):
+        pkg.QuantLinear.new(2, 128, 256, 64, False)
+    with pytest.raises(ValueError, match="bits=4"):
+        pkg.ExllamaQuantLinear(pkg.GPTQWeight(qw, qz, sc, None, 8, 128, False, True), None)
+    with pytest.raises(NotImplementedError, match="4-bit"):
+        pkg.WQLinear(8, 128, qw, qz, sc, None)
+    # bits read from a marker tensor arrive as a float (tests/utils/test_weights.py:671-672)
+    assert pkg.QuantLinear(qw, qz, sc, None, None, 4.0, 128).bits == 4
+
+
+def test_quant_linear_new_geometry(pkg):
+    lin = pkg.QuantLinear.new(4, 128, 1024, 512, True)
+    assert lin.qweight.shape == (128, 512) and lin.qweight.dtype == torch.int32
+    assert lin.qzeros.shape == (8, 64) and lin.scales.shape == (8, 512)
+    assert lin.g_idx.tolist() == [i // 128 for i in range(1024)]
+    assert lin.bias.shape == (512,) and lin.bias.dtype == torch.float16
+    one_group = pkg.QuantLinear.new(4, -1, 1024, 512, False)
+    assert one_group.qzeros.shape == (1, 64) and one_group.bias is None
+
+
+def test_wqlinear_contract(pkg, oracle):
+    aq, az, sc = oracle.make_awq(256, 64, 128, seed=0)
+    lin = pkg.WQLinear(4, 128, torch.from_numpy(aq), torch.from_numpy(az), torch.from_numpy(sc), None)
+    assert (lin.in_features, lin.out_features, lin.w_bit, lin.group_size) == (256, 64, 4, 128)
+    assert pkg.WQLinear(4, -1, torch.from_numpy(aq), torch.from_numpy(az[:1]), torch.from_numpy(sc[:1]), None).group_size == 256
+    with pytest.raises(AssertionError):
+        pkg.WQLinear(4, 96, torch.from_numpy(aq), torch.from_numpy(az), torch.from_numpy(sc), None)
+    w = pkg.GPTQWeight(torch.from_numpy(aq), torch.from_numpy(az), torch.from_numpy(sc), None, 4, 128, True, False)
+    assert type(pkg.get_linear(w, None)).__name__ == "WQLinear"  # no ROCm refusal here
+
+
+def test_no_cpu_fallback(pkg, oracle):
+    """CPU tensors are refused loudly: the package has no host compute path."""
+    qw, qz, sc, _ = _cpu_gptq_tensors(oracle)
+    lin = pkg.QuantLinear(qw, qz, sc, None, None, 4, 128)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        lin(torch.zeros(1, 256, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        lin.dequantize()
+
+
+def test_make_packed_validation(pkg, oracle):
+    qw, qz, sc, gi = _cpu_gptq_tensors(oracle, act_order=True)
+    mk = pkg.ops.make_packed
+    pk = mk(qw, qz, sc, gi, 128, 0)
+    assert (pk.K, pk.N, pk.groupsize, pk.num_groups) == (256, 64, 128, 2)
+    assert mk(qw, qz[:1], sc[:1], None, -1, 0).groupsize == 256
+    with pytest.raises(TypeError):
+        mk(qw.to(torch.int64), qz, sc, None, 128, 0)
+    with pytest.raises(TypeError):
+        mk(qw, qz, sc.float(), None, 128, 0)
+    with pytest.raises(ValueError, match="inconsistent"):
+        mk(qw, qz[:, :4], sc, None, 128, 0)
+    with pytest.raises(ValueError, match="do not cover"):
+        mk(qw, qz[:1], sc[:1], None, 128, 0)
+    with pytest.raises(ValueError, match="g_idx has"):
+        mk(qw, qz, sc, gi[:100], 128, 0)
+    with pytest.raises(ValueError, match="AWQ"):
+        mk(torch.zeros(256, 8, dtype=torch.int32), qz, sc, gi, 128, 1)
+
+
+def test_trivial_g_idx_detection(pkg):
+    from importlib import import_module
+    ql = import_module("text-generation-inference_amd.layers.gptq.quant_linear")
+    seq = (torch.arange(512) // 128).to(torch.int32)
+    assert ql.is_trivial_g_idx(seq, 128)
+    assert ql.is_trivial_g_idx(torch.zeros(512, dtype=torch.int32), -1)
+    assert not ql.is_trivial_g_idx(seq.flip(0), 128)
+    assert not ql.is_trivial_g_idx(seq, 64)
+
+
+def test_conversion_utils_match_oracle(pkg, oracle):
+    """The torch layout helpers (loader-side host logic) agree with the oracle's NumPy ones."""
+    cu = pkg.conversion_utils
+    aq, az, sc = oracle.make_awq(128, 64, 32, seed=3)
+    gq, gz = cu.fast_awq_to_gptq(torch.from_numpy(aq), torch.from_numpy(az))
+    oq, oz = oracle.fast_awq_to_gptq(aq, az)
+    assert np.array_equal(gq.numpy(), oq) and np.array_equal(gz.numpy(), oz)
+    m = torch.randint(0, 16, (32, 64), generator=torch.Generator().manual_seed(0))
+    for d in ("row", "column"):
+        assert torch.equal(cu.unpack(cu.pack(m, d), d).to(torch.int64), m)
+    assert np.array_equal(cu.pack(m, "row").numpy(), oracle.pack_rows(m.numpy()))
+    assert np.array_equal(cu.pack(m, "column").numpy(), oracle.pack_cols(m.numpy()))
+    assert cu.AWQ_PACK_ORDER == oracle.AWQ_PACK_ORDER
+
+
+def test_exllama_hooks_are_noops(pkg):
+    pkg.set_device(torch.device("cpu"))
+    assert pkg.create_exllama_buffers(4096) is None
