@@ -78,13 +78,14 @@ def test_gemv_groupsizes(pkg, oracle, gpu, gs):
 @pytest.mark.parametrize("cfg", [(1, 1, 1), (1, 1, 8), (2, 1, 4), (4, 1, 2), (1, 4, 2), (2, 2, 2), (4, 2, 1), (1, 8, 1), (2, 4, 1), (4, 1, 16)])
 @pytest.mark.parametrize("M", [1, 6, 16])
 def test_gemv_decompositions(pkg, oracle, gpu, cfg, M):
-    if M * (2048 // cfg[2] * 2 + 16) > 65536:
-        # the activation slab of this decomposition does not fit 64 KB of LDS: the library
-        # must refuse it with a clear error instead of launching
-        with pytest.raises(pkg._lib.Q4Error, match="LDS"):
-            _run(pkg, oracle, gpu, 2048, 1024, 128, M, sym=False, cfg=cfg, seed=1)
-        return
     _run(pkg, oracle, gpu, 2048, 1024, 128, M, sym=False, bias=(M == 6), cfg=cfg, seed=sum(cfg) + M)
+
+
+def test_gemv_config_that_exceeds_lds_is_refused(pkg, oracle, gpu):
+    """16 rows x 14336 K values do not fit the 160 KB of LDS in one split: the library must
+    refuse the decomposition with a clear error instead of launching."""
+    with pytest.raises(pkg._lib.Q4Error, match="LDS"):
+        _run(pkg, oracle, gpu, 14336, 256, 128, 16, cfg=(1, 1, 1), seed=1)
 
 
 def test_gemv_bf16(pkg, oracle, gpu):
@@ -158,3 +159,71 @@ def test_auto_dispatch(pkg, oracle, gpu):
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 40, 0)
     assert pkg.ops.select_path(pk, 1) == "generic"
     assert pkg.ops.select_path(pk, 2048) == "generic"
+
+
+# --------------------------------------------------------------------------- AWQ and act-order decode kernels
+
+
+@pytest.mark.parametrize("K,N", [(4096, 14336), (14336, 4096)])
+@pytest.mark.parametrize("M", [1, 2, 4, 16])
+def test_awq_decode_mistral(pkg, oracle, gpu, K, N, M):
+    """cfg5: AWQ GEMM layout, asymmetric zeros, Mistral-7B shapes, decode kernel."""
+    _run(pkg, oracle, gpu, K, N, 128, M, layout="awq", path=1, seed=K // 256 + M)
+
+
+@pytest.mark.parametrize("M", [3, 7, 16, 17, 40, 64, 256])
+def test_awq_m_sweep_chunked(pkg, oracle, gpu, M):
+    """The AWQ decode kernel takes any M in row chunks of 16 (cfg5 sweeps M up to 256)."""
+    _run(pkg, oracle, gpu, 1024, 512, 128, M, layout="awq", bias=(M % 2 == 1), seed=M)
+
+
+@pytest.mark.parametrize("gs", [32, 64, 128, 256, -1])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_awq_groupsizes_dtypes(pkg, oracle, gpu, gs, dtype):
+    _run(pkg, oracle, gpu, 512, 256, gs, 5, dtype=dtype, layout="awq", path=1, seed=gs + 7)
+
+
+@pytest.mark.parametrize("cfg", [(1, 1, 1), (1, 4, 2), (2, 2, 1), (1, 8, 1), (2, 1, 4)])
+def test_awq_decompositions(pkg, oracle, gpu, cfg):
+    _run(pkg, oracle, gpu, 1024, 512, 128, 6, layout="awq", cfg=cfg, seed=sum(cfg))
+
+
+def test_awq_auto_path_is_native(pkg, oracle, gpu):
+    qw, qz, sc = oracle.make_awq(1024, 512, 128, seed=0)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 1)
+    for M in (1, 16, 100, 256):
+        assert pkg.ops.select_path(pk, M) == "gemv"
+
+
+@pytest.mark.parametrize("K,N", [(8192, 10240), (28672, 8192)])
+@pytest.mark.parametrize("M", [1, 16])
+def test_act_order_decode_llama70b(pkg, oracle, gpu, K, N, M):
+    """cfg4: desc_act=True with a random row permutation, Llama-3-70B per-layer shapes."""
+    _run(pkg, oracle, gpu, K, N, 128, M, act=True, path=1, seed=K // 1024 + M)
+
+
+@pytest.mark.parametrize("M", [1, 5, 16, 33, 128])
+def test_act_order_small(pkg, oracle, gpu, M):
+    _run(pkg, oracle, gpu, 1024, 256, 128, M, sym=False, act=True, bias=True, seed=M + 300)
+
+
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("cfg", [(1, 1, 1), (1, 4, 2), (2, 2, 2), (1, 8, 1)])
+def test_act_order_groupsizes_decompositions(pkg, oracle, gpu, gs, cfg):
+    _run(pkg, oracle, gpu, 2048, 256, gs, 4, sym=False, act=True, cfg=cfg, seed=gs + sum(cfg))
+
+
+def test_act_order_bit_exact_weights_through_identity(pkg, oracle, gpu):
+    """One-hot activations read the unpacked act-order weights back exactly."""
+    K, N, gs = 256, 128, 32
+    qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=21, sym=False, act_order=True)
+    w = oracle.dequant_gptq(qw, qz, sc, gi, gs, "f16")
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), gs, 0)
+    eye = torch.eye(K, dtype=torch.float16, device=gpu)
+    got = pkg.ops.linear(pk, eye, None, path=1)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), w.view(np.uint16))
+
+
+def test_gptq_decode_m_chunks(pkg, oracle, gpu):
+    """The GPTQ decode kernel also runs M > 16 in row chunks when forced."""
+    _run(pkg, oracle, gpu, 1024, 512, 128, 50, sym=False, bias=True, path=1, seed=50)

@@ -82,28 +82,42 @@ int q4_dequant(const q4_weight* w, void* w_out, int dtype, void* stream) {
 
 int q4_select_path(const q4_weight* w, int M, int dtype) {
   if (validate_weight(w, "q4_select_path") != Q4_OK) return Q4_ERR_INVALID_ARGUMENT;
-  if (M <= 16 && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
-  if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;
+  const bool contiguous_gptq = w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr;
+  if (contiguous_gptq) {
+    // decode kernel up to one MFMA row block, the MFMA GEMM above
+    if (M <= 16 && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
+    if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;
+    if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
+    return Q4_PATH_GENERIC;
+  }
+  // AWQ and act-order: the decode kernels take any M in row chunks of 16
+  if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
   return Q4_PATH_GENERIC;
 }
 
 size_t q4_workspace_bytes(int M, int K, int N) {
   if (M < 1 || K < 1 || N < 1) return Q4_WORKSPACE_COUNTER_BYTES;
-  const int rows = M < 16 ? M : 16;
-  q4_weight w = {};
-  w.K = K;
-  w.N = N;
-  w.layout = Q4_LAYOUT_GPTQ;
-  w.groupsize = 128;
-  w.num_groups = (K + 127) / 128;
+  // Upper bound over the three decode kernels (their column tiles and split choices differ).
   int splits = 1;
   if (K % 128 == 0 && N % 64 == 0) {
-    for (int m = 1; m <= rows; ++m) {
-      const int s = gemv_pick_config(&w, m).splits;
-      if (s > splits) splits = s;
+    static const int32_t fake_idx = 0;
+    q4_weight w = {};
+    w.K = K;
+    w.N = N;
+    w.groupsize = 128;
+    w.num_groups = K / 128;
+    const int m_lo = M <= 16 ? 1 : M, m_hi = M;
+    for (int variant = 0; variant < 3; ++variant) {
+      w.layout = variant == 1 ? Q4_LAYOUT_AWQ : Q4_LAYOUT_GPTQ;
+      w.g_idx = variant == 2 ? &fake_idx : nullptr;  // only tested against NULL
+      if (variant == 1 && N % 256 != 0) continue;
+      for (int m = m_lo; m <= m_hi; ++m) {
+        const int s = gemv_pick_config(&w, m).splits;
+        if (s > splits) splits = s;
+      }
     }
   }
-  return (size_t)Q4_WORKSPACE_COUNTER_BYTES + (size_t)splits * rows * N * sizeof(float);
+  return (size_t)Q4_WORKSPACE_COUNTER_BYTES + (size_t)splits * M * N * sizeof(float);
 }
 
 int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,

@@ -1,35 +1,42 @@
-// Decode path: y[M<=16, N] = x @ dequant(W), GPTQ layout, groups contiguous in K.
+// Decode path: y[M, N] = x @ dequant(W) for small M (16 rows per workgroup row-chunk).
 //
-// HBM-bound: the packed weights are read exactly once with 128-bit loads and never
-// written back.  Work decomposition (all wave64):
-//   * a wave owns 64 columns; lane l covers columns n0 + 4*(l%16) .. +3 and the packed row
-//     r0 + l/16, so one global_load_dwordx4 per lane fetches a 4-row x 256-byte patch
-//     (32 K rows x 64 columns) whose rows are contiguous 256-byte segments;
-//   * a packed word already holds 8 consecutive K values of one column, which is exactly
-//     what one lane of a 16x16x32 MFMA supplies for the B operand (column l%16, K block
-//     l/16).  Word t of the dwordx4 feeds MFMA t; the four MFMAs produce columns
-//     n0 + 4*j + t.  The matrix core performs both the multiply and the reduction across
-//     the four K blocks of the wave, so the VALU only unpacks nibbles;
-//   * nibbles become halves with one AND+OR each pair (see q4_common.cuh) in the order
-//     [0,4,1,5,2,6,3,7]; the activation slab is staged once per workgroup in LDS in that
-//     same order, so no weight is ever repacked;
-//   * zero points are subtracted exactly in fp16 ((1024+q) - (1024+z)); the group scale
-//     is factored out of the K sum and applied to the fp32 group accumulator, so a weight
-//     costs ~1.1 VALU operations;
-//   * split-K: `wk` waves of a workgroup take consecutive K ranges and are combined
-//     through LDS in fixed order; `splits` workgroups write fp32 partials to the
-//     workspace and the last one to arrive (ticket counter) adds them in split order and
-//     writes the output.  The result is deterministic and needs no memset: the last
-//     workgroup resets its ticket.
+// HBM-bound: the packed weights are read exactly once with wide loads and never written
+// back.  All three kernels share one structure (wave64):
+//   * the B operand of a 16x16x32 MFMA wants, per lane, 8 consecutive K values of one
+//     column (column = lane % 16, K block = lane / 16).  The matrix core then performs both
+//     the multiply and the reduction across the four K blocks of the wave; the VALU only
+//     unpacks nibbles (about one operation per weight);
+//   * nibbles become halves by splicing them into the mantissa of 1024.0 (q4_common.cuh),
+//     zero points are subtracted exactly in fp16 and, when groups are contiguous in K, the
+//     group scale is factored out of the K sum and applied to the fp32 group accumulator;
+//   * the activation slab of the workgroup is staged once in LDS in the K order the unpack
+//     produces, so no weight is ever repacked;
+//   * split-K: `wk` waves of a workgroup take consecutive K ranges and are combined through
+//     LDS in fixed order; `splits` workgroups write fp32 partials to the workspace and the
+//     last one to arrive (ticket counter) adds them in split order and writes the output.
+//     The result is deterministic and needs no memset: the last workgroup resets its ticket.
+//
+// gemv_gptq_kernel      GPTQ layout, groups contiguous in K.  A packed word *is* one lane's
+//                       B operand; a lane loads 4 adjacent columns x 1 packed row with one
+//                       128-bit load (256-byte row segments per 16 lanes), word t feeds
+//                       MFMA t.
+// gemv_gptq_act_kernel  GPTQ layout with g_idx (act-order): every K row has its own group.
+//                       Scales and zero points of the workgroup's columns sit in an LDS
+//                       table indexed by g_idx[k]; they are applied per weight.
+// gemv_awq_kernel       AWQ layout: a word holds 8 interleaved columns of one K row.  A lane
+//                       loads an 8-row x 2-word patch and transposes nibbles in registers
+//                       (one byte permute per row pair and byte) into 16 B operands.
+//
 // Workgroup ids are laid out split-major so that all splits of a column tile land on the
 // same XCD (id % 8) and the partials stay in that XCD's L2.
 #include "q4_common.cuh"
 
 namespace q4 {
 
-constexpr int kChunkSteps = 4;              // 32-row MFMA steps per software-pipelined chunk
+constexpr int kChunkSteps = 4;                // 32-row MFMA steps per software-pipelined chunk
 constexpr int kChunkRows = 32 * kChunkSteps;  // 128 K rows
 constexpr int kPrefetch = 4;                  // chunks of weight loads in flight per wave
+constexpr int kRowsPerBlock = 16;             // activation rows per workgroup (MFMA M)
 
 struct GemvParams {
   Problem p;
@@ -37,6 +44,7 @@ struct GemvParams {
   uint32_t* __restrict__ tickets;
   int wcol, wk, splits;
   int slab_stride;  // bytes between activation rows in LDS
+  int slab_bytes;   // size of the activation slab region
 };
 
 // Constants of the nibble splice, hidden from constant folding (empty asm, no instruction
@@ -65,22 +73,23 @@ __device__ __forceinline__ void unpack_word_f16(uint32_t w, half2_t czlo, half2_
   out[3] = as_half2((w8 & k.mask_hi) | k.magic) * sixteenth + czhi;
 }
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
+// half2 of exact small integers -> packed bf16 pair (exact; v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint32_t pack_bf16_pair(half2_t h) {
-  // Small integers are exact in fp32 with a zero low half, so truncation is exact.
-  const uint32_t lo = __builtin_bit_cast(uint32_t, (float)h.x);
-  const uint32_t hi = __builtin_bit_cast(uint32_t, (float)h.y);
-  return (lo >> 16) | (hi & 0xFFFF0000u);
+  const float2_t f = {(float)h.x, (float)h.y};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
 }
 
+// One 16x16x32 MFMA; `b` holds eight weights as four half2.
 template <int DTYPE>
 __device__ __forceinline__ float4_t mfma16(const uint4_t a, const half2_t b[4], float4_t c) {
   if constexpr (DTYPE == Q4_DTYPE_F16) {
-    union {
-      half2_t h[4];
-      half8_t v;
-    } bu;
-    bu.h[0] = b[0]; bu.h[1] = b[1]; bu.h[2] = b[2]; bu.h[3] = b[3];
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), bu.v, c, 0, 0, 0);
+    uint4_t bu;
+    bu.x = as_u32(b[0]); bu.y = as_u32(b[1]); bu.z = as_u32(b[2]); bu.w = as_u32(b[3]);
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
+                                                  __builtin_bit_cast(half8_t, bu), c, 0, 0, 0);
   } else {
     uint4_t bb;
     bb.x = pack_bf16_pair(b[0]);
@@ -92,69 +101,221 @@ __device__ __forceinline__ float4_t mfma16(const uint4_t a, const half2_t b[4], 
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Work decomposition shared by the kernels.
+struct Decomp {
+  int tid, lane, wave, wc, wkk, j, kq, nthreads;
+  int tile_cols, ntiles, tile, split;
+  int KR, KW, kwg0, kw0;
+  int mb, mloc;  // first activation row of this workgroup and number of live rows (<= 16)
+};
+
+__device__ __forceinline__ Decomp make_decomp(const GemvParams& gp, int wave_cols) {
+  Decomp d;
+  d.tid = threadIdx.x;
+  d.lane = d.tid & 63;
+  d.wave = __builtin_amdgcn_readfirstlane(d.tid >> 6);  // wave-uniform: keeps index math scalar
+  d.wc = d.wave % gp.wcol;
+  d.wkk = d.wave / gp.wcol;
+  d.j = d.lane & 15;
+  d.kq = d.lane >> 4;
+  d.nthreads = blockDim.x;
+  d.tile_cols = wave_cols * gp.wcol;
+  d.ntiles = gp.p.N / d.tile_cols;
+  d.tile = blockIdx.x % d.ntiles;
+  d.split = blockIdx.x / d.ntiles;
+  d.KR = gp.p.K / gp.splits;
+  d.KW = d.KR / gp.wk;
+  d.kwg0 = d.split * d.KR;
+  d.kw0 = d.kwg0 + d.wkk * d.KW;
+  d.mb = blockIdx.y * kRowsPerBlock;
+  d.mloc = min(kRowsPerBlock, gp.p.M - d.mb);
+  return d;
+}
+
+// Activation slab [mloc][KR] -> LDS.  The global loads are issued before the weight loads
+// (memory returns in issue order, so L2 hits must not queue behind the HBM stream they are
+// needed to consume) and stored after them.  PERMUTE stores every 8-block in the K order
+// [0,4,1,5,2,6,3,7] of the GPTQ nibble splice.
+template <bool PERMUTE>
+struct SlabStager {
+  static constexpr int kLoads = 2;  // 16-byte activation loads per thread kept in flight
+  uint4_t xv[kLoads];
+  const uint16_t* xs;
+  int kb_per_row, items;
+
+  __device__ __forceinline__ uint4_t fetch(const GemvParams& gp, int idx) const {
+    const int m = idx / kb_per_row;
+    const int kb = idx - m * kb_per_row;
+    return *(const uint4_t*)(xs + (size_t)m * gp.p.K + kb * 8);
+  }
+  __device__ __forceinline__ void issue(const GemvParams& gp, const Decomp& d) {
+    xs = (const uint16_t*)gp.p.x + (size_t)d.mb * gp.p.K + d.kwg0;
+    kb_per_row = d.KR >> 3;
+    items = d.mloc * kb_per_row;
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+      const int idx = d.tid + u * d.nthreads;
+      if (idx < items) xv[u] = fetch(gp, idx);
+    }
+  }
+  __device__ __forceinline__ void put(const GemvParams& gp, unsigned char* smem, int idx,
+                                      uint4_t v) const {
+    const int m = idx / kb_per_row;
+    const int kb = idx - m * kb_per_row;
+    uint4_t o = v;
+    if constexpr (PERMUTE) {
+      o.x = (v.x & 0xFFFFu) | (v.z << 16);
+      o.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
+      o.z = (v.y & 0xFFFFu) | (v.w << 16);
+      o.w = (v.y >> 16) | (v.w & 0xFFFF0000u);
+    }
+    *(uint4_t*)(smem + (size_t)m * gp.slab_stride + kb * 16) = o;
+  }
+  __device__ __forceinline__ void store(const GemvParams& gp, const Decomp& d,
+                                        unsigned char* smem) {
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+      const int idx = d.tid + u * d.nthreads;
+      if (idx < items) put(gp, smem, idx, xv[u]);
+    }
+    for (int idx = d.tid + kLoads * d.nthreads; idx < items; idx += d.nthreads)
+      put(gp, smem, idx, fetch(gp, idx));
+  }
+};
+
+// Everything after the K loop.  out[t][r] is the fp32 sum of output row 4*kq + r (relative
+// to the workgroup's first row) and column col0 + t: every lane owns NT adjacent columns.
+template <int DTYPE, int NT, int RMAX>
+__device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& d,
+                                            float (&out)[NT][RMAX], int col0,
+                                            unsigned char* smem) {
+  const Problem& p = gp.p;
+  const int N = p.N;
+  // ---- combine the wk waves of the workgroup through LDS (fixed order)
+  if (gp.wk > 1) {
+    __syncthreads();  // everyone is done with the slab / tables
+    float* red = (float*)smem;
+    if (d.wkk > 0) {
+      float* dst = red + ((size_t)((d.wkk - 1) * gp.wcol + d.wc) * NT * RMAX) * 64 + d.lane;
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) dst[(t * RMAX + r) * 64] = out[t][r];
+    }
+    __syncthreads();
+    if (d.wkk == 0) {
+      for (int w = 1; w < gp.wk; ++w) {
+        const float* src = red + ((size_t)((w - 1) * gp.wcol + d.wc) * NT * RMAX) * 64 + d.lane;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int r = 0; r < RMAX; ++r) out[t][r] += src[(t * RMAX + r) * 64];
+      }
+    }
+  }
+
+  uint16_t* y = (uint16_t*)p.y;
+  if (gp.splits == 1) {
+    if (d.wkk == 0) {
+#pragma unroll
+      for (int r = 0; r < RMAX; ++r) {
+        const int m = 4 * d.kq + r;
+        if (m < d.mloc) {
+          uint16_t* dst = y + (size_t)(d.mb + m) * N + col0;
+#pragma unroll
+          for (int t = 0; t < NT; t += 4) {
+            uint16_t o[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+              o[u] = finish_output<DTYPE>(out[t + u][r], p.bias, col0 + t + u);
+            uint2_t packed;
+            packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+            packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+            *(uint2_t*)(dst + t) = packed;
+          }
+        }
+      }
+    }
+    return;
+  }
+
+  // ---- cross-workgroup split-K: write the partial, take a ticket, last one reduces.
+  // Partials and the ticket move with agent-scope relaxed atomics (coherent loads/stores
+  // that bypass the per-XCD L2 state) instead of release/acquire fences: a fence here
+  // would write back and invalidate the whole L2 once per workgroup, which costs more
+  // than the kernel itself.  Ordering comes from waiting for the stores to be
+  // acknowledged (vmcnt(0)) before the workgroup barrier that precedes the ticket.
+  if (d.wkk == 0) {
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) {
+      const int m = 4 * d.kq + r;
+      if (m < d.mloc) {
+        float* dst = gp.partials + ((size_t)d.split * p.M + d.mb + m) * N + col0;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          __hip_atomic_store(dst + t, out[t][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  __shared__ uint32_t ticket_s;
+  uint32_t* ticket = gp.tickets + blockIdx.y * d.ntiles + d.tile;
+  if (d.tid == 0) {
+    ticket_s = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (ticket_s != (uint32_t)(gp.splits - 1)) return;
+  {
+    const int items = d.mloc * d.tile_cols;
+    const int nbase = d.tile * d.tile_cols;
+    for (int idx = d.tid; idx < items; idx += d.nthreads) {
+      const int m = idx / d.tile_cols;
+      const int n = nbase + (idx - m * d.tile_cols);
+      const float* src = gp.partials + (size_t)(d.mb + m) * N + n;
+      const size_t sstride = (size_t)p.M * N;
+      float sum = 0.f;
+      int sp = 0;
+      for (; sp + 8 <= gp.splits; sp += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          v[u] = __hip_atomic_load(src + (size_t)(sp + u) * sstride, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += v[u];
+      }
+      for (; sp < gp.splits; ++sp)
+        sum += __hip_atomic_load(src + (size_t)sp * sstride, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+      y[(size_t)(d.mb + m) * N + n] = finish_output<DTYPE>(sum, p.bias, n);
+    }
+    if (d.tid == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// GPTQ, contiguous groups.
 // GSTEPS: MFMA steps (32 rows) per quantisation group inside a chunk: 1, 2 or 4.
 // STATIC128: groupsize is exactly 128, so every chunk is one whole group.
 template <int DTYPE, int RMAX, int GSTEPS, bool STATIC128>
 __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   extern __shared__ __align__(16) unsigned char smem[];
   const Problem& p = gp.p;
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps tile/K-range math scalar
-  const int wc = wave % gp.wcol;
-  const int wkk = wave / gp.wcol;
-  const int j = lane & 15;
-  const int kq = lane >> 4;
-  const int nthreads = blockDim.x;
-
-  const int tile_cols = 64 * gp.wcol;
-  const int ntiles = p.N / tile_cols;
-  const int tile = blockIdx.x % ntiles;
-  const int split = blockIdx.x / ntiles;
-  const int nl = tile * tile_cols + wc * 64 + 4 * j;  // first of this lane's 4 columns
-
-  const int KR = p.K / gp.splits;  // rows of this workgroup
-  const int KW = KR / gp.wk;       // rows of this wave
-  const int kwg0 = split * KR;
-  const int kw0 = kwg0 + wkk * KW;
-  const int nchunks = KW / kChunkRows;
+  const Decomp d = make_decomp(gp, 64);
   const int N = p.N;
+  const int nl = d.tile * d.tile_cols + d.wc * 64 + 4 * d.j;  // first of this lane's 4 columns
+  const int nchunks = d.KW / kChunkRows;
   constexpr int GPC = kChunkSteps / GSTEPS;  // groups per chunk
 
-  // ---- activation slab [M][KR] -> LDS, each 8-block in K order 0,4,1,5,2,6,3,7.  The
-  // global loads are issued before the weight loads: memory returns in issue order, so the
-  // slab (L2 hits) must not queue behind the HBM stream it is needed to consume.
-  constexpr int kSlabLoads = 2;  // 16-byte activation loads per thread kept in flight
-  const int kb_per_row = KR >> 3;
-  const int slab_items = p.M * kb_per_row;
-  const uint16_t* xs = (const uint16_t*)p.x;
-  uint4_t xv[kSlabLoads];
-#pragma unroll
-  for (int u = 0; u < kSlabLoads; ++u) {
-    const int idx = tid + u * nthreads;
-    if (idx < slab_items) {
-      const int m = idx / kb_per_row;
-      const int kb = idx - m * kb_per_row;
-      xv[u] = *(const uint4_t*)(xs + (size_t)m * p.K + kwg0 + kb * 8);
-    }
-  }
-  auto store_slab = [&](int idx, uint4_t v) {
-    const int m = idx / kb_per_row;
-    const int kb = idx - m * kb_per_row;
-    uint4_t o;
-    o.x = (v.x & 0xFFFFu) | (v.z << 16);
-    o.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
-    o.z = (v.y & 0xFFFFu) | (v.w << 16);
-    o.w = (v.y >> 16) | (v.w & 0xFFFF0000u);
-    *(uint4_t*)(smem + (size_t)m * gp.slab_stride + kb * 16) = o;
-  };
+  SlabStager<true> slab;
+  slab.issue(gp, d);
 
-  // ---- issue the first kPrefetch chunks of weight loads before anything else
-  // Addresses are a wave-uniform 64-bit base (scalar registers, advanced per step) plus a
-  // per-lane 32-bit byte offset, so the loads use the scalar-base addressing mode and the
-  // VALU does no address arithmetic in the loop.
-  const char* wbase = (const char*)(p.qweight + (size_t)(kw0 / 8) * N);
-  const uint32_t w_lane = ((uint32_t)kq * (uint32_t)N + (uint32_t)nl) * 4u;
+  // ---- issue the first kPrefetch chunks of weight loads.  Addresses are a wave-uniform
+  // 64-bit base plus a per-lane 32-bit byte offset.
+  const char* wbase = (const char*)(p.qweight + (size_t)(d.kw0 / 8) * N);
+  const uint32_t w_lane = ((uint32_t)d.kq * (uint32_t)N + (uint32_t)nl) * 4u;
   const size_t step_bytes = (size_t)N * 16;  // four packed rows
   const uint32_t s_lane = (uint32_t)nl * 2u;
   const uint32_t z_lane = (uint32_t)(nl >> 3) * 4u;
@@ -169,7 +330,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
           (const uint4_t*)(wbase + (size_t)(c * kChunkSteps + st) * step_bytes + w_lane));
 #pragma unroll
     for (int g = 0; g < GPC; ++g) {
-      int gi = (kw0 + c * kChunkRows + g * GSTEPS * 32) / p.groupsize;
+      int gi = (d.kw0 + c * kChunkRows + g * GSTEPS * 32) / p.groupsize;
       gi = min(gi, p.num_groups - 1);
       s[g] = *(const uint2_t*)((const char*)p.scales + (size_t)gi * N * 2 + s_lane);
       z[g] = *(const uint32_t*)((const char*)p.qzeros + (size_t)gi * (N >> 3) * 4 + z_lane);
@@ -179,20 +340,12 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   for (int b = 0; b < kPrefetch; ++b)
     if (b < nchunks) load_chunk(b, wq[b], sc[b], zw[b]);
 
-#pragma unroll
-  for (int u = 0; u < kSlabLoads; ++u) {
-    const int idx = tid + u * nthreads;
-    if (idx < slab_items) store_slab(idx, xv[u]);
-  }
-  for (int idx = tid + kSlabLoads * nthreads; idx < slab_items; idx += nthreads) {
-    const int m = idx / kb_per_row;
-    const int kb = idx - m * kb_per_row;
-    store_slab(idx, *(const uint4_t*)(xs + (size_t)m * p.K + kwg0 + kb * 8));
-  }
+  slab.store(gp, d, smem);
   __syncthreads();
 
-  const bool row_live = j < p.M;  // A-operand row of this lane
-  const unsigned char* a_base = smem + (size_t)j * gp.slab_stride + (size_t)(wkk * KW + kq * 8) * 2;
+  const bool row_live = d.j < d.mloc;  // A-operand row of this lane
+  const unsigned char* a_base =
+      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.wkk * d.KW + d.kq * 8) * 2;
 
   const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   float4_t tot[4] = {zero4, zero4, zero4, zero4};
@@ -202,7 +355,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
 
   auto process_chunk = [&](int c, const uint4_t (&w)[kChunkSteps], const uint2_t (&s)[GPC],
                            const uint32_t (&z)[GPC]) {
-    const int kc = kw0 + c * kChunkRows;
+    const int kc = d.kw0 + c * kChunkRows;
     bool group_start = true, group_end = true;
     if constexpr (!STATIC128 && GSTEPS == kChunkSteps) {
       group_start = (c == 0) || (kc % p.groupsize == 0);
@@ -262,99 +415,273 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
     }
   }
 
-  // ---- combine the wk waves of the workgroup through LDS (fixed order)
-  if (gp.wk > 1) {
-    __syncthreads();  // everyone is done with the activation slab
-    float* red = (float*)smem;
-    if (wkk > 0) {
-      float* dst = red + ((size_t)((wkk - 1) * gp.wcol + wc) * 4 * RMAX) * 64 + lane;
+  float out[4][RMAX];
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+  for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int r = 0; r < RMAX; ++r) dst[(t * RMAX + r) * 64] = tot[t][r];
+    for (int r = 0; r < RMAX; ++r) out[t][r] = tot[t][r];
+  gemv_finish<DTYPE, 4, RMAX>(gp, d, out, nl, smem);
+}
+
+// ---------------------------------------------------------------------------------------
+// GPTQ with g_idx (act-order), fp16.  LDS: [slab][g_idx slice as uint16][table G x tile_cols].
+// Table entry (g, column) = fp16 scale | fp16 -(1024 + zero) << 16.
+template <int RMAX>
+__global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const Problem& p = gp.p;
+  const Decomp d = make_decomp(gp, 64);
+  const int N = p.N;
+  const int nl = d.tile * d.tile_cols + d.wc * 64 + 4 * d.j;
+  const int nsteps = d.KW / 32;
+  constexpr int PF = 8;  // 32-row steps of weight loads in flight per wave
+
+  SlabStager<true> slab;
+  slab.issue(gp, d);
+
+  const char* wbase = (const char*)(p.qweight + (size_t)(d.kw0 / 8) * N);
+  const uint32_t w_lane = ((uint32_t)d.kq * (uint32_t)N + (uint32_t)nl) * 4u;
+  const size_t step_bytes = (size_t)N * 16;
+  uint4_t wq[PF];
+  auto load_step = [&](int st) {
+    return __builtin_nontemporal_load((const uint4_t*)(wbase + (size_t)st * step_bytes + w_lane));
+  };
+#pragma unroll
+  for (int b = 0; b < PF; ++b)
+    if (b < nsteps) wq[b] = load_step(b);
+
+  slab.store(gp, d, smem);
+
+  // ---- g_idx slice of this workgroup, clamped to the table, as uint16
+  uint16_t* gidx_s = (uint16_t*)(smem + gp.slab_bytes);
+  for (int i = d.tid; i < d.KR; i += d.nthreads) {
+    int g = p.g_idx[d.kwg0 + i];
+    g = min(max(g, 0), p.num_groups - 1);
+    gidx_s[i] = (uint16_t)g;
+  }
+  // ---- scale / zero table of the workgroup's columns, all groups
+  uint32_t* table = (uint32_t*)(smem + gp.slab_bytes + ((d.KR * 2 + 15) & ~15));
+  const int tc = d.tile_cols;
+  {
+    const int nbase = d.tile * tc;
+    const int words_per_row = tc >> 3;  // one qzeros word covers 8 columns
+    for (int i = d.tid; i < p.num_groups * words_per_row; i += d.nthreads) {
+      const int g = i / words_per_row;
+      const int c8 = i - g * words_per_row;
+      const uint32_t z8 = gptq_zero_plus_one(p.qzeros[(size_t)g * (N >> 3) + (nbase >> 3) + c8]);
+      const uint4_t s8 = *(const uint4_t*)(p.scales + (size_t)g * N + nbase + c8 * 8);
+      const uint32_t su[4] = {s8.x, s8.y, s8.z, s8.w};
+      uint32_t e[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const uint32_t s16 = (u & 1) ? (su[u >> 1] >> 16) : (su[u >> 1] & 0xFFFFu);
+        const uint32_t z = (z8 >> (4 * u)) & 0xFu;
+        e[u] = s16 | ((0xE400u | z) << 16);
+      }
+      uint4_t* dst = (uint4_t*)(table + (size_t)g * tc + c8 * 8);
+      dst[0] = uint4_t{e[0], e[1], e[2], e[3]};
+      dst[1] = uint4_t{e[4], e[5], e[6], e[7]};
     }
-    __syncthreads();
-    if (wkk == 0) {
-      for (int w = 1; w < gp.wk; ++w) {
-        const float* src = red + ((size_t)((w - 1) * gp.wcol + wc) * 4 * RMAX) * 64 + lane;
+  }
+  __syncthreads();
+
+  const bool row_live = d.j < d.mloc;
+  const unsigned char* a_base =
+      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.wkk * d.KW + d.kq * 8) * 2;
+  const uint16_t* g_base = gidx_s + d.wkk * d.KW + d.kq * 8;
+  const uint32_t* t_lane = table + d.wc * 64 + 4 * d.j;
+
+  const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  float4_t acc[4] = {zero4, zero4, zero4, zero4};
+  const SpliceConsts splice = splice_consts();
+
+  auto process_step = [&](int st, const uint4_t w) {
+    uint4_t a = {0u, 0u, 0u, 0u};
+    if (row_live) a = *(const uint4_t*)(a_base + (size_t)st * 64);
+    // groups of the 8 rows of this lane's K block, then their table rows (4 columns each)
+    const uint4_t g8 = *(const uint4_t*)(g_base + st * 32);
+    const uint32_t gw[4] = {g8.x, g8.y, g8.z, g8.w};
+    uint32_t e[8][4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+    for (int r = 0; r < 8; ++r) {
+      const uint32_t g = (r & 1) ? (gw[r >> 1] >> 16) : (gw[r >> 1] & 0xFFFFu);
+      const uint4_t row = *(const uint4_t*)(t_lane + (size_t)g * tc);
+      e[r][0] = row.x; e[r][1] = row.y; e[r][2] = row.z; e[r][3] = row.w;
+    }
+    const uint32_t words[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-          for (int r = 0; r < RMAX; ++r) tot[t][r] += src[(t * RMAX + r) * 64];
+    for (int t = 0; t < 4; ++t) {
+      half2_t b[4];
+#pragma unroll
+      for (int pr = 0; pr < 4; ++pr) {
+        // rows pr and pr + 4 of the K block share one splice (nibbles 16 bits apart)
+        const uint32_t ea = e[pr][t], eb = e[pr + 4][t];
+        const uint32_t s2 = (ea & 0xFFFFu) | (eb << 16);
+        const uint32_t c2 = (ea >> 16) | (eb & 0xFFFF0000u);
+        const uint32_t q2 = ((words[t] >> (4 * pr)) & splice.mask_lo) | splice.magic;
+        const half2_t dq = as_half2(q2) + as_half2(c2);  // exact q - z
+        b[pr] = dq * as_half2(s2);                       // one fp16 rounding, as the reference
+      }
+      // b is in K order [0,4,1,5,2,6,3,7], the order of the staged activations
+      acc[t] = mfma16<Q4_DTYPE_F16>(a, b, acc[t]);
+    }
+  };
+
+  for (int s0 = 0; s0 < nsteps; s0 += PF) {
+#pragma unroll
+    for (int b = 0; b < PF; ++b) {
+      const int st = s0 + b;
+      if (st < nsteps) {
+        process_step(st, wq[b]);
+        if (st + PF < nsteps) wq[b] = load_step(st + PF);
       }
     }
   }
 
-  uint16_t* y = (uint16_t*)p.y;
-  if (gp.splits == 1) {
-    if (wkk == 0) {
+  float out[4][RMAX];
 #pragma unroll
-      for (int r = 0; r < RMAX; ++r) {
-        const int m = 4 * kq + r;
-        if (m < p.M) {
-          uint16_t o[4];
+  for (int t = 0; t < 4; ++t)
 #pragma unroll
-          for (int t = 0; t < 4; ++t) o[t] = finish_output<DTYPE>(tot[t][r], p.bias, nl + t);
-          uint2_t packed;
-          packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
-          packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
-          *(uint2_t*)(y + (size_t)m * N + nl) = packed;
+    for (int r = 0; r < RMAX; ++r) out[t][r] = acc[t][r];
+  gemv_finish<Q4_DTYPE_F16, 4, RMAX>(gp, d, out, nl, smem);
+}
+
+// ---------------------------------------------------------------------------------------
+// AWQ layout.  Wave tile: 256 columns (32 packed words) x 32 rows per step; lane (j, kq)
+// loads words [8 rows of K block kq][2 adjacent words] and owns the 16 adjacent columns
+// starting at 8 * (first word of the wave + 2 j).
+template <int DTYPE, int RMAX>
+__global__ __launch_bounds__(512) void gemv_awq_kernel(GemvParams gp) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const Problem& p = gp.p;
+  const Decomp d = make_decomp(gp, 256);
+  const int N = p.N;
+  const int NC = N >> 3;                                             // packed words per row
+  const int cw = (d.tile * d.tile_cols + d.wc * 256) / 8 + 2 * d.j;  // first of this lane's 2 words
+  const int col0 = cw * 8;
+  const int nsteps = d.KW / 32;
+  constexpr int PF = 3;  // 32-row steps (8 x 64-bit loads each) in flight per wave
+
+  SlabStager<false> slab;
+  slab.issue(gp, d);
+
+  const char* wbase = (const char*)(p.qweight + (size_t)d.kw0 * NC);
+  const uint32_t w_lane = ((uint32_t)(d.kq * 8) * (uint32_t)NC + (uint32_t)cw) * 4u;
+  const size_t row_bytes = (size_t)NC * 4;
+  uint2_t wq[PF][8];
+  auto load_step = [&](int st, uint2_t (&w)[8]) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+      w[r] = __builtin_nontemporal_load(
+          (const uint2_t*)(wbase + (size_t)(st * 32 + r) * row_bytes + w_lane));
+  };
+#pragma unroll
+  for (int b = 0; b < PF; ++b)
+    if (b < nsteps) load_step(b, wq[b]);
+
+  slab.store(gp, d, smem);
+  __syncthreads();
+
+  const bool row_live = d.j < d.mloc;
+  const unsigned char* a_base =
+      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.wkk * d.KW + d.kq * 8) * 2;
+
+  const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  float4_t acc[16];
+  float tot[16][RMAX];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    acc[t] = zero4;
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) tot[t][r] = 0.f;
+  }
+  half2_t cz[2][8];  // per word h and nibble position: -(1024 + z) (even) or -(64 + z) (odd)
+  const SpliceConsts splice = splice_consts();
+  const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+
+  auto flush = [&](int g) {
+    // scales of the lane's 16 columns: position pos of word h is column 8h + awq_order(pos)
+    const uint4_t* sp = (const uint4_t*)(p.scales + (size_t)g * N + col0);
+    const uint4_t s0 = sp[0], s1 = sp[1];
+    const uint32_t su[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int pos = 0; pos < 8; ++pos) {
+        const int col = 8 * h + (((pos & 3) << 1) | (pos >> 2));
+        const half2_t pr = as_half2(su[col >> 1]);
+        const float sf = (float)((col & 1) ? pr.y : pr.x);
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r)
+          tot[h * 8 + pos][r] = fmaf(sf, acc[h * 8 + pos][r], tot[h * 8 + pos][r]);
+      }
+  };
+
+  auto process_step = [&](int st, const uint2_t (&w)[8]) {
+    const int k = d.kw0 + st * 32;
+    const int g = min(k / p.groupsize, p.num_groups - 1);
+    const bool group_start = (st == 0) || (k % p.groupsize == 0);
+    const bool group_end = (st == nsteps - 1) || ((k + 32) % p.groupsize == 0);
+    if (group_start) {
+      const uint2_t zw = *(const uint2_t*)(p.qzeros + (size_t)g * NC + cw);
+      const uint32_t zz[2] = {zw.x, zw.y};
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int pos = 0; pos < 8; ++pos) {
+          const uint32_t z = (zz[h] >> (4 * pos)) & 0xFu;  // AWQ zero points are used as stored
+          cz[h][pos] = (pos & 1) ? as_half2(0xD400D400u | (z << 4) | (z << 20))
+                                 : as_half2(0xE400E400u | z | (z << 16));
+        }
+#pragma unroll
+      for (int t = 0; t < 16; ++t) acc[t] = zero4;
+    }
+    uint4_t a = {0u, 0u, 0u, 0u};
+    if (row_live) a = *(const uint4_t*)(a_base + (size_t)st * 64);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      half2_t b[8][4];  // [nibble position][row pair]
+#pragma unroll
+      for (int rp = 0; rp < 4; ++rp) {
+        const uint32_t w0 = h == 0 ? w[2 * rp].x : w[2 * rp].y;
+        const uint32_t w1 = h == 0 ? w[2 * rp + 1].x : w[2 * rp + 1].y;
+#pragma unroll
+        for (int by = 0; by < 4; ++by) {
+          // byte `by` of both rows side by side: low nibble = position 2*by, high = 2*by + 1
+          const uint32_t sel = 0x0C000C00u | (uint32_t)by | ((uint32_t)(4 + by) << 16);
+          const uint32_t t2 = __builtin_amdgcn_perm(w1, w0, sel);
+          b[2 * by][rp] = as_half2((t2 & splice.mask_lo) | splice.magic) + cz[h][2 * by];
+          b[2 * by + 1][rp] =
+              as_half2((t2 & splice.mask_hi) | splice.magic) * sixteenth + cz[h][2 * by + 1];
         }
       }
+#pragma unroll
+      for (int pos = 0; pos < 8; ++pos) acc[h * 8 + pos] = mfma16<DTYPE>(a, b[pos], acc[h * 8 + pos]);
     }
-    return;
+    if (group_end) flush(g);
+  };
+
+  for (int s0 = 0; s0 < nsteps; s0 += PF) {
+#pragma unroll
+    for (int b = 0; b < PF; ++b) {
+      const int st = s0 + b;
+      if (st < nsteps) {
+        process_step(st, wq[b]);
+        if (st + PF < nsteps) load_step(st + PF, wq[b]);
+      }
+    }
   }
 
-  // ---- cross-workgroup split-K: write the partial, take a ticket, last one reduces.
-  // Partials and the ticket move with agent-scope relaxed atomics (coherent loads/stores
-  // that bypass the per-XCD L2 state) instead of release/acquire fences: a fence here
-  // would write back and invalidate the whole L2 once per workgroup, which costs more
-  // than the kernel itself.  Ordering comes from waiting for the stores to be
-  // acknowledged (vmcnt(0)) before the workgroup barrier that precedes the ticket.
-  if (wkk == 0) {
+  // accumulator (h, pos) is column 8h + awq_order(pos) of the lane's 16
+  float out[16][RMAX];
 #pragma unroll
-    for (int r = 0; r < RMAX; ++r) {
-      const int m = 4 * kq + r;
-      if (m < p.M) {
-        float* dst = gp.partials + ((size_t)split * p.M + m) * N + nl;
+  for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-          __hip_atomic_store(dst + t, tot[t][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  __shared__ uint32_t ticket_s;
-  if (tid == 0) {
-    ticket_s = __hip_atomic_fetch_add(gp.tickets + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  __syncthreads();
-  if (ticket_s != (uint32_t)(gp.splits - 1)) return;
-  {
-    const int items = p.M * tile_cols;
-    const int nbase = tile * tile_cols;
-    for (int idx = tid; idx < items; idx += nthreads) {
-      const int m = idx / tile_cols;
-      const int n = nbase + (idx - m * tile_cols);
-      const float* src = gp.partials + (size_t)m * N + n;
-      const size_t sstride = (size_t)p.M * N;
-      float sum = 0.f;
-      int sp = 0;
-      for (; sp + 8 <= gp.splits; sp += 8) {
-        float v[8];
+    for (int pos = 0; pos < 8; ++pos)
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-          v[u] = __hip_atomic_load(src + (size_t)(sp + u) * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) sum += v[u];
-      }
-      for (; sp < gp.splits; ++sp)
-        sum += __hip_atomic_load(src + (size_t)sp * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      y[(size_t)m * N + n] = finish_output<DTYPE>(sum, p.bias, n);
-    }
-    if (tid == 0) __hip_atomic_store(gp.tickets + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+      for (int r = 0; r < RMAX; ++r)
+        out[8 * h + (((pos & 3) << 1) | (pos >> 2))][r] = tot[h * 8 + pos][r];
+  gemv_finish<DTYPE, 16, RMAX>(gp, d, out, col0, smem);
 }
 
 }  // namespace q4
@@ -364,61 +691,95 @@ namespace q4host {
 using q4::GemvParams;
 using q4::Problem;
 
+static bool groupsize_ok_contiguous(int gs) {
+  return gs == 32 || gs == 64 || (gs >= 128 && gs % 128 == 0);
+}
+
 bool gemv_supported(const q4_weight* w, int M, int dtype) {
-  (void)dtype;
-  if (w->layout != Q4_LAYOUT_GPTQ || w->g_idx != nullptr) return false;
-  if (M < 1 || M > 16) return false;
-  if (w->K % 128 != 0 || w->N % 64 != 0) return false;
-  const int gs = w->groupsize;
-  if (!(gs == 32 || gs == 64 || (gs >= 128 && gs % 128 == 0))) return false;
-  if ((long)w->num_groups * gs < w->K) return false;
-  if (w->N / 64 > Q4_WORKSPACE_COUNTER_BYTES / 4) return false;
-  return true;
+  if (M < 1) return false;
+  if (w->K % 128 != 0) return false;
+  const long chunks = (M + q4::kRowsPerBlock - 1) / q4::kRowsPerBlock;
+  if (chunks > 65535) return false;
+  if (w->layout == Q4_LAYOUT_AWQ) {
+    if (w->N % 256 != 0 || w->groupsize % 32 != 0) return false;
+    if ((long)w->num_groups * w->groupsize < w->K) return false;
+    return chunks * (w->N / 256) <= Q4_WORKSPACE_COUNTER_BYTES / 4;
+  }
+  if (w->N % 64 != 0) return false;
+  if (chunks * (w->N / 64) > Q4_WORKSPACE_COUNTER_BYTES / 4) return false;
+  if (w->g_idx != nullptr) {
+    // act-order: the table of all groups for 64 columns must fit LDS next to the slab
+    if (dtype != Q4_DTYPE_F16) return false;
+    return w->num_groups <= 65535 && (long)w->num_groups * 64 * 4 <= 96 * 1024;
+  }
+  if (!groupsize_ok_contiguous(w->groupsize)) return false;
+  return (long)w->num_groups * w->groupsize >= w->K;
 }
 
 GemvConfig gemv_pick_config(const q4_weight* w, int M) {
-  // Measured on MI355X (Llama-3-8B shapes, M=1): 64-column tiles with 4 waves along K per
-  // workgroup and about two workgroups per CU (512 in flight) is the best point; wider
+  // Measured on MI355X (Llama-3-8B shapes, M=1): narrow column tiles with 4 waves along K
+  // per workgroup and about two workgroups per CU (512 in flight) is the best point; wider
   // workgroups start too slowly and more splits lengthen the reduction tail.  The
-  // activation slab (M rows x K/splits) must fit 60 KB of LDS.
+  // activation slab (rows x K/splits) must fit its share of LDS.
   GemvConfig c;
+  const int rows = M < q4::kRowsPerBlock ? M : q4::kRowsPerBlock;
+  const int mchunks = (M + q4::kRowsPerBlock - 1) / q4::kRowsPerBlock;
   const int chunks = w->K / 128;
   c.wcol = 1;
   c.wk = chunks % 4 == 0 ? 4 : (chunks % 2 == 0 ? 2 : 1);
-  const int per_wg = chunks / c.wk;  // chunks left to distribute over splits x per-wave work
-  const int ntiles = w->N / 64;
+  const bool act = w->layout == Q4_LAYOUT_GPTQ && w->g_idx != nullptr;
+  if (act && chunks % 8 == 0) c.wk = 8;  // the group table is built once per workgroup
+  const int per_wg = chunks / c.wk;      // chunks left to distribute over splits x per-wave work
+  const int wave_cols = w->layout == Q4_LAYOUT_AWQ ? 256 : 64;
+  const int ntiles = (w->N / wave_cols) * mchunks;
   const int target_wgs = M <= 4 ? 512 : 384;  // partial-sum traffic grows with M
   int want = (target_wgs + ntiles / 2) / ntiles;
   if (want < 1) want = 1;
-  const long lds_budget = 60000 - 16L * M;
-  int min_splits = (int)(((long)M * w->K * 2 + lds_budget - 1) / lds_budget);
+  long lds_budget = 60000 - 16L * rows;
+  if (act) lds_budget = 150000 - (long)w->num_groups * 64 * 4 - 16L * rows;
+  // bytes per K row in LDS: activations, plus the uint16 g_idx slice for act-order
+  const long per_row = (long)rows * 2 + (act ? 2 : 0);
+  int min_splits = lds_budget > 0 ? (int)(((long)w->K * per_row + lds_budget - 1) / lds_budget) : per_wg;
   if (min_splits < 1) min_splits = 1;
   int best = per_wg;  // always legal: one chunk per wave
   long best_cost = -1;
-  for (int d = 1; d <= per_wg; ++d) {
-    if (per_wg % d != 0 || d < min_splits) continue;
-    const long cost = d > want ? (long)d * 1000 / want : (long)want * 1000 / d;
+  for (int dv = 1; dv <= per_wg; ++dv) {
+    if (per_wg % dv != 0 || dv < min_splits) continue;
+    const long cost = dv > want ? (long)dv * 1000 / want : (long)want * 1000 / dv;
     if (best_cost < 0 || cost < best_cost) {
       best_cost = cost;
-      best = d;
+      best = dv;
     }
   }
   c.splits = best;
   return c;
 }
 
+template <typename Kernel>
+static void launch_kernel(Kernel k, const GemvParams& gp, dim3 grid, dim3 block, size_t smem,
+                          hipStream_t stream) {
+  if (smem > 64 * 1024)
+    (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  hipLaunchKernelGGL(k, grid, block, smem, stream, gp);
+}
+
 template <int DTYPE, int RMAX>
-static void launch_rmax(const GemvParams& gp, int gs, dim3 grid, dim3 block, size_t smem,
-                        hipStream_t stream) {
+static void launch_rmax(const q4_weight* w, const GemvParams& gp, dim3 grid, dim3 block,
+                        size_t smem, hipStream_t stream) {
   using namespace q4;
-  if (gs == 128) {
-    hipLaunchKernelGGL((gemv_gptq_kernel<DTYPE, RMAX, 4, true>), grid, block, smem, stream, gp);
+  const int gs = w->groupsize;
+  if (w->layout == Q4_LAYOUT_AWQ) {
+    launch_kernel(gemv_awq_kernel<DTYPE, RMAX>, gp, grid, block, smem, stream);
+  } else if (w->g_idx != nullptr) {
+    launch_kernel(gemv_gptq_act_kernel<RMAX>, gp, grid, block, smem, stream);
+  } else if (gs == 128) {
+    launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, true>, gp, grid, block, smem, stream);
   } else if (gs > 128) {
-    hipLaunchKernelGGL((gemv_gptq_kernel<DTYPE, RMAX, 4, false>), grid, block, smem, stream, gp);
+    launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, false>, gp, grid, block, smem, stream);
   } else if (gs == 64) {
-    hipLaunchKernelGGL((gemv_gptq_kernel<DTYPE, RMAX, 2, false>), grid, block, smem, stream, gp);
+    launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 2, false>, gp, grid, block, smem, stream);
   } else {
-    hipLaunchKernelGGL((gemv_gptq_kernel<DTYPE, RMAX, 1, false>), grid, block, smem, stream, gp);
+    launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 1, false>, gp, grid, block, smem, stream);
   }
 }
 
@@ -427,28 +788,41 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
                 hipStream_t stream) {
   using namespace q4;
   if (!gemv_supported(w, M, dtype)) {
-    set_error("q4_linear(gemv): unsupported problem (layout=%d g_idx=%p M=%d K=%d N=%d groupsize=%d)",
-              w->layout, (const void*)w->g_idx, M, w->K, w->N, w->groupsize);
+    set_error("q4_linear(gemv): unsupported problem (layout=%d g_idx=%p M=%d K=%d N=%d groupsize=%d dtype=%d)",
+              w->layout, (const void*)w->g_idx, M, w->K, w->N, w->groupsize, dtype);
     return Q4_ERR_UNSUPPORTED;
   }
+  const bool awq = w->layout == Q4_LAYOUT_AWQ;
+  const bool act = !awq && w->g_idx != nullptr;
+  const int wave_cols = awq ? 256 : 64;
   const GemvConfig cfg = cfg_in ? *cfg_in : gemv_pick_config(w, M);
   if (cfg.wcol < 1 || cfg.wk < 1 || cfg.splits < 1 || cfg.wcol * cfg.wk > 8 ||
-      w->N % (64 * cfg.wcol) != 0 || w->K % (cfg.splits * cfg.wk * 128) != 0) {
+      w->N % (wave_cols * cfg.wcol) != 0 || w->K % (cfg.splits * cfg.wk * 128) != 0) {
     set_error("q4_linear(gemv): bad config wcol=%d wk=%d splits=%d for K=%d N=%d", cfg.wcol, cfg.wk,
               cfg.splits, w->K, w->N);
     return Q4_ERR_INVALID_ARGUMENT;
   }
+  const int rows = M < kRowsPerBlock ? M : kRowsPerBlock;
+  const int mchunks = (M + kRowsPerBlock - 1) / kRowsPerBlock;
   const int KR = w->K / cfg.splits;
   const int slab_stride = KR * 2 + 16;
   const int rmax = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
-  size_t smem = (size_t)M * slab_stride;
-  const size_t red = (size_t)(cfg.wk - 1) * cfg.wcol * 4 * rmax * 64 * sizeof(float);
+  const int nt = awq ? 16 : 4;
+  const size_t slab_bytes = ((size_t)rows * slab_stride + 15) & ~(size_t)15;
+  size_t smem = slab_bytes;
+  if (act) smem += (((size_t)KR * 2 + 15) & ~(size_t)15) + (size_t)w->num_groups * 64 * cfg.wcol * 4;
+  const size_t red = (size_t)(cfg.wk - 1) * cfg.wcol * nt * rmax * 64 * sizeof(float);
   if (red > smem) smem = red;
-  if (smem > 64 * 1024) {
-    set_error("q4_linear(gemv): config needs %zu bytes of LDS (> 64 KB)", smem);
+  const size_t smem_limit = 160 * 1024 - 1024;  // gfx950: 160 KB of LDS per workgroup
+  if (smem > smem_limit) {
+    set_error("q4_linear(gemv): config needs %zu bytes of LDS (> %zu)", smem, smem_limit);
     return Q4_ERR_INVALID_ARGUMENT;
   }
-  const int ntiles = w->N / (64 * cfg.wcol);
+  const int ntiles = w->N / (wave_cols * cfg.wcol);
+  if ((long)ntiles * mchunks > Q4_WORKSPACE_COUNTER_BYTES / 4) {
+    set_error("q4_linear(gemv): too many tiles (%d x %d)", ntiles, mchunks);
+    return Q4_ERR_UNSUPPORTED;
+  }
   float* partials = nullptr;
   uint32_t* tickets = nullptr;
   if (cfg.splits > 1) {
@@ -461,7 +835,7 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
     partials = (float*)((char*)workspace + Q4_WORKSPACE_COUNTER_BYTES);
   }
   GemvParams gp;
-  gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, nullptr, x, bias, y,
+  gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, w->g_idx, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
   gp.partials = partials;
   gp.tickets = tickets;
@@ -469,17 +843,17 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.wk = cfg.wk;
   gp.splits = cfg.splits;
   gp.slab_stride = slab_stride;
-  dim3 grid((unsigned)(ntiles * cfg.splits));
+  gp.slab_bytes = (int)slab_bytes;
+  dim3 grid((unsigned)(ntiles * cfg.splits), (unsigned)mchunks);
   dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
-  const int gs = w->groupsize;
   if (dtype == Q4_DTYPE_F16) {
-    if (rmax == 1) launch_rmax<Q4_DTYPE_F16, 1>(gp, gs, grid, block, smem, stream);
-    else if (rmax == 2) launch_rmax<Q4_DTYPE_F16, 2>(gp, gs, grid, block, smem, stream);
-    else launch_rmax<Q4_DTYPE_F16, 4>(gp, gs, grid, block, smem, stream);
+    if (rmax == 1) launch_rmax<Q4_DTYPE_F16, 1>(w, gp, grid, block, smem, stream);
+    else if (rmax == 2) launch_rmax<Q4_DTYPE_F16, 2>(w, gp, grid, block, smem, stream);
+    else launch_rmax<Q4_DTYPE_F16, 4>(w, gp, grid, block, smem, stream);
   } else {
-    if (rmax == 1) launch_rmax<Q4_DTYPE_BF16, 1>(gp, gs, grid, block, smem, stream);
-    else if (rmax == 2) launch_rmax<Q4_DTYPE_BF16, 2>(gp, gs, grid, block, smem, stream);
-    else launch_rmax<Q4_DTYPE_BF16, 4>(gp, gs, grid, block, smem, stream);
+    if (rmax == 1) launch_rmax<Q4_DTYPE_BF16, 1>(w, gp, grid, block, smem, stream);
+    else if (rmax == 2) launch_rmax<Q4_DTYPE_BF16, 2>(w, gp, grid, block, smem, stream);
+    else launch_rmax<Q4_DTYPE_BF16, 4>(w, gp, grid, block, smem, stream);
   }
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {

@@ -186,7 +186,15 @@ def linear(
     lib = _lib.load()
     with torch.cuda.device(x.device):
         stream = _stream_handle(x.device)
-        ws = reserve_workspace(x.device, workspace_bytes(min(M, 16), w.K, w.N), stream)
+        st = w.struct()
+        # only the decode kernels use the workspace (split-K partials + tickets)
+        chosen = path
+        if chosen == PATH_AUTO and gemv_config is None:
+            chosen = lib.q4_select_path(ctypes.byref(st), M, _DTYPES[x.dtype])
+        need = _lib.WORKSPACE_COUNTER_BYTES
+        if chosen == _lib.PATH_GEMV:
+            need = workspace_bytes(M, w.K, w.N)
+        ws = reserve_workspace(x.device, need, stream)
         st = w.struct()
         if gemv_config is not None:
             wcol, wk, splits = gemv_config
