@@ -153,8 +153,8 @@ def test_auto_dispatch(pkg, oracle, gpu):
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
     assert pkg.ops.select_path(pk, 1) == "gemv"
     assert pkg.ops.select_path(pk, 16) == "gemv"
-    assert pkg.ops.select_path(pk, 17) == "gemm"
-    assert pkg.ops.select_path(pk, 2048) == "gemm"
+    assert pkg.ops.select_path(pk, 2048) == "gemv"   # M * N <= 2^20: row-chunked decode
+    assert pkg.ops.select_path(pk, 2049) == "gemm"
     qw, qz, sc, _ = oracle.make_gptq(1000, 264, 40, seed=3)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 40, 0)
     assert pkg.ops.select_path(pk, 1) == "generic"

@@ -84,8 +84,11 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   if (validate_weight(w, "q4_select_path") != Q4_OK) return Q4_ERR_INVALID_ARGUMENT;
   const bool contiguous_gptq = w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr;
   if (contiguous_gptq) {
-    // decode kernel up to one MFMA row block, the MFMA GEMM above
-    if (M <= 16 && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
+    // Measured crossover on MI355X (Llama-3-8B shapes): the row-chunked decode kernel wins
+    // while M * N <= 2^20 (the GEMM grid of 128 x 256 tiles does not fill the 256 CUs
+    // below that); the MFMA GEMM wins above.
+    const bool small = M <= 16 || (long)M * w->N <= (1L << 20);
+    if (small && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
     if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;
     if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
     return Q4_PATH_GENERIC;

@@ -727,11 +727,15 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M) {
   const int chunks = w->K / 128;
   c.wcol = 1;
   c.wk = chunks % 4 == 0 ? 4 : (chunks % 2 == 0 ? 2 : 1);
+  // wide layers with many rows: two column tiles per workgroup halve the slab staging
+  if (w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && M >= 8 && w->N % 128 == 0 &&
+      w->N / 64 >= 256)
+    c.wcol = 2;
   const bool act = w->layout == Q4_LAYOUT_GPTQ && w->g_idx != nullptr;
   if (act && chunks % 8 == 0) c.wk = 8;  // the group table is built once per workgroup
   const int per_wg = chunks / c.wk;      // chunks left to distribute over splits x per-wave work
   const int wave_cols = w->layout == Q4_LAYOUT_AWQ ? 256 : 64;
-  const int ntiles = (w->N / wave_cols) * mchunks;
+  const int ntiles = (w->N / (wave_cols * c.wcol)) * mchunks;
   const int target_wgs = M <= 4 ? 512 : 384;  // partial-sum traffic grows with M
   int want = (target_wgs + ntiles / 2) / ntiles;
   if (want < 1) want = 1;
