@@ -33,6 +33,9 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E peak
 MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16/bf16 MFMA peak
 
+# FETCH_SIZE 14334.3 KiB x 2.000 (copy-kernel calibration) + WRITE_SIZE 369.3 KiB x 1.000
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 29734758
+
 SHAPES = [  # name, K, N
     ("qkv_proj", 4096, 6144),
     ("o_proj", 4096, 4096),
@@ -265,7 +268,10 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": None,
+        # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this
+        # workload (mean over the four projections, calibrated with a 256 MiB copy kernel);
+        # only valid for the default M=1 workload, null otherwise
+        "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if M == 1 else None,
         "bytes_per_launch": all_bytes // len(SHAPES),
         "us_per_launch": round(sum(all_durs) / len(SHAPES) * 1e6, 2),
     }
