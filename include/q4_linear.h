@@ -96,12 +96,15 @@ int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, i
 /*
  * Decode kernel with an explicit work decomposition, for tuning sweeps: `wcol` waves
  * across columns and `wk` waves across K per workgroup (wcol * wk <= 8), `splits`
- * workgroups across K.  K must be a multiple of 128 * wk * splits and N of 64 * wcol.
+ * workgroups across K, `words` packed words per lane (4, 2 or 1: column tiles of 64, 32 or
+ * 16 per wave; GPTQ layout with contiguous groups of at least 128 rows, otherwise forced to
+ * 4; the AWQ kernel's tile is 256 columns).  K must be a multiple of 128 * wk * splits and
+ * N of tile * wcol.
  * Plays the role of exllama's `set_tuning_params`
  * (server/exllama_kernels/exllama_kernels/exllama_ext.cpp:78-100) without global state.
  */
 int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
-                  void* workspace, size_t workspace_bytes, int wcol, int wk, int splits,
+                  void* workspace, size_t workspace_bytes, int wcol, int wk, int splits, int words,
                   void* stream);
 
 /*

@@ -227,3 +227,15 @@ def test_act_order_bit_exact_weights_through_identity(pkg, oracle, gpu):
 def test_gptq_decode_m_chunks(pkg, oracle, gpu):
     """The GPTQ decode kernel also runs M > 16 in row chunks when forced."""
     _run(pkg, oracle, gpu, 1024, 512, 128, 50, sym=False, bias=True, path=1, seed=50)
+
+
+@pytest.mark.parametrize("cfg", [(1, 8, 1, 1), (1, 4, 2, 1), (2, 4, 1, 2), (1, 8, 1, 2), (4, 2, 1, 1), (1, 1, 4, 2)])
+@pytest.mark.parametrize("M", [1, 2, 7, 16])
+def test_gemv_narrow_column_tiles(pkg, oracle, gpu, cfg, M):
+    """16- and 32-column tiles per wave (1 or 2 packed words per lane) of the GPTQ decode kernel."""
+    _run(pkg, oracle, gpu, 1024, 512, 128, M, sym=False, bias=(M == 7), cfg=cfg, seed=sum(cfg) + M)
+
+
+@pytest.mark.parametrize("gs", [256, -1])
+def test_gemv_narrow_tiles_large_groups(pkg, oracle, gpu, gs):
+    _run(pkg, oracle, gpu, 1024, 256, gs, 3, sym=False, cfg=(1, 4, 1, 1), seed=gs + 1)

@@ -61,7 +61,7 @@ SIGNATURES = {
     ),
     "q4_gemv_tuned": (
         c_int,
-        [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_size_t, c_int, c_int, c_int, c_void_p],
+        [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p],
     ),
     "q4_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "q4_select_path": (c_int, [POINTER(Q4Weight), c_int, c_int]),

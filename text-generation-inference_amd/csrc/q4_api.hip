@@ -158,7 +158,7 @@ int q4_linear(const q4_weight* w, const void* x, const void* bias, void* y, int 
 }
 
 int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
-                  void* workspace, size_t workspace_bytes, int wcol, int wk, int splits,
+                  void* workspace, size_t workspace_bytes, int wcol, int wk, int splits, int words,
                   void* stream) {
   int rc = validate_weight(w, "q4_gemv_tuned");
   if (rc == Q4_OK) rc = validate_dtype(dtype, "q4_gemv_tuned");
@@ -167,7 +167,7 @@ int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, 
     set_error("q4_gemv_tuned: bad M=%d or null x/y", M);
     return Q4_ERR_INVALID_ARGUMENT;
   }
-  GemvConfig cfg{wcol, wk, splits};
+  GemvConfig cfg{wcol, wk, splits, words};
   return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, &cfg, (hipStream_t)stream);
 }
 

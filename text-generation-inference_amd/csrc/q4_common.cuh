@@ -123,9 +123,10 @@ int launch_dequant(const q4_weight* w, void* w_out, int dtype, hipStream_t strea
 int launch_generic(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                    hipStream_t stream);
 struct GemvConfig {
-  int wcol;    // waves across columns in a workgroup (64 columns each)
+  int wcol;    // waves across columns in a workgroup (one column tile each)
   int wk;      // waves across K in a workgroup
   int splits;  // workgroups across K (cross-workgroup reduction through the workspace)
+  int words;   // GPTQ contiguous-group kernel: packed words per lane (4, 2, 1 -> 64/32/16-column tiles)
 };
 bool gemv_supported(const q4_weight* w, int M, int dtype);
 GemvConfig gemv_pick_config(const q4_weight* w, int M);

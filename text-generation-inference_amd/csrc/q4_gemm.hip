@@ -118,22 +118,34 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
   const int kq = lane >> 5;
   const int N = p.N, K = p.K, M = p.M;
 
-  // XCD-aware tile order: consecutive workgroup ids go to different XCDs, so a group of 8
-  // consecutive ids shares nothing; ids that land on one XCD (id % 8 equal) walk the M
-  // tiles of one column block first and re-use its packed weights from that XCD's L2.
+  // XCD-aware tile order.  Workgroup ids are dealt round-robin to the 8 XCDs (id % 8), each
+  // with its own L2.  Every XCD is given its own slice of M tiles and walks all column
+  // blocks of it: the activation rows of the slice (BM x K, a few MB) stay resident in that
+  // XCD's L2 and are re-read from there by every column block, while the packed weights are
+  // the streamed operand (each column block is read once per XCD, prefetched ahead).
+  // (A grid of a single round, at most one workgroup per CU, measured faster the other way
+  // round: each XCD takes a few column blocks and all M tiles of them.)
   const int tiles_m = (M + BM - 1) / BM;
   const int tiles_n = N / kBN;
-  int bid = blockIdx.x;
+  int tm, tn;
   {
+    const int bid = blockIdx.x;
     const int total = tiles_m * tiles_n;
-    const int per_xcd = (total + 7) / 8;
-    const int xcd = bid & 7;
-    const int local = bid >> 3;
-    const int lin = xcd * per_xcd + local;
-    bid = lin < total && (total % 8 == 0) ? lin : bid;
+    if (tiles_m % 8 == 0 && total > 256) {
+      const int mpx = tiles_m >> 3;  // M tiles per XCD
+      const int xcd = bid & 7;
+      const int local = bid >> 3;
+      tm = xcd * mpx + local % mpx;
+      tn = local / mpx;
+    } else if (total % 8 == 0) {
+      const int lin = (bid & 7) * (total >> 3) + (bid >> 3);
+      tm = lin % tiles_m;
+      tn = lin / tiles_m;
+    } else {
+      tm = bid % tiles_m;
+      tn = bid / tiles_m;
+    }
   }
-  const int tm = bid % tiles_m;
-  const int tn = bid / tiles_m;
   const int m0 = tm * BM;
   const int n0 = tn * kBN;
   const int nw = n0 + wave * 64;   // first column of this wave

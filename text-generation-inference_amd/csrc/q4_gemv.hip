@@ -223,16 +223,21 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
         const int m = 4 * d.kq + r;
         if (m < d.mloc) {
           uint16_t* dst = y + (size_t)(d.mb + m) * N + col0;
+          uint16_t o[NT];
 #pragma unroll
-          for (int t = 0; t < NT; t += 4) {
-            uint16_t o[4];
+          for (int t = 0; t < NT; ++t) o[t] = finish_output<DTYPE>(out[t][r], p.bias, col0 + t);
+          if constexpr (NT == 1) {
+            dst[0] = o[0];
+          } else if constexpr (NT == 2) {
+            *(uint32_t*)dst = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+          } else {
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
-              o[u] = finish_output<DTYPE>(out[t + u][r], p.bias, col0 + t + u);
-            uint2_t packed;
-            packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
-            packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
-            *(uint2_t*)(dst + t) = packed;
+            for (int t = 0; t < NT; t += 4) {
+              uint2_t packed;
+              packed.x = (uint32_t)o[t] | ((uint32_t)o[t + 1] << 16);
+              packed.y = (uint32_t)o[t + 2] | ((uint32_t)o[t + 3] << 16);
+              *(uint2_t*)(dst + t) = packed;
+            }
           }
         }
       }
@@ -299,45 +304,71 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
 // GPTQ, contiguous groups.
 // GSTEPS: MFMA steps (32 rows) per quantisation group inside a chunk: 1, 2 or 4.
 // STATIC128: groupsize is exactly 128, so every chunk is one whole group.
-template <int DTYPE, int RMAX, int GSTEPS, bool STATIC128>
+// WORDS: adjacent packed words (columns) per lane: 4, 2 or 1, i.e. column tiles of 64, 32
+// or 16 per wave.  Narrow tiles give enough workgroups to fill the chip without splitting
+// K across workgroups, which removes the cross-workgroup reduction tail of small layers.
+template <int DTYPE, int RMAX, int GSTEPS, bool STATIC128, int WORDS>
 __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   extern __shared__ __align__(16) unsigned char smem[];
   const Problem& p = gp.p;
-  const Decomp d = make_decomp(gp, 64);
+  const Decomp d = make_decomp(gp, 16 * WORDS);
   const int N = p.N;
-  const int nl = d.tile * d.tile_cols + d.wc * 64 + 4 * d.j;  // first of this lane's 4 columns
+  const int nl = d.tile * d.tile_cols + d.wc * 16 * WORDS + WORDS * d.j;  // lane's first column
   const int nchunks = d.KW / kChunkRows;
   constexpr int GPC = kChunkSteps / GSTEPS;  // groups per chunk
+  constexpr int PF = kPrefetch * 4 / WORDS;  // chunks in flight: same bytes for every WORDS
 
   SlabStager<true> slab;
   slab.issue(gp, d);
 
-  // ---- issue the first kPrefetch chunks of weight loads.  Addresses are a wave-uniform
-  // 64-bit base plus a per-lane 32-bit byte offset.
+  // ---- issue the first PF chunks of weight loads.  Addresses are a wave-uniform 64-bit
+  // base plus a per-lane 32-bit byte offset.
   const char* wbase = (const char*)(p.qweight + (size_t)(d.kw0 / 8) * N);
   const uint32_t w_lane = ((uint32_t)d.kq * (uint32_t)N + (uint32_t)nl) * 4u;
   const size_t step_bytes = (size_t)N * 16;  // four packed rows
   const uint32_t s_lane = (uint32_t)nl * 2u;
   const uint32_t z_lane = (uint32_t)(nl >> 3) * 4u;
-  const int zshift = (nl & 4) * 4;
-  uint4_t wq[kPrefetch][kChunkSteps];
-  uint2_t sc[kPrefetch][GPC];
-  uint32_t zw[kPrefetch][GPC];
-  auto load_chunk = [&](int c, uint4_t (&w)[kChunkSteps], uint2_t (&s)[GPC], uint32_t (&z)[GPC]) {
+  const int zshift = (nl & 7) * 4;
+  struct Words { uint32_t v[WORDS]; };
+  struct Scales { uint32_t v[(WORDS + 1) / 2]; };  // WORDS fp16 scales
+  Words wq[PF][kChunkSteps];
+  Scales sc[PF][GPC];
+  uint32_t zw[PF][GPC];
+  auto load_words = [&](const char* addr) {
+    Words r;
+    if constexpr (WORDS == 4) {
+      const uint4_t t = __builtin_nontemporal_load((const uint4_t*)addr);
+      r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w;
+    } else if constexpr (WORDS == 2) {
+      const uint2_t t = __builtin_nontemporal_load((const uint2_t*)addr);
+      r.v[0] = t.x; r.v[1] = t.y;
+    } else {
+      r.v[0] = __builtin_nontemporal_load((const uint32_t*)addr);
+    }
+    return r;
+  };
+  auto load_chunk = [&](int c, Words (&w)[kChunkSteps], Scales (&s)[GPC], uint32_t (&z)[GPC]) {
 #pragma unroll
     for (int st = 0; st < kChunkSteps; ++st)
-      w[st] = __builtin_nontemporal_load(
-          (const uint4_t*)(wbase + (size_t)(c * kChunkSteps + st) * step_bytes + w_lane));
+      w[st] = load_words(wbase + (size_t)(c * kChunkSteps + st) * step_bytes + w_lane);
 #pragma unroll
     for (int g = 0; g < GPC; ++g) {
       int gi = (d.kw0 + c * kChunkRows + g * GSTEPS * 32) / p.groupsize;
       gi = min(gi, p.num_groups - 1);
-      s[g] = *(const uint2_t*)((const char*)p.scales + (size_t)gi * N * 2 + s_lane);
+      const char* sp = (const char*)p.scales + (size_t)gi * N * 2 + s_lane;
+      if constexpr (WORDS == 4) {
+        const uint2_t t = *(const uint2_t*)sp;
+        s[g].v[0] = t.x; s[g].v[1] = t.y;
+      } else if constexpr (WORDS == 2) {
+        s[g].v[0] = *(const uint32_t*)sp;
+      } else {
+        s[g].v[0] = *(const uint16_t*)sp;
+      }
       z[g] = *(const uint32_t*)((const char*)p.qzeros + (size_t)gi * (N >> 3) * 4 + z_lane);
     }
   };
 #pragma unroll
-  for (int b = 0; b < kPrefetch; ++b)
+  for (int b = 0; b < PF; ++b)
     if (b < nchunks) load_chunk(b, wq[b], sc[b], zw[b]);
 
   slab.store(gp, d, smem);
@@ -348,12 +379,13 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
       smem + (size_t)d.j * gp.slab_stride + (size_t)(d.wkk * d.KW + d.kq * 8) * 2;
 
   const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-  float4_t tot[4] = {zero4, zero4, zero4, zero4};
-  float4_t acc[4] = {zero4, zero4, zero4, zero4};
-  half2_t czlo[4], czhi[4];
+  float4_t tot[WORDS], acc[WORDS];
+#pragma unroll
+  for (int t = 0; t < WORDS; ++t) tot[t] = acc[t] = zero4;
+  half2_t czlo[WORDS], czhi[WORDS];
   const SpliceConsts splice = splice_consts();
 
-  auto process_chunk = [&](int c, const uint4_t (&w)[kChunkSteps], const uint2_t (&s)[GPC],
+  auto process_chunk = [&](int c, const Words (&w)[kChunkSteps], const Scales (&s)[GPC],
                            const uint32_t (&z)[GPC]) {
     const int kc = d.kw0 + c * kChunkRows;
     bool group_start = true, group_end = true;
@@ -371,7 +403,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
         // zero-point constants of the group: z = (stored + 1) & 15 per column
         const uint32_t z4 = gptq_zero_plus_one(z[gi]) >> zshift;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < WORDS; ++t) {
           const uint32_t zz = (z4 >> (4 * t)) & 0xFu;
           czlo[t] = as_half2(0xE400E400u | zz | (zz << 16));        // -(1024 + z)
           czhi[t] = as_half2(0xD400D400u | (zz << 4) | (zz << 20));  // -(64 + z)
@@ -379,11 +411,10 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
       }
       uint4_t a = {0u, 0u, 0u, 0u};
       if (row_live) a = *(const uint4_t*)(a_base + (size_t)(c * kChunkRows + st * 32) * 2);
-      const uint32_t words[4] = {w[st].x, w[st].y, w[st].z, w[st].w};
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
+      for (int t = 0; t < WORDS; ++t) {
         half2_t b[4];
-        unpack_word_f16(words[t], czlo[t], czhi[t], splice, b);
+        unpack_word_f16(w[st].v[t], czlo[t], czhi[t], splice, b);
         if (first && kStaticGroups) {
           acc[t] = mfma16<DTYPE>(a, b, zero4);
         } else {
@@ -392,35 +423,35 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
         }
       }
       if (last && (kStaticGroups || group_end)) {
-        const half2_t s01 = as_half2(s[gi].x), s23 = as_half2(s[gi].y);
-        const float sf[4] = {(float)s01.x, (float)s01.y, (float)s23.x, (float)s23.y};
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < WORDS; ++t) {
+          const half2_t pr = as_half2(s[gi].v[t >> 1]);
+          const float sf = (float)((t & 1) ? pr.y : pr.x);
 #pragma unroll
-          for (int r = 0; r < RMAX; ++r) tot[t][r] = fmaf(sf[t], acc[t][r], tot[t][r]);
+          for (int r = 0; r < RMAX; ++r) tot[t][r] = fmaf(sf, acc[t][r], tot[t][r]);
         }
       }
     }
   };
 
-  // ring of kPrefetch chunk buffers: consume slot b, then refill it with chunk c + kPrefetch
-  for (int c0 = 0; c0 < nchunks; c0 += kPrefetch) {
+  // ring of PF chunk buffers: consume slot b, then refill it with chunk c + PF
+  for (int c0 = 0; c0 < nchunks; c0 += PF) {
 #pragma unroll
-    for (int b = 0; b < kPrefetch; ++b) {
+    for (int b = 0; b < PF; ++b) {
       const int c = c0 + b;
       if (c < nchunks) {
         process_chunk(c, wq[b], sc[b], zw[b]);
-        if (c + kPrefetch < nchunks) load_chunk(c + kPrefetch, wq[b], sc[b], zw[b]);
+        if (c + PF < nchunks) load_chunk(c + PF, wq[b], sc[b], zw[b]);
       }
     }
   }
 
-  float out[4][RMAX];
+  float out[WORDS][RMAX];
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int t = 0; t < WORDS; ++t)
 #pragma unroll
     for (int r = 0; r < RMAX; ++r) out[t][r] = tot[t][r];
-  gemv_finish<DTYPE, 4, RMAX>(gp, d, out, nl, smem);
+  gemv_finish<DTYPE, WORDS, RMAX>(gp, d, out, nl, smem);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -706,7 +737,7 @@ bool gemv_supported(const q4_weight* w, int M, int dtype) {
     return chunks * (w->N / 256) <= Q4_WORKSPACE_COUNTER_BYTES / 4;
   }
   if (w->N % 64 != 0) return false;
-  if (chunks * (w->N / 64) > Q4_WORKSPACE_COUNTER_BYTES / 4) return false;
+  if (chunks * (w->N / 16) > Q4_WORKSPACE_COUNTER_BYTES / 4 && M > 16) return false;
   if (w->g_idx != nullptr) {
     // act-order: the table of all groups for 64 columns must fit LDS next to the slab
     if (dtype != Q4_DTYPE_F16) return false;
@@ -722,6 +753,7 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M) {
   // workgroups start too slowly and more splits lengthen the reduction tail.  The
   // activation slab (rows x K/splits) must fit its share of LDS.
   GemvConfig c;
+  c.words = 4;
   const int rows = M < q4::kRowsPerBlock ? M : q4::kRowsPerBlock;
   const int mchunks = (M + q4::kRowsPerBlock - 1) / q4::kRowsPerBlock;
   const int chunks = w->K / 128;
@@ -768,7 +800,7 @@ static void launch_kernel(Kernel k, const GemvParams& gp, dim3 grid, dim3 block,
 }
 
 template <int DTYPE, int RMAX>
-static void launch_rmax(const q4_weight* w, const GemvParams& gp, dim3 grid, dim3 block,
+static void launch_rmax(const q4_weight* w, const GemvParams& gp, int words, dim3 grid, dim3 block,
                         size_t smem, hipStream_t stream) {
   using namespace q4;
   const int gs = w->groupsize;
@@ -777,13 +809,17 @@ static void launch_rmax(const q4_weight* w, const GemvParams& gp, dim3 grid, dim
   } else if (w->g_idx != nullptr) {
     launch_kernel(gemv_gptq_act_kernel<RMAX>, gp, grid, block, smem, stream);
   } else if (gs == 128) {
-    launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, true>, gp, grid, block, smem, stream);
+    if (words == 4) launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, true, 4>, gp, grid, block, smem, stream);
+    else if (words == 2) launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, true, 2>, gp, grid, block, smem, stream);
+    else launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, true, 1>, gp, grid, block, smem, stream);
   } else if (gs > 128) {
-    launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, false>, gp, grid, block, smem, stream);
+    if (words == 4) launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, false, 4>, gp, grid, block, smem, stream);
+    else if (words == 2) launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, false, 2>, gp, grid, block, smem, stream);
+    else launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, false, 1>, gp, grid, block, smem, stream);
   } else if (gs == 64) {
-    launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 2, false>, gp, grid, block, smem, stream);
+    launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 2, false, 4>, gp, grid, block, smem, stream);
   } else {
-    launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 1, false>, gp, grid, block, smem, stream);
+    launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 1, false, 4>, gp, grid, block, smem, stream);
   }
 }
 
@@ -798,8 +834,14 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   }
   const bool awq = w->layout == Q4_LAYOUT_AWQ;
   const bool act = !awq && w->g_idx != nullptr;
-  const int wave_cols = awq ? 256 : 64;
-  const GemvConfig cfg = cfg_in ? *cfg_in : gemv_pick_config(w, M);
+  GemvConfig cfg = cfg_in ? *cfg_in : gemv_pick_config(w, M);
+  const bool contiguous = !awq && !act;
+  if (!contiguous || w->groupsize < 128) cfg.words = 4;  // only the contiguous-group kernel has narrow tiles
+  if (cfg.words != 1 && cfg.words != 2 && cfg.words != 4) {
+    set_error("q4_linear(gemv): words per lane must be 1, 2 or 4 (got %d)", cfg.words);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  const int wave_cols = awq ? 256 : 16 * cfg.words;
   if (cfg.wcol < 1 || cfg.wk < 1 || cfg.splits < 1 || cfg.wcol * cfg.wk > 8 ||
       w->N % (wave_cols * cfg.wcol) != 0 || w->K % (cfg.splits * cfg.wk * 128) != 0) {
     set_error("q4_linear(gemv): bad config wcol=%d wk=%d splits=%d for K=%d N=%d", cfg.wcol, cfg.wk,
@@ -811,7 +853,7 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   const int KR = w->K / cfg.splits;
   const int slab_stride = KR * 2 + 16;
   const int rmax = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
-  const int nt = awq ? 16 : 4;
+  const int nt = awq ? 16 : cfg.words;
   const size_t slab_bytes = ((size_t)rows * slab_stride + 15) & ~(size_t)15;
   size_t smem = slab_bytes;
   if (act) smem += (((size_t)KR * 2 + 15) & ~(size_t)15) + (size_t)w->num_groups * 64 * cfg.wcol * 4;
@@ -851,13 +893,13 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   dim3 grid((unsigned)(ntiles * cfg.splits), (unsigned)mchunks);
   dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
   if (dtype == Q4_DTYPE_F16) {
-    if (rmax == 1) launch_rmax<Q4_DTYPE_F16, 1>(w, gp, grid, block, smem, stream);
-    else if (rmax == 2) launch_rmax<Q4_DTYPE_F16, 2>(w, gp, grid, block, smem, stream);
-    else launch_rmax<Q4_DTYPE_F16, 4>(w, gp, grid, block, smem, stream);
+    if (rmax == 1) launch_rmax<Q4_DTYPE_F16, 1>(w, gp, cfg.words, grid, block, smem, stream);
+    else if (rmax == 2) launch_rmax<Q4_DTYPE_F16, 2>(w, gp, cfg.words, grid, block, smem, stream);
+    else launch_rmax<Q4_DTYPE_F16, 4>(w, gp, cfg.words, grid, block, smem, stream);
   } else {
-    if (rmax == 1) launch_rmax<Q4_DTYPE_BF16, 1>(w, gp, grid, block, smem, stream);
-    else if (rmax == 2) launch_rmax<Q4_DTYPE_BF16, 2>(w, gp, grid, block, smem, stream);
-    else launch_rmax<Q4_DTYPE_BF16, 4>(w, gp, grid, block, smem, stream);
+    if (rmax == 1) launch_rmax<Q4_DTYPE_BF16, 1>(w, gp, cfg.words, grid, block, smem, stream);
+    else if (rmax == 2) launch_rmax<Q4_DTYPE_BF16, 2>(w, gp, cfg.words, grid, block, smem, stream);
+    else launch_rmax<Q4_DTYPE_BF16, 4>(w, gp, cfg.words, grid, block, smem, stream);
   }
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {

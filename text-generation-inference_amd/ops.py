@@ -154,7 +154,7 @@ def linear(
     x: torch.Tensor,
     bias: Optional[torch.Tensor] = None,
     path: int = PATH_AUTO,
-    gemv_config: Optional[tuple[int, int, int]] = None,
+    gemv_config: Optional[tuple] = None,
     out: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """y[M, N] = x[M, K] @ dequant(W) (+ bias) on the current stream of x's device.
@@ -197,13 +197,14 @@ def linear(
         ws = reserve_workspace(x.device, need, stream)
         st = w.struct()
         if gemv_config is not None:
-            wcol, wk, splits = gemv_config
+            wcol, wk, splits = gemv_config[:3]
+            words = gemv_config[3] if len(gemv_config) > 3 else 4
             need = _lib.WORKSPACE_COUNTER_BYTES + splits * M * w.N * 4
             if ws.numel() < need:
                 ws = reserve_workspace(x.device, need, stream)
             rc = lib.q4_gemv_tuned(
                 ctypes.byref(st), x.data_ptr(), bias_ptr, y.data_ptr(), M, _DTYPES[x.dtype],
-                ws.data_ptr(), ws.numel(), wcol, wk, splits, stream,
+                ws.data_ptr(), ws.numel(), wcol, wk, splits, words, stream,
             )
         else:
             rc = lib.q4_linear_ex(
