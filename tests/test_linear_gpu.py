@@ -192,7 +192,7 @@ def test_awq_auto_path_is_native(pkg, oracle, gpu):
     qw, qz, sc = oracle.make_awq(1024, 512, 128, seed=0)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 1)
     for M in (1, 16, 100, 256):
-        assert pkg.ops.select_path(pk, M) == "gemv"
+        assert pkg.ops.select_path(pk, M) == "gemv"  # M * N <= 0.75 * 2^20 for N = 512
 
 
 @pytest.mark.parametrize("K,N", [(8192, 10240), (28672, 8192)])
@@ -239,3 +239,35 @@ def test_gemv_narrow_column_tiles(pkg, oracle, gpu, cfg, M):
 @pytest.mark.parametrize("gs", [256, -1])
 def test_gemv_narrow_tiles_large_groups(pkg, oracle, gpu, gs):
     _run(pkg, oracle, gpu, 1024, 256, gs, 3, sym=False, cfg=(1, 4, 1, 1), seed=gs + 1)
+
+
+# --------------------------------------------------------------------------- AWQ prefill GEMM
+
+
+@pytest.mark.parametrize("K,N,M", [(4096, 14336, 256), (14336, 4096, 512), (1024, 512, 130)])
+def test_awq_gemm(pkg, oracle, gpu, K, N, M):
+    """AWQ layout through the MFMA kernel that unpacks the weight tile into LDS."""
+    _run(pkg, oracle, gpu, K, N, 128, M, layout="awq", path=2, bias=(M == 130), seed=K // 512 + M)
+
+
+@pytest.mark.parametrize("gs", [32, 64, 128, -1])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_awq_gemm_groupsizes_dtypes(pkg, oracle, gpu, gs, dtype):
+    _run(pkg, oracle, gpu, 512, 256, gs, 100, dtype=dtype, layout="awq", path=2, seed=gs + 11)
+
+
+def test_awq_gemm_bit_exact_weights_through_identity(pkg, oracle, gpu):
+    K, N, gs = 512, 256, 128
+    qw, qz, sc = oracle.make_awq(K, N, gs, seed=31)
+    w = oracle.dequant_awq(qw, qz, sc, gs, "f16")
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, gs, 1)
+    eye = torch.eye(K, dtype=torch.float16, device=gpu)
+    got = pkg.ops.linear(pk, eye, None, path=2)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), w.view(np.uint16))
+
+
+def test_awq_dispatch_large_m(pkg, oracle, gpu):
+    qw, qz, sc = oracle.make_awq(1024, 14336, 128, seed=0)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 1)
+    assert pkg.ops.select_path(pk, 48) == "gemv"
+    assert pkg.ops.select_path(pk, 64) == "gemm"

@@ -132,6 +132,9 @@ bool gemv_supported(const q4_weight* w, int M, int dtype);
 GemvConfig gemv_pick_config(const q4_weight* w, int M);
 int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                 void* workspace, size_t workspace_bytes, const GemvConfig* cfg, hipStream_t stream);
+bool gemm_awq_supported(const q4_weight* w, int M, int dtype);
+int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                    hipStream_t stream);
 bool gemm_supported(const q4_weight* w, int M, int dtype);
 int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                 hipStream_t stream);

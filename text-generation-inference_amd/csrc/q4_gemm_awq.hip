@@ -1,0 +1,263 @@
+// Prefill path for the AWQ layout: y[M, N] = x @ dequant(W) on the MFMA units (gfx950).
+//
+// An AWQ word holds 8 interleaved columns of ONE K row, so it is not an MFMA operand by
+// itself.  The weight tile is therefore unpacked cooperatively into LDS (the classic
+// dequantize-to-LDS stage) and both operands are read from there:
+//   * workgroup = 4 waves in a 2 x 2 arrangement, tile 128 x 128, K tile 64; each wave owns
+//     a 64 x 64 block = 2 x 2 MFMA tiles of v_mfma_f32_32x32x16 (64 accumulator VGPRs),
+//     so two or three workgroups share a CU and cover each other's barriers;
+//   * producer: thread t < 128 owns an 8-row x 1-word patch (8 rows of one K block, 8
+//     columns).  One byte permute per row pair and byte puts the same nibble positions of
+//     two rows side by side, the mantissa splice turns them into halves, zero points are
+//     subtracted exactly and each weight is multiplied once by its fp16 scale (the
+//     reference's rounding).  The patch becomes eight 16-byte units (one per column,
+//     8 consecutive K values each) written to LDS at [K block][column];
+//   * LDS layouts: activations [row][K block] with the row stride padded to 9 units,
+//     weights [K block][column]; both give conflict-free 128-bit fragment reads;
+//   * double-buffered LDS, global loads for tile k+2 in flight while tile k is multiplied.
+#include "q4_common.cuh"
+
+namespace q4 {
+
+constexpr int kABM = 128;  // rows per workgroup
+constexpr int kABN = 128;  // columns per workgroup
+constexpr int kABK = 64;   // K rows per tile
+constexpr int kAUnits = kABK / 8 + 1;  // padded units per activation row
+
+struct AwqGemmParams {
+  Problem p;
+};
+
+struct AwqSplice {
+  uint32_t mask_lo, mask_hi, magic;
+};
+__device__ __forceinline__ AwqSplice awq_splice_consts() {
+  // registers instead of literals so that (w & mask) | magic selects v_and_or_b32
+  AwqSplice k{0x000F000Fu, 0x00F000F0u, 0x64006400u};
+  asm volatile("" : "+s"(k.mask_lo), "+s"(k.mask_hi), "+v"(k.magic));
+  return k;
+}
+
+typedef __bf16 awq_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float awq_float2_t __attribute__((ext_vector_type(2)));
+
+template <int DTYPE>
+__global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
+  constexpr int A_TILE = kABM * kAUnits * 16;   // bytes
+  constexpr int B_TILE = (kABK / 8) * kABN * 16;
+  constexpr int A_LOADS = kABM * (kABK / 8) / 256;  // 16-byte activation loads per thread
+  extern __shared__ __align__(16) unsigned char smem[];  // [A0][A1][B0][B1]
+  const Problem& p = gp.p;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int j = lane & 31;
+  const int kq = lane >> 5;
+  const int N = p.N, K = p.K, M = p.M;
+  const int NC = N >> 3;
+  const int tiles_m = (M + kABM - 1) / kABM;
+  const int tm = blockIdx.x % tiles_m;
+  const int tn = blockIdx.x / tiles_m;
+  const int m0 = tm * kABM;
+  const int n0 = tn * kABN;
+  const int KT = K / kABK;
+  const int last_tile = KT - 1;
+  const AwqSplice splice = awq_splice_consts();
+
+  // ---- producer state: threads 0..127 own K block pb (8 rows) x word pc (8 columns)
+  const bool producer = tid < 128;
+  const int pb = (tid >> 4) & 7;
+  const int pc = tid & 15;
+  const uint32_t* wsrc = p.qweight + (size_t)(pb * 8) * NC + (n0 >> 3) + pc;
+  uint32_t braw[8];
+  uint4_t sraw;   // 8 fp16 scales of the word's columns
+  uint32_t zraw;  // 8 zero-point nibbles
+  auto load_b = [&](int kt) {
+    if (producer) {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) braw[r] = wsrc[(size_t)(kt * kABK + r) * NC];
+      const int g = min((kt * kABK + pb * 8) / p.groupsize, p.num_groups - 1);
+      sraw = *(const uint4_t*)(p.scales + (size_t)g * N + n0 + pc * 8);
+      zraw = p.qzeros[(size_t)g * NC + (n0 >> 3) + pc];
+    }
+  };
+  auto store_b = [&](int buf) {
+    if (!producer) return;
+    unsigned char* base = smem + 2 * A_TILE + buf * B_TILE;
+    const uint32_t su[4] = {sraw.x, sraw.y, sraw.z, sraw.w};
+    const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+    half2_t d[8][4];  // [nibble position][row pair]: exact q - z
+#pragma unroll
+    for (int rp = 0; rp < 4; ++rp) {
+#pragma unroll
+      for (int by = 0; by < 4; ++by) {
+        const uint32_t sel = 0x0C000C00u | (uint32_t)by | ((uint32_t)(4 + by) << 16);
+        const uint32_t t2 = __builtin_amdgcn_perm(braw[2 * rp + 1], braw[2 * rp], sel);
+        const uint32_t ze = (zraw >> (8 * by)) & 0xFu;       // position 2*by
+        const uint32_t zo = (zraw >> (8 * by + 4)) & 0xFu;   // position 2*by + 1
+        d[2 * by][rp] = as_half2((t2 & splice.mask_lo) | splice.magic) +
+                        as_half2(0xE400E400u | ze | (ze << 16));
+        d[2 * by + 1][rp] = as_half2((t2 & splice.mask_hi) | splice.magic) * sixteenth +
+                            as_half2(0xD400D400u | (zo << 4) | (zo << 20));
+      }
+    }
+#pragma unroll
+    for (int pos = 0; pos < 8; ++pos) {
+      const int col = ((pos & 3) << 1) | (pos >> 2);  // logical column of this nibble position
+      const half2_t pr = as_half2(su[col >> 1]);
+      const half_t s = (col & 1) ? pr.y : pr.x;
+      uint4_t unit;
+      uint32_t o[4];
+#pragma unroll
+      for (int rp = 0; rp < 4; ++rp) {
+        if constexpr (DTYPE == Q4_DTYPE_F16) {
+          o[rp] = as_u32(d[pos][rp] * half2_t{s, s});  // one fp16 rounding per weight
+        } else {
+          const awq_float2_t f = {(float)d[pos][rp].x * (float)s, (float)d[pos][rp].y * (float)s};
+          o[rp] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, awq_bf16x2_t));
+        }
+      }
+      unit.x = o[0]; unit.y = o[1]; unit.z = o[2]; unit.w = o[3];
+      *(uint4_t*)(base + ((size_t)pb * kABN + pc * 8 + col) * 16) = unit;
+    }
+  };
+
+  // ---- activation tile: global -> registers -> LDS (natural K order)
+  const uint16_t* xs = (const uint16_t*)p.x;
+  uint4_t areg[A_LOADS];
+  auto load_a = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int u = tid + 256 * i;
+      const int m = u >> 3, kb = u & 7;
+      const int row = min(m0 + m, M - 1);  // rows past M re-read the last row, never stored
+      areg[i] = *(const uint4_t*)(xs + (size_t)row * K + kt * kABK + kb * 8);
+    }
+  };
+  auto store_a = [&](int buf) {
+    unsigned char* base = smem + buf * A_TILE;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int u = tid + 256 * i;
+      const int m = u >> 3, kb = u & 7;
+      *(uint4_t*)(base + (m * kAUnits + kb) * 16) = areg[i];
+    }
+  };
+
+  float16_t acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  load_a(0);
+  load_b(0);
+  store_a(0);
+  store_b(0);
+  load_a(min(1, last_tile));
+  load_b(min(1, last_tile));
+  __syncthreads();
+
+  const int a_off = ((wm * 64 + j) * kAUnits + kq) * 16;
+  const int b_off = (kq * kABN + wn * 64 + j) * 16;
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const int cur = kt & 1;
+    // the other buffer was last read in tile kt-1, before the barrier that ended it
+    store_a(cur ^ 1);
+    store_b(cur ^ 1);
+    const int kt2 = min(kt + 2, last_tile);
+    load_a(kt2);
+    load_b(kt2);
+    const unsigned char* ab = smem + cur * A_TILE + a_off;
+    const unsigned char* bb = smem + 2 * A_TILE + cur * B_TILE + b_off;
+#pragma unroll
+    for (int s = 0; s < kABK / 16; ++s) {
+      uint4_t af[2], bf[2];
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) af[mt] = *(const uint4_t*)(ab + (mt * 32 * kAUnits + 2 * s) * 16);
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) bf[nt] = *(const uint4_t*)(bb + ((2 * s) * kABN + nt * 32) * 16);
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+          if constexpr (DTYPE == Q4_DTYPE_F16) {
+            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                __builtin_bit_cast(half8_t, af[mt]), __builtin_bit_cast(half8_t, bf[nt]), acc[mt][nt], 0, 0, 0);
+          } else {
+            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                __builtin_bit_cast(bf16x8_t, af[mt]), __builtin_bit_cast(bf16x8_t, bf[nt]), acc[mt][nt], 0, 0, 0);
+          }
+        }
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: register r of lane (j, kq) is row 8*(r/4) + 4*kq + r%4, column j
+  uint16_t* y = (uint16_t*)p.y;
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const int n = n0 + wn * 64 + nt * 32 + j;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 64 + mt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
+        if (m < M) y[(size_t)m * N + n] = finish_output<DTYPE>(acc[mt][nt][r], p.bias, n);
+      }
+    }
+  }
+}
+
+}  // namespace q4
+
+namespace q4host {
+
+bool gemm_awq_supported(const q4_weight* w, int M, int dtype) {
+  (void)dtype;
+  if (w->layout != Q4_LAYOUT_AWQ || M < 1) return false;
+  if (w->K % q4::kABK != 0 || w->N % q4::kABN != 0) return false;
+  // one group per 8-row K block
+  if (w->groupsize % 8 != 0) return false;
+  return (long)w->num_groups * w->groupsize >= w->K;
+}
+
+int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                    hipStream_t stream) {
+  using namespace q4;
+  if (!gemm_awq_supported(w, M, dtype)) {
+    set_error("q4_linear(gemm/awq): unsupported problem (M=%d K=%d N=%d groupsize=%d)", M, w->K, w->N,
+              w->groupsize);
+    return Q4_ERR_UNSUPPORTED;
+  }
+  AwqGemmParams gp;
+  gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, nullptr, x, bias, y,
+                 M,          w->K,      w->N,                     w->groupsize, w->num_groups};
+  const long total = (long)((M + kABM - 1) / kABM) * (w->N / kABN);
+  if (total > 0x7fffffffL) {
+    set_error("q4_linear(gemm/awq): grid too large");
+    return Q4_ERR_UNSUPPORTED;
+  }
+  const size_t smem = 2 * (size_t)kABM * kAUnits * 16 + 2 * (size_t)(kABK / 8) * kABN * 16;
+  if (dtype == Q4_DTYPE_F16) {
+    auto k = gemm_awq_kernel<Q4_DTYPE_F16>;
+    (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL(k, dim3((unsigned)total), dim3(256), smem, stream, gp);
+  } else {
+    auto k = gemm_awq_kernel<Q4_DTYPE_BF16>;
+    (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL(k, dim3((unsigned)total), dim3(256), smem, stream, gp);
+  }
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    set_error("q4_linear(gemm/awq): launch failed: %s", hipGetErrorString(err));
+    return Q4_ERR_LAUNCH;
+  }
+  return Q4_OK;
+}
+
+}  // namespace q4host
