@@ -271,3 +271,8 @@ def test_awq_dispatch_large_m(pkg, oracle, gpu):
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 1)
     assert pkg.ops.select_path(pk, 48) == "gemv"
     assert pkg.ops.select_path(pk, 64) == "gemm"
+
+
+def test_gemm_n_multiple_of_128_only(pkg, oracle, gpu):
+    """N = 384 is not a multiple of 256: the GEMM takes its 128-column tile."""
+    _run(pkg, oracle, gpu, 1024, 384, 128, 3000, sym=False, bias=True, path=2, seed=384)

@@ -28,7 +28,6 @@ namespace q4 {
 constexpr int kBK = 64;            // K rows per tile
 constexpr int kKSteps = kBK / 16;  // MFMA K steps per tile
 constexpr int kAUnitsPerRow = kBK / 8 + 1;  // 16-byte units per LDS row, padded
-constexpr int kBN = 256;           // columns per workgroup (4 waves x 64)
 
 struct GemmParams {
   Problem p;
@@ -104,8 +103,9 @@ __device__ __forceinline__ float16_t mfma32(const uint4_t a, const uint4_t b, fl
 }
 
 // BM: rows per workgroup (128 or 256).  GPT: quantisation groups per K tile (1 or 2).
-template <int DTYPE, int BM, int GPT>
-__global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(GemmParams gp) {
+// NW: packed words (columns) per lane and K step: 2 -> 256-column workgroup tile, 1 -> 128.
+template <int DTYPE, int BM, int GPT, int NW>
+__global__ __launch_bounds__(256, (BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm_gptq_kernel(GemmParams gp) {
   constexpr int MT = BM / 32;                      // MFMA row tiles per wave
   constexpr int A_LOADS = BM * (kBK / 8) / 256;    // 16-byte activation loads per thread per tile
   constexpr int A_TILE_BYTES = BM * kAUnitsPerRow * 16;
@@ -126,7 +126,8 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
   // (A grid of a single round, at most one workgroup per CU, measured faster the other way
   // round: each XCD takes a few column blocks and all M tiles of them.)
   const int tiles_m = (M + BM - 1) / BM;
-  const int tiles_n = N / kBN;
+  constexpr int BN = 4 * 32 * NW;
+  const int tiles_n = N / BN;
   int tm, tn;
   {
     const int bid = blockIdx.x;
@@ -147,9 +148,9 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
     }
   }
   const int m0 = tm * BM;
-  const int n0 = tn * kBN;
-  const int nw = n0 + wave * 64;   // first column of this wave
-  const int ncol = nw + 2 * j;     // first of this lane's two columns
+  const int n0 = tn * BN;
+  const int nw = n0 + wave * 32 * NW;  // first column of this wave
+  const int ncol = nw + NW * j;        // first of this lane's NW columns
 
   const SpliceK splice = gemm_splice_consts();
   const int KT = K / kBK;
@@ -158,16 +159,25 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
   const char* wbase = (const char*)p.qweight;
   const uint32_t w_lane = ((uint32_t)kq * (uint32_t)N + (uint32_t)ncol) * 4u;
   const size_t kstep_bytes = (size_t)N * 8;  // two packed rows per MFMA K step
-  uint2_t bq[2][kKSteps];
-  auto load_b = [&](int kt, uint2_t (&dst)[kKSteps]) {
+  struct BWords { uint32_t v[NW]; };
+  BWords bq[2][kKSteps];
+  auto load_b = [&](int kt, BWords (&dst)[kKSteps]) {
 #pragma unroll
     for (int s = 0; s < kKSteps; ++s)
-      dst[s] = *(const uint2_t*)(wbase + (size_t)(kt * kKSteps + s) * kstep_bytes + w_lane);
+    {
+      const char* addr = wbase + (size_t)(kt * kKSteps + s) * kstep_bytes + w_lane;
+      if constexpr (NW == 2) {
+        const uint2_t t = *(const uint2_t*)addr;
+        dst[s].v[0] = t.x; dst[s].v[1] = t.y;
+      } else {
+        dst[s].v[0] = *(const uint32_t*)addr;
+      }
+    }
   };
 
   // ---- group constants for this lane's two columns.  They are rebuilt for every tile
   // from two tiny (cached) loads, which keeps the steady-state loop free of branches.
-  ColConsts cc[GPT][2], cc_next[GPT][2];
+  ColConsts cc[GPT][NW], cc_next[GPT][NW];
   uint32_t sraw[GPT], zraw[GPT];
   const int zshift = (ncol & 7) * 4;
   auto load_group_raw = [&](int kt) {
@@ -175,40 +185,46 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
     for (int g = 0; g < GPT; ++g) {
       int gi = (kt * kBK + g * (kBK / GPT)) / p.groupsize;
       gi = min(gi, p.num_groups - 1);
-      sraw[g] = *(const uint32_t*)(p.scales + (size_t)gi * N + ncol);
+      if constexpr (NW == 2) sraw[g] = *(const uint32_t*)(p.scales + (size_t)gi * N + ncol);
+      else sraw[g] = *(const uint16_t*)(p.scales + (size_t)gi * N + ncol);
       zraw[g] = p.qzeros[(size_t)gi * (N >> 3) + (ncol >> 3)];
     }
   };
-  auto make_group = [&](ColConsts (&dst)[GPT][2]) {
+  auto make_group = [&](ColConsts (&dst)[GPT][NW]) {
 #pragma unroll
     for (int g = 0; g < GPT; ++g) {
       const uint32_t z2 = gptq_zero_plus_one(zraw[g]) >> zshift;
       const half2_t s01 = as_half2(sraw[g]);
       dst[g][0] = make_col_consts(z2 & 0xFu, s01.x);
-      dst[g][1] = make_col_consts((z2 >> 4) & 0xFu, s01.y);
+      if constexpr (NW == 2) dst[g][1] = make_col_consts((z2 >> 4) & 0xFu, s01.y);
     }
   };
 
   // ---- activation tile: global -> registers -> (permuted) LDS
   const uint16_t* xs = (const uint16_t*)p.x;
-  uint4_t areg[A_LOADS];
-  auto load_a = [&](int kt) {
+  // Register staging sets: with two sets (128-row tiles) a tile's loads are issued two
+  // tiles before they are written to LDS; the 256-row tile has registers for one set only.
+  constexpr int ASETS = BM == 128 ? 2 : 1;
+  uint4_t areg[ASETS][A_LOADS];
+  auto load_a = [&](int kt, auto set_c) {
+    constexpr int set = decltype(set_c)::value % ASETS;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
       const int u = tid + 256 * i;
       const int m = u >> 3, kb = u & 7;
       // rows past M re-read the last row: their results are never stored
       const int row = min(m0 + m, M - 1);
-      areg[i] = *(const uint4_t*)(xs + (size_t)row * K + kt * kBK + kb * 8);
+      areg[set][i] = *(const uint4_t*)(xs + (size_t)row * K + kt * kBK + kb * 8);
     }
   };
-  auto store_a = [&](int buf) {
+  auto store_a = [&](int buf, auto set_c) {
+    constexpr int set = decltype(set_c)::value % ASETS;
     unsigned char* base = smem + buf * A_TILE_BYTES;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
       const int u = tid + 256 * i;
       const int m = u >> 3, kb = u & 7;
-      const uint4_t v = areg[i];
+      const uint4_t v = areg[set][i];
       uint4_t o;
       o.x = (v.x & 0xFFFFu) | (v.z << 16);
       o.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
@@ -218,17 +234,17 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
     }
   };
 
-  float16_t acc[MT][2];
+  float16_t acc[MT][NW];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int f = 0; f < 2; ++f)
+    for (int f = 0; f < NW; ++f)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[mt][f][r] = 0.f;
 
   const int a_lane_off = (j * kAUnitsPerRow + kq) * 16;
   uint4_t afrag[2][MT];  // A fragments of the current / next MFMA K step
-  uint4_t bfrag[2][2];   // unpacked B fragments of the current / next step
+  uint4_t bfrag[2][NW];  // unpacked B fragments of the current / next step
   auto read_a = [&](int buf, int s, uint4_t (&dst)[MT]) {
     const unsigned char* abase = smem + buf * A_TILE_BYTES + a_lane_off;
 #pragma unroll
@@ -239,17 +255,21 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
 
   // ---- prologue: tile 0 staged, tile 1 in flight, first fragments ready
   const int last_tile = KT - 1;
-  load_a(0);
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  load_a(0, I0{});
   load_b(0, bq[0]);
   load_b(min(1, last_tile), bq[1]);
   load_group_raw(0);
-  store_a(0);
-  load_a(min(1, last_tile));
+  if constexpr (ASETS == 2) load_a(min(1, last_tile), I1{});
+  store_a(0, I0{});
+  if constexpr (ASETS == 2) load_a(min(2, last_tile), I0{});
+  else load_a(min(1, last_tile), I0{});
   make_group(cc);
   __syncthreads();
   read_a(0, 0, afrag[0]);
-  bfrag[0][0] = dequant_word<DTYPE>(bq[0][0].x, cc[0][0], splice);
-  bfrag[0][1] = dequant_word<DTYPE>(bq[0][0].y, cc[0][1], splice);
+#pragma unroll
+  for (int f = 0; f < NW; ++f) bfrag[0][f] = dequant_word<DTYPE>(bq[0][0].v[f], cc[0][f], splice);
 
   // One K tile, software pipelined: while the MFMAs of step s run, the VALU unpacks the
   // weights of step s+1 and the LDS returns its A fragments; the global loads of tile
@@ -272,29 +292,36 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
       // (2) unpack the next step's weights
       if (s + 1 < kKSteps) {
         const int g = group_of_step(s + 1);
-        bfrag[sb ^ 1][0] = dequant_word<DTYPE>(bq[cur][s + 1].x, cc[g][0], splice);
-        bfrag[sb ^ 1][1] = dequant_word<DTYPE>(bq[cur][s + 1].y, cc[g][1], splice);
+#pragma unroll
+        for (int f = 0; f < NW; ++f)
+          bfrag[sb ^ 1][f] = dequant_word<DTYPE>(bq[cur][s + 1].v[f], cc[g][f], splice);
       } else {
-        bfrag[sb ^ 1][0] = dequant_word<DTYPE>(bq[cur ^ 1][0].x, cc_next[0][0], splice);
-        bfrag[sb ^ 1][1] = dequant_word<DTYPE>(bq[cur ^ 1][0].y, cc_next[0][1], splice);
+#pragma unroll
+        for (int f = 0; f < NW; ++f)
+          bfrag[sb ^ 1][f] = dequant_word<DTYPE>(bq[cur ^ 1][0].v[f], cc_next[0][f], splice);
       }
       // (3) side work of this step
       if (s == 0) {
-        store_a(cur ^ 1);       // tile kt+1 (held in areg) -> the other LDS buffer
+        // tile kt+1 (staged in register set (kt+1) % ASETS) -> the other LDS buffer
+        store_a(cur ^ 1, std::integral_constant<int, cur ^ 1>{});
         load_group_raw(kt1);    // scales / zero points the next tile starts with
       }
-      if (s == 1) load_a(kt2);
+      if (s == 1) {
+        // refill the set that was just written out: tile kt+3 with two sets, kt+2 with one
+        if constexpr (ASETS == 2) load_a(min(kt + 3, last_tile), std::integral_constant<int, cur ^ 1>{});
+        else load_a(kt2, I0{});
+      }
       if (s == 2) make_group(cc_next);
       // (4) the MFMAs of this step
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        acc[mt][0] = mfma32<DTYPE>(afrag[sb][mt], bfrag[sb][0], acc[mt][0]);
-        acc[mt][1] = mfma32<DTYPE>(afrag[sb][mt], bfrag[sb][1], acc[mt][1]);
+#pragma unroll
+        for (int f = 0; f < NW; ++f) acc[mt][f] = mfma32<DTYPE>(afrag[sb][mt], bfrag[sb][f], acc[mt][f]);
       }
       if (s == kKSteps - 1) load_b(kt2, bq[cur]);
       // interleave: after every MFMA a few VALU ops, one LDS op and one global load
 #pragma unroll
-      for (int i = 0; i < 2 * MT; ++i) {
+      for (int i = 0; i < NW * MT; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
         __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
@@ -310,8 +337,8 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
     }
 #pragma unroll
     for (int g = 0; g < GPT; ++g) {
-      cc[g][0] = cc_next[g][0];
-      cc[g][1] = cc_next[g][1];
+#pragma unroll
+      for (int f = 0; f < NW; ++f) cc[g][f] = cc_next[g][f];
     }
   };
   {
@@ -326,11 +353,11 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
   // ---- epilogue: C layout of the 32x32 MFMA: register r of lane (j, kq) is row
   // 8*(r/4) + 4*kq + r%4, column j.  Fragments 0/1 are adjacent columns -> one 32-bit store.
   uint16_t* y = (uint16_t*)p.y;
-  float bias_f[2] = {0.f, 0.f};
+  float bias_f[NW] = {};
   const bool has_bias = p.bias != nullptr;
   if (has_bias) {
-    bias_f[0] = load_act<DTYPE>(p.bias, ncol);
-    bias_f[1] = load_act<DTYPE>(p.bias, ncol + 1);
+#pragma unroll
+    for (int f = 0; f < NW; ++f) bias_f[f] = load_act<DTYPE>(p.bias, ncol + f);
   }
   // The sum is rounded to the activation dtype first and the bias added in that dtype
   // (one more rounding), like `out + bias` on a half tensor.
@@ -351,8 +378,12 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void gemm_gptq_kernel(Gem
       const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
       if (m < M) {
         const uint32_t lo = finish(acc[mt][0][r], bias_f[0]);
-        const uint32_t hi = finish(acc[mt][1][r], bias_f[1]);
-        *(uint32_t*)(y + (size_t)m * N + ncol) = lo | (hi << 16);
+        if constexpr (NW == 2) {
+          const uint32_t hi = finish(acc[mt][1][r], bias_f[1]);
+          *(uint32_t*)(y + (size_t)m * N + ncol) = lo | (hi << 16);
+        } else {
+          y[(size_t)m * N + ncol] = (uint16_t)lo;
+        }
       }
     }
   }
@@ -369,23 +400,23 @@ bool gemm_supported(const q4_weight* w, int M, int dtype) {
   (void)dtype;
   if (w->layout != Q4_LAYOUT_GPTQ || w->g_idx != nullptr) return false;
   if (M < 1) return false;
-  if (w->K % q4::kBK != 0 || w->N % q4::kBN != 0) return false;
+  if (w->K % q4::kBK != 0 || w->N % 128 != 0) return false;
   const int gs = w->groupsize;
   if (!(gs == 32 || (gs >= 64 && gs % 64 == 0))) return false;
   if ((long)w->num_groups * gs < w->K) return false;
   return true;
 }
 
-template <int DTYPE, int BM>
-static void launch_bm(const GemmParams& gp, int gs, dim3 grid, size_t smem, hipStream_t stream) {
+template <int DTYPE, int BM, int NW>
+static void launch_tile(const GemmParams& gp, int gs, dim3 grid, size_t smem, hipStream_t stream) {
   using namespace q4;
   if (gs == 32) {
-    auto k = gemm_gptq_kernel<DTYPE, BM, 2>;
+    auto k = gemm_gptq_kernel<DTYPE, BM, 2, NW>;
     if (smem > 64 * 1024)
       (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     hipLaunchKernelGGL(k, grid, dim3(256), smem, stream, gp);
   } else {
-    auto k = gemm_gptq_kernel<DTYPE, BM, 1>;
+    auto k = gemm_gptq_kernel<DTYPE, BM, 1, NW>;
     if (smem > 64 * 1024)
       (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     hipLaunchKernelGGL(k, grid, dim3(256), smem, stream, gp);
@@ -403,25 +434,34 @@ int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, in
   GemmParams gp;
   gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, nullptr, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
-  const int tiles_n = w->N / kBN;
-  // 256-row tiles halve the unpacking work per flop (and run at a higher clock for it) but
-  // need one wave per SIMD and a grid of at least two rounds over the 256 CUs; otherwise
-  // 128-row tiles with two workgroups per CU.
-  const int bm = ((long)((M + 255) / 256) * tiles_n >= 512) ? 256 : 128;
+  // Tile choice (all with 4 waves side by side along N):
+  //   256 x 256  grids of at least two rounds over the 256 CUs: half the unpacking per flop,
+  //              one wave per SIMD, runs at a higher clock;
+  //   128 x 256  the default; two workgroups per CU once there are more than 256 of them;
+  //   128 x 128  only when N is not a multiple of 256 (measured slower than 128 x 256
+  //              everywhere else: twice the activation-fragment reads per MFMA).
+  const bool n256 = w->N % 256 == 0;
+  const long t256 = n256 ? (long)((M + 255) / 256) * (w->N / 256) : 0;
+  int bm = 128, nw = n256 ? 2 : 1;
+  if (t256 >= 512) bm = 256;
+  const int bn = 128 * nw;
   const int tiles_m = (M + bm - 1) / bm;
-  const long total = (long)tiles_m * tiles_n;
+  const long total = (long)tiles_m * (w->N / bn);
   if (total > 0x7fffffffL) {
     set_error("q4_linear(gemm): grid too large");
     return Q4_ERR_UNSUPPORTED;
   }
   const size_t smem = 2 * (size_t)bm * kAUnitsPerRow * 16;
   dim3 grid((unsigned)total);
-  if (bm == 256) {
-    if (dtype == Q4_DTYPE_F16) launch_bm<Q4_DTYPE_F16, 256>(gp, w->groupsize, grid, smem, stream);
-    else launch_bm<Q4_DTYPE_BF16, 256>(gp, w->groupsize, grid, smem, stream);
+  const int gs = w->groupsize;
+  if (dtype == Q4_DTYPE_F16) {
+    if (bm == 256) launch_tile<Q4_DTYPE_F16, 256, 2>(gp, gs, grid, smem, stream);
+    else if (nw == 2) launch_tile<Q4_DTYPE_F16, 128, 2>(gp, gs, grid, smem, stream);
+    else launch_tile<Q4_DTYPE_F16, 128, 1>(gp, gs, grid, smem, stream);
   } else {
-    if (dtype == Q4_DTYPE_F16) launch_bm<Q4_DTYPE_F16, 128>(gp, w->groupsize, grid, smem, stream);
-    else launch_bm<Q4_DTYPE_BF16, 128>(gp, w->groupsize, grid, smem, stream);
+    if (bm == 256) launch_tile<Q4_DTYPE_BF16, 256, 2>(gp, gs, grid, smem, stream);
+    else if (nw == 2) launch_tile<Q4_DTYPE_BF16, 128, 2>(gp, gs, grid, smem, stream);
+    else launch_tile<Q4_DTYPE_BF16, 128, 1>(gp, gs, grid, smem, stream);
   }
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {
