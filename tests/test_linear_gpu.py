@@ -276,3 +276,37 @@ def test_awq_dispatch_large_m(pkg, oracle, gpu):
 def test_gemm_n_multiple_of_128_only(pkg, oracle, gpu):
     """N = 384 is not a multiple of 256: the GEMM takes its 128-column tile."""
     _run(pkg, oracle, gpu, 1024, 384, 128, 3000, sym=False, bias=True, path=2, seed=384)
+
+
+# --------------------------------------------------------------------------- act-order prefill GEMM
+
+
+@pytest.mark.parametrize("K,N,M", [(8192, 10240, 1024), (1024, 256, 200), (2048, 128, 64)])
+def test_act_order_gemm(pkg, oracle, gpu, K, N, M):
+    """cfg4 prefill: desc_act through the MFMA kernel (per-row scale/zero gathered by g_idx)."""
+    _run(pkg, oracle, gpu, K, N, 128, M, sym=(K == 8192), act=True, path=2, bias=(M == 200), seed=K // 512 + M)
+
+
+@pytest.mark.parametrize("gs", [32, 128])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_act_order_gemm_groupsizes_dtypes(pkg, oracle, gpu, gs, dtype):
+    _run(pkg, oracle, gpu, 512, 256, gs, 70, dtype=dtype, sym=False, act=True, path=2, seed=gs + 13)
+
+
+def test_act_order_gemm_bit_exact_weights_through_identity(pkg, oracle, gpu):
+    K, N, gs = 512, 128, 64
+    qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=33, sym=False, act_order=True)
+    w = oracle.dequant_gptq(qw, qz, sc, gi, gs, "f16")
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), gs, 0)
+    eye = torch.eye(K, dtype=torch.float16, device=gpu)
+    got = pkg.ops.linear(pk, eye, None, path=2)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), w.view(np.uint16))
+
+
+def test_act_order_dispatch(pkg, oracle, gpu):
+    qw, qz, sc, gi = oracle.make_gptq(1024, 10240, 128, seed=0, act_order=True)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), 128, 0)
+    assert pkg.ops.select_path(pk, 16) == "gemv"
+    assert pkg.ops.select_path(pk, 1024) == "gemm"
+    assert pkg.ops.select_path(pk, 1024, torch.bfloat16) == "gemm"
+    assert pkg.ops.select_path(pk, 4, torch.bfloat16) == "generic"  # the act-order decode kernel is fp16 only

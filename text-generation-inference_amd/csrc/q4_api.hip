@@ -97,9 +97,9 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   // kernel (weights unpacked into LDS) for the sizes where a GEMM grid fills the chip
   // (measured crossover for the 128 x 128 AWQ tiles: M * N around 0.75 * 2^20)
   const bool small = M <= 16 || (long)M * w->N <= (3L << 18);
-  if (w->layout == Q4_LAYOUT_AWQ && !small && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
+  if (!small && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
   if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
-  if (w->layout == Q4_LAYOUT_AWQ && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
+  if (M > 16 && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
   return Q4_PATH_GENERIC;
 }
 
@@ -148,7 +148,8 @@ int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, i
       return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, nullptr,
                          (hipStream_t)stream);
     case Q4_PATH_GEMM:
-      if (w->layout == Q4_LAYOUT_AWQ) return launch_gemm_awq(w, x, bias, y, M, dtype, (hipStream_t)stream);
+      if (w->layout == Q4_LAYOUT_AWQ || w->g_idx != nullptr)
+        return launch_gemm_awq(w, x, bias, y, M, dtype, (hipStream_t)stream);
       return launch_gemm(w, x, bias, y, M, dtype, (hipStream_t)stream);
     case Q4_PATH_GENERIC:
       return launch_generic(w, x, bias, y, M, dtype, (hipStream_t)stream);

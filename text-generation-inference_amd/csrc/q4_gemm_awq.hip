@@ -1,8 +1,10 @@
-// Prefill path for the AWQ layout: y[M, N] = x @ dequant(W) on the MFMA units (gfx950).
+// Prefill path for the layouts whose packed words cannot feed the MFMA directly:
+// y[M, N] = x @ dequant(W) for AWQ and for GPTQ with g_idx (act-order), gfx950.
 //
-// An AWQ word holds 8 interleaved columns of ONE K row, so it is not an MFMA operand by
-// itself.  The weight tile is therefore unpacked cooperatively into LDS (the classic
-// dequantize-to-LDS stage) and both operands are read from there:
+// An AWQ word holds 8 interleaved columns of ONE K row; an act-order GPTQ word holds 8 K
+// rows that each belong to a different group.  In both cases the weight tile is unpacked
+// cooperatively into LDS (the classic dequantize-to-LDS stage) and both MFMA operands are
+// read from there:
 //   * workgroup = 4 waves in a 2 x 2 arrangement, tile 128 x 128, K tile 64; each wave owns
 //     a 64 x 64 block = 2 x 2 MFMA tiles of v_mfma_f32_32x32x16 (64 accumulator VGPRs),
 //     so two or three workgroups share a CU and cover each other's barriers;
@@ -12,6 +14,10 @@
 //     subtracted exactly and each weight is multiplied once by its fp16 scale (the
 //     reference's rounding).  The patch becomes eight 16-byte units (one per column,
 //     8 consecutive K values each) written to LDS at [K block][column];
+//   * act-order producer: every thread owns 4 packed words (8 K rows x 1 column each).  The
+//     groups of the 8 rows are wave-uniform (g_idx[k]); scale and zero point of each row
+//     are gathered from the checkpoint tensors (coalesced across the 64 columns of a wave,
+//     L2 resident) and applied per weight -- no row of qweight is ever moved;
 //   * LDS layouts: activations [row][K block] with the row stride padded to 9 units,
 //     weights [K block][column]; both give conflict-free 128-bit fragment reads;
 //   * double-buffered LDS, global loads for tile k+2 in flight while tile k is multiplied.
@@ -41,7 +47,8 @@ __device__ __forceinline__ AwqSplice awq_splice_consts() {
 typedef __bf16 awq_bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float awq_float2_t __attribute__((ext_vector_type(2)));
 
-template <int DTYPE>
+// ACT = false: AWQ layout.  ACT = true: GPTQ layout with g_idx.
+template <int DTYPE, bool ACT>
 __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   constexpr int A_TILE = kABM * kAUnits * 16;   // bytes
   constexpr int B_TILE = (kABK / 8) * kABN * 16;
@@ -65,16 +72,24 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   const int last_tile = KT - 1;
   const AwqSplice splice = awq_splice_consts();
 
-  // ---- producer state: threads 0..127 own K block pb (8 rows) x word pc (8 columns)
-  const bool producer = tid < 128;
+  // ---- producer state
+  // AWQ: threads 0..127 own K block pb (8 rows) x word pc (8 columns).
+  // act-order: every thread owns column pn and K blocks pkb0, pkb0 + 2, pkb0 + 4, pkb0 + 6.
+  const bool producer = ACT || tid < 128;
   const int pb = (tid >> 4) & 7;
   const int pc = tid & 15;
-  const uint32_t* wsrc = p.qweight + (size_t)(pb * 8) * NC + (n0 >> 3) + pc;
-  uint32_t braw[8];
-  uint4_t sraw;   // 8 fp16 scales of the word's columns
-  uint32_t zraw;  // 8 zero-point nibbles
+  const int pn = tid & 127;
+  const int pkb0 = __builtin_amdgcn_readfirstlane(tid >> 7);  // wave-uniform
+  const uint32_t* wsrc = ACT ? p.qweight + (size_t)pkb0 * N + n0 + pn
+                             : p.qweight + (size_t)(pb * 8) * NC + (n0 >> 3) + pc;
+  uint32_t braw[8];  // AWQ: 8 rows of one word column; act-order: 4 words (K blocks)
+  uint4_t sraw;      // AWQ: 8 fp16 scales of the word's columns
+  uint32_t zraw;     // AWQ: 8 zero-point nibbles
   auto load_b = [&](int kt) {
-    if (producer) {
+    if constexpr (ACT) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) braw[i] = wsrc[(size_t)(kt * (kABK / 8) + 2 * i) * N];
+    } else if (producer) {
 #pragma unroll
       for (int r = 0; r < 8; ++r) braw[r] = wsrc[(size_t)(kt * kABK + r) * NC];
       const int g = min((kt * kABK + pb * 8) / p.groupsize, p.num_groups - 1);
@@ -82,7 +97,49 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
       zraw = p.qzeros[(size_t)g * NC + (n0 >> 3) + pc];
     }
   };
-  auto store_b = [&](int buf) {
+  auto store_b_act = [&](int buf, int kt) {
+    unsigned char* base = smem + 2 * A_TILE + buf * B_TILE;
+    const int n = n0 + pn;
+    const int zshift = (n & 7) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int kb = pkb0 + 2 * i;
+      const int k0 = kt * kABK + kb * 8;
+      // scale and -(1024 + zero) of the 8 rows of this word: groups are wave-uniform
+      uint32_t sc[8], cz[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        int g = p.g_idx[k0 + r];
+        g = min(max(g, 0), p.num_groups - 1);
+        sc[r] = *(const uint16_t*)(p.scales + (size_t)g * N + n);
+        const uint32_t z = (gptq_zero_plus_one(p.qzeros[(size_t)g * NC + (n >> 3)]) >> zshift) & 0xFu;
+        cz[r] = 0xE400u | z;
+      }
+      const uint32_t w = braw[i];
+      uint32_t o[4];
+#pragma unroll
+      for (int pr = 0; pr < 4; ++pr) {
+        // rows pr and pr + 4 share one splice (nibbles 16 bits apart)
+        const uint32_t q2 = ((w >> (4 * pr)) & splice.mask_lo) | splice.magic;
+        const half2_t dq = as_half2(q2) + as_half2(cz[pr] | (cz[pr + 4] << 16));  // exact q - z
+        if constexpr (DTYPE == Q4_DTYPE_F16) {
+          o[pr] = as_u32(dq * as_half2(sc[pr] | (sc[pr + 4] << 16)));  // one fp16 rounding
+        } else {
+          const half2_t s2 = as_half2(sc[pr] | (sc[pr + 4] << 16));
+          const awq_float2_t f = {(float)dq.x * (float)s2.x, (float)dq.y * (float)s2.y};
+          o[pr] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, awq_bf16x2_t));
+        }
+      }
+      // o holds rows (0,4),(1,5),(2,6),(3,7): back to natural K order for the unit
+      uint4_t unit;
+      unit.x = (o[0] & 0xFFFFu) | (o[1] << 16);
+      unit.y = (o[2] & 0xFFFFu) | (o[3] << 16);
+      unit.z = (o[0] >> 16) | (o[1] & 0xFFFF0000u);
+      unit.w = (o[2] >> 16) | (o[3] & 0xFFFF0000u);
+      *(uint4_t*)(base + ((size_t)kb * kABN + pn) * 16) = unit;
+    }
+  };
+  auto store_b_awq = [&](int buf) {
     if (!producer) return;
     unsigned char* base = smem + 2 * A_TILE + buf * B_TILE;
     const uint32_t su[4] = {sraw.x, sraw.y, sraw.z, sraw.w};
@@ -123,6 +180,11 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
     }
   };
 
+  auto store_b = [&](int buf, int kt) {
+    if constexpr (ACT) store_b_act(buf, kt);
+    else store_b_awq(buf);
+  };
+
   // ---- activation tile: global -> registers -> LDS (natural K order)
   const uint16_t* xs = (const uint16_t*)p.x;
   uint4_t areg[A_LOADS];
@@ -156,7 +218,7 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   load_a(0);
   load_b(0);
   store_a(0);
-  store_b(0);
+  store_b(0, 0);
   load_a(min(1, last_tile));
   load_b(min(1, last_tile));
   __syncthreads();
@@ -168,7 +230,7 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
     const int cur = kt & 1;
     // the other buffer was last read in tile kt-1, before the barrier that ended it
     store_a(cur ^ 1);
-    store_b(cur ^ 1);
+    store_b(cur ^ 1, min(kt + 1, last_tile));
     const int kt2 = min(kt + 2, last_tile);
     load_a(kt2);
     load_b(kt2);
@@ -219,9 +281,10 @@ namespace q4host {
 
 bool gemm_awq_supported(const q4_weight* w, int M, int dtype) {
   (void)dtype;
-  if (w->layout != Q4_LAYOUT_AWQ || M < 1) return false;
+  if (M < 1) return false;
   if (w->K % q4::kABK != 0 || w->N % q4::kABN != 0) return false;
-  // one group per 8-row K block
+  if (w->layout == Q4_LAYOUT_GPTQ) return w->g_idx != nullptr;  // act-order
+  // AWQ: one group per 8-row K block
   if (w->groupsize % 8 != 0) return false;
   return (long)w->num_groups * w->groupsize >= w->K;
 }
@@ -235,7 +298,7 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
     return Q4_ERR_UNSUPPORTED;
   }
   AwqGemmParams gp;
-  gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, nullptr, x, bias, y,
+  gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, w->g_idx, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
   const long total = (long)((M + kABM - 1) / kABM) * (w->N / kABN);
   if (total > 0x7fffffffL) {
@@ -243,14 +306,17 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
     return Q4_ERR_UNSUPPORTED;
   }
   const size_t smem = 2 * (size_t)kABM * kAUnits * 16 + 2 * (size_t)(kABK / 8) * kABN * 16;
+  const bool act = w->layout == Q4_LAYOUT_GPTQ;
+  auto launch = [&](auto k) {
+    (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL(k, dim3((unsigned)total), dim3(256), smem, stream, gp);
+  };
   if (dtype == Q4_DTYPE_F16) {
-    auto k = gemm_awq_kernel<Q4_DTYPE_F16>;
-    (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipLaunchKernelGGL(k, dim3((unsigned)total), dim3(256), smem, stream, gp);
+    if (act) launch(gemm_awq_kernel<Q4_DTYPE_F16, true>);
+    else launch(gemm_awq_kernel<Q4_DTYPE_F16, false>);
   } else {
-    auto k = gemm_awq_kernel<Q4_DTYPE_BF16>;
-    (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipLaunchKernelGGL(k, dim3((unsigned)total), dim3(256), smem, stream, gp);
+    if (act) launch(gemm_awq_kernel<Q4_DTYPE_BF16, true>);
+    else launch(gemm_awq_kernel<Q4_DTYPE_BF16, false>);
   }
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {

@@ -737,7 +737,9 @@ bool gemv_supported(const q4_weight* w, int M, int dtype) {
     return chunks * (w->N / 256) <= Q4_WORKSPACE_COUNTER_BYTES / 4;
   }
   if (w->N % 64 != 0) return false;
-  if (chunks * (w->N / 16) > Q4_WORKSPACE_COUNTER_BYTES / 4 && M > 16) return false;
+  // one ticket per (row chunk, column tile); the narrowest tile of each kernel decides
+  const long tile = w->g_idx != nullptr ? 64 : 16;
+  if (chunks * (w->N / tile) > Q4_WORKSPACE_COUNTER_BYTES / 4 && M > 16) return false;
   if (w->g_idx != nullptr) {
     // act-order: the table of all groups for 64 columns must fit LDS next to the slab
     if (dtype != Q4_DTYPE_F16) return false;
