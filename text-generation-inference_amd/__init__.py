@@ -11,6 +11,7 @@ from . import _lib, ops  # noqa: F401
 from .layers.linear import get_linear  # noqa: F401
 from .layers.gptq import (  # noqa: F401
     GPTQWeight,
+    GPTQWeightsLoader,
     QuantLinear,
     ExllamaQuantLinear,
     create_exllama_buffers,
@@ -18,9 +19,15 @@ from .layers.gptq import (  # noqa: F401
 )
 from .layers.awq.quantize import WQLinear  # noqa: F401
 from .layers.awq import conversion_utils  # noqa: F401
+from .utils.weights import Weights, WeightsLoader, DefaultWeightsLoader, UnquantizedWeight  # noqa: F401
+from .utils.quantization import get_loader, get_quantizer_config  # noqa: F401
 
 __all__ = [
     "GPTQWeight",
+    "GPTQWeightsLoader",
+    "Weights",
+    "get_loader",
+    "get_quantizer_config",
     "QuantLinear",
     "ExllamaQuantLinear",
     "WQLinear",

@@ -18,6 +18,7 @@ from .exllama import (  # noqa: F401
     create_exllama_buffers,
     set_device,
 )
+from .loader import GPTQWeightsLoader  # noqa: F401
 
 # The reference sets this to "1"/"2" when an exllama extension imported; here the native
 # library always plays that role.
