@@ -322,7 +322,7 @@ def main():
         if gm:
             out["gemm"] = {
                 "M": Mg, "per_shape": gm,
-                "roofline": {"bound": "mfma", "kernel": "q4::gemm_kernel", "achieved": round(tot_f / tot_t / 1e12, 1),
+                "roofline": {"bound": "mfma", "kernel": "q4::gemm_gptq_kernel", "achieved": round(tot_f / tot_t / 1e12, 1),
                              "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                              "frac": round(tot_f / tot_t / 1e12 / MFMA_PEAK_TFLOPS, 4), "traffic": None},
             }

@@ -35,8 +35,12 @@ FLAGS = [
 ]
 
 
-def build_library(verbose: bool = False, extra_flags: list[str] | None = None) -> Path:
-    """Compile every kernel translation unit and link the shared library."""
+def build_library(verbose: bool = False, extra_flags: list[str] | None = None,
+                  only: list[str] | None = None) -> Path:
+    """Compile every kernel translation unit and link the shared library.
+
+    `only` (development aid) recompiles just the named sources and links them with the
+    objects a previous full build left in build/."""
     objs = []
     procs = []
     build_dir = HERE / "build"
@@ -44,11 +48,13 @@ def build_library(verbose: bool = False, extra_flags: list[str] | None = None) -
     flags = FLAGS + (extra_flags or [])
     for src in SOURCES:
         obj = build_dir / (Path(src).stem + ".o")
+        objs.append(str(obj))
+        if only and src not in only and obj.exists():
+            continue
         cmd = [HIPCC, *flags, "-c", str(CSRC / src), "-o", str(obj)]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
-        objs.append(str(obj))
     failed = False
     for src, proc in procs:
         out, _ = proc.communicate()
@@ -70,4 +76,4 @@ def build_library(verbose: bool = False, extra_flags: list[str] | None = None) -
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    print(build_library(verbose=True, only=sys.argv[1:] or None))
