@@ -94,6 +94,28 @@ int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, i
                  void* workspace, size_t workspace_bytes, int path, void* stream);
 
 /*
+ * First half of a gated MLP in one launch: W packs [gate | up] along N and
+ *   y[M, N/2] = act(x @ gate (+ bias[:N/2])) * (x @ up (+ bias[N/2:])),
+ * with the roundings of the unfused sequence (both products rounded to `dtype`, the
+ * activation evaluated in fp32 and rounded, the product rounded).  Replaces
+ * `gate_up_proj(x)` followed by `act(gate_up[:, 0]) * gate_up[:, 1]`
+ * (server/text_generation_server/models/custom_modeling/flash_llama_modeling.py:400-404;
+ * the reference fuses this only for unquantized ROCm decode, `ops.LLMM_Silu`, :378-397).
+ * Fused in the decode kernel of the GPTQ layout with contiguous groups.  Returns
+ * Q4_ERR_UNSUPPORTED otherwise (AWQ layout, g_idx, odd shapes, and M large enough for the
+ * prefill GEMM, where the separate elementwise pass is the faster route): the caller then
+ * runs q4_linear into an [M, N] buffer and q4_act_mul.
+ */
+#define Q4_ACT_SILU 0       /* x * sigmoid(x) */
+#define Q4_ACT_GELU_TANH 1  /* gelu(approximate="tanh"): "gelu_fast", "gelu_pytorch_tanh" */
+#define Q4_ACT_GELU 2       /* gelu(approximate="none") */
+int q4_linear_gate_up(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                      int act, void* workspace, size_t workspace_bytes, void* stream);
+
+/* y[M, inter] = act(gate_up[:, :inter]) * gate_up[:, inter:] for gate_up [M, 2 * inter]. */
+int q4_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, void* stream);
+
+/*
  * Decode kernel with an explicit work decomposition, for tuning sweeps: `wcol` waves
  * across columns and `wk` waves across K per workgroup (wcol * wk <= 8), `splits`
  * workgroups across K, `words` packed words per lane (4, 2 or 1: column tiles of 64, 32 or

@@ -250,6 +250,44 @@ def linear_forward(x, w, bias=None, dtype="f16"):
     return y.reshape(lead + (N,)), yc.reshape(lead + (N,))
 
 
+def activation_f32(g: np.ndarray, act: str) -> np.ndarray:
+    """The reference's MLP activations in fp32 (ACT2FN / torch.nn.functional.gelu selection,
+    server/text_generation_server/models/custom_modeling/flash_llama_modeling.py:309-321):
+    "silu" = g * sigmoid(g); "gelu_tanh" = gelu(approximate="tanh"); "gelu" = erf form."""
+    g = g.astype(np.float32)
+    if act == "silu":
+        return (g / (np.float32(1.0) + np.exp(-g, dtype=np.float32))).astype(np.float32)
+    if act == "gelu_tanh":
+        inner = np.float32(0.7978845608028654) * (g + np.float32(0.044715) * g * g * g)
+        return (np.float32(0.5) * g * (np.float32(1.0) + np.tanh(inner, dtype=np.float32))).astype(np.float32)
+    if act == "gelu":
+        from math import erf
+
+        e = np.vectorize(erf, otypes=[np.float64])(g.astype(np.float64) * 0.7071067811865476)
+        return (0.5 * g.astype(np.float64) * (1.0 + e)).astype(np.float32)
+    raise ValueError(f"unknown activation {act}")
+
+
+def gate_up_forward(x, w, act="silu", bias=None, dtype="f16"):
+    """act(gate) * up of a gated MLP whose first linear packs [gate | up] along N
+    (flash_llama_modeling.py:400-404), with eager PyTorch's roundings on half tensors:
+    the linear output is rounded to `dtype`, the activation is evaluated in fp32 and
+    rounded, the product is rounded.  Returns (y_f32 from the unrounded fp32 linear output,
+    y_cast in `dtype`); both [..., N/2]."""
+    y32, yc = linear_forward(x, w, bias, dtype)
+    inter = w.shape[1] // 2
+    exact = activation_f32(y32[..., :inter], act) * y32[..., inter:]
+    yr = to_f32(yc, dtype)
+    a = activation_f32(yr[..., :inter], act)
+    if dtype == "f16":
+        a = a.astype(np.float16).astype(np.float32)
+        out = (a * yr[..., inter:]).astype(np.float16)
+    else:
+        a = bf16_bits_to_f32(f32_to_bf16_bits(a))
+        out = f32_to_bf16_bits(a * yr[..., inter:])
+    return exact, out
+
+
 # --------------------------------------------------------------------------- synthetic inputs
 
 

@@ -23,7 +23,7 @@ def declared_functions():
 def test_header_functions_are_exported_and_bound(pkg):
     lib = pkg._lib.load()
     names = declared_functions()
-    assert {"q4_dequant", "q4_linear", "q4_linear_ex", "q4_gemv_tuned", "q4_workspace_bytes",
+    assert {"q4_dequant", "q4_linear", "q4_linear_ex", "q4_gemv_tuned", "q4_linear_gate_up", "q4_act_mul", "q4_workspace_bytes",
             "q4_select_path", "q4_last_error", "q4_abi_version"} <= set(names)
     for name in names:
         assert hasattr(lib, name), f"{name} declared in q4_linear.h but not exported"

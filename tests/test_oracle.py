@@ -274,3 +274,34 @@ def test_synthetic_generators_match_config():
     assert sorted(np.bincount(gi).tolist()) == [128, 128]  # every group has exactly 128 rows
     q = o.unpack_rows(qw)
     assert q.min() == 0 and q.max() == 15
+
+
+def test_activations_known_values(oracle):
+    """Closed forms: silu(0) = 0, silu(x) + silu(-x) = x; gelu(x) - gelu(-x) = x for both
+    variants; large |x| limits; a dropped factor or sign fails one of them."""
+    x = np.linspace(-6, 6, 97, dtype=np.float32)
+    for act in ("silu", "gelu", "gelu_tanh"):
+        a = oracle.activation_f32(x, act)
+        assert a[48] == 0.0
+        assert np.allclose(a - oracle.activation_f32(-x, act), x, atol=2e-6)
+        assert abs(a[-1] - 6.0) < 2e-2 and abs(a[0]) < 2e-2
+    assert np.isclose(oracle.activation_f32(np.float32([1.0]), "silu")[0], 1.0 / (1.0 + np.exp(-1.0)), rtol=1e-6)
+    assert np.isclose(oracle.activation_f32(np.float32([1.0]), "gelu")[0], 0.8413447460685429, rtol=1e-6)
+    assert np.isclose(oracle.activation_f32(np.float32([1.0]), "gelu_tanh")[0], 0.8411919906082768, rtol=1e-6)
+
+
+def test_gate_up_forward_roundings(oracle):
+    """act(gate) * up on a hand-made case: every intermediate is rounded to fp16."""
+    w = np.zeros((2, 4), dtype=np.float16)
+    w[0, 0] = 1.0      # gate_0 = x_0
+    w[1, 1] = 1.0      # gate_1 = x_1
+    w[0, 2] = 3.0      # up_0 = 3 x_0
+    w[1, 3] = 0.5      # up_1 = x_1 / 2
+    x = np.array([[1.0, -2.0]], dtype=np.float16)
+    exact, out = oracle.gate_up_forward(x, w, "silu")
+    s1 = np.float16(1.0 / (1.0 + np.exp(-1.0)))
+    s2 = np.float16(-2.0 / (1.0 + np.exp(2.0)))
+    assert out.dtype == np.float16 and out.shape == (1, 2)
+    assert out[0, 0] == np.float16(np.float32(s1) * np.float32(3.0))
+    assert out[0, 1] == np.float16(np.float32(s2) * np.float32(-1.0))
+    assert np.allclose(exact[0], [3.0 / (1.0 + np.exp(-1.0)), 2.0 / (1.0 + np.exp(2.0))], rtol=1e-6)

@@ -9,6 +9,7 @@ on sys.path.
 
 from . import _lib, ops  # noqa: F401
 from .layers.linear import get_linear  # noqa: F401
+from .layers.mlp import gate_up_act  # noqa: F401
 from .layers.gptq import (  # noqa: F401
     GPTQWeight,
     GPTQWeightsLoader,
@@ -32,6 +33,7 @@ __all__ = [
     "ExllamaQuantLinear",
     "WQLinear",
     "get_linear",
+    "gate_up_act",
     "create_exllama_buffers",
     "set_device",
     "conversion_utils",

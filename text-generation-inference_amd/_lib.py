@@ -29,6 +29,10 @@ ERR_UNSUPPORTED = -2
 ERR_WORKSPACE = -3
 ERR_LAUNCH = -4
 
+# Q4_ACT_*: the MLP activations the fused gate_up epilogue knows, by the names the reference's
+# configs use (hidden_act)
+ACTIVATIONS = {"silu": 0, "gelu_fast": 1, "gelu_pytorch_tanh": 1, "gelu_tanh": 1, "gelu": 2}
+
 
 class Q4Weight(Structure):
     """Mirror of `struct q4_weight`."""
@@ -63,6 +67,11 @@ SIGNATURES = {
         c_int,
         [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p],
     ),
+    "q4_linear_gate_up": (
+        c_int,
+        [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "q4_act_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "q4_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "q4_select_path": (c_int, [POINTER(Q4Weight), c_int, c_int]),
 }

@@ -120,8 +120,12 @@ size_t q4_workspace_bytes(int M, int K, int N) {
       w.g_idx = variant == 2 ? &fake_idx : nullptr;  // only tested against NULL
       if (variant == 1 && N % 256 != 0) continue;
       for (int m = m_lo; m <= m_hi; ++m) {
-        const int s = gemv_pick_config(&w, m).splits;
+        int s = gemv_pick_config(&w, m).splits;
         if (s > splits) splits = s;
+        if (variant == 0 && N % 128 == 0) {  // the gated-MLP variant tiles N differently
+          s = gemv_pick_config(&w, m, true).splits;
+          if (s > splits) splits = s;
+        }
       }
     }
   }
@@ -157,6 +161,55 @@ int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, i
       set_error("q4_linear: unknown path %d", path);
       return Q4_ERR_INVALID_ARGUMENT;
   }
+}
+
+int q4_linear_gate_up(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                      int act, void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = validate_weight(w, "q4_linear_gate_up");
+  if (rc == Q4_OK) rc = validate_dtype(dtype, "q4_linear_gate_up");
+  if (rc != Q4_OK) return rc;
+  if (act != Q4_ACT_SILU && act != Q4_ACT_GELU_TANH && act != Q4_ACT_GELU) {
+    set_error("q4_linear_gate_up: unknown activation %d", act);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M < 0 || (w->N & 1)) {
+    set_error("q4_linear_gate_up: bad M=%d or odd N=%d", M, w->N);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M == 0 || w->N == 0) return Q4_OK;
+  if (y == nullptr || (x == nullptr && w->K > 0)) {
+    set_error("q4_linear_gate_up: null x or y");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  // Fused on the decode path only.  In the prefill GEMM the exp / tanh of a 256 x 256 tile
+  // would run with the matrix cores idle and the lane's gate and up columns are no longer
+  // neighbours in memory; measured slower (571 us against 476 + 36 us for the Llama-3-8B
+  // gate_up projection at M = 2048) than the GEMM followed by q4_act_mul, so the caller gets
+  // Q4_ERR_UNSUPPORTED there and runs the two kernels.
+  if (q4_select_path(w, M, dtype) == Q4_PATH_GEMV && gemv_gate_up_supported(w, M, dtype))
+    return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, nullptr, (hipStream_t)stream, act + 1);
+  set_error("q4_linear_gate_up: no fused kernel for this problem (layout=%d g_idx=%p M=%d K=%d N=%d groupsize=%d)",
+            w->layout, (const void*)w->g_idx, M, w->K, w->N, w->groupsize);
+  return Q4_ERR_UNSUPPORTED;
+}
+
+int q4_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, void* stream) {
+  int rc = validate_dtype(dtype, "q4_act_mul");
+  if (rc != Q4_OK) return rc;
+  if (act != Q4_ACT_SILU && act != Q4_ACT_GELU_TANH && act != Q4_ACT_GELU) {
+    set_error("q4_act_mul: unknown activation %d", act);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M < 0 || inter < 0) {
+    set_error("q4_act_mul: negative M=%d or intermediate size %d", M, inter);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M == 0 || inter == 0) return Q4_OK;
+  if (gate_up == nullptr || y == nullptr) {
+    set_error("q4_act_mul: null pointer");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  return launch_act_mul(gate_up, y, M, inter, dtype, act, (hipStream_t)stream);
 }
 
 int q4_linear(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,

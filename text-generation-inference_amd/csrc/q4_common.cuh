@@ -102,6 +102,37 @@ __device__ __forceinline__ uint16_t finish_output(float acc, const void* bias, i
   return y;
 }
 
+// Gated-MLP epilogue: act(gate) * up on values already rounded to the activation dtype, with
+// the roundings of the unfused sequence `act(g) * u` on half tensors (the activation is
+// evaluated in fp32 and rounded, then the product is rounded):
+// server/text_generation_server/models/custom_modeling/flash_llama_modeling.py:400-404.
+// `act` is a Q4_ACT_* value.
+template <int DTYPE>
+__device__ __forceinline__ uint16_t act_mul(uint16_t g_bits, uint16_t u_bits, int act) {
+  float g, u;
+  if constexpr (DTYPE == Q4_DTYPE_F16) {
+    g = (float)__builtin_bit_cast(half_t, g_bits);
+    u = (float)__builtin_bit_cast(half_t, u_bits);
+  } else {
+    g = bf16_bits_to_f32(g_bits);
+    u = bf16_bits_to_f32(u_bits);
+  }
+  float a;
+  if (act == Q4_ACT_SILU) {
+    a = g / (1.0f + expf(-g));
+  } else if (act == Q4_ACT_GELU_TANH) {
+    const float inner = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    a = 0.5f * g * (1.0f + tanhf(inner));
+  } else {
+    a = 0.5f * g * (1.0f + erff(g * 0.7071067811865476f));
+  }
+  const uint16_t a_bits = store_act<DTYPE>(a);
+  float ar;
+  if constexpr (DTYPE == Q4_DTYPE_F16) ar = (float)__builtin_bit_cast(half_t, a_bits);
+  else ar = bf16_bits_to_f32(a_bits);
+  return store_act<DTYPE>(ar * u);
+}
+
 // Kernel-side view of q4_weight plus the activation-side pointers.
 struct Problem {
   const uint32_t* __restrict__ qweight;
@@ -112,6 +143,10 @@ struct Problem {
   const void* __restrict__ bias;
   void* __restrict__ y;
   int M, K, N, groupsize, num_groups;
+  // 0: y[M, N] = x @ W (+ bias).  Q4_ACT_* + 1: gated-MLP epilogue, W = [gate | up] along N
+  // and y[M, N/2] = act(x @ gate (+ bias)) * (x @ up (+ bias)); only kernels that say so
+  // support it.
+  int gate_up_act;
 };
 
 }  // namespace q4
@@ -130,8 +165,12 @@ struct GemvConfig {
 };
 bool gemv_supported(const q4_weight* w, int M, int dtype);
 GemvConfig gemv_pick_config(const q4_weight* w, int M);
+GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up);
 int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
-                void* workspace, size_t workspace_bytes, const GemvConfig* cfg, hipStream_t stream);
+                void* workspace, size_t workspace_bytes, const GemvConfig* cfg, hipStream_t stream,
+                int gate_up_act = 0);
+bool gemv_gate_up_supported(const q4_weight* w, int M, int dtype);
+int launch_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, hipStream_t stream);
 bool gemm_awq_supported(const q4_weight* w, int M, int dtype);
 int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                     hipStream_t stream);

@@ -1,0 +1,790 @@
+// Decode kernels (device code shared by the translation units that instantiate them).
+//
+// Decode path: y[M, N] = x @ dequant(W) for small M (16 rows per workgroup row-chunk).
+//
+// HBM-bound: the packed weights are read exactly once with wide loads and never written
+// back.  All three kernels share one structure (wave64):
+//   * the B operand of a 16x16x32 MFMA wants, per lane, 8 consecutive K values of one
+//     column (column = lane % 16, K block = lane / 16).  The matrix core then performs both
+//     the multiply and the reduction across the four K blocks of the wave; the VALU only
+//     unpacks nibbles (about one operation per weight);
+//   * nibbles become halves by splicing them into the mantissa of 1024.0 (q4_common.cuh),
+//     zero points are subtracted exactly in fp16 and, when groups are contiguous in K, the
+//     group scale is factored out of the K sum and applied to the fp32 group accumulator;
+//   * the activation slab of the workgroup is staged once in LDS in the K order the unpack
+//     produces, so no weight is ever repacked;
+//   * split-K: `wk` waves of a workgroup take consecutive K ranges and are combined through
+//     LDS in fixed order; `splits` workgroups write fp32 partials to the workspace and the
+//     last one to arrive (ticket counter) adds them in split order and writes the output.
+//     The result is deterministic and needs no memset: the last workgroup resets its ticket.
+//
+// gemv_gptq_kernel      GPTQ layout, groups contiguous in K.  A packed word *is* one lane's
+//                       B operand; a lane loads 4 adjacent columns x 1 packed row with one
+//                       128-bit load (256-byte row segments per 16 lanes), word t feeds
+//                       MFMA t.
+// gemv_gptq_act_kernel  GPTQ layout with g_idx (act-order): every K row has its own group.
+//                       Scales and zero points of the workgroup's columns sit in an LDS
+//                       table indexed by g_idx[k]; they are applied per weight.
+// gemv_awq_kernel       AWQ layout: a word holds 8 interleaved columns of one K row.  A lane
+//                       loads an 8-row x 2-word patch and transposes nibbles in registers
+//                       (one byte permute per row pair and byte) into 16 B operands.
+//
+// Workgroup ids are laid out split-major so that all splits of a column tile land on the
+// same XCD (id % 8) and the partials stay in that XCD's L2.
+#pragma once
+
+#include "q4_common.cuh"
+
+namespace q4 {
+
+constexpr int kChunkSteps = 4;                // 32-row MFMA steps per software-pipelined chunk
+constexpr int kChunkRows = 32 * kChunkSteps;  // 128 K rows
+constexpr int kPrefetch = 4;                  // chunks of weight loads in flight per wave
+constexpr int kRowsPerBlock = 16;             // activation rows per workgroup (MFMA M)
+
+struct GemvParams {
+  Problem p;
+  float* __restrict__ partials;
+  uint32_t* __restrict__ tickets;
+  int wcol, wk, splits;
+  int slab_stride;  // bytes between activation rows in LDS
+  int slab_bytes;   // size of the activation slab region
+};
+
+// Constants of the nibble splice, hidden from constant folding (empty asm, no instruction
+// is emitted): as literals the compiler must split (w & mask) | magic into v_and + v_or
+// because a three-operand VALU instruction cannot carry a literal; as register operands it
+// selects the fused v_and_or_b32.  The asm must stay empty: an instruction inside inline
+// asm is invisible to the MFMA hazard recognizer.
+struct SpliceConsts {
+  uint32_t mask_lo, mask_hi, magic;
+};
+__device__ __forceinline__ SpliceConsts splice_consts() {
+  SpliceConsts k{0x000F000Fu, 0x00F000F0u, 0x64006400u};
+  asm volatile("" : "+s"(k.mask_lo), "+s"(k.mask_hi), "+v"(k.magic));
+  return k;
+}
+
+// Eight exact (q - z) values of one packed word, as four half2 in K order [0,4,1,5,2,6,3,7].
+// czlo = half2(-(1024 + z)), czhi = half2(-(64 + z)).
+__device__ __forceinline__ void unpack_word_f16(uint32_t w, half2_t czlo, half2_t czhi,
+                                                const SpliceConsts& k, half2_t out[4]) {
+  const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+  const uint32_t w8 = w >> 8;
+  out[0] = as_half2((w & k.mask_lo) | k.magic) + czlo;
+  out[1] = as_half2((w & k.mask_hi) | k.magic) * sixteenth + czhi;
+  out[2] = as_half2((w8 & k.mask_lo) | k.magic) + czlo;
+  out[3] = as_half2((w8 & k.mask_hi) | k.magic) * sixteenth + czhi;
+}
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
+// half2 of exact small integers -> packed bf16 pair (exact; v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t pack_bf16_pair(half2_t h) {
+  const float2_t f = {(float)h.x, (float)h.y};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+
+// One 16x16x32 MFMA; `b` holds eight weights as four half2.
+template <int DTYPE>
+__device__ __forceinline__ float4_t mfma16(const uint4_t a, const half2_t b[4], float4_t c) {
+  if constexpr (DTYPE == Q4_DTYPE_F16) {
+    uint4_t bu;
+    bu.x = as_u32(b[0]); bu.y = as_u32(b[1]); bu.z = as_u32(b[2]); bu.w = as_u32(b[3]);
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
+                                                  __builtin_bit_cast(half8_t, bu), c, 0, 0, 0);
+  } else {
+    uint4_t bb;
+    bb.x = pack_bf16_pair(b[0]);
+    bb.y = pack_bf16_pair(b[1]);
+    bb.z = pack_bf16_pair(b[2]);
+    bb.w = pack_bf16_pair(b[3]);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                   __builtin_bit_cast(bf16x8_t, bb), c, 0, 0, 0);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Work decomposition shared by the kernels.
+struct Decomp {
+  int tid, lane, wave, wc, wkk, j, kq, nthreads;
+  int tile_cols, ntiles, tile, split;
+  int KR, KW, kwg0, kw0;
+  int mb, mloc;  // first activation row of this workgroup and number of live rows (<= 16)
+};
+
+__device__ __forceinline__ Decomp make_decomp(const GemvParams& gp, int wave_cols) {
+  Decomp d;
+  d.tid = threadIdx.x;
+  d.lane = d.tid & 63;
+  d.wave = __builtin_amdgcn_readfirstlane(d.tid >> 6);  // wave-uniform: keeps index math scalar
+  d.wc = d.wave % gp.wcol;
+  d.wkk = d.wave / gp.wcol;
+  d.j = d.lane & 15;
+  d.kq = d.lane >> 4;
+  d.nthreads = blockDim.x;
+  d.tile_cols = wave_cols * gp.wcol;
+  d.ntiles = gp.p.N / d.tile_cols;
+  d.tile = blockIdx.x % d.ntiles;
+  d.split = blockIdx.x / d.ntiles;
+  d.KR = gp.p.K / gp.splits;
+  d.KW = d.KR / gp.wk;
+  d.kwg0 = d.split * d.KR;
+  d.kw0 = d.kwg0 + d.wkk * d.KW;
+  d.mb = blockIdx.y * kRowsPerBlock;
+  d.mloc = min(kRowsPerBlock, gp.p.M - d.mb);
+  return d;
+}
+
+// Activation slab [mloc][KR] -> LDS.  The global loads are issued before the weight loads
+// (memory returns in issue order, so L2 hits must not queue behind the HBM stream they are
+// needed to consume) and stored after them.  PERMUTE stores every 8-block in the K order
+// [0,4,1,5,2,6,3,7] of the GPTQ nibble splice.
+template <bool PERMUTE>
+struct SlabStager {
+  static constexpr int kLoads = 2;  // 16-byte activation loads per thread kept in flight
+  uint4_t xv[kLoads];
+  const uint16_t* xs;
+  int kb_per_row, items;
+
+  __device__ __forceinline__ uint4_t fetch(const GemvParams& gp, int idx) const {
+    const int m = idx / kb_per_row;
+    const int kb = idx - m * kb_per_row;
+    return *(const uint4_t*)(xs + (size_t)m * gp.p.K + kb * 8);
+  }
+  __device__ __forceinline__ void issue(const GemvParams& gp, const Decomp& d) {
+    xs = (const uint16_t*)gp.p.x + (size_t)d.mb * gp.p.K + d.kwg0;
+    kb_per_row = d.KR >> 3;
+    items = d.mloc * kb_per_row;
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+      const int idx = d.tid + u * d.nthreads;
+      if (idx < items) xv[u] = fetch(gp, idx);
+    }
+  }
+  __device__ __forceinline__ void put(const GemvParams& gp, unsigned char* smem, int idx,
+                                      uint4_t v) const {
+    const int m = idx / kb_per_row;
+    const int kb = idx - m * kb_per_row;
+    uint4_t o = v;
+    if constexpr (PERMUTE) {
+      o.x = (v.x & 0xFFFFu) | (v.z << 16);
+      o.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
+      o.z = (v.y & 0xFFFFu) | (v.w << 16);
+      o.w = (v.y >> 16) | (v.w & 0xFFFF0000u);
+    }
+    *(uint4_t*)(smem + (size_t)m * gp.slab_stride + kb * 16) = o;
+  }
+  __device__ __forceinline__ void store(const GemvParams& gp, const Decomp& d,
+                                        unsigned char* smem) {
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+      const int idx = d.tid + u * d.nthreads;
+      if (idx < items) put(gp, smem, idx, xv[u]);
+    }
+    for (int idx = d.tid + kLoads * d.nthreads; idx < items; idx += d.nthreads)
+      put(gp, smem, idx, fetch(gp, idx));
+  }
+};
+
+// Everything after the K loop.  out[t][r] is the fp32 sum of output row 4*kq + r (relative
+// to the workgroup's first row) and column col0 + t: every lane owns NT adjacent columns.
+// FUSE (NT = 8): gated-MLP epilogue.  out[0..3] are four gate columns col0 .. col0 + 3 and
+// out[4..7] the matching up columns N/2 + col0 ..; the output is act(gate) * up, [M, N/2].
+template <int DTYPE, int NT, int RMAX, bool FUSE = false>
+__device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& d,
+                                            float (&out)[NT][RMAX], int col0,
+                                            unsigned char* smem) {
+  const Problem& p = gp.p;
+  const int N = p.N;
+  // ---- combine the wk waves of the workgroup through LDS (fixed order)
+  if (gp.wk > 1) {
+    __syncthreads();  // everyone is done with the slab / tables
+    float* red = (float*)smem;
+    if (d.wkk > 0) {
+      float* dst = red + ((size_t)((d.wkk - 1) * gp.wcol + d.wc) * NT * RMAX) * 64 + d.lane;
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) dst[(t * RMAX + r) * 64] = out[t][r];
+    }
+    __syncthreads();
+    if (d.wkk == 0) {
+      for (int w = 1; w < gp.wk; ++w) {
+        const float* src = red + ((size_t)((w - 1) * gp.wcol + d.wc) * NT * RMAX) * 64 + d.lane;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int r = 0; r < RMAX; ++r) out[t][r] += src[(t * RMAX + r) * 64];
+      }
+    }
+  }
+
+  uint16_t* y = (uint16_t*)p.y;
+  const int half_n = N >> 1;
+  if constexpr (FUSE) {
+    if (gp.splits == 1) {
+      if (d.wkk == 0) {
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) {
+          const int m = 4 * d.kq + r;
+          if (m < d.mloc) {
+            uint32_t o[NT / 2];
+#pragma unroll
+            for (int t = 0; t < NT / 2; ++t) {
+              const uint16_t g = finish_output<DTYPE>(out[t][r], p.bias, col0 + t);
+              const uint16_t u = finish_output<DTYPE>(out[NT / 2 + t][r], p.bias, half_n + col0 + t);
+              o[t] = act_mul<DTYPE>(g, u, p.gate_up_act - 1);
+            }
+            uint2_t packed;
+            packed.x = o[0] | (o[1] << 16);
+            packed.y = o[2] | (o[3] << 16);
+            *(uint2_t*)(y + (size_t)(d.mb + m) * half_n + col0) = packed;
+          }
+        }
+      }
+      return;
+    }
+  }
+  if (gp.splits == 1) {
+    if (d.wkk == 0) {
+#pragma unroll
+      for (int r = 0; r < RMAX; ++r) {
+        const int m = 4 * d.kq + r;
+        if (m < d.mloc) {
+          uint16_t* dst = y + (size_t)(d.mb + m) * N + col0;
+          uint16_t o[NT];
+#pragma unroll
+          for (int t = 0; t < NT; ++t) o[t] = finish_output<DTYPE>(out[t][r], p.bias, col0 + t);
+          if constexpr (NT == 1) {
+            dst[0] = o[0];
+          } else if constexpr (NT == 2) {
+            *(uint32_t*)dst = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+          } else {
+#pragma unroll
+            for (int t = 0; t < NT; t += 4) {
+              uint2_t packed;
+              packed.x = (uint32_t)o[t] | ((uint32_t)o[t + 1] << 16);
+              packed.y = (uint32_t)o[t + 2] | ((uint32_t)o[t + 3] << 16);
+              *(uint2_t*)(dst + t) = packed;
+            }
+          }
+        }
+      }
+    }
+    return;
+  }
+
+  // ---- cross-workgroup split-K: write the partial, take a ticket, last one reduces.
+  // Partials and the ticket move with agent-scope relaxed atomics (coherent loads/stores
+  // that bypass the per-XCD L2 state) instead of release/acquire fences: a fence here
+  // would write back and invalidate the whole L2 once per workgroup, which costs more
+  // than the kernel itself.  Ordering comes from waiting for the stores to be
+  // acknowledged (vmcnt(0)) before the workgroup barrier that precedes the ticket.
+  if (d.wkk == 0) {
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) {
+      const int m = 4 * d.kq + r;
+      if (m < d.mloc) {
+        float* dst = gp.partials + ((size_t)d.split * p.M + d.mb + m) * N + col0;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          __hip_atomic_store(dst + (FUSE && t >= NT / 2 ? half_n + t - NT / 2 : t), out[t][r], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  __shared__ uint32_t ticket_s;
+  uint32_t* ticket = gp.tickets + blockIdx.y * d.ntiles + d.tile;
+  if (d.tid == 0) {
+    ticket_s = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (ticket_s != (uint32_t)(gp.splits - 1)) return;
+  {
+    const size_t sstride = (size_t)p.M * N;
+    // sum of the partials of one output element, in split order
+    auto total = [&](int m, int n) {
+      const float* src = gp.partials + (size_t)(d.mb + m) * N + n;
+      float sum = 0.f;
+      int sp = 0;
+      for (; sp + 8 <= gp.splits; sp += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          v[u] = __hip_atomic_load(src + (size_t)(sp + u) * sstride, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += v[u];
+      }
+      for (; sp < gp.splits; ++sp)
+        sum += __hip_atomic_load(src + (size_t)sp * sstride, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+      return sum;
+    };
+    if constexpr (FUSE) {
+      // the tile holds tile_cols / 2 gate columns and as many up columns
+      const int half_cols = d.tile_cols >> 1;
+      const int items = d.mloc * half_cols;
+      for (int idx = d.tid; idx < items; idx += d.nthreads) {
+        const int m = idx / half_cols;
+        const int n = d.tile * half_cols + (idx - m * half_cols);
+        const uint16_t g = finish_output<DTYPE>(total(m, n), p.bias, n);
+        const uint16_t u = finish_output<DTYPE>(total(m, half_n + n), p.bias, half_n + n);
+        y[(size_t)(d.mb + m) * half_n + n] = act_mul<DTYPE>(g, u, p.gate_up_act - 1);
+      }
+    } else {
+      const int items = d.mloc * d.tile_cols;
+      const int nbase = d.tile * d.tile_cols;
+      for (int idx = d.tid; idx < items; idx += d.nthreads) {
+        const int m = idx / d.tile_cols;
+        const int n = nbase + (idx - m * d.tile_cols);
+        y[(size_t)(d.mb + m) * N + n] = finish_output<DTYPE>(total(m, n), p.bias, n);
+      }
+    }
+    if (d.tid == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// GPTQ, contiguous groups.
+// GSTEPS: MFMA steps (32 rows) per quantisation group inside a chunk: 1, 2 or 4.
+// STATIC128: groupsize is exactly 128, so every chunk is one whole group.
+// WORDS: adjacent packed words (columns) per lane: 4, 2 or 1, i.e. column tiles of 64, 32
+// or 16 per wave.  Narrow tiles give enough workgroups to fill the chip without splitting
+// K across workgroups, which removes the cross-workgroup reduction tail of small layers.
+// FUSE (WORDS = 8): gated-MLP epilogue, W = [gate | up] along N.  The lane's eight words are
+// four neighbouring gate columns and the four up columns N/2 further (two 128-bit loads per
+// packed row); a wave covers 64 gate and 64 up columns, and the activation and the product
+// happen in the lane that owns both sums.
+template <int DTYPE, int RMAX, int GSTEPS, bool STATIC128, int WORDS, bool FUSE = false>
+__global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
+  static_assert(FUSE == (WORDS == 8), "eight words per lane = four gate + four up columns (fused only)");
+  extern __shared__ __align__(16) unsigned char smem[];
+  const Problem& p = gp.p;
+  const Decomp d = make_decomp(gp, 16 * WORDS);
+  const int N = p.N;
+  // lane's first column (fused: its first gate column)
+  const int nl = FUSE ? d.tile * (d.tile_cols >> 1) + d.wc * 64 + 4 * d.j
+                      : d.tile * d.tile_cols + d.wc * 16 * WORDS + WORDS * d.j;
+  const size_t up_cols = (size_t)(N >> 1);  // distance from a gate column to its up column
+  const int nchunks = d.KW / kChunkRows;
+  constexpr int GPC = kChunkSteps / GSTEPS;  // groups per chunk
+  constexpr int PF = kPrefetch * 4 / WORDS;  // chunks in flight: same bytes for every WORDS
+
+  SlabStager<true> slab;
+  slab.issue(gp, d);
+
+  // ---- issue the first PF chunks of weight loads.  Addresses are a wave-uniform 64-bit
+  // base plus a per-lane 32-bit byte offset.
+  const char* wbase = (const char*)(p.qweight + (size_t)(d.kw0 / 8) * N);
+  const uint32_t w_lane = ((uint32_t)d.kq * (uint32_t)N + (uint32_t)nl) * 4u;
+  const size_t step_bytes = (size_t)N * 16;  // four packed rows
+  const uint32_t s_lane = (uint32_t)nl * 2u;
+  const uint32_t z_lane = (uint32_t)(nl >> 3) * 4u;
+  const int zshift = (nl & 7) * 4;
+  struct Words { uint32_t v[WORDS]; };
+  struct Scales { uint32_t v[(WORDS + 1) / 2]; };  // WORDS fp16 scales
+  struct Zeros { uint32_t v[FUSE ? 2 : 1]; };      // packed zero points (fused: gate, up)
+  Words wq[PF][kChunkSteps];
+  Scales sc[PF][GPC];
+  Zeros zw[PF][GPC];
+  auto load_words = [&](const char* addr) {
+    Words r;
+    if constexpr (FUSE) {
+      const uint4_t g = __builtin_nontemporal_load((const uint4_t*)addr);
+      const uint4_t u = __builtin_nontemporal_load((const uint4_t*)(addr + up_cols * 4));
+      r.v[0] = g.x; r.v[1] = g.y; r.v[2] = g.z; r.v[3] = g.w;
+      r.v[4] = u.x; r.v[5] = u.y; r.v[6] = u.z; r.v[7] = u.w;
+    } else if constexpr (WORDS == 4) {
+      const uint4_t t = __builtin_nontemporal_load((const uint4_t*)addr);
+      r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w;
+    } else if constexpr (WORDS == 2) {
+      const uint2_t t = __builtin_nontemporal_load((const uint2_t*)addr);
+      r.v[0] = t.x; r.v[1] = t.y;
+    } else {
+      r.v[0] = __builtin_nontemporal_load((const uint32_t*)addr);
+    }
+    return r;
+  };
+  auto load_chunk = [&](int c, Words (&w)[kChunkSteps], Scales (&s)[GPC], Zeros (&z)[GPC]) {
+#pragma unroll
+    for (int st = 0; st < kChunkSteps; ++st)
+      w[st] = load_words(wbase + (size_t)(c * kChunkSteps + st) * step_bytes + w_lane);
+#pragma unroll
+    for (int g = 0; g < GPC; ++g) {
+      int gi = (d.kw0 + c * kChunkRows + g * GSTEPS * 32) / p.groupsize;
+      gi = min(gi, p.num_groups - 1);
+      const char* sp = (const char*)p.scales + (size_t)gi * N * 2 + s_lane;
+      if constexpr (FUSE) {
+        const uint2_t tg = *(const uint2_t*)sp;
+        const uint2_t tu = *(const uint2_t*)(sp + up_cols * 2);
+        s[g].v[0] = tg.x; s[g].v[1] = tg.y; s[g].v[2] = tu.x; s[g].v[3] = tu.y;
+      } else if constexpr (WORDS == 4) {
+        const uint2_t t = *(const uint2_t*)sp;
+        s[g].v[0] = t.x; s[g].v[1] = t.y;
+      } else if constexpr (WORDS == 2) {
+        s[g].v[0] = *(const uint32_t*)sp;
+      } else {
+        s[g].v[0] = *(const uint16_t*)sp;
+      }
+      const char* zp = (const char*)p.qzeros + (size_t)gi * (N >> 3) * 4 + z_lane;
+      z[g].v[0] = *(const uint32_t*)zp;
+      if constexpr (FUSE) z[g].v[1] = *(const uint32_t*)(zp + (up_cols >> 3) * 4);
+    }
+  };
+#pragma unroll
+  for (int b = 0; b < PF; ++b)
+    if (b < nchunks) load_chunk(b, wq[b], sc[b], zw[b]);
+
+  slab.store(gp, d, smem);
+  __syncthreads();
+
+  const bool row_live = d.j < d.mloc;  // A-operand row of this lane
+  const unsigned char* a_base =
+      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.wkk * d.KW + d.kq * 8) * 2;
+
+  const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  float4_t tot[WORDS], acc[WORDS];
+#pragma unroll
+  for (int t = 0; t < WORDS; ++t) tot[t] = acc[t] = zero4;
+  half2_t czlo[WORDS], czhi[WORDS];
+  const SpliceConsts splice = splice_consts();
+
+  auto process_chunk = [&](int c, const Words (&w)[kChunkSteps], const Scales (&s)[GPC],
+                           const Zeros (&z)[GPC]) {
+    const int kc = d.kw0 + c * kChunkRows;
+    bool group_start = true, group_end = true;
+    if constexpr (!STATIC128 && GSTEPS == kChunkSteps) {
+      group_start = (c == 0) || (kc % p.groupsize == 0);
+      group_end = (c == nchunks - 1) || ((kc + kChunkRows) % p.groupsize == 0);
+    }
+#pragma unroll
+    for (int st = 0; st < kChunkSteps; ++st) {
+      const int gi = st / GSTEPS;
+      const bool first = (st % GSTEPS) == 0;
+      const bool last = (st % GSTEPS) == GSTEPS - 1;
+      constexpr bool kStaticGroups = STATIC128 || GSTEPS != kChunkSteps;
+      if (first && (kStaticGroups || group_start)) {
+        // zero-point constants of the group: z = (stored + 1) & 15 per column
+        // (N/2 is a multiple of 8, so the up columns sit at the same nibbles of their word)
+        const uint32_t z4 = gptq_zero_plus_one(z[gi].v[0]) >> zshift;
+        uint32_t z4u = 0;
+        if constexpr (FUSE) z4u = gptq_zero_plus_one(z[gi].v[1]) >> zshift;
+#pragma unroll
+        for (int t = 0; t < WORDS; ++t) {
+          const uint32_t zz = FUSE && t >= 4 ? (z4u >> (4 * (t - 4))) & 0xFu : (z4 >> (4 * t)) & 0xFu;
+          czlo[t] = as_half2(0xE400E400u | zz | (zz << 16));        // -(1024 + z)
+          czhi[t] = as_half2(0xD400D400u | (zz << 4) | (zz << 20));  // -(64 + z)
+        }
+      }
+      uint4_t a = {0u, 0u, 0u, 0u};
+      if (row_live) a = *(const uint4_t*)(a_base + (size_t)(c * kChunkRows + st * 32) * 2);
+#pragma unroll
+      for (int t = 0; t < WORDS; ++t) {
+        half2_t b[4];
+        unpack_word_f16(w[st].v[t], czlo[t], czhi[t], splice, b);
+        if (first && kStaticGroups) {
+          acc[t] = mfma16<DTYPE>(a, b, zero4);
+        } else {
+          if (first && group_start) acc[t] = zero4;
+          acc[t] = mfma16<DTYPE>(a, b, acc[t]);
+        }
+      }
+      if (last && (kStaticGroups || group_end)) {
+#pragma unroll
+        for (int t = 0; t < WORDS; ++t) {
+          const half2_t pr = as_half2(s[gi].v[t >> 1]);
+          const float sf = (float)((t & 1) ? pr.y : pr.x);
+#pragma unroll
+          for (int r = 0; r < RMAX; ++r) tot[t][r] = fmaf(sf, acc[t][r], tot[t][r]);
+        }
+      }
+    }
+  };
+
+  // ring of PF chunk buffers: consume slot b, then refill it with chunk c + PF
+  for (int c0 = 0; c0 < nchunks; c0 += PF) {
+#pragma unroll
+    for (int b = 0; b < PF; ++b) {
+      const int c = c0 + b;
+      if (c < nchunks) {
+        process_chunk(c, wq[b], sc[b], zw[b]);
+        if (c + PF < nchunks) load_chunk(c + PF, wq[b], sc[b], zw[b]);
+      }
+    }
+  }
+
+  float out[WORDS][RMAX];
+#pragma unroll
+  for (int t = 0; t < WORDS; ++t)
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) out[t][r] = tot[t][r];
+  gemv_finish<DTYPE, WORDS, RMAX, FUSE>(gp, d, out, nl, smem);
+}
+
+// ---------------------------------------------------------------------------------------
+// GPTQ with g_idx (act-order), fp16.  LDS: [slab][g_idx slice as uint16][table G x tile_cols].
+// Table entry (g, column) = fp16 scale | fp16 -(1024 + zero) << 16.
+template <int RMAX>
+__global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const Problem& p = gp.p;
+  const Decomp d = make_decomp(gp, 64);
+  const int N = p.N;
+  const int nl = d.tile * d.tile_cols + d.wc * 64 + 4 * d.j;
+  const int nsteps = d.KW / 32;
+  constexpr int PF = 8;  // 32-row steps of weight loads in flight per wave
+
+  SlabStager<true> slab;
+  slab.issue(gp, d);
+
+  const char* wbase = (const char*)(p.qweight + (size_t)(d.kw0 / 8) * N);
+  const uint32_t w_lane = ((uint32_t)d.kq * (uint32_t)N + (uint32_t)nl) * 4u;
+  const size_t step_bytes = (size_t)N * 16;
+  uint4_t wq[PF];
+  auto load_step = [&](int st) {
+    return __builtin_nontemporal_load((const uint4_t*)(wbase + (size_t)st * step_bytes + w_lane));
+  };
+#pragma unroll
+  for (int b = 0; b < PF; ++b)
+    if (b < nsteps) wq[b] = load_step(b);
+
+  slab.store(gp, d, smem);
+
+  // ---- g_idx slice of this workgroup, clamped to the table, as uint16
+  uint16_t* gidx_s = (uint16_t*)(smem + gp.slab_bytes);
+  for (int i = d.tid; i < d.KR; i += d.nthreads) {
+    int g = p.g_idx[d.kwg0 + i];
+    g = min(max(g, 0), p.num_groups - 1);
+    gidx_s[i] = (uint16_t)g;
+  }
+  // ---- scale / zero table of the workgroup's columns, all groups
+  uint32_t* table = (uint32_t*)(smem + gp.slab_bytes + ((d.KR * 2 + 15) & ~15));
+  const int tc = d.tile_cols;
+  {
+    const int nbase = d.tile * tc;
+    const int words_per_row = tc >> 3;  // one qzeros word covers 8 columns
+    for (int i = d.tid; i < p.num_groups * words_per_row; i += d.nthreads) {
+      const int g = i / words_per_row;
+      const int c8 = i - g * words_per_row;
+      const uint32_t z8 = gptq_zero_plus_one(p.qzeros[(size_t)g * (N >> 3) + (nbase >> 3) + c8]);
+      const uint4_t s8 = *(const uint4_t*)(p.scales + (size_t)g * N + nbase + c8 * 8);
+      const uint32_t su[4] = {s8.x, s8.y, s8.z, s8.w};
+      uint32_t e[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const uint32_t s16 = (u & 1) ? (su[u >> 1] >> 16) : (su[u >> 1] & 0xFFFFu);
+        const uint32_t z = (z8 >> (4 * u)) & 0xFu;
+        e[u] = s16 | ((0xE400u | z) << 16);
+      }
+      uint4_t* dst = (uint4_t*)(table + (size_t)g * tc + c8 * 8);
+      dst[0] = uint4_t{e[0], e[1], e[2], e[3]};
+      dst[1] = uint4_t{e[4], e[5], e[6], e[7]};
+    }
+  }
+  __syncthreads();
+
+  const bool row_live = d.j < d.mloc;
+  const unsigned char* a_base =
+      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.wkk * d.KW + d.kq * 8) * 2;
+  const uint16_t* g_base = gidx_s + d.wkk * d.KW + d.kq * 8;
+  const uint32_t* t_lane = table + d.wc * 64 + 4 * d.j;
+
+  const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  float4_t acc[4] = {zero4, zero4, zero4, zero4};
+  const SpliceConsts splice = splice_consts();
+
+  auto process_step = [&](int st, const uint4_t w) {
+    uint4_t a = {0u, 0u, 0u, 0u};
+    if (row_live) a = *(const uint4_t*)(a_base + (size_t)st * 64);
+    // groups of the 8 rows of this lane's K block, then their table rows (4 columns each)
+    const uint4_t g8 = *(const uint4_t*)(g_base + st * 32);
+    const uint32_t gw[4] = {g8.x, g8.y, g8.z, g8.w};
+    uint32_t e[8][4];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const uint32_t g = (r & 1) ? (gw[r >> 1] >> 16) : (gw[r >> 1] & 0xFFFFu);
+      const uint4_t row = *(const uint4_t*)(t_lane + (size_t)g * tc);
+      e[r][0] = row.x; e[r][1] = row.y; e[r][2] = row.z; e[r][3] = row.w;
+    }
+    const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      half2_t b[4];
+#pragma unroll
+      for (int pr = 0; pr < 4; ++pr) {
+        // rows pr and pr + 4 of the K block share one splice (nibbles 16 bits apart)
+        const uint32_t ea = e[pr][t], eb = e[pr + 4][t];
+        const uint32_t s2 = (ea & 0xFFFFu) | (eb << 16);
+        const uint32_t c2 = (ea >> 16) | (eb & 0xFFFF0000u);
+        const uint32_t q2 = ((words[t] >> (4 * pr)) & splice.mask_lo) | splice.magic;
+        const half2_t dq = as_half2(q2) + as_half2(c2);  // exact q - z
+        b[pr] = dq * as_half2(s2);                       // one fp16 rounding, as the reference
+      }
+      // b is in K order [0,4,1,5,2,6,3,7], the order of the staged activations
+      acc[t] = mfma16<Q4_DTYPE_F16>(a, b, acc[t]);
+    }
+  };
+
+  for (int s0 = 0; s0 < nsteps; s0 += PF) {
+#pragma unroll
+    for (int b = 0; b < PF; ++b) {
+      const int st = s0 + b;
+      if (st < nsteps) {
+        process_step(st, wq[b]);
+        if (st + PF < nsteps) wq[b] = load_step(st + PF);
+      }
+    }
+  }
+
+  float out[4][RMAX];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) out[t][r] = acc[t][r];
+  gemv_finish<Q4_DTYPE_F16, 4, RMAX>(gp, d, out, nl, smem);
+}
+
+// ---------------------------------------------------------------------------------------
+// AWQ layout.  Wave tile: 256 columns (32 packed words) x 32 rows per step; lane (j, kq)
+// loads words [8 rows of K block kq][2 adjacent words] and owns the 16 adjacent columns
+// starting at 8 * (first word of the wave + 2 j).
+template <int DTYPE, int RMAX>
+__global__ __launch_bounds__(512) void gemv_awq_kernel(GemvParams gp) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const Problem& p = gp.p;
+  const Decomp d = make_decomp(gp, 256);
+  const int N = p.N;
+  const int NC = N >> 3;                                             // packed words per row
+  const int cw = (d.tile * d.tile_cols + d.wc * 256) / 8 + 2 * d.j;  // first of this lane's 2 words
+  const int col0 = cw * 8;
+  const int nsteps = d.KW / 32;
+  constexpr int PF = 3;  // 32-row steps (8 x 64-bit loads each) in flight per wave
+
+  SlabStager<false> slab;
+  slab.issue(gp, d);
+
+  const char* wbase = (const char*)(p.qweight + (size_t)d.kw0 * NC);
+  const uint32_t w_lane = ((uint32_t)(d.kq * 8) * (uint32_t)NC + (uint32_t)cw) * 4u;
+  const size_t row_bytes = (size_t)NC * 4;
+  uint2_t wq[PF][8];
+  auto load_step = [&](int st, uint2_t (&w)[8]) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+      w[r] = __builtin_nontemporal_load(
+          (const uint2_t*)(wbase + (size_t)(st * 32 + r) * row_bytes + w_lane));
+  };
+#pragma unroll
+  for (int b = 0; b < PF; ++b)
+    if (b < nsteps) load_step(b, wq[b]);
+
+  slab.store(gp, d, smem);
+  __syncthreads();
+
+  const bool row_live = d.j < d.mloc;
+  const unsigned char* a_base =
+      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.wkk * d.KW + d.kq * 8) * 2;
+
+  const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  float4_t acc[16];
+  float tot[16][RMAX];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    acc[t] = zero4;
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) tot[t][r] = 0.f;
+  }
+  half2_t cz[2][8];  // per word h and nibble position: -(1024 + z) (even) or -(64 + z) (odd)
+  const SpliceConsts splice = splice_consts();
+  const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+
+  auto flush = [&](int g) {
+    // scales of the lane's 16 columns: position pos of word h is column 8h + awq_order(pos)
+    const uint4_t* sp = (const uint4_t*)(p.scales + (size_t)g * N + col0);
+    const uint4_t s0 = sp[0], s1 = sp[1];
+    const uint32_t su[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int pos = 0; pos < 8; ++pos) {
+        const int col = 8 * h + (((pos & 3) << 1) | (pos >> 2));
+        const half2_t pr = as_half2(su[col >> 1]);
+        const float sf = (float)((col & 1) ? pr.y : pr.x);
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r)
+          tot[h * 8 + pos][r] = fmaf(sf, acc[h * 8 + pos][r], tot[h * 8 + pos][r]);
+      }
+  };
+
+  auto process_step = [&](int st, const uint2_t (&w)[8]) {
+    const int k = d.kw0 + st * 32;
+    const int g = min(k / p.groupsize, p.num_groups - 1);
+    const bool group_start = (st == 0) || (k % p.groupsize == 0);
+    const bool group_end = (st == nsteps - 1) || ((k + 32) % p.groupsize == 0);
+    if (group_start) {
+      const uint2_t zw = *(const uint2_t*)(p.qzeros + (size_t)g * NC + cw);
+      const uint32_t zz[2] = {zw.x, zw.y};
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int pos = 0; pos < 8; ++pos) {
+          const uint32_t z = (zz[h] >> (4 * pos)) & 0xFu;  // AWQ zero points are used as stored
+          cz[h][pos] = (pos & 1) ? as_half2(0xD400D400u | (z << 4) | (z << 20))
+                                 : as_half2(0xE400E400u | z | (z << 16));
+        }
+#pragma unroll
+      for (int t = 0; t < 16; ++t) acc[t] = zero4;
+    }
+    uint4_t a = {0u, 0u, 0u, 0u};
+    if (row_live) a = *(const uint4_t*)(a_base + (size_t)st * 64);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      half2_t b[8][4];  // [nibble position][row pair]
+#pragma unroll
+      for (int rp = 0; rp < 4; ++rp) {
+        const uint32_t w0 = h == 0 ? w[2 * rp].x : w[2 * rp].y;
+        const uint32_t w1 = h == 0 ? w[2 * rp + 1].x : w[2 * rp + 1].y;
+#pragma unroll
+        for (int by = 0; by < 4; ++by) {
+          // byte `by` of both rows side by side: low nibble = position 2*by, high = 2*by + 1
+          const uint32_t sel = 0x0C000C00u | (uint32_t)by | ((uint32_t)(4 + by) << 16);
+          const uint32_t t2 = __builtin_amdgcn_perm(w1, w0, sel);
+          b[2 * by][rp] = as_half2((t2 & splice.mask_lo) | splice.magic) + cz[h][2 * by];
+          b[2 * by + 1][rp] =
+              as_half2((t2 & splice.mask_hi) | splice.magic) * sixteenth + cz[h][2 * by + 1];
+        }
+      }
+#pragma unroll
+      for (int pos = 0; pos < 8; ++pos) acc[h * 8 + pos] = mfma16<DTYPE>(a, b[pos], acc[h * 8 + pos]);
+    }
+    if (group_end) flush(g);
+  };
+
+  for (int s0 = 0; s0 < nsteps; s0 += PF) {
+#pragma unroll
+    for (int b = 0; b < PF; ++b) {
+      const int st = s0 + b;
+      if (st < nsteps) {
+        process_step(st, wq[b]);
+        if (st + PF < nsteps) load_step(st + PF, wq[b]);
+      }
+    }
+  }
+
+  // accumulator (h, pos) is column 8h + awq_order(pos) of the lane's 16
+  float out[16][RMAX];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int pos = 0; pos < 8; ++pos)
+#pragma unroll
+      for (int r = 0; r < RMAX; ++r)
+        out[8 * h + (((pos & 3) << 1) | (pos >> 2))][r] = tot[h * 8 + pos][r];
+  gemv_finish<DTYPE, 16, RMAX>(gp, d, out, col0, smem);
+}
+
+}  // namespace q4

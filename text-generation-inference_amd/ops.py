@@ -220,6 +220,76 @@ def linear(
     return y
 
 
+def act_mul(gate_up: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """act(gate_up[:, :I]) * gate_up[:, I:] for a contiguous [M, 2I] fp16/bf16 tensor."""
+    _require_cuda(gate_up, "gate_up")
+    if gate_up.dtype not in _DTYPES:
+        raise TypeError(f"gate_up must be float16 or bfloat16, got {gate_up.dtype}")
+    if gate_up.dim() != 2 or gate_up.shape[1] % 2:
+        raise ValueError(f"gate_up must be [M, 2I], got {tuple(gate_up.shape)}")
+    if act not in _lib.ACTIVATIONS:
+        raise ValueError(f"unknown activation {act!r}; known: {sorted(_lib.ACTIVATIONS)}")
+    gate_up = gate_up.contiguous()
+    M, inter = gate_up.shape[0], gate_up.shape[1] // 2
+    y = out if out is not None else torch.empty((M, inter), dtype=gate_up.dtype, device=gate_up.device)
+    if tuple(y.shape) != (M, inter) or y.dtype != gate_up.dtype or not y.is_contiguous():
+        raise ValueError(f"out must be a contiguous [{M}, {inter}] {gate_up.dtype} tensor")
+    with torch.cuda.device(gate_up.device):
+        _lib.check(_lib.load().q4_act_mul(gate_up.data_ptr(), y.data_ptr(), M, inter, _DTYPES[gate_up.dtype],
+                                          _lib.ACTIVATIONS[act], _stream_handle(gate_up.device)))
+    return y
+
+
+def linear_gate_up(
+    w: PackedWeight,
+    x: torch.Tensor,
+    act: str = "silu",
+    bias: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+    fused: Optional[bool] = None,
+) -> torch.Tensor:
+    """y[M, N/2] = act(x @ W[:, :N/2]) * (x @ W[:, N/2:]) for a weight that packs [gate | up].
+
+    One launch where a fused kernel covers the weight (GPTQ layout with contiguous groups);
+    otherwise the linear kernel followed by the elementwise act_mul kernel.  `fused`
+    forces one of the two (True raises if there is no fused kernel).
+    """
+    _require_cuda(x, "x")
+    _require_cuda(w.qweight, "qweight")
+    if x.dtype not in _DTYPES:
+        raise TypeError(f"x must be float16 or bfloat16, got {x.dtype}")
+    if x.dim() != 2 or x.shape[1] != w.K:
+        raise ValueError(f"x must be [M, {w.K}], got {tuple(x.shape)}")
+    if w.N % 2:
+        raise ValueError(f"N={w.N} cannot hold a gate and an up half")
+    if act not in _lib.ACTIVATIONS:
+        raise ValueError(f"unknown activation {act!r}; known: {sorted(_lib.ACTIVATIONS)}")
+    x = x.contiguous()
+    M, inter = x.shape[0], w.N // 2
+    y = out if out is not None else torch.empty((M, inter), dtype=x.dtype, device=x.device)
+    if tuple(y.shape) != (M, inter) or y.dtype != x.dtype or y.device != x.device or not y.is_contiguous():
+        raise ValueError(f"out must be a contiguous [{M}, {inter}] {x.dtype} tensor on {x.device}")
+    if M == 0 or inter == 0:
+        return y
+    fusable_bias = bias is None or (bias.dtype == x.dtype and bias.is_cuda and bias.numel() == w.N)
+    if fused is not False and fusable_bias:
+        lib = _lib.load()
+        with torch.cuda.device(x.device):
+            stream = _stream_handle(x.device)
+            ws = reserve_workspace(x.device, workspace_bytes(M, w.K, w.N), stream)
+            st = w.struct()
+            rc = lib.q4_linear_gate_up(
+                ctypes.byref(st), x.data_ptr(), bias.contiguous().data_ptr() if bias is not None else None,
+                y.data_ptr(), M, _DTYPES[x.dtype], _lib.ACTIVATIONS[act], ws.data_ptr(), ws.numel(), stream,
+            )
+        if rc != _lib.ERR_UNSUPPORTED or fused:
+            _lib.check(rc)
+            return y
+    elif fused:
+        raise ValueError("the fused kernel needs a bias of x's dtype with N entries (or none)")
+    return act_mul(linear(w, x, bias), act, out=y)
+
+
 def select_path(w: PackedWeight, M: int, dtype: torch.dtype = torch.float16) -> str:
     st = w.struct()
     rc = _lib.load().q4_select_path(ctypes.byref(st), int(M), _DTYPES[dtype])
