@@ -61,6 +61,8 @@ def parse_args():
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--gemm-m", type=int, default=2048)
     ap.add_argument("--copies", type=int, default=0, help="weight copies to rotate over (0 = auto)")
+    ap.add_argument("--no-dense-ref", action="store_true",
+                    help="skip timing torch's dense fp16 matmul (hipBLASLt) on the GEMM shapes")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="eager launches only (a 256 MiB copy kernel, then each decode shape and one GEMM), "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs; prints no JSON line")
@@ -318,6 +320,14 @@ def main():
                         "frac_of_mfma_peak": round(fl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)}
             tot_f += fl
             tot_t += avg
+            if not args.no_dense_ref:
+                # context, not the product: the vendor library's dense fp16 GEMM on the same
+                # shape and box (weights already dequantized, 4x the weight bytes), timed the same way
+                dense = [torch.randn((K, N), device=dev, dtype=torch.float16) * 0.02 for _ in range(2)]
+                dfns = [(lambda c=c: torch.matmul(xg, dense[c], out=yg)) for c in range(2)]
+                davg, _ = time_kernel_launches(torch, dfns, 20)
+                gm[name]["dense_fp16_matmul_TFLOPs"] = round(fl / davg / 1e12, 1)
+                del dense
             del xg, yg
         if gm:
             out["gemm"] = {
