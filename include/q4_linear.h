@@ -82,9 +82,10 @@ int q4_dequant(const q4_weight* w, void* w_out, int dtype, void* stream);
  * server/text_generation_server/layers/awq/quantize/cuda.py:45-47).
  *
  * workspace: device buffer of at least q4_workspace_bytes(M, K, N) bytes whose first
- * Q4_WORKSPACE_COUNTER_BYTES bytes were zero before the first call that used it; the
- * kernels leave them zero again.  Calls that share a workspace must be ordered on
- * one stream.
+ * Q4_WORKSPACE_COUNTER_BYTES bytes (split-K tickets, then fixed-point accumulation cells)
+ * were zero before the first call that used it; the kernels leave them zero again.  The
+ * rest holds fp32 partial sums and needs no initialisation.  Calls that share a workspace
+ * must be ordered on one stream.
  */
 int q4_linear(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
               void* workspace, size_t workspace_bytes, void* stream);
@@ -135,7 +136,9 @@ int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, 
  * server/text_generation_server/layers/gptq/exllamav2.py:233-240
  * (temp_dq_size / temp_fwd_size / scratch_space_fixed).
  */
-#define Q4_WORKSPACE_COUNTER_BYTES 16384
+#define Q4_WORKSPACE_TICKET_BYTES 16384   /* split-K arrival tickets, one per column tile */
+#define Q4_WORKSPACE_CELL_BYTES 1048576   /* 64-bit fixed-point accumulation cells (fp16 decode, few rows) */
+#define Q4_WORKSPACE_COUNTER_BYTES 1064960 /* = tickets + cells: the part that must start zero */
 size_t q4_workspace_bytes(int M, int K, int N);
 
 /* The Q4_PATH_* value q4_linear would take for this problem (negative on bad arguments). */

@@ -102,6 +102,48 @@ def test_gemv_deterministic_and_tickets_reset(pkg, oracle, gpu):
         assert int(ws[: pkg._lib.WORKSPACE_COUNTER_BYTES].sum().item()) == 0
 
 
+@pytest.mark.parametrize("K,N", [(4096, 4096), (14336, 4096), (4096, 6144), (8192, 1024)])
+def test_gemv_single_row_fixed_point_combine(pkg, oracle, gpu, K, N):
+    """M = 1, fp16: the K splits meet in 64-bit fixed-point cells (integer adds, so the sum does
+    not depend on arrival order).  Bit-reproducible, cells back at zero, and the same row
+    computed through the ticket path (the row duplicated to M = 2) agrees to fp16 rounding."""
+    qw, qz, sc, _ = oracle.make_gptq(K, N, 128, seed=K + N, sym=False)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
+    x = to_dev(oracle.make_x(1, K, seed=5), gpu)
+    a = pkg.ops.linear(pk, x, None, path=1)
+    b = pkg.ops.linear(pk, x, None, path=1)
+    two = pkg.ops.linear(pk, torch.cat([x, x]), None, path=1)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    for ws in pkg.ops._workspaces.values():
+        assert int(ws[: pkg._lib.WORKSPACE_COUNTER_BYTES].sum().item()) == 0
+    w = oracle.dequant_gptq(qw, qz, sc, None, 128, "f16")
+    y32, _ = oracle.linear_forward(x.cpu().numpy(), w, None, "f16")
+    assert max_rel_err(to_f32(a), y32) <= TOL
+    assert max_rel_err(to_f32(a), to_f32(two[:1])) <= 1e-3
+    assert float((a == two[:1]).float().mean()) > 0.9
+
+
+def test_gemv_single_row_non_finite_input_leaves_the_cells_clean(pkg, oracle, gpu):
+    """inf / NaN activations in different K splits make every output non-finite (as in the
+    reference; opposite infinities must not cancel) and must not leave anything behind in the
+    accumulation cells: the next call is exact again."""
+    K, N = 4096, 4096
+    qw, qz, sc, _ = oracle.make_gptq(K, N, 128, seed=3, sym=False)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
+    good = to_dev(oracle.make_x(1, K, seed=8), gpu)
+    want = pkg.ops.linear(pk, good, None, path=1).clone()
+    bad = good.clone()
+    bad[0, 5] = float("inf")
+    bad[0, 4000] = float("nan")
+    y = pkg.ops.linear(pk, bad, None, path=1)
+    torch.cuda.synchronize()
+    assert not bool(torch.isfinite(y).any())
+    for ws in pkg.ops._workspaces.values():
+        assert int(ws[: pkg._lib.WORKSPACE_COUNTER_BYTES].sum().item()) == 0
+    assert torch.equal(pkg.ops.linear(pk, good, None, path=1), want)
+
+
 @pytest.mark.parametrize("layout,act", [("gptq", True), ("awq", False), ("gptq", False)])
 @pytest.mark.parametrize("M", [1, 5, 33])
 def test_generic_path(pkg, oracle, gpu, layout, act, M):

@@ -23,12 +23,12 @@ bool gemv_supported(const q4_weight* w, int M, int dtype) {
   if (w->layout == Q4_LAYOUT_AWQ) {
     if (w->N % 256 != 0 || w->groupsize % 32 != 0) return false;
     if ((long)w->num_groups * w->groupsize < w->K) return false;
-    return chunks * (w->N / 256) <= Q4_WORKSPACE_COUNTER_BYTES / 4;
+    return chunks * (w->N / 256) <= Q4_WORKSPACE_TICKET_BYTES / 4;
   }
   if (w->N % 64 != 0) return false;
   // one ticket per (row chunk, column tile); the narrowest tile of each kernel decides
   const long tile = w->g_idx != nullptr ? 64 : 16;
-  if (chunks * (w->N / tile) > Q4_WORKSPACE_COUNTER_BYTES / 4 && M > 16) return false;
+  if (chunks * (w->N / tile) > Q4_WORKSPACE_TICKET_BYTES / 4 && M > 16) return false;
   if (w->g_idx != nullptr) {
     // act-order: the table of all groups for 64 columns must fit LDS next to the slab
     if (dtype != Q4_DTYPE_F16) return false;
@@ -182,7 +182,7 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
     return Q4_ERR_INVALID_ARGUMENT;
   }
   const int ntiles = w->N / (wave_cols * cfg.wcol);
-  if ((long)ntiles * mchunks > Q4_WORKSPACE_COUNTER_BYTES / 4) {
+  if ((long)ntiles * mchunks > Q4_WORKSPACE_TICKET_BYTES / 4) {
     set_error("q4_linear(gemv): too many tiles (%d x %d)", ntiles, mchunks);
     return Q4_ERR_UNSUPPORTED;
   }
@@ -206,6 +206,14 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.wcol = cfg.wcol;
   gp.wk = cfg.wk;
   gp.splits = cfg.splits;
+  // fp16, one row, plain epilogue, four columns per lane: one atomic per element beats the
+  // ticket (measured on MI355X at M = 1: 12.3 against 13.6 us for 14336 x 4096, 8.3 / 9.0 us
+  // for 4096 x 6144, 7.1 / 7.8 us for 4096 x 4096).  Every further row doubles the atomics,
+  // which execute at the memory side: already slower at M = 2 (9.3 against 8.0 us) and for the
+  // AWQ kernel's 16 columns per lane (16.5 against 13.8 us).
+  gp.fixed_point_split = cfg.splits > 1 && cfg.splits <= 14 && dtype == Q4_DTYPE_F16 && gate_up_act == 0 &&
+                         !awq && M == 1 && (size_t)w->N * 8 <= Q4_WORKSPACE_CELL_BYTES;
+  gp.cells = cfg.splits > 1 ? (unsigned long long*)((char*)workspace + Q4_WORKSPACE_TICKET_BYTES) : nullptr;
   gp.slab_stride = slab_stride;
   gp.slab_bytes = (int)slab_bytes;
   dim3 grid((unsigned)(ntiles * cfg.splits), (unsigned)mchunks);

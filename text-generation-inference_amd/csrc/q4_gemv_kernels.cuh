@@ -47,6 +47,8 @@ struct GemvParams {
   float* __restrict__ partials;
   uint32_t* __restrict__ tickets;
   int wcol, wk, splits;
+  unsigned long long* __restrict__ cells;  // fixed-point accumulation cells [M][N] (workspace)
+  int fixed_point_split;  // fp16 outputs: combine the splits with one 64-bit atomic per element
   int slab_stride;  // bytes between activation rows in LDS
   int slab_bytes;   // size of the activation slab region
 };
@@ -274,6 +276,53 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
       }
     }
     return;
+  }
+
+  // ---- cross-workgroup split-K, fp16: one 64-bit atomic per output element and workgroup.
+  // The cell of an element accumulates the partial sums in fixed point (28 fractional bits,
+  // integer addition: the total does not depend on the arrival order) and, in its top byte,
+  // the number of arrivals.  The add returns the previous contents, so the workgroup that
+  // brings the count to `splits` holds the complete sum, writes the output and clears the
+  // cell: one memory round trip where partial store -> ticket -> re-read takes three.
+  // Finite partials are clamped to +-2^17 (twice the largest fp16) and a non-finite partial
+  // (inf or NaN activations) counts as +2^23, more than all finite partials of up to 14
+  // splits can cancel: the output is then +inf where the reference's would be inf or NaN.
+  // |sum| stays below 2^55 fixed-point units, clear of the count.  The cells must be zero
+  // before the first call; they are left zero.
+  if constexpr (DTYPE == Q4_DTYPE_F16 && !FUSE) {
+    if (gp.fixed_point_split) {
+      if (d.wkk == 0) {
+        unsigned long long* cells = gp.cells;
+        constexpr unsigned long long kOne = 1ull << 56, kHalf = 1ull << 55;
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) {
+          const int m = 4 * d.kq + r;
+          if (m < d.mloc) {
+            unsigned long long* cell = cells + (size_t)(d.mb + m) * N + col0;
+            unsigned long long before[NT], inc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+              const float v = out[t][r];
+              long long q = 1ll << 51;  // non-finite
+              if (fabsf(v) <= 3.0e38f) q = __float2ll_rn(fminf(fmaxf(v, -131072.f), 131072.f) * 268435456.f);
+              inc[t] = kOne + (unsigned long long)q;
+              before[t] = __hip_atomic_fetch_add(cell + t, inc[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+              const unsigned long long now = before[t] + inc[t];
+              if ((long long)(now + kHalf) >> 56 == (long long)gp.splits) {
+                const long long sum = (long long)(now - ((unsigned long long)gp.splits << 56));
+                y[(size_t)(d.mb + m) * N + col0 + t] =
+                    finish_output<DTYPE>((float)sum * (1.0f / 268435456.f), p.bias, col0 + t);
+                __hip_atomic_store(cell + t, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              }
+            }
+          }
+        }
+      }
+      return;
+    }
   }
 
   // ---- cross-workgroup split-K: write the partial, take a ticket, last one reduces.
