@@ -63,8 +63,10 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   c.wcol = 1;
   c.wk = chunks % 4 == 0 ? 4 : (chunks % 2 == 0 ? 2 : 1);
   // wide layers with many rows: two column tiles per workgroup halve the slab staging
-  if (w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && M >= 8 && w->N % 128 == 0 &&
-      w->N / 64 >= 256)
+  // (and at any M once the tiles alone are well over the CU count: 4096 x 28672 at M = 1
+  // measured 16.7 against 17.0-17.8 us)
+  if (w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && w->N % 128 == 0 &&
+      ((M >= 8 && w->N / 64 >= 256) || w->N / 64 >= 384))
     c.wcol = 2;
   const bool act = w->layout == Q4_LAYOUT_GPTQ && w->g_idx != nullptr;
   if (act && chunks % 8 == 0) c.wk = 8;  // the group table is built once per workgroup
@@ -79,9 +81,15 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   const int wave_cols = w->layout == Q4_LAYOUT_AWQ ? 256 : (gate_up ? 128 : 64);
   const int ntiles = (w->N / (wave_cols * c.wcol)) * mchunks;
   int target_wgs = M <= 4 ? 512 : 384;  // partial-sum traffic grows with M
+  // a single fp16 row combines its splits with one atomic per element: more, shorter
+  // workgroups pay (4096 x 6144: 7.7 us with 8 splits against 8.4 us with 4)
+  const bool cheap_combine = M == 1 && w->layout == Q4_LAYOUT_GPTQ && !gate_up;
+  if (cheap_combine) target_wgs = 768;
   if (gate_up) target_wgs = 256;        // 512-thread workgroups: one per CU
   int want = (target_wgs + ntiles / 2) / ntiles;
-  if (want < 1) want = 1;
+  // tiles that fill the chip on their own are not split (4096 x 28672: 18.5 us with two
+  // splits against 16.7 us with one)
+  if (want < 1 || ntiles * c.wcol >= 256) want = 1;
   long lds_budget = 60000 - 16L * rows;
   if (act) lds_budget = 150000 - (long)w->num_groups * 64 * 4 - 16L * rows;
   // bytes per K row in LDS: activations, plus the uint16 g_idx slice for act-order
