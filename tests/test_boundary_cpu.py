@@ -88,7 +88,7 @@ def test_path_selection_and_workspace(pkg):
     lib = pkg._lib.load()
     L = pkg._lib
     w = _weight(pkg, 4096, 4096, 128)
-    for M, want in [(1, L.PATH_GEMV), (16, L.PATH_GEMV), (256, L.PATH_GEMV), (257, L.PATH_GEMM), (2048, L.PATH_GEMM)]:
+    for M, want in [(1, L.PATH_GEMV), (16, L.PATH_GEMV), (48, L.PATH_GEMV), (49, L.PATH_GEMM), (2048, L.PATH_GEMM)]:
         assert lib.q4_select_path(ctypes.byref(w), M, 0) == want
     odd = _weight(pkg, 4104, 4104, 8)
     assert lib.q4_select_path(ctypes.byref(odd), 1, 0) == L.PATH_GENERIC

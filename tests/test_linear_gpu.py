@@ -189,14 +189,45 @@ def test_gemm_bit_exact_weights_through_identity(pkg, oracle, gpu):
     assert np.array_equal(got.cpu().numpy().view(np.uint16), w.view(np.uint16))
 
 
+@pytest.mark.parametrize("K,N,M,dtype", [(4096, 4096, 512, "f16"), (14336, 4096, 300, "f16"), (4096, 6144, 129, "bf16"),
+                                         (1024, 512, 100, "f16"), (2048, 1280, 64, "f16"), (4096, 1024, 1000, "bf16")])
+def test_gemm_split_k(pkg, oracle, gpu, K, N, M, dtype):
+    """Few output tiles: the K loop is split over workgroups, fp32 partial tiles meet in the
+    reduction kernel (fixed split order: bit-reproducible), bias and rounding happen there."""
+    a, _ = _run(pkg, oracle, gpu, K, N, 128, M, dtype=dtype, sym=False, bias=True, path=2, seed=K // 64 + N // 64 + M)
+    b, _ = _run(pkg, oracle, gpu, K, N, 128, M, dtype=dtype, sym=False, bias=True, path=2, seed=K // 64 + N // 64 + M)
+    assert np.array_equal(a, b)
+
+
+def test_gemm_without_workspace_runs_unsplit(pkg, oracle, gpu):
+    """No workspace -> one workgroup per whole tile; same result to the parity bar."""
+    import ctypes
+
+    K, N, M, gs = 4096, 1024, 300, 128
+    qw, qz, sc, _ = oracle.make_gptq(K, N, gs, seed=5, sym=False)
+    w = oracle.dequant_gptq(qw, qz, sc, None, gs, "f16")
+    x = oracle.make_x(M, K, seed=5)
+    y32, _ = oracle.linear_forward(x, w, None, "f16")
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, gs, 0)
+    xt = to_dev(x, gpu)
+    y = torch.empty((M, N), dtype=torch.float16, device=gpu)
+    st = pk.struct()
+    rc = pkg._lib.load().q4_linear_ex(ctypes.byref(st), xt.data_ptr(), None, y.data_ptr(), M, 0, None, 0, 2,
+                                      torch.cuda.current_stream().cuda_stream)
+    pkg._lib.check(rc)
+    torch.cuda.synchronize()
+    assert max_rel_err(to_f32(y), y32) <= TOL
+    assert max_rel_err(to_f32(pkg.ops.linear(pk, xt, None, path=2)), y32) <= TOL
+
+
 def test_auto_dispatch(pkg, oracle, gpu):
     """q4_linear picks decode for M <= 16 and the MFMA GEMM above, generic for odd shapes."""
     qw, qz, sc, _ = oracle.make_gptq(1024, 512, 128, seed=3)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
     assert pkg.ops.select_path(pk, 1) == "gemv"
     assert pkg.ops.select_path(pk, 16) == "gemv"
-    assert pkg.ops.select_path(pk, 2048) == "gemv"   # M * N <= 2^20: row-chunked decode
-    assert pkg.ops.select_path(pk, 2049) == "gemm"
+    assert pkg.ops.select_path(pk, 48) == "gemv"   # small matrix: row-chunked decode up to 48 rows
+    assert pkg.ops.select_path(pk, 49) == "gemm"
     qw, qz, sc, _ = oracle.make_gptq(1000, 264, 40, seed=3)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 40, 0)
     assert pkg.ops.select_path(pk, 1) == "generic"

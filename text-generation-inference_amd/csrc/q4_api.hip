@@ -84,10 +84,13 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   if (validate_weight(w, "q4_select_path") != Q4_OK) return Q4_ERR_INVALID_ARGUMENT;
   const bool contiguous_gptq = w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr;
   if (contiguous_gptq) {
-    // Measured crossover on MI355X (Llama-3-8B shapes): the row-chunked decode kernel wins
-    // while M * N <= 2^20 (the GEMM grid of 128 x 256 tiles does not fill the 256 CUs
-    // below that); the MFMA GEMM wins above.
-    const bool small = M <= 16 || (long)M * w->N <= (1L << 20);
+    // Measured crossover on MI355X (Llama-3-8B shapes).  The decode kernel's cost grows with
+    // every 16-row chunk, the split-K GEMM's is nearly flat up to a few hundred rows:
+    // 4096 x 4096 (2^24 weights) decode 15.2 / 17.1 / 22.7 us against GEMM 17.3 / 18.6 / 19.1 us
+    // at M = 32 / 48 / 64; 4096 x 6144 decode 17.1 / 20.3 against 18.6 / 19.5 us at M = 32 / 40;
+    // 14336 x 4096 and 4096 x 28672 are faster through the GEMM from M = 17 on.
+    const long weights = (long)w->K * w->N;
+    const bool small = M <= 16 || (M <= 32 && weights <= (1L << 25)) || (M <= 48 && weights <= (1L << 24));
     if (small && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
     if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;
     if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
@@ -129,7 +132,10 @@ size_t q4_workspace_bytes(int M, int K, int N) {
       }
     }
   }
-  return (size_t)Q4_WORKSPACE_COUNTER_BYTES + (size_t)splits * M * N * sizeof(float);
+  // decode: split-K partial sums; prefill: split-K partial tiles of under-filled GEMM grids
+  const size_t decode = (size_t)splits * M * N * sizeof(float);
+  const size_t prefill = gemm_workspace_bytes(M, K, N);
+  return (size_t)Q4_WORKSPACE_COUNTER_BYTES + (decode > prefill ? decode : prefill);
 }
 
 int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
@@ -154,7 +160,7 @@ int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, i
     case Q4_PATH_GEMM:
       if (w->layout == Q4_LAYOUT_AWQ || w->g_idx != nullptr)
         return launch_gemm_awq(w, x, bias, y, M, dtype, (hipStream_t)stream);
-      return launch_gemm(w, x, bias, y, M, dtype, (hipStream_t)stream);
+      return launch_gemm(w, x, bias, y, M, dtype, workspace, workspace_bytes, (hipStream_t)stream);
     case Q4_PATH_GENERIC:
       return launch_generic(w, x, bias, y, M, dtype, (hipStream_t)stream);
     default:

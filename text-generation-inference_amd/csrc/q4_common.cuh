@@ -176,5 +176,6 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
                     hipStream_t stream);
 bool gemm_supported(const q4_weight* w, int M, int dtype);
 int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
-                hipStream_t stream);
+                void* workspace, size_t workspace_bytes, hipStream_t stream);
+size_t gemm_workspace_bytes(int M, int K, int N);
 }  // namespace q4host

@@ -31,7 +31,15 @@ constexpr int kAUnitsPerRow = kBK / 8 + 1;  // 16-byte units per LDS row, padded
 
 struct GemmParams {
   Problem p;
+  // Split-K for grids that do not fill the chip: `splits` workgroups share an output tile,
+  // each takes a contiguous range of K tiles and writes its fp32 partial tile to
+  // partials[split][M][N]; gemm_reduce_kernel adds them in split order.  splits == 1:
+  // the output is written directly.
+  float* __restrict__ partials;
+  int splits;
 };
+
+typedef float float2_t __attribute__((ext_vector_type(2)));
 
 struct SpliceK {
   uint32_t mask_lo, mask_hi, magic;
@@ -129,9 +137,11 @@ __global__ __launch_bounds__(256, (BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm
   constexpr int BN = 4 * 32 * NW;
   const int tiles_n = N / BN;
   int tm, tn;
+  const int total_tiles = tiles_m * tiles_n;
+  const int split = blockIdx.x / total_tiles;  // workgroups of one split are neighbours in id
   {
-    const int bid = blockIdx.x;
-    const int total = tiles_m * tiles_n;
+    const int bid = blockIdx.x - split * total_tiles;
+    const int total = total_tiles;
     if (tiles_m % 8 == 0 && total > 256) {
       const int mpx = tiles_m >> 3;  // M tiles per XCD
       const int xcd = bid & 7;
@@ -153,7 +163,10 @@ __global__ __launch_bounds__(256, (BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm
   const int ncol = nw + NW * j;        // first of this lane's NW columns
 
   const SpliceK splice = gemm_splice_consts();
-  const int KT = K / kBK;
+  const int KT_all = K / kBK;
+  // this workgroup's K tiles [kt_begin, KT)
+  const int kt_begin = (int)((long)split * KT_all / gp.splits);
+  const int KT = (int)((long)(split + 1) * KT_all / gp.splits);
 
   // ---- packed-weight stream: words [K/8 + kq][ncol, ncol+1], two K tiles ahead
   const char* wbase = (const char*)p.qweight;
@@ -257,14 +270,14 @@ __global__ __launch_bounds__(256, (BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm
   const int last_tile = KT - 1;
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
-  load_a(0, I0{});
-  load_b(0, bq[0]);
-  load_b(min(1, last_tile), bq[1]);
-  load_group_raw(0);
-  if constexpr (ASETS == 2) load_a(min(1, last_tile), I1{});
+  load_a(kt_begin, I0{});
+  load_b(kt_begin, bq[0]);
+  load_b(min(kt_begin + 1, last_tile), bq[1]);
+  load_group_raw(kt_begin);
+  if constexpr (ASETS == 2) load_a(min(kt_begin + 1, last_tile), I1{});
   store_a(0, I0{});
-  if constexpr (ASETS == 2) load_a(min(2, last_tile), I0{});
-  else load_a(min(1, last_tile), I0{});
+  if constexpr (ASETS == 2) load_a(min(kt_begin + 2, last_tile), I0{});
+  else load_a(min(kt_begin + 1, last_tile), I0{});
   make_group(cc);
   __syncthreads();
   read_a(0, 0, afrag[0]);
@@ -342,7 +355,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm
     }
   };
   {
-    int kt = 0;
+    int kt = kt_begin;
     for (; kt + 1 < KT; kt += 2) {
       tile_step(kt, std::integral_constant<int, 0>{});
       tile_step(kt + 1, std::integral_constant<int, 1>{});
@@ -352,6 +365,22 @@ __global__ __launch_bounds__(256, (BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm
 
   // ---- epilogue: C layout of the 32x32 MFMA: register r of lane (j, kq) is row
   // 8*(r/4) + 4*kq + r%4, column j.  Fragments 0/1 are adjacent columns -> one 32-bit store.
+  if (gp.splits > 1) {
+    // fp32 partial tile; bias, rounding and the store to y happen in the reduction kernel
+    float* part = gp.partials + (size_t)split * M * N;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
+        if (m < M) {
+          if constexpr (NW == 2) *(float2_t*)(part + (size_t)m * N + ncol) = float2_t{acc[mt][0][r], acc[mt][1][r]};
+          else part[(size_t)m * N + ncol] = acc[mt][0][r];
+        }
+      }
+    }
+    return;
+  }
   uint16_t* y = (uint16_t*)p.y;
   float bias_f[NW] = {};
   const bool has_bias = p.bias != nullptr;
@@ -389,6 +418,28 @@ __global__ __launch_bounds__(256, (BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm
   }
 }
 
+// y[m][n] = round(sum over splits of partials[s][m][n]) (+ bias), four columns per thread.
+template <int DTYPE>
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restrict__ partials,
+                                                          const void* __restrict__ bias, uint16_t* __restrict__ y,
+                                                          int M, int N, int splits) {
+  const long quads = (long)M * (N >> 2);
+  const size_t stride = (size_t)M * N;
+  for (long q = (long)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (long)gridDim.x * blockDim.x) {
+    const size_t e = (size_t)q * 4;
+    const int n = (int)(e % (size_t)N);
+    float4_t sum = *(const float4_t*)(partials + e);
+    for (int sp = 1; sp < splits; ++sp) {
+      const float4_t v = *(const float4_t*)(partials + (size_t)sp * stride + e);
+      sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+    }
+    uint2_t o;
+    o.x = (uint32_t)finish_output<DTYPE>(sum.x, bias, n) | ((uint32_t)finish_output<DTYPE>(sum.y, bias, n + 1) << 16);
+    o.y = (uint32_t)finish_output<DTYPE>(sum.z, bias, n + 2) | ((uint32_t)finish_output<DTYPE>(sum.w, bias, n + 3) << 16);
+    *(uint2_t*)(y + e) = o;
+  }
+}
+
 }  // namespace q4
 
 namespace q4host {
@@ -423,8 +474,65 @@ static void launch_tile(const GemmParams& gp, int gs, dim3 grid, size_t smem, hi
   }
 }
 
+// Tile shape and split factor for a problem; shared by the launcher and the workspace sizing.
+struct GemmPlan {
+  int bm, nw, splits;
+  long tiles;
+};
+
+static GemmPlan gemm_plan(int M, int K, int N) {
+  // Tile choice (all with 4 waves side by side along N):
+  //   256 x 256  grids of at least two rounds over the 256 CUs: half the unpacking per flop,
+  //              one wave per SIMD, runs at a higher clock;
+  //   128 x 256  the default; two workgroups per CU once there are more than 256 of them;
+  //   128 x 128  only when N is not a multiple of 256 (measured slower than 128 x 256
+  //              everywhere else: twice the activation-fragment reads per MFMA).
+  GemmPlan g;
+  const bool n256 = N % 256 == 0;
+  const long t256 = n256 ? (long)((M + 255) / 256) * (N / 256) : 0;
+  g.bm = 128;
+  g.nw = n256 ? 2 : 1;
+  if (t256 >= 512) g.bm = 256;
+  const int bn = 128 * g.nw;
+  g.tiles = (long)((M + g.bm - 1) / g.bm) * (N / bn);
+  // Split-K when the tiles alone leave CUs idle (one workgroup runs the whole K loop at
+  // ~0.9 us per 64-row K tile whatever M is: 14336 x 4096 took 200 us for every M up to
+  // 1024).  Aim at two workgroups per CU, keep at least 8 K tiles per workgroup.
+  // The split factor minimises a cost model fitted to measurements on MI355X: a workgroup
+  // takes ~0.9 us per K tile alone on its CU and ~1.3 us when two share one; the partial
+  // tiles cost a second launch (~5 us) plus S * M * N * 8 bytes of traffic at ~5 TB/s.
+  // (4096 x 6144 at M = 1024: 70 us unsplit, 86 us with three splits; 14336 x 4096 at
+  // M = 512: 200 us unsplit, 78 us with eight.)
+  g.splits = 1;
+  const int KT = K / q4::kBK;
+  if (g.bm == 128 && g.tiles < 256) {
+    static const int kCandidates[] = {1, 2, 3, 4, 6, 8, 12, 16};
+    double best = -1.0;
+    for (int sp : kCandidates) {
+      if (sp > 1 && KT / sp < 8) break;  // at least 8 K tiles (512 rows) per workgroup
+      const long wgs = g.tiles * sp;
+      const long rounds = (wgs + 511) / 512;
+      const double per_tile = wgs <= 256 ? 0.9 : 1.3;
+      double t = (double)rounds * ((KT + sp - 1) / sp) * per_tile;
+      if (sp > 1) t += 5.0 + (double)sp * M * N * 8.0 / 5.0e6;
+      if (best < 0.0 || t < best) {
+        best = t;
+        g.splits = sp;
+      }
+    }
+  }
+  return g;
+}
+
+// fp32 partial tiles of the split-K variant: splits x M x N floats.
+size_t gemm_workspace_bytes(int M, int K, int N) {
+  if (M <= 16 || K % q4::kBK != 0 || N % 128 != 0) return 0;
+  const GemmPlan g = gemm_plan(M, K, N);
+  return g.splits > 1 ? (size_t)g.splits * M * N * sizeof(float) : 0;
+}
+
 int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
-                hipStream_t stream) {
+                void* workspace, size_t workspace_bytes, hipStream_t stream) {
   using namespace q4;
   if (!gemm_supported(w, M, dtype)) {
     set_error("q4_linear(gemm): unsupported problem (layout=%d g_idx=%p M=%d K=%d N=%d groupsize=%d)",
@@ -434,19 +542,16 @@ int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, in
   GemmParams gp;
   gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, nullptr, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
-  // Tile choice (all with 4 waves side by side along N):
-  //   256 x 256  grids of at least two rounds over the 256 CUs: half the unpacking per flop,
-  //              one wave per SIMD, runs at a higher clock;
-  //   128 x 256  the default; two workgroups per CU once there are more than 256 of them;
-  //   128 x 128  only when N is not a multiple of 256 (measured slower than 128 x 256
-  //              everywhere else: twice the activation-fragment reads per MFMA).
-  const bool n256 = w->N % 256 == 0;
-  const long t256 = n256 ? (long)((M + 255) / 256) * (w->N / 256) : 0;
-  int bm = 128, nw = n256 ? 2 : 1;
-  if (t256 >= 512) bm = 256;
-  const int bn = 128 * nw;
-  const int tiles_m = (M + bm - 1) / bm;
-  const long total = (long)tiles_m * (w->N / bn);
+  GemmPlan g = gemm_plan(M, w->K, w->N);
+  // without room for the partial tiles every workgroup owns a whole tile (slower, same result
+  // up to fp32 summation order)
+  const size_t partial_bytes = (size_t)g.splits * M * w->N * sizeof(float);
+  if (g.splits > 1 && (workspace == nullptr || workspace_bytes < Q4_WORKSPACE_COUNTER_BYTES + partial_bytes))
+    g.splits = 1;
+  gp.splits = g.splits;
+  gp.partials = g.splits > 1 ? (float*)((char*)workspace + Q4_WORKSPACE_COUNTER_BYTES) : nullptr;
+  const int bm = g.bm, nw = g.nw;
+  const long total = g.tiles * g.splits;
   if (total > 0x7fffffffL) {
     set_error("q4_linear(gemm): grid too large");
     return Q4_ERR_UNSUPPORTED;
@@ -462,6 +567,17 @@ int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, in
     if (bm == 256) launch_tile<Q4_DTYPE_BF16, 256, 2>(gp, gs, grid, smem, stream);
     else if (nw == 2) launch_tile<Q4_DTYPE_BF16, 128, 2>(gp, gs, grid, smem, stream);
     else launch_tile<Q4_DTYPE_BF16, 128, 1>(gp, gs, grid, smem, stream);
+  }
+  if (g.splits > 1) {
+    const long quads = (long)M * (w->N / 4);
+    long blocks = (quads + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (dtype == Q4_DTYPE_F16)
+      hipLaunchKernelGGL(gemm_reduce_kernel<Q4_DTYPE_F16>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                         gp.partials, bias, (uint16_t*)y, M, w->N, g.splits);
+    else
+      hipLaunchKernelGGL(gemm_reduce_kernel<Q4_DTYPE_BF16>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                         gp.partials, bias, (uint16_t*)y, M, w->N, g.splits);
   }
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {

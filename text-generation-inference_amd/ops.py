@@ -187,12 +187,13 @@ def linear(
     with torch.cuda.device(x.device):
         stream = _stream_handle(x.device)
         st = w.struct()
-        # only the decode kernels use the workspace (split-K partials + tickets)
+        # decode: split-K partial sums, tickets, accumulation cells; prefill GEMM: split-K
+        # partial tiles when the tile grid alone would leave CUs idle
         chosen = path
         if chosen == PATH_AUTO and gemv_config is None:
             chosen = lib.q4_select_path(ctypes.byref(st), M, _DTYPES[x.dtype])
         need = _lib.WORKSPACE_COUNTER_BYTES
-        if chosen == _lib.PATH_GEMV:
+        if chosen in (_lib.PATH_GEMV, _lib.PATH_GEMM):
             need = workspace_bytes(M, w.K, w.N)
         ws = reserve_workspace(x.device, need, stream)
         st = w.struct()
