@@ -199,6 +199,14 @@ def test_gemm_split_k(pkg, oracle, gpu, K, N, M, dtype):
     assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("layout,act", [("awq", False), ("gptq", True)])
+@pytest.mark.parametrize("K,N,M", [(4096, 512, 200), (14336, 1024, 96), (2048, 4096, 130)])
+def test_gemm_split_k_awq_and_act_order(pkg, oracle, gpu, layout, act, K, N, M):
+    a, _ = _run(pkg, oracle, gpu, K, N, 128, M, layout=layout, act=act, sym=False, bias=True, path=2, seed=K // 64 + N + M)
+    b, _ = _run(pkg, oracle, gpu, K, N, 128, M, layout=layout, act=act, sym=False, bias=True, path=2, seed=K // 64 + N + M)
+    assert np.array_equal(a, b)
+
+
 def test_gemm_without_workspace_runs_unsplit(pkg, oracle, gpu):
     """No workspace -> one workgroup per whole tile; same result to the parity bar."""
     import ctypes
@@ -264,8 +272,13 @@ def test_awq_decompositions(pkg, oracle, gpu, cfg):
 def test_awq_auto_path_is_native(pkg, oracle, gpu):
     qw, qz, sc = oracle.make_awq(1024, 512, 128, seed=0)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 1)
-    for M in (1, 16, 100, 256):
-        assert pkg.ops.select_path(pk, M) == "gemv"  # M * N <= 0.75 * 2^20 for N = 512
+    for M in (1, 16):
+        assert pkg.ops.select_path(pk, M) == "gemv"
+    for M in (17, 100, 256):
+        assert pkg.ops.select_path(pk, M) == "gemm"  # the LDS-unpack MFMA kernel, split-K on small grids
+    qw, qz, sc, gi = oracle.make_gptq(1024, 512, 128, seed=0, act_order=True)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), 128, 0)
+    assert pkg.ops.select_path(pk, 48) == "gemv" and pkg.ops.select_path(pk, 49) == "gemm"
 
 
 @pytest.mark.parametrize("K,N", [(8192, 10240), (28672, 8192)])
@@ -342,7 +355,8 @@ def test_awq_gemm_bit_exact_weights_through_identity(pkg, oracle, gpu):
 def test_awq_dispatch_large_m(pkg, oracle, gpu):
     qw, qz, sc = oracle.make_awq(1024, 14336, 128, seed=0)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 1)
-    assert pkg.ops.select_path(pk, 48) == "gemv"
+    assert pkg.ops.select_path(pk, 16) == "gemv"
+    assert pkg.ops.select_path(pk, 17) == "gemm"
     assert pkg.ops.select_path(pk, 64) == "gemm"
 
 

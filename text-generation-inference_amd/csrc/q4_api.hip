@@ -96,10 +96,13 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
     if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
     return Q4_PATH_GENERIC;
   }
-  // AWQ and act-order: the decode kernels take any M in row chunks of 16; AWQ has an MFMA
-  // kernel (weights unpacked into LDS) for the sizes where a GEMM grid fills the chip
-  // (measured crossover for the 128 x 128 AWQ tiles: M * N around 0.75 * 2^20)
-  const bool small = M <= 16 || (long)M * w->N <= (3L << 18);
+  // AWQ and act-order: the decode kernels take any M in row chunks of 16; the MFMA kernel
+  // that unpacks the weights into LDS (split-K when its tile grid is small) takes over where
+  // it measured faster on MI355X: AWQ from M = 17 on (4096 x 14336: 37.7 against 46.8 us at
+  // M = 17, 49 against 110 us at M = 64), act-order from about M = 48 on (14336 x 4096:
+  // 86.9 / 86.5 us at M = 48, 87.6 against 105 us at M = 64; its gathered scales make the
+  // kernel ~2x slower per tile).
+  const bool small = M <= 16 || (w->layout == Q4_LAYOUT_GPTQ && M <= 48);
   if (!small && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
   if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
   if (M > 16 && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
@@ -159,7 +162,7 @@ int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, i
                          (hipStream_t)stream);
     case Q4_PATH_GEMM:
       if (w->layout == Q4_LAYOUT_AWQ || w->g_idx != nullptr)
-        return launch_gemm_awq(w, x, bias, y, M, dtype, (hipStream_t)stream);
+        return launch_gemm_awq(w, x, bias, y, M, dtype, workspace, workspace_bytes, (hipStream_t)stream);
       return launch_gemm(w, x, bias, y, M, dtype, workspace, workspace_bytes, (hipStream_t)stream);
     case Q4_PATH_GENERIC:
       return launch_generic(w, x, bias, y, M, dtype, (hipStream_t)stream);

@@ -173,9 +173,15 @@ bool gemv_gate_up_supported(const q4_weight* w, int M, int dtype);
 int launch_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, hipStream_t stream);
 bool gemm_awq_supported(const q4_weight* w, int M, int dtype);
 int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
-                    hipStream_t stream);
+                    void* workspace, size_t workspace_bytes, hipStream_t stream);
 bool gemm_supported(const q4_weight* w, int M, int dtype);
 int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                 void* workspace, size_t workspace_bytes, hipStream_t stream);
 size_t gemm_workspace_bytes(int M, int K, int N);
+// Split factor of an under-filled tile grid from the fitted cost model (us per K tile of a
+// workgroup alone on its CU / sharing it).
+int gemm_pick_splits(long tiles, int KT, int M, int N, double us_alone, double us_shared);
+int gemm_awq_splits(int M, int K, int N);
+void launch_gemm_reduce(const float* partials, const void* bias, void* y, int M, int N, int splits, int dtype,
+                        hipStream_t stream);
 }  // namespace q4host

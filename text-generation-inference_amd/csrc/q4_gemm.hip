@@ -504,31 +504,50 @@ static GemmPlan gemm_plan(int M, int K, int N) {
   // (4096 x 6144 at M = 1024: 70 us unsplit, 86 us with three splits; 14336 x 4096 at
   // M = 512: 200 us unsplit, 78 us with eight.)
   g.splits = 1;
-  const int KT = K / q4::kBK;
-  if (g.bm == 128 && g.tiles < 256) {
-    static const int kCandidates[] = {1, 2, 3, 4, 6, 8, 12, 16};
-    double best = -1.0;
-    for (int sp : kCandidates) {
-      if (sp > 1 && KT / sp < 8) break;  // at least 8 K tiles (512 rows) per workgroup
-      const long wgs = g.tiles * sp;
-      const long rounds = (wgs + 511) / 512;
-      const double per_tile = wgs <= 256 ? 0.9 : 1.3;
-      double t = (double)rounds * ((KT + sp - 1) / sp) * per_tile;
-      if (sp > 1) t += 5.0 + (double)sp * M * N * 8.0 / 5.0e6;
-      if (best < 0.0 || t < best) {
-        best = t;
-        g.splits = sp;
-      }
-    }
-  }
+  if (g.bm == 128 && g.tiles < 256) g.splits = gemm_pick_splits(g.tiles, K / q4::kBK, M, N, 0.9, 1.3);
   return g;
 }
 
-// fp32 partial tiles of the split-K variant: splits x M x N floats.
+int gemm_pick_splits(long tiles, int KT, int M, int N, double us_alone, double us_shared) {
+  static const int kCandidates[] = {1, 2, 3, 4, 6, 8, 12, 16};
+  double best = -1.0;
+  int splits = 1;
+  for (int sp : kCandidates) {
+    if (sp > 1 && KT / sp < 8) break;  // at least 8 K tiles (512 rows) per workgroup
+    const long wgs = tiles * sp;
+    const long rounds = (wgs + 511) / 512;
+    const double per_tile = wgs <= 256 ? us_alone : us_shared;
+    double t = (double)rounds * ((KT + sp - 1) / sp) * per_tile;
+    if (sp > 1) t += 5.0 + (double)sp * M * N * 8.0 / 5.0e6;
+    if (best < 0.0 || t < best) {
+      best = t;
+      splits = sp;
+    }
+  }
+  return splits;
+}
+
+void launch_gemm_reduce(const float* partials, const void* bias, void* y, int M, int N, int splits, int dtype,
+                        hipStream_t stream) {
+  const long quads = (long)M * (N / 4);
+  long blocks = (quads + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  if (dtype == Q4_DTYPE_F16)
+    hipLaunchKernelGGL(q4::gemm_reduce_kernel<Q4_DTYPE_F16>, dim3((unsigned)blocks), dim3(256), 0, stream, partials,
+                       bias, (uint16_t*)y, M, N, splits);
+  else
+    hipLaunchKernelGGL(q4::gemm_reduce_kernel<Q4_DTYPE_BF16>, dim3((unsigned)blocks), dim3(256), 0, stream, partials,
+                       bias, (uint16_t*)y, M, N, splits);
+}
+
+// fp32 partial tiles of the split-K variants: splits x M x N floats (upper bound over the
+// GPTQ kernel and the AWQ / act-order kernel, whose tiles differ).
 size_t gemm_workspace_bytes(int M, int K, int N) {
   if (M <= 16 || K % q4::kBK != 0 || N % 128 != 0) return 0;
-  const GemmPlan g = gemm_plan(M, K, N);
-  return g.splits > 1 ? (size_t)g.splits * M * N * sizeof(float) : 0;
+  int splits = gemm_plan(M, K, N).splits;
+  const int other = gemm_awq_splits(M, K, N);
+  if (other > splits) splits = other;
+  return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
 
 int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
@@ -568,17 +587,7 @@ int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, in
     else if (nw == 2) launch_tile<Q4_DTYPE_BF16, 128, 2>(gp, gs, grid, smem, stream);
     else launch_tile<Q4_DTYPE_BF16, 128, 1>(gp, gs, grid, smem, stream);
   }
-  if (g.splits > 1) {
-    const long quads = (long)M * (w->N / 4);
-    long blocks = (quads + 255) / 256;
-    if (blocks > 4096) blocks = 4096;
-    if (dtype == Q4_DTYPE_F16)
-      hipLaunchKernelGGL(gemm_reduce_kernel<Q4_DTYPE_F16>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                         gp.partials, bias, (uint16_t*)y, M, w->N, g.splits);
-    else
-      hipLaunchKernelGGL(gemm_reduce_kernel<Q4_DTYPE_BF16>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                         gp.partials, bias, (uint16_t*)y, M, w->N, g.splits);
-  }
+  if (g.splits > 1) launch_gemm_reduce(gp.partials, bias, y, M, w->N, g.splits, dtype, stream);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {
     set_error("q4_linear(gemm): launch failed: %s", hipGetErrorString(err));

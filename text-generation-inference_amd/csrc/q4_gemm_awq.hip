@@ -31,6 +31,10 @@ constexpr int kABK = 64;   // K rows per tile
 constexpr int kAUnits = kABK / 8 + 1;  // padded units per activation row
 
 struct AwqGemmParams {
+  // split-K as in the GPTQ GEMM: `splits` workgroups per output tile, fp32 partial tiles in
+  // partials[split][M][N], combined by gemm_reduce_kernel
+  float* __restrict__ partials;
+  int splits;
   Problem p;
 };
 
@@ -64,11 +68,16 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   const int N = p.N, K = p.K, M = p.M;
   const int NC = N >> 3;
   const int tiles_m = (M + kABM - 1) / kABM;
-  const int tm = blockIdx.x % tiles_m;
-  const int tn = blockIdx.x / tiles_m;
+  const int tiles_all = tiles_m * (N / kABN);
+  const int split = blockIdx.x / tiles_all;
+  const int tile_id = blockIdx.x - split * tiles_all;
+  const int tm = tile_id % tiles_m;
+  const int tn = tile_id / tiles_m;
   const int m0 = tm * kABM;
   const int n0 = tn * kABN;
-  const int KT = K / kABK;
+  const int KT_all = K / kABK;
+  const int kt_begin = (int)((long)split * KT_all / gp.splits);  // this workgroup's K tiles
+  const int KT = (int)((long)(split + 1) * KT_all / gp.splits);
   const int last_tile = KT - 1;
   const AwqSplice splice = awq_splice_consts();
 
@@ -215,19 +224,19 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
-  load_a(0);
-  load_b(0);
+  load_a(kt_begin);
+  load_b(kt_begin);
   store_a(0);
-  store_b(0, 0);
-  load_a(min(1, last_tile));
-  load_b(min(1, last_tile));
+  store_b(0, kt_begin);
+  load_a(min(kt_begin + 1, last_tile));
+  load_b(min(kt_begin + 1, last_tile));
   __syncthreads();
 
   const int a_off = ((wm * 64 + j) * kAUnits + kq) * 16;
   const int b_off = (kq * kABN + wn * 64 + j) * 16;
 
-  for (int kt = 0; kt < KT; ++kt) {
-    const int cur = kt & 1;
+  for (int kt = kt_begin; kt < KT; ++kt) {
+    const int cur = (kt - kt_begin) & 1;
     // the other buffer was last read in tile kt-1, before the barrier that ended it
     store_a(cur ^ 1);
     store_b(cur ^ 1, min(kt + 1, last_tile));
@@ -260,6 +269,22 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   }
 
   // ---- epilogue: register r of lane (j, kq) is row 8*(r/4) + 4*kq + r%4, column j
+  if (gp.splits > 1) {
+    float* part = gp.partials + (size_t)split * M * N;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int n = n0 + wn * 64 + nt * 32 + j;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm * 64 + mt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
+          if (m < M) part[(size_t)m * N + n] = acc[mt][nt][r];
+        }
+      }
+    }
+    return;
+  }
   uint16_t* y = (uint16_t*)p.y;
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
@@ -289,8 +314,15 @@ bool gemm_awq_supported(const q4_weight* w, int M, int dtype) {
   return (long)w->num_groups * w->groupsize >= w->K;
 }
 
+// 128 x 128 tiles, ~1.0 us per K tile alone on a CU, ~1.9 us when two workgroups share it
+int gemm_awq_splits(int M, int K, int N) {
+  if (K % q4::kABK != 0 || N % q4::kABN != 0) return 1;
+  const long tiles = (long)((M + q4::kABM - 1) / q4::kABM) * (N / q4::kABN);
+  return tiles < 256 ? gemm_pick_splits(tiles, K / q4::kABK, M, N, 1.0, 1.9) : 1;
+}
+
 int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
-                    hipStream_t stream) {
+                    void* workspace, size_t workspace_bytes, hipStream_t stream) {
   using namespace q4;
   if (!gemm_awq_supported(w, M, dtype)) {
     set_error("q4_linear(gemm/awq): unsupported problem (M=%d K=%d N=%d groupsize=%d)", M, w->K, w->N,
@@ -300,7 +332,13 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
   AwqGemmParams gp;
   gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, w->g_idx, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
-  const long total = (long)((M + kABM - 1) / kABM) * (w->N / kABN);
+  int splits = gemm_awq_splits(M, w->K, w->N);
+  if (splits > 1 && (workspace == nullptr ||
+                     workspace_bytes < Q4_WORKSPACE_COUNTER_BYTES + (size_t)splits * M * w->N * sizeof(float)))
+    splits = 1;  // no room for partial tiles: one workgroup per whole tile
+  gp.splits = splits;
+  gp.partials = splits > 1 ? (float*)((char*)workspace + Q4_WORKSPACE_COUNTER_BYTES) : nullptr;
+  const long total = (long)((M + kABM - 1) / kABM) * (w->N / kABN) * splits;
   if (total > 0x7fffffffL) {
     set_error("q4_linear(gemm/awq): grid too large");
     return Q4_ERR_UNSUPPORTED;
@@ -318,6 +356,7 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
     if (act) launch(gemm_awq_kernel<Q4_DTYPE_BF16, true>);
     else launch(gemm_awq_kernel<Q4_DTYPE_BF16, false>);
   }
+  if (splits > 1) launch_gemm_reduce(gp.partials, bias, y, M, w->N, splits, dtype, stream);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {
     set_error("q4_linear(gemm/awq): launch failed: %s", hipGetErrorString(err));
