@@ -39,7 +39,7 @@ namespace q4 {
 
 constexpr int kChunkSteps = 4;                // 32-row MFMA steps per software-pipelined chunk
 constexpr int kChunkRows = 32 * kChunkSteps;  // 128 K rows
-constexpr int kPrefetch = 4;                  // chunks of weight loads in flight per wave
+constexpr int kPrefetch = 2;                  // chunks of weight loads in flight per wave
 constexpr int kRowsPerBlock = 16;             // activation rows per workgroup (MFMA M)
 
 struct GemvParams {
