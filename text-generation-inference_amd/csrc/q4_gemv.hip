@@ -41,11 +41,12 @@ bool gemv_supported(const q4_weight* w, int M, int dtype) {
 bool gemv_gate_up_supported(const q4_weight* w, int M, int dtype) {
   // the contiguous-group GPTQ kernel with groups of whole chunks; both halves of W in whole
   // 64-column wave tiles.  Measured on the Llama-3-8B gate_up projection against the plain
-  // kernel followed by the elementwise kernel: 17.7 / 19.6 us at M = 1, 28.5 / 30.0 us at
-  // M = 8, 44.1 / 43.4 us at M = 16 (the wider workgroups stage twice the activation slab),
-  // so the fused kernel is offered up to 8 rows.
+  // kernel followed by the elementwise kernel: 16.1 / 18.2 us at M = 1, 17.2 / 18.4 us at
+  // M = 2, 19.6 / 19.3 us at M = 4, 26.0 / 22.4 us at M = 8 (the fused workgroups are twice
+  // as wide and stage twice the activation slab), so the fused kernel is offered for one and
+  // two rows.
   return w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && w->groupsize >= 128 && w->N % 128 == 0 &&
-         M <= 8 && gemv_supported(w, M, dtype);
+         M <= 2 && gemv_supported(w, M, dtype);
 }
 
 GemvConfig gemv_pick_config(const q4_weight* w, int M) { return gemv_pick_config(w, M, false); }

@@ -1,5 +1,6 @@
 // Decode kernel instantiations with the gated-MLP epilogue (act(x @ gate) * (x @ up)), kept in
-// their own translation unit so that they compile in parallel with the plain ones.
+// their own translation unit so that they compile in parallel with the plain ones.  The
+// launcher offers them for one and two activation rows only.
 #include "q4_gemv_kernels.cuh"
 
 namespace q4host {
@@ -27,12 +28,10 @@ void launch_gemv_gate_up(const GemvParams& gp, int dtype, int rmax, bool static1
                          size_t smem, hipStream_t stream) {
   if (dtype == Q4_DTYPE_F16) {
     if (rmax == 1) launch_fused<Q4_DTYPE_F16, 1>(gp, static128, grid, block, smem, stream);
-    else if (rmax == 2) launch_fused<Q4_DTYPE_F16, 2>(gp, static128, grid, block, smem, stream);
-    else launch_fused<Q4_DTYPE_F16, 4>(gp, static128, grid, block, smem, stream);
+    else launch_fused<Q4_DTYPE_F16, 2>(gp, static128, grid, block, smem, stream);
   } else {
     if (rmax == 1) launch_fused<Q4_DTYPE_BF16, 1>(gp, static128, grid, block, smem, stream);
-    else if (rmax == 2) launch_fused<Q4_DTYPE_BF16, 2>(gp, static128, grid, block, smem, stream);
-    else launch_fused<Q4_DTYPE_BF16, 4>(gp, static128, grid, block, smem, stream);
+    else launch_fused<Q4_DTYPE_BF16, 2>(gp, static128, grid, block, smem, stream);
   }
 }
 
