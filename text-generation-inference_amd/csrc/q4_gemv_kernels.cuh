@@ -586,7 +586,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
   const int N = p.N;
   const int nl = d.tile * d.tile_cols + d.wc * 64 + 4 * d.j;
   const int nsteps = d.KW / 32;
-  constexpr int PF = 8;  // 32-row steps of weight loads in flight per wave
+  constexpr int PF = 2;  // 32-row steps of weight loads in flight per wave
 
   SlabStager<true> slab;
   slab.issue(gp, d);
