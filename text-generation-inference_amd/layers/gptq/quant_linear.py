@@ -12,6 +12,7 @@ from __future__ import annotations
 import math
 from typing import Optional
 
+import numpy as np
 import torch
 import torch.nn as nn
 
@@ -68,6 +69,42 @@ class QuantLinear(nn.Module):
         g_idx = (torch.arange(infeatures, dtype=torch.int64) // gs).to(torch.int32)
         bias_t = torch.zeros((outfeatures,), dtype=torch.float16) if bias else None
         return cls(qweight, qzeros, scales, g_idx, bias_t, bits, groupsize)
+
+    def pack(self, linear, scales, zeros, g_idx=None):
+        """Quantize a dense layer into this module's packed buffers (triton.py:294-349).
+
+        `linear.weight` is [outfeatures, infeatures]; `scales` and `zeros` are
+        [outfeatures, groups] as a GPTQ quantizer emits them.  Row k of the integer
+        matrix is round((W[:, k] + zero*scale) / fp16(scale)) with its group's
+        parameters (round half to even); eight consecutive rows fill one qweight word
+        from the low nibble up, eight consecutive columns one qzeros word, and the
+        stored zero point is zero - 1.  Like the reference, nothing is clamped: the
+        quantizer is expected to hand in weights that land on 0..15 and zeros in 1..16.
+        Runs on the CPU at conversion time; the caller moves the module afterwards.
+        """
+        if g_idx is not None:
+            self.g_idx = g_idx.clone()
+        gi = self.g_idx.to(torch.int64).cpu()
+        scales = scales.detach().cpu().t().contiguous()
+        zeros = zeros.detach().cpu().t().contiguous()
+        scale_zeros = zeros * scales
+        self.scales = scales.clone().half()
+        if getattr(linear, "bias", None) is not None:
+            self.bias = linear.bias.detach().clone().half()
+
+        w = linear.weight.detach().cpu().t()  # [K, N]
+        q = torch.round((w + scale_zeros[gi]) / self.scales[gi]).to(torch.int32)
+        per_word = 32 // self.bits
+        shifts = (np.arange(per_word, dtype=np.uint32) * np.uint32(self.bits))
+        qi = q.numpy().astype(np.uint32).reshape(-1, per_word, q.shape[1])
+        qweight = np.bitwise_or.reduce(qi << shifts[None, :, None], axis=1)
+        self.qweight = torch.from_numpy(qweight.astype(np.int32))
+
+        z = (zeros - 1).to(torch.int64).numpy().astype(np.uint32)  # -1 wraps to all ones
+        zi = z.reshape(z.shape[0], -1, per_word)
+        qzeros = np.bitwise_or.reduce(zi << shifts[None, None, :], axis=2)
+        self.qzeros = torch.from_numpy(qzeros.astype(np.int32))
+        self._packed = None
 
     def packed(self) -> ops.PackedWeight:
         """Validated kernel view of the buffers, rebuilt if they moved (e.g. `.to(device)`)."""
