@@ -278,6 +278,10 @@ def test_awq_auto_path_is_native(pkg, oracle, gpu):
         assert pkg.ops.select_path(pk, M) == "gemm"  # the LDS-unpack MFMA kernel, split-K on small grids
     qw, qz, sc, gi = oracle.make_gptq(1024, 512, 128, seed=0, act_order=True)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), 128, 0)
+    assert pkg.ops.select_path(pk, 16) == "gemv" and pkg.ops.select_path(pk, 17) == "gemm"
+    # too many groups for an LDS parameter table: the gathering kernel pays off later
+    qw, qz, sc, gi = oracle.make_gptq(8192, 128, 32, seed=0, act_order=True)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), 32, 0)
     assert pkg.ops.select_path(pk, 48) == "gemv" and pkg.ops.select_path(pk, 49) == "gemm"
 
 
@@ -380,11 +384,40 @@ def test_act_order_gemm_groupsizes_dtypes(pkg, oracle, gpu, gs, dtype):
     _run(pkg, oracle, gpu, 512, 256, gs, 70, dtype=dtype, sym=False, act=True, path=2, seed=gs + 13)
 
 
-def test_act_order_gemm_bit_exact_weights_through_identity(pkg, oracle, gpu):
-    K, N, gs = 512, 128, 64
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("K,gs,N,M", [(2048, 128, 256, 100),      # 16 groups: 32-bit LDS table
+                                       (6400, 32, 256, 100),       # 200 groups: scale + zero-byte LDS table
+                                       (8192, 32, 128, 100),       # 256 groups: per-row global gather
+                                       (4096, 128, 11008, 300)])   # 258 tiles: the table that lets two share a CU
+def test_act_order_gemm_parameter_sources(pkg, oracle, gpu, K, gs, N, M, dtype):
+    """Every way the act-order MFMA kernel fetches a row's scale and zero point."""
+    _run(pkg, oracle, gpu, K, N, gs, M, dtype=dtype, sym=False, act=True, path=2, bias=True, seed=K // 64 + gs)
+
+
+@pytest.mark.parametrize("K,gs", [(512, 64), (6400, 32), (8192, 32)])
+def test_act_order_gemm_bit_exact_weights_through_identity(pkg, oracle, gpu, K, gs):
+    N = 128
     qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=33, sym=False, act_order=True)
     w = oracle.dequant_gptq(qw, qz, sc, gi, gs, "f16")
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), gs, 0)
+    eye = torch.eye(K, dtype=torch.float16, device=gpu)
+    got = pkg.ops.linear(pk, eye, None, path=2)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), w.view(np.uint16))
+
+
+def test_act_order_gemm_out_of_range_group_index_is_clamped(pkg, oracle, gpu):
+    """A corrupt g_idx must not send the kernel outside its table: entries are clamped to
+    the first and last group, as in the dequantize kernel."""
+    K, N, gs = 1024, 128, 128
+    qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=4, sym=False, act_order=True)
+    bad = gi.copy()
+    bad[5] = 1000
+    bad[77] = -3
+    clamped = gi.copy()
+    clamped[5] = K // gs - 1
+    clamped[77] = 0
+    w = oracle.dequant_gptq(qw, qz, sc, clamped, gs, "f16")
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(bad, gpu), gs, 0)
     eye = torch.eye(K, dtype=torch.float16, device=gpu)
     got = pkg.ops.linear(pk, eye, None, path=2)
     assert np.array_equal(got.cpu().numpy().view(np.uint16), w.view(np.uint16))

@@ -99,13 +99,14 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   // AWQ and act-order: the decode kernels take any M in row chunks of 16; the MFMA kernel
   // that unpacks the weights into LDS (split-K when its tile grid is small) takes over where
   // it measured faster on MI355X: AWQ from M = 17 on (4096 x 14336: 37.7 against 46.8 us at
-  // M = 17, 49 against 110 us at M = 64), act-order from about M = 48 on (14336 x 4096:
-  // 86.9 / 86.5 us at M = 48, 87.6 against 105 us at M = 64; its gathered scales make the
-  // kernel ~2x slower per tile).
+  // M = 17, 49 against 110 us at M = 64); act-order from M = 17 on when its parameter table
+  // fits in LDS (8192 x 10240: 57 against 67 us at M = 24, 52 against 140 us at M = 64; the
+  // kernel's time is flat in M up to 128 rows), from about M = 48 on when it has to gather
+  // scales and zero points from global memory (~2x slower per tile).
   // Below 17 rows the AWQ decode kernel's time grows with every row (16 accumulator sets, ~250
   // VGPRs) while the split-K GEMM stays flat at ~38 us for these sizes: 4096 x 14336 decode
   // 35.9 / 43.9 us at M = 12 / 16, 14336 x 4096 decode 40.9 / 71.6 us at M = 8 / 16.
-  bool small = M <= 16 || (w->layout == Q4_LAYOUT_GPTQ && M <= 48);
+  bool small = M <= 16 || (w->layout == Q4_LAYOUT_GPTQ && M <= 48 && !gemm_act_order_table(w));
   if (w->layout == Q4_LAYOUT_AWQ && (M > 12 || (M > 7 && w->K > 8192))) small = false;
   if (!small && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
   if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;

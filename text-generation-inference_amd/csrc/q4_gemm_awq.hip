@@ -15,9 +15,13 @@
 //     reference's rounding).  The patch becomes eight 16-byte units (one per column,
 //     8 consecutive K values each) written to LDS at [K block][column];
 //   * act-order producer: every thread owns 4 packed words (8 K rows x 1 column each).  The
-//     groups of the 8 rows are wave-uniform (g_idx[k]); scale and zero point of each row
-//     are gathered from the checkpoint tensors (coalesced across the 64 columns of a wave,
-//     L2 resident) and applied per weight -- no row of qweight is ever moved;
+//     groups of the 8 rows (g_idx[k], the same for every lane, requested one tile ahead)
+//     index a per-workgroup LDS table of all groups x the tile's 128 columns, filled once
+//     in the prologue, and scale and zero point are applied per weight -- no row of
+//     qweight is ever moved.  The table holds one 32-bit entry per group and column
+//     (fp16 scale | fp16 -(1024 + zero), one LDS read per row) for up to 184 groups, or
+//     an fp16 scale and a zero-point byte (two reads per row) for up to 245 groups;
+//     layers with more groups gather the two values per row from the checkpoint tensors;
 //   * LDS layouts: activations [row][K block] with the row stride padded to 9 units,
 //     weights [K block][column]; both give conflict-free 128-bit fragment reads;
 //   * double-buffered LDS, global loads for tile k+2 in flight while tile k is multiplied.
@@ -29,6 +33,7 @@ constexpr int kABM = 128;  // rows per workgroup
 constexpr int kABN = 128;  // columns per workgroup
 constexpr int kABK = 64;   // K rows per tile
 constexpr int kAUnits = kABK / 8 + 1;  // padded units per activation row
+constexpr size_t kLdsBytesPerWorkgroup = 160 * 1024;  // gfx950: 160 KB of LDS per CU
 
 struct AwqGemmParams {
   // split-K as in the GPTQ GEMM: `splits` workgroups per output tile, fp32 partial tiles in
@@ -51,9 +56,18 @@ __device__ __forceinline__ AwqSplice awq_splice_consts() {
 typedef __bf16 awq_bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float awq_float2_t __attribute__((ext_vector_type(2)));
 
-// ACT = false: AWQ layout.  ACT = true: GPTQ layout with g_idx.
-template <int DTYPE, bool ACT>
+constexpr int kModeAwq = 0;        // AWQ layout
+constexpr int kModeActGather = 1;  // GPTQ layout with g_idx, per-row parameters from global memory
+constexpr int kModeActWide = 2;    // GPTQ layout with g_idx, LDS table of 32-bit (scale | -(1024 + zero)) entries
+constexpr int kModeActNarrow = 3;  // GPTQ layout with g_idx, LDS table of fp16 scales and zero-point bytes
+constexpr int kActWideGroupBytes = kABN * 4;
+constexpr int kActNarrowGroupBytes = kABN * 3;  // 128 fp16 scales, then 128 zero-point bytes
+
+template <int DTYPE, int MODE>
 __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
+  constexpr bool ACT = MODE != kModeAwq;
+  constexpr bool TABLE = MODE == kModeActWide || MODE == kModeActNarrow;
+  constexpr int GROUP_BYTES = MODE == kModeActWide ? kActWideGroupBytes : kActNarrowGroupBytes;
   constexpr int A_TILE = kABM * kAUnits * 16;   // bytes
   constexpr int B_TILE = (kABK / 8) * kABN * 16;
   constexpr int A_LOADS = kABM * (kABK / 8) / 256;  // 16-byte activation loads per thread
@@ -94,10 +108,25 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   uint32_t braw[8];  // AWQ: 8 rows of one word column; act-order: 4 words (K blocks)
   uint4_t sraw;      // AWQ: 8 fp16 scales of the word's columns
   uint32_t zraw;     // AWQ: 8 zero-point nibbles
+  int graw[4][8];    // act-order table modes: groups of the thread's 32 rows
+  // The groups are the same in every lane, but they are wanted in vector registers (LDS
+  // addresses are per lane): an offset the compiler cannot see through keeps the loads
+  // and the address arithmetic on the vector unit instead of a detour through scalars.
+  int lane_zero = 0;
+  asm volatile("" : "+v"(lane_zero));
+  // act-order: word i of the thread (K block pkb0 + 2 i) and, in table modes, its rows' groups
+  auto load_b_word = [&](int kt, int i) {
+    braw[i] = wsrc[(size_t)(kt * (kABK / 8) + 2 * i) * N];
+    if constexpr (TABLE) {
+      const int* gsrc = p.g_idx + kt * kABK + (pkb0 + 2 * i) * 8 + lane_zero;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) graw[i][r] = gsrc[r];
+    }
+  };
   auto load_b = [&](int kt) {
     if constexpr (ACT) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) braw[i] = wsrc[(size_t)(kt * (kABK / 8) + 2 * i) * N];
+      for (int i = 0; i < 4; ++i) load_b_word(kt, i);
     } else if (producer) {
 #pragma unroll
       for (int r = 0; r < 8; ++r) braw[r] = wsrc[(size_t)(kt * kABK + r) * NC];
@@ -106,47 +135,71 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
       zraw = p.qzeros[(size_t)g * NC + (n0 >> 3) + pc];
     }
   };
-  auto store_b_act = [&](int buf, int kt) {
-    unsigned char* base = smem + 2 * A_TILE + buf * B_TILE;
+  const unsigned char* table = smem + 2 * A_TILE + 2 * B_TILE;  // act-order table modes only
+  const int last_group = p.num_groups - 1;
+  // The act-order producer works on one word (8 K rows of the thread's column) in three
+  // phases, so that the main loop can place MFMAs between them.
+  // Phase 1: the parameters of the word's 8 rows.  Wide table: ra = scale | -(1024 + zero) << 16.
+  // Otherwise ra = scale bits, rb = zero point.
+  auto word_params = [&](int kt, int i, uint32_t (&ra)[8], uint32_t (&rb)[8]) {
     const int n = n0 + pn;
     const int zshift = (n & 7) * 4;
+    const int k0 = kt * kABK + (pkb0 + 2 * i) * 8;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int kb = pkb0 + 2 * i;
-      const int k0 = kt * kABK + kb * 8;
-      // scale and -(1024 + zero) of the 8 rows of this word: groups are wave-uniform
-      uint32_t sc[8], cz[8];
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
+    for (int r = 0; r < 8; ++r) {
+      if constexpr (TABLE) {
+        // a corrupt index stays inside the table: clamp to [0, groups - 1] in one instruction
+        int g;
+        asm("v_med3_i32 %0, %1, 0, %2" : "=v"(g) : "v"(graw[i][r]), "s"(last_group));
+        if constexpr (MODE == kModeActWide) {
+          ra[r] = *(const uint32_t*)(table + g * GROUP_BYTES + 4 * pn);
+        } else {
+          ra[r] = *(const uint16_t*)(table + g * GROUP_BYTES + 2 * pn);
+          rb[r] = table[g * GROUP_BYTES + 2 * kABN + pn];
+        }
+      } else {
         int g = p.g_idx[k0 + r];
         g = min(max(g, 0), p.num_groups - 1);
-        sc[r] = *(const uint16_t*)(p.scales + (size_t)g * N + n);
-        const uint32_t z = (gptq_zero_plus_one(p.qzeros[(size_t)g * NC + (n >> 3)]) >> zshift) & 0xFu;
-        cz[r] = 0xE400u | z;
+        ra[r] = *(const uint16_t*)(p.scales + (size_t)g * N + n);
+        rb[r] = (gptq_zero_plus_one(p.qzeros[(size_t)g * NC + (n >> 3)]) >> zshift) & 0xFu;
       }
-      const uint32_t w = braw[i];
-      uint32_t o[4];
-#pragma unroll
-      for (int pr = 0; pr < 4; ++pr) {
-        // rows pr and pr + 4 share one splice (nibbles 16 bits apart)
-        const uint32_t q2 = ((w >> (4 * pr)) & splice.mask_lo) | splice.magic;
-        const half2_t dq = as_half2(q2) + as_half2(cz[pr] | (cz[pr + 4] << 16));  // exact q - z
-        if constexpr (DTYPE == Q4_DTYPE_F16) {
-          o[pr] = as_u32(dq * as_half2(sc[pr] | (sc[pr + 4] << 16)));  // one fp16 rounding
-        } else {
-          const half2_t s2 = as_half2(sc[pr] | (sc[pr + 4] << 16));
-          const awq_float2_t f = {(float)dq.x * (float)s2.x, (float)dq.y * (float)s2.y};
-          o[pr] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, awq_bf16x2_t));
-        }
-      }
-      // o holds rows (0,4),(1,5),(2,6),(3,7): back to natural K order for the unit
-      uint4_t unit;
-      unit.x = (o[0] & 0xFFFFu) | (o[1] << 16);
-      unit.y = (o[2] & 0xFFFFu) | (o[3] << 16);
-      unit.z = (o[0] >> 16) | (o[1] & 0xFFFF0000u);
-      unit.w = (o[2] >> 16) | (o[3] & 0xFFFF0000u);
-      *(uint4_t*)(base + ((size_t)kb * kABN + pn) * 16) = unit;
     }
+  };
+  // Phase 2: rows pr and pr + 4 share one splice (their nibbles sit 16 bits apart).
+  auto word_pair = [&](uint32_t w, int pr, const uint32_t (&ra)[8], const uint32_t (&rb)[8]) -> uint32_t {
+    const uint32_t q2 = ((w >> (4 * pr)) & splice.mask_lo) | splice.magic;
+    half2_t s2, cz2;
+    if constexpr (MODE == kModeActWide) {
+      s2 = as_half2(__builtin_amdgcn_perm(ra[pr + 4], ra[pr], 0x05040100u));
+      cz2 = as_half2(__builtin_amdgcn_perm(ra[pr + 4], ra[pr], 0x07060302u));
+    } else {
+      s2 = as_half2(ra[pr] | (ra[pr + 4] << 16));
+      cz2 = as_half2(0xE400E400u | rb[pr] | (rb[pr + 4] << 16));
+    }
+    const half2_t dq = as_half2(q2) + cz2;  // exact q - z
+    if constexpr (DTYPE == Q4_DTYPE_F16) {
+      return as_u32(dq * s2);  // one fp16 rounding
+    } else {
+      const awq_float2_t f = {(float)dq.x * (float)s2.x, (float)dq.y * (float)s2.y};
+      return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, awq_bf16x2_t));
+    }
+  };
+  // Phase 3: o holds rows (0,4),(1,5),(2,6),(3,7): back to natural K order, one 16-byte unit.
+  auto word_store = [&](int buf, int i, const uint32_t (&o)[4]) {
+    unsigned char* base = smem + 2 * A_TILE + buf * B_TILE;
+    uint4_t unit;
+    unit.x = (o[0] & 0xFFFFu) | (o[1] << 16);
+    unit.y = (o[2] & 0xFFFFu) | (o[3] << 16);
+    unit.z = (o[0] >> 16) | (o[1] & 0xFFFF0000u);
+    unit.w = (o[2] >> 16) | (o[3] & 0xFFFF0000u);
+    *(uint4_t*)(base + ((size_t)(pkb0 + 2 * i) * kABN + pn) * 16) = unit;
+  };
+  auto store_b_act_word = [&](int buf, int kt, int i) {
+    uint32_t ra[8], rb[8], o[4];
+    word_params(kt, i, ra, rb);
+#pragma unroll
+    for (int pr = 0; pr < 4; ++pr) o[pr] = word_pair(braw[i], pr, ra, rb);
+    word_store(buf, i, o);
   };
   auto store_b_awq = [&](int buf) {
     if (!producer) return;
@@ -190,8 +243,12 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   };
 
   auto store_b = [&](int buf, int kt) {
-    if constexpr (ACT) store_b_act(buf, kt);
-    else store_b_awq(buf);
+    if constexpr (ACT) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) store_b_act_word(buf, kt, i);
+    } else {
+      store_b_awq(buf);
+    }
   };
 
   // ---- activation tile: global -> registers -> LDS (natural K order)
@@ -224,6 +281,34 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
+  if constexpr (TABLE) {
+    // every group's parameters for this tile's 128 columns: 16 scale units + 16 zero words each
+    unsigned char* tab = smem + 2 * A_TILE + 2 * B_TILE;
+    for (int u = tid; u < p.num_groups * 16; u += 256) {
+      const int g = u >> 4, c = u & 15;
+      const uint4_t s8 = *(const uint4_t*)(p.scales + (size_t)g * N + n0 + c * 8);
+      const uint32_t zw = gptq_zero_plus_one(p.qzeros[(size_t)g * NC + (n0 >> 3) + c]);
+      if constexpr (MODE == kModeActWide) {
+        const uint32_t sp[4] = {s8.x, s8.y, s8.z, s8.w};
+        uint32_t e[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const uint32_t sbits = (q & 1) ? sp[q >> 1] >> 16 : sp[q >> 1] & 0xFFFFu;
+          e[q] = sbits | ((0xE400u | ((zw >> (4 * q)) & 0xFu)) << 16);
+        }
+        uint4_t* dst = (uint4_t*)(tab + g * GROUP_BYTES + c * 32);
+        dst[0] = uint4_t{e[0], e[1], e[2], e[3]};
+        dst[1] = uint4_t{e[4], e[5], e[6], e[7]};
+      } else {
+        uint2_t zb;  // one byte per zero point, column order
+        zb.x = (zw & 0xFu) | ((zw & 0xF0u) << 4) | ((zw & 0xF00u) << 8) | ((zw & 0xF000u) << 12);
+        zb.y = ((zw >> 16) & 0xFu) | ((zw >> 12) & 0xF00u) | ((zw >> 8) & 0xF0000u) | ((zw >> 4) & 0xF000000u);
+        *(uint4_t*)(tab + g * GROUP_BYTES + c * 16) = s8;
+        *(uint2_t*)(tab + g * GROUP_BYTES + 2 * kABN + c * 8) = zb;
+      }
+    }
+    __syncthreads();
+  }
   load_a(kt_begin);
   load_b(kt_begin);
   store_a(0);
@@ -235,35 +320,76 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   const int a_off = ((wm * 64 + j) * kAUnits + kq) * 16;
   const int b_off = (kq * kABN + wn * 64 + j) * 16;
 
+  auto read_frags = [&](const unsigned char* ab, const unsigned char* bb, int s, uint4_t (&af)[2], uint4_t (&bf)[2]) {
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) af[mt] = *(const uint4_t*)(ab + (mt * 32 * kAUnits + 2 * s) * 16);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) bf[nt] = *(const uint4_t*)(bb + ((2 * s) * kABN + nt * 32) * 16);
+  };
+  auto mfma_one = [&](const uint4_t& a, const uint4_t& b, float16_t& c) {
+    if constexpr (DTYPE == Q4_DTYPE_F16) {
+      c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+    } else {
+      c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+  };
+  auto mfma_frags = [&](const uint4_t (&af)[2], const uint4_t (&bf)[2]) {
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) mfma_one(af[mt], bf[nt], acc[mt][nt]);
+  };
+  auto mfma_step = [&](const unsigned char* ab, const unsigned char* bb, int s) {
+    uint4_t af[2], bf[2];
+    read_frags(ab, bb, s, af, bf);
+    mfma_frags(af, bf);
+  };
+
   for (int kt = kt_begin; kt < KT; ++kt) {
     const int cur = (kt - kt_begin) & 1;
-    // the other buffer was last read in tile kt-1, before the barrier that ended it
-    store_a(cur ^ 1);
-    store_b(cur ^ 1, min(kt + 1, last_tile));
+    const int kt1 = min(kt + 1, last_tile);
     const int kt2 = min(kt + 2, last_tile);
-    load_a(kt2);
-    load_b(kt2);
     const unsigned char* ab = smem + cur * A_TILE + a_off;
     const unsigned char* bb = smem + 2 * A_TILE + cur * B_TILE + b_off;
+    // the other buffer was last read in tile kt-1, before the barrier that ended it
+    store_a(cur ^ 1);
+    load_a(kt2);
+    if constexpr (ACT) {
+      // one word of the next tile is unpacked in phases with one MFMA of this tile's K step
+      // between them (the order is pinned: the matrix pipe runs under the unpack even when
+      // the LDS table leaves room for a single workgroup per CU), then the word two tiles
+      // ahead is requested
+      static_assert(kABK / 16 == 4, "one producer word per MFMA K step");
 #pragma unroll
-    for (int s = 0; s < kABK / 16; ++s) {
-      uint4_t af[2], bf[2];
+      for (int s = 0; s < 4; ++s) {
+        uint4_t af[2], bf[2];
+        uint32_t ra[8], rb[8], o[4];
+        read_frags(ab, bb, s, af, bf);
+        word_params(kt1, s, ra, rb);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_one(af[0], bf[0], acc[0][0]);
+        __builtin_amdgcn_sched_barrier(0);
+        o[0] = word_pair(braw[s], 0, ra, rb);
+        o[1] = word_pair(braw[s], 1, ra, rb);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_one(af[0], bf[1], acc[0][1]);
+        __builtin_amdgcn_sched_barrier(0);
+        o[2] = word_pair(braw[s], 2, ra, rb);
+        o[3] = word_pair(braw[s], 3, ra, rb);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_one(af[1], bf[0], acc[1][0]);
+        __builtin_amdgcn_sched_barrier(0);
+        word_store(cur ^ 1, s, o);
+        load_b_word(kt2, s);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_one(af[1], bf[1], acc[1][1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+      store_b(cur ^ 1, kt1);
+      load_b(kt2);
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) af[mt] = *(const uint4_t*)(ab + (mt * 32 * kAUnits + 2 * s) * 16);
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt) bf[nt] = *(const uint4_t*)(bb + ((2 * s) * kABN + nt * 32) * 16);
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-          if constexpr (DTYPE == Q4_DTYPE_F16) {
-            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                __builtin_bit_cast(half8_t, af[mt]), __builtin_bit_cast(half8_t, bf[nt]), acc[mt][nt], 0, 0, 0);
-          } else {
-            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                __builtin_bit_cast(bf16x8_t, af[mt]), __builtin_bit_cast(bf16x8_t, bf[nt]), acc[mt][nt], 0, 0, 0);
-          }
-        }
+      for (int s = 0; s < kABK / 16; ++s) mfma_step(ab, bb, s);
     }
     __syncthreads();
   }
@@ -314,6 +440,28 @@ bool gemm_awq_supported(const q4_weight* w, int M, int dtype) {
   return (long)w->num_groups * w->groupsize >= w->K;
 }
 
+constexpr size_t kAwqTilesLdsBytes = 2 * (size_t)q4::kABM * q4::kAUnits * 16 + 2 * (size_t)(q4::kABK / 8) * q4::kABN * 16;
+
+// Kernel variant for a weight: act-order takes the 32-bit parameter table where it fits
+// beside the tiles, except that the smaller table is taken when only it leaves room for two
+// workgroups per CU and the grid has more than one workgroup per CU to offer; layers with
+// too many groups for either table gather from global memory.
+static int gemm_awq_mode(const q4_weight* w, long workgroups) {
+  using namespace q4;
+  if (w->layout != Q4_LAYOUT_GPTQ) return kModeAwq;
+  const size_t wide = kAwqTilesLdsBytes + (size_t)w->num_groups * kActWideGroupBytes;
+  const size_t narrow = kAwqTilesLdsBytes + (size_t)w->num_groups * kActNarrowGroupBytes;
+  const bool narrow_doubles =
+      workgroups > 256 && wide > kLdsBytesPerWorkgroup / 2 && narrow <= kLdsBytesPerWorkgroup / 2;
+  if (wide <= kLdsBytesPerWorkgroup && !narrow_doubles) return kModeActWide;
+  if (narrow <= kLdsBytesPerWorkgroup) return kModeActNarrow;
+  return kModeActGather;
+}
+
+bool gemm_act_order_table(const q4_weight* w) {
+  return w->layout == Q4_LAYOUT_GPTQ && w->g_idx != nullptr && gemm_awq_mode(w, 0) != q4::kModeActGather;
+}
+
 // 128 x 128 tiles, ~1.0 us per K tile alone on a CU, ~1.9 us when two workgroups share it
 int gemm_awq_splits(int M, int K, int N) {
   if (K % q4::kABK != 0 || N % q4::kABN != 0) return 1;
@@ -343,19 +491,26 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
     set_error("q4_linear(gemm/awq): grid too large");
     return Q4_ERR_UNSUPPORTED;
   }
-  const size_t smem = 2 * (size_t)kABM * kAUnits * 16 + 2 * (size_t)(kABK / 8) * kABN * 16;
-  const bool act = w->layout == Q4_LAYOUT_GPTQ;
+  const size_t tiles_smem = kAwqTilesLdsBytes;
+  const int mode = gemm_awq_mode(w, total);
+  const size_t smem = tiles_smem + (mode == kModeActWide     ? (size_t)w->num_groups * kActWideGroupBytes
+                                    : mode == kModeActNarrow ? (size_t)w->num_groups * kActNarrowGroupBytes
+                                                             : 0);
   auto launch = [&](auto k) {
     (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     hipLaunchKernelGGL(k, dim3((unsigned)total), dim3(256), smem, stream, gp);
   };
-  if (dtype == Q4_DTYPE_F16) {
-    if (act) launch(gemm_awq_kernel<Q4_DTYPE_F16, true>);
-    else launch(gemm_awq_kernel<Q4_DTYPE_F16, false>);
-  } else {
-    if (act) launch(gemm_awq_kernel<Q4_DTYPE_BF16, true>);
-    else launch(gemm_awq_kernel<Q4_DTYPE_BF16, false>);
-  }
+  auto launch_dtype = [&](auto dt) {
+    constexpr int DT = decltype(dt)::value;
+    switch (mode) {
+      case kModeAwq: launch(gemm_awq_kernel<DT, kModeAwq>); break;
+      case kModeActWide: launch(gemm_awq_kernel<DT, kModeActWide>); break;
+      case kModeActNarrow: launch(gemm_awq_kernel<DT, kModeActNarrow>); break;
+      default: launch(gemm_awq_kernel<DT, kModeActGather>); break;
+    }
+  };
+  if (dtype == Q4_DTYPE_F16) launch_dtype(std::integral_constant<int, Q4_DTYPE_F16>{});
+  else launch_dtype(std::integral_constant<int, Q4_DTYPE_BF16>{});
   if (splits > 1) launch_gemm_reduce(gp.partials, bias, y, M, w->N, splits, dtype, stream);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {
