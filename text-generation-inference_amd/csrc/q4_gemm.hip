@@ -508,15 +508,17 @@ static GemmPlan gemm_plan(int M, int K, int N) {
   return g;
 }
 
-int gemm_pick_splits(long tiles, int KT, int M, int N, double us_alone, double us_shared) {
+// per_cu: workgroups of this kernel that fit on a CU together (1 or 2)
+int gemm_pick_splits(long tiles, int KT, int M, int N, double us_alone, double us_shared, int per_cu) {
   static const int kCandidates[] = {1, 2, 3, 4, 6, 8, 12, 16};
   double best = -1.0;
   int splits = 1;
   for (int sp : kCandidates) {
     if (sp > 1 && KT / sp < 8) break;  // at least 8 K tiles (512 rows) per workgroup
     const long wgs = tiles * sp;
-    const long rounds = (wgs + 511) / 512;
-    const double per_tile = wgs <= 256 ? us_alone : us_shared;
+    const long slots = 256L * per_cu;
+    const long rounds = (wgs + slots - 1) / slots;
+    const double per_tile = (per_cu == 1 || wgs <= 256) ? us_alone : us_shared;
     double t = (double)rounds * ((KT + sp - 1) / sp) * per_tile;
     if (sp > 1) t += 5.0 + (double)sp * M * N * 8.0 / 5.0e6;
     if (best < 0.0 || t < best) {
@@ -545,8 +547,10 @@ void launch_gemm_reduce(const float* partials, const void* bias, void* y, int M,
 size_t gemm_workspace_bytes(int M, int K, int N) {
   if (M <= 16 || K % q4::kBK != 0 || N % 128 != 0) return 0;
   int splits = gemm_plan(M, K, N).splits;
-  const int other = gemm_awq_splits(M, K, N);
-  if (other > splits) splits = other;
+  for (const bool one_per_cu : {false, true}) {
+    const int other = gemm_awq_splits(M, K, N, one_per_cu);
+    if (other > splits) splits = other;
+  }
   return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
 

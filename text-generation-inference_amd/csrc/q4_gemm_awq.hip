@@ -462,10 +462,15 @@ bool gemm_act_order_table(const q4_weight* w) {
   return w->layout == Q4_LAYOUT_GPTQ && w->g_idx != nullptr && gemm_awq_mode(w, 0) != q4::kModeActGather;
 }
 
-// 128 x 128 tiles, ~1.0 us per K tile alone on a CU, ~1.9 us when two workgroups share it
-int gemm_awq_splits(int M, int K, int N) {
+// 128 x 128 tiles, ~1.0 us per K tile alone on a CU, ~1.9 us when two workgroups share it.
+// one_per_cu: act-order with its parameter table in LDS, which leaves room for a single
+// workgroup per CU (~1.0 us per K tile).  There a grid of a few hundred tiles runs in
+// rounds of 256 and a last, mostly empty round costs as much as a full one, so split-K is
+// also weighed above 256 tiles (8192 x 10240 at M = 512: 320 tiles, 2 rounds).
+int gemm_awq_splits(int M, int K, int N, bool one_per_cu) {
   if (K % q4::kABK != 0 || N % q4::kABN != 0) return 1;
   const long tiles = (long)((M + q4::kABM - 1) / q4::kABM) * (N / q4::kABN);
+  if (one_per_cu) return tiles < 1024 ? gemm_pick_splits(tiles, K / q4::kABK, M, N, 1.0, 1.0, 1) : 1;
   return tiles < 256 ? gemm_pick_splits(tiles, K / q4::kABK, M, N, 1.0, 1.9) : 1;
 }
 
@@ -480,7 +485,7 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
   AwqGemmParams gp;
   gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, w->g_idx, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
-  int splits = gemm_awq_splits(M, w->K, w->N);
+  int splits = gemm_awq_splits(M, w->K, w->N, gemm_act_order_table(w));
   if (splits > 1 && (workspace == nullptr ||
                      workspace_bytes < Q4_WORKSPACE_COUNTER_BYTES + (size_t)splits * M * w->N * sizeof(float)))
     splits = 1;  // no room for partial tiles: one workgroup per whole tile
