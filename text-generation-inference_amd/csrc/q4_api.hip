@@ -83,13 +83,13 @@ int q4_dequant(const q4_weight* w, void* w_out, int dtype, void* stream) {
 int q4_select_path(const q4_weight* w, int M, int dtype) {
   if (validate_weight(w, "q4_select_path") != Q4_OK) return Q4_ERR_INVALID_ARGUMENT;
   const bool contiguous_gptq = w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr;
+  const long weights = (long)w->K * w->N;
   if (contiguous_gptq) {
     // Measured crossover on MI355X (Llama-3-8B shapes).  The decode kernel's cost grows with
     // every 16-row chunk, the split-K GEMM's is nearly flat up to a few hundred rows:
     // 4096 x 4096 (2^24 weights) decode 15.2 / 17.1 / 22.7 us against GEMM 17.3 / 18.6 / 19.1 us
     // at M = 32 / 48 / 64; 4096 x 6144 decode 17.1 / 20.3 against 18.6 / 19.5 us at M = 32 / 40;
     // 14336 x 4096 and 4096 x 28672 are faster through the GEMM from M = 17 on.
-    const long weights = (long)w->K * w->N;
     const bool small = M <= 16 || (M <= 32 && weights <= (1L << 25)) || (M <= 48 && weights <= (1L << 24));
     if (small && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
     if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;
@@ -98,16 +98,24 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   }
   // AWQ and act-order: the decode kernels take any M in row chunks of 16; the MFMA kernel
   // that unpacks the weights into LDS (split-K when its tile grid is small) takes over where
-  // it measured faster on MI355X: AWQ from M = 17 on (4096 x 14336: 37.7 against 46.8 us at
-  // M = 17, 49 against 110 us at M = 64); act-order from M = 17 on when its parameter table
-  // fits in LDS (8192 x 10240: 57 against 67 us at M = 24, 52 against 140 us at M = 64; the
-  // kernel's time is flat in M up to 128 rows), from about M = 48 on when it has to gather
-  // scales and zero points from global memory (~2x slower per tile).
-  // Below 17 rows the AWQ decode kernel's time grows with every row (16 accumulator sets, ~250
-  // VGPRs) while the split-K GEMM stays flat at ~38 us for these sizes: 4096 x 14336 decode
-  // 35.9 / 43.9 us at M = 12 / 16, 14336 x 4096 decode 40.9 / 71.6 us at M = 8 / 16.
+  // it measured faster on MI355X.
+  // Act-order: from M = 17 on when its parameter table fits in LDS (8192 x 10240: 57 against
+  // 67 us at M = 24, 52 against 140 us at M = 64; the kernel's time is flat in M up to 128
+  // rows), from about M = 48 on when it has to gather scales and zero points from global
+  // memory (~2x slower per tile).
+  // AWQ: the decode kernel's time grows with every row (16 accumulator sets, ~250 VGPRs)
+  // while the split-K GEMM is flat in M (17 us for 4096 x 4096, 30 us for 4096 x 14336,
+  // 40 us for 8192 x 10240, 88 / 103 us for 28672 x 8192 / 8192 x 28672).  First M at which
+  // the GEMM was faster: 4096 x 4096 7, 4096 x 14336 10, 8192 x 8192 8, 5120 x 13824 8,
+  // 8192 x 10240 13, 14336 x 4096 6, 13824 x 5120 5, 28672 x 8192 14, 8192 x 28672 above 16.
   bool small = M <= 16 || (w->layout == Q4_LAYOUT_GPTQ && M <= 48 && !gemm_act_order_table(w));
-  if (w->layout == Q4_LAYOUT_AWQ && (M > 12 || (M > 7 && w->K > 8192))) small = false;
+  if (w->layout == Q4_LAYOUT_AWQ) {
+    int first_gemm_m = 8;
+    if (weights >= (1L << 27)) first_gemm_m = w->K >= 16384 ? 14 : 17;
+    else if (w->K > 8192) first_gemm_m = 6;
+    else if (w->K >= 8192 && weights > (1L << 26)) first_gemm_m = 12;
+    small = M < first_gemm_m;
+  }
   if (!small && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
   if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
   if (M > 16 && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;

@@ -23,7 +23,9 @@
 //     an fp16 scale and a zero-point byte (two reads per row) for up to 245 groups;
 //     layers with more groups gather the two values per row from the checkpoint tensors;
 //   * LDS layouts: activations [row][K block] with the row stride padded to 9 units,
-//     weights [K block][column]; both give conflict-free 128-bit fragment reads;
+//     weights [K block][column] with the low column bits XORed with the word index; both
+//     give conflict-free 128-bit fragment reads, and the swizzle spreads the AWQ
+//     producer's stores (16 words, columns 8 apart) over all banks;
 //   * double-buffered LDS, global loads for tile k+2 in flight while tile k is multiplied.
 #include "q4_common.cuh"
 
@@ -52,6 +54,12 @@ __device__ __forceinline__ AwqSplice awq_splice_consts() {
   asm volatile("" : "+s"(k.mask_lo), "+s"(k.mask_hi), "+v"(k.magic));
   return k;
 }
+
+// LDS slot of a weight unit inside its K block: the low three column bits are XORed with the
+// column's word index.  The AWQ producer stores one nibble position of 16 words per
+// instruction (columns 8 apart: without the swizzle every lane would hit the same banks);
+// consumers read 32 consecutive columns, which the swizzle only permutes.
+__device__ __forceinline__ int b_slot(int n) { return n ^ ((n >> 3) & 7); }
 
 typedef __bf16 awq_bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float awq_float2_t __attribute__((ext_vector_type(2)));
@@ -192,7 +200,7 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
     unit.y = (o[2] & 0xFFFFu) | (o[3] << 16);
     unit.z = (o[0] >> 16) | (o[1] & 0xFFFF0000u);
     unit.w = (o[2] >> 16) | (o[3] & 0xFFFF0000u);
-    *(uint4_t*)(base + ((size_t)(pkb0 + 2 * i) * kABN + pn) * 16) = unit;
+    *(uint4_t*)(base + ((size_t)(pkb0 + 2 * i) * kABN + b_slot(pn)) * 16) = unit;
   };
   auto store_b_act_word = [&](int buf, int kt, int i) {
     uint32_t ra[8], rb[8], o[4];
@@ -238,7 +246,7 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
         }
       }
       unit.x = o[0]; unit.y = o[1]; unit.z = o[2]; unit.w = o[3];
-      *(uint4_t*)(base + ((size_t)pb * kABN + pc * 8 + col) * 16) = unit;
+      *(uint4_t*)(base + ((size_t)pb * kABN + b_slot(pc * 8 + col)) * 16) = unit;
     }
   };
 
@@ -318,13 +326,13 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   __syncthreads();
 
   const int a_off = ((wm * 64 + j) * kAUnits + kq) * 16;
-  const int b_off = (kq * kABN + wn * 64 + j) * 16;
+  const int b_off[2] = {(kq * kABN + b_slot(wn * 64 + j)) * 16, (kq * kABN + b_slot(wn * 64 + 32 + j)) * 16};
 
   auto read_frags = [&](const unsigned char* ab, const unsigned char* bb, int s, uint4_t (&af)[2], uint4_t (&bf)[2]) {
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) af[mt] = *(const uint4_t*)(ab + (mt * 32 * kAUnits + 2 * s) * 16);
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) bf[nt] = *(const uint4_t*)(bb + ((2 * s) * kABN + nt * 32) * 16);
+    for (int nt = 0; nt < 2; ++nt) bf[nt] = *(const uint4_t*)(bb + b_off[nt] + (2 * s) * kABN * 16);
   };
   auto mfma_one = [&](const uint4_t& a, const uint4_t& b, float16_t& c) {
     if constexpr (DTYPE == Q4_DTYPE_F16) {
@@ -350,7 +358,7 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
     const int kt1 = min(kt + 1, last_tile);
     const int kt2 = min(kt + 2, last_tile);
     const unsigned char* ab = smem + cur * A_TILE + a_off;
-    const unsigned char* bb = smem + 2 * A_TILE + cur * B_TILE + b_off;
+    const unsigned char* bb = smem + 2 * A_TILE + cur * B_TILE;
     // the other buffer was last read in tile kt-1, before the barrier that ended it
     store_a(cur ^ 1);
     load_a(kt2);
