@@ -141,6 +141,54 @@ int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, 
 #define Q4_WORKSPACE_COUNTER_BYTES 1064960 /* = tickets + cells: the part that must start zero */
 size_t q4_workspace_bytes(int M, int K, int N);
 
+/*
+ * ---- Mixture of experts: the same linear layer, grouped over experts -----------------
+ *
+ * Replaces, for GPTQ checkpoints, what the reference's sparse MoE layer
+ * (server/text_generation_server/layers/moe/gptq_marlin.py:116-146 -> fused_marlin_moe,
+ * :232-351) gets from the un-vendored `kernels-community/moe` package (fused_topk +
+ * fused_marlin_moe): routing, the two grouped projections and the weighted sum.  The
+ * expert tensors stay in checkpoint layout, stacked along a leading expert dimension
+ * (what _pack_weight, gptq_marlin.py:186-229, builds) -- there is no Marlin repack.
+ *
+ * Rows are (token, expert) pairs sorted by expert.  q4_moe_route writes, all on the
+ * device and without a host round trip:
+ *   topk_weights f32 [tokens, topk], topk_ids int32 [tokens, topk]   routing result
+ *   sorted_tokens int32 [tokens*topk]   token of every sorted row
+ *   pair_slot     int32 [tokens*topk]   sorted row of pair (t, j) = pair_slot[t*topk + j]
+ *   expert_offsets int32 [experts + 1]  first sorted row of every expert
+ * The order of the rows of one expert is not specified (no output depends on it).
+ */
+typedef struct q4_moe_weight {
+  q4_weight expert0;      /* geometry and the tensors of expert 0: GPTQ layout, g_idx NULL */
+  int32_t num_experts;
+  int64_t qweight_stride; /* elements between consecutive experts' qweight / qzeros / scales */
+  int64_t qzeros_stride;
+  int64_t scales_stride;
+} q4_moe_weight;
+
+#define Q4_DTYPE_F32 2 /* gating logits only */
+
+/* softmax over experts, top-k (ties: lowest expert), optional renormalisation to sum 1,
+ * then the sort by expert described above.  experts <= 256, topk <= 8. */
+int q4_moe_route(const void* gating, int gating_dtype, int tokens, int experts, int topk, int renormalize,
+                 float* topk_weights, int32_t* topk_ids, int32_t* sorted_tokens, int32_t* pair_slot,
+                 int32_t* expert_offsets, void* stream);
+
+/* y[r, :] = x[x_rows ? x_rows[r] : r, :] @ W_e for every sorted row r of every expert e.
+ * y is [tokens*topk, N] in sorted order.  Up to 16 tokens the decode kernel runs once per
+ * expert that has rows; above, the MFMA kernel.  Workspace as for q4_linear, sized by
+ * q4_moe_workspace_bytes, zero-initialised once. */
+int q4_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_rows, const int32_t* expert_offsets,
+                  void* y, int tokens, int topk, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* out[t, :] = sum_j topk_weights[t, j] * y_sorted[pair_slot[t*topk + j], :], summed in fp32
+ * in the order j = 0, 1, ..., rounded once. */
+int q4_moe_combine(const void* y_sorted, const float* topk_weights, const int32_t* pair_slot, void* out,
+                   int tokens, int topk, int N, int dtype, void* stream);
+
+size_t q4_moe_workspace_bytes(const q4_moe_weight* w, int tokens, int topk);
+
 /* The Q4_PATH_* value q4_linear would take for this problem (negative on bad arguments). */
 int q4_select_path(const q4_weight* w, int M, int dtype);
 

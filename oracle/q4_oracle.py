@@ -26,6 +26,15 @@ Pinning status (what proves each function right, other than itself):
   matmul_fp32 / linear_forward
         pinned: float64 matmul, linearity, identity/one-hot activations that read
         single weight rows back.
+  moe_fused_topk
+        pinned: scipy.special.softmax + argsort brute force, hand-computed two-expert case,
+        weights sum to 1 after renormalisation; follows the in-tree pure-PyTorch routine.
+  moe_forward
+        structure pinned by the in-tree dense formulation it follows (every expert applied
+        to every token, weighted by the scattered top-k weights) through its already pinned
+        parts (linear_forward, gate_up_forward).  The reference's GPTQ MoE kernels
+        (kernels-community/moe, fused_marlin_moe) are not in the tree: their internal
+        roundings are parity unpinned; GPU results are compared within the GEMM tolerance.
   awq_inference_engine.gemm_forward_cuda (third-party, huggingface/llm-awq @ bd1dc2d5,
   not in the reference tree): parity unpinned by any runnable reference test; covered
   through the in-tree equivalence fast_awq_to_gptq (awq/conversion_utils.py:83-97).
@@ -286,6 +295,45 @@ def gate_up_forward(x, w, act="silu", bias=None, dtype="f16"):
         a = bf16_bits_to_f32(f32_to_bf16_bits(a))
         out = f32_to_bf16_bits(a * yr[..., inter:])
     return exact, out
+
+
+# --------------------------------------------------------------------------- mixture of experts
+
+
+def moe_fused_topk(gating: np.ndarray, topk: int, renormalize: bool):
+    """Routing of the sparse MoE layers (server/text_generation_server/layers/moe/
+    fused_moe_ipex.py:53-65): softmax over the experts in fp32, the `topk` largest
+    probabilities per token (descending; equal values: lowest expert first), optionally
+    renormalised to sum 1.  Returns (weights f32 [T, topk], ids int32 [T, topk])."""
+    g = np.asarray(gating).astype(np.float32)
+    e = np.exp(g - g.max(axis=1, keepdims=True), dtype=np.float32)
+    prob = (e / e.sum(axis=1, keepdims=True, dtype=np.float32)).astype(np.float32)
+    ids = np.argsort(-prob, axis=1, kind="stable")[:, :topk]
+    w = np.take_along_axis(prob, ids, axis=1)
+    if renormalize:
+        w = w / w.sum(axis=1, keepdims=True, dtype=np.float32)
+    return w.astype(np.float32), ids.astype(np.int32)
+
+
+def moe_forward(x, gating, gate_up_w, down_w, topk, renormalize=True, act="silu", dtype="f16"):
+    """Sparse MoE block, following the reference's dense formulation
+    (layers/moe/__init__.py:158-194): out = sum_e weights[:, e] * down_e(act(gate_e(x)) * up_e(x))
+    with weights the top-k routing weights scattered over the experts (zero elsewhere, so
+    only chosen experts are evaluated here).  gate_up_w[e] is the dense [K, 2I] weight that
+    packs [gate | up], down_w[e] the dense [I, K] one.  Every expert's projections carry the
+    roundings of linear_forward / gate_up_forward; the weighted sum is kept in fp32 and
+    rounded once.  Returns (out_f32, out_cast)."""
+    T = x.shape[0]
+    w, ids = moe_fused_topk(gating, topk, renormalize)
+    H = down_w[0].shape[1]
+    out = np.zeros((T, H), dtype=np.float32)
+    for e in sorted(set(ids.reshape(-1).tolist())):
+        rows, slots = np.nonzero(ids == e)
+        _, h = gate_up_forward(x[rows], gate_up_w[e], act, None, dtype)
+        _, d = linear_forward(h, down_w[e], None, dtype)
+        out[rows] += w[rows, slots][:, None] * to_f32(d, dtype)
+    cast = out.astype(np.float16) if dtype == "f16" else f32_to_bf16_bits(out)
+    return out, cast
 
 
 # --------------------------------------------------------------------------- synthetic inputs

@@ -19,6 +19,7 @@ from .layers.gptq import (  # noqa: F401
     set_device,
 )
 from .layers.awq.quantize import WQLinear  # noqa: F401
+from .layers.moe import GPTQSparseMoELayer, GPTQMoEWeight  # noqa: F401
 from .layers.awq import conversion_utils  # noqa: F401
 from .utils.weights import Weights, WeightsLoader, DefaultWeightsLoader, UnquantizedWeight  # noqa: F401
 from .utils.quantization import get_loader, get_quantizer_config  # noqa: F401
@@ -32,6 +33,8 @@ __all__ = [
     "QuantLinear",
     "ExllamaQuantLinear",
     "WQLinear",
+    "GPTQSparseMoELayer",
+    "GPTQMoEWeight",
     "get_linear",
     "gate_up_act",
     "create_exllama_buffers",

@@ -7,7 +7,7 @@ with an error that says how to build it; nothing falls back to PyTorch or the CP
 from __future__ import annotations
 
 import ctypes
-from ctypes import POINTER, Structure, c_char_p, c_int, c_int32, c_size_t, c_void_p
+from ctypes import POINTER, Structure, c_char_p, c_int, c_int32, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
 HERE = Path(__file__).resolve().parent
@@ -17,6 +17,7 @@ LAYOUT_GPTQ = 0
 LAYOUT_AWQ = 1
 DTYPE_F16 = 0
 DTYPE_BF16 = 1
+DTYPE_F32 = 2  # gating logits of the mixture-of-experts router only
 PATH_AUTO = 0
 PATH_GEMV = 1
 PATH_GEMM = 2
@@ -50,6 +51,18 @@ class Q4Weight(Structure):
     ]
 
 
+class Q4MoeWeight(Structure):
+    """Mirror of `struct q4_moe_weight`: expert 0's view plus the strides to the next expert."""
+
+    _fields_ = [
+        ("expert0", Q4Weight),
+        ("num_experts", c_int32),
+        ("qweight_stride", c_int64),
+        ("qzeros_stride", c_int64),
+        ("scales_stride", c_int64),
+    ]
+
+
 # name -> (restype, argtypes); the single source for binding and for the export test
 SIGNATURES = {
     "q4_abi_version": (c_int, []),
@@ -74,6 +87,16 @@ SIGNATURES = {
     "q4_act_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "q4_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "q4_select_path": (c_int, [POINTER(Q4Weight), c_int, c_int]),
+    "q4_moe_route": (
+        c_int,
+        [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
+    "q4_moe_linear": (
+        c_int,
+        [POINTER(Q4MoeWeight), c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "q4_moe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "q4_moe_workspace_bytes": (c_size_t, [POINTER(Q4MoeWeight), c_int, c_int]),
 }
 
 _lib = None

@@ -149,6 +149,30 @@ struct Problem {
   int gate_up_act;
 };
 
+// Grouped launch over the experts of a mixture-of-experts layer.  The rows of the problem are
+// the (token, expert) pairs sorted by expert: expert e owns sorted rows offsets[e] ..
+// offsets[e + 1] - 1, its tensors sit e * stride elements behind expert 0's, and it writes
+// the same rows of y.  x_rows, when given, names the row of x every sorted row reads (the
+// first projection reads tokens); otherwise x is in sorted order like y.
+struct MoeView {
+  const int32_t* __restrict__ offsets;  // [experts + 1], device memory
+  const int32_t* __restrict__ x_rows;   // [pairs] or nullptr
+  long qweight_stride, qzeros_stride, scales_stride;
+};
+
+// Narrows `p` to expert e.  Returns the expert's first sorted row; p.M becomes its row count
+// (possibly 0).  With x_rows the activation pointer stays whole (rows are looked up).
+__device__ __forceinline__ int moe_enter(Problem& p, const MoeView& mv, int e) {
+  const int row0 = mv.offsets[e];
+  p.M = mv.offsets[e + 1] - row0;
+  p.qweight += (size_t)e * mv.qweight_stride;
+  p.qzeros += (size_t)e * mv.qzeros_stride;
+  p.scales += (size_t)e * mv.scales_stride;
+  p.y = (uint16_t*)p.y + (size_t)row0 * p.N;
+  if (mv.x_rows == nullptr) p.x = (const uint16_t*)p.x + (size_t)row0 * p.K;
+  return row0;
+}
+
 }  // namespace q4
 
 // Host-side launchers implemented by the kernel translation units.

@@ -1,0 +1,467 @@
+// Prefill kernels (device code shared by the translation units that instantiate them).
+//
+// Prefill path: y[M, N] = x @ dequant(W) for large M on the MFMA units (gfx950).
+//
+// MFMA-bound: 2*M*N*K flops against 0.5 B/weight of HBM traffic.  Tiling (wave64):
+//   * a workgroup of 4 waves owns a BM x 256 output tile; wave w owns columns
+//     n0 + 64 w .. + 63 for all BM rows (4 waves side by side along N);
+//   * the B operand never touches LDS: a packed GPTQ word holds 8 consecutive K values of
+//     one column, which is exactly what lane (column j, K block kq) of a
+//     v_mfma_f32_32x32x16 supplies.  Each lane loads two adjacent words (columns
+//     nw + 2j, nw + 2j + 1) of packed row K/8 + kq with one 64-bit load (256 contiguous
+//     bytes per half-wave), unpacks them in registers to the reference's fp16 weight
+//     round_once(s * (q - z)) -- bit-identical to the dense dequantized matrix -- and feeds
+//     BM/32 MFMAs with each fragment.  Because the waves split N, no weight is unpacked
+//     twice inside a workgroup;
+//   * the A operand (activations) is staged through LDS, double buffered, in 16-byte
+//     units [row][K block] whose 8 values are stored in the order [0,4,1,5,2,6,3,7] that
+//     the nibble splice produces (see q4_common.cuh), so weights are never repacked;
+//     the row stride is padded to 9 units, which makes the 128-bit fragment reads
+//     conflict free;
+//   * packed weights are prefetched two K tiles (128 rows) ahead in registers, activations
+//     one tile ahead; fp32 accumulators live in VGPRs (BM = 128: 128 of them, two
+//     workgroups per CU so one wave's unpacking overlaps the other's MFMAs).
+#pragma once
+
+#include <type_traits>
+
+#include "q4_common.cuh"
+
+namespace q4 {
+
+constexpr int kBK = 64;            // K rows per tile
+constexpr int kKSteps = kBK / 16;  // MFMA K steps per tile
+constexpr int kAUnitsPerRow = kBK / 8 + 1;  // 16-byte units per LDS row, padded
+
+struct GemmParams {
+  Problem p;
+  // Split-K for grids that do not fill the chip: `splits` workgroups share an output tile,
+  // each takes a contiguous range of K tiles and writes its fp32 partial tile to
+  // partials[split][M][N]; gemm_reduce_kernel adds them in split order.  splits == 1:
+  // the output is written directly.
+  float* __restrict__ partials;
+  int splits;
+  MoeView moe;  // grouped launches only (MOE kernels): blockIdx.y is the expert
+};
+
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
+struct SpliceK {
+  uint32_t mask_lo, mask_hi, magic;
+};
+__device__ __forceinline__ SpliceK gemm_splice_consts() {
+  // Hidden from constant folding so that (w & mask) | magic selects v_and_or_b32 (a
+  // three-operand VALU op cannot carry literals).  The asm is empty on purpose.
+  SpliceK k{0x000F000Fu, 0x00F000F0u, 0x64006400u};
+  asm volatile("" : "+s"(k.mask_lo), "+s"(k.mask_hi), "+v"(k.magic));
+  return k;
+}
+
+// Per-column constants of one quantisation group.
+struct ColConsts {
+  half2_t czlo, czhi;  // -(1024 + z), -(64 + z), both halves equal
+  half2_t s2;          // (s, s)
+  float sf;            // float(s), bf16 path
+};
+
+__device__ __forceinline__ ColConsts make_col_consts(uint32_t z, half_t s) {
+  ColConsts c;
+  c.czlo = as_half2(0xE400E400u | z | (z << 16));
+  c.czhi = as_half2(0xD400D400u | (z << 4) | (z << 20));
+  c.s2 = half2_t{s, s};
+  c.sf = (float)s;
+  return c;
+}
+
+// One packed word -> MFMA B fragment (8 weights of one column, K order 0,4,1,5,2,6,3,7).
+template <int DTYPE>
+__device__ __forceinline__ uint4_t dequant_word(uint32_t w, const ColConsts& c, const SpliceK& k) {
+  const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+  const uint32_t w8 = w >> 8;
+  half2_t d[4];  // exact (q - z)
+  d[0] = as_half2((w & k.mask_lo) | k.magic) + c.czlo;
+  d[1] = as_half2((w & k.mask_hi) | k.magic) * sixteenth + c.czhi;
+  d[2] = as_half2((w8 & k.mask_lo) | k.magic) + c.czlo;
+  d[3] = as_half2((w8 & k.mask_hi) | k.magic) * sixteenth + c.czhi;
+  uint4_t out;
+  if constexpr (DTYPE == Q4_DTYPE_F16) {
+    // one fp16 multiply per weight: the reference's rounding
+    out.x = as_u32(d[0] * c.s2);
+    out.y = as_u32(d[1] * c.s2);
+    out.z = as_u32(d[2] * c.s2);
+    out.w = as_u32(d[3] * c.s2);
+  } else {
+    // bf16: exact fp32 product, rounded once
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float lo = (float)d[i].x * c.sf;
+      const float hi = (float)d[i].y * c.sf;
+      o[i] = (uint32_t)f32_to_bf16_rne(lo) | ((uint32_t)f32_to_bf16_rne(hi) << 16);
+    }
+    out.x = o[0]; out.y = o[1]; out.z = o[2]; out.w = o[3];
+  }
+  return out;
+}
+
+template <int DTYPE>
+__device__ __forceinline__ float16_t mfma32(const uint4_t a, const uint4_t b, float16_t c) {
+  if constexpr (DTYPE == Q4_DTYPE_F16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a),
+                                                  __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+}
+
+// BM: rows per workgroup (128 or 256).  GPT: quantisation groups per K tile (1 or 2).
+// NW: packed words (columns) per lane and K step: 2 -> 256-column workgroup tile, 1 -> 128.
+// MOE: grouped launch, blockIdx.y is the expert; its row count is read from device memory, so
+// the grid covers the largest possible count and surplus workgroups leave at once.
+template <int DTYPE, int BM, int GPT, int NW, bool MOE = false>
+__global__ __launch_bounds__(256, (BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm_gptq_kernel(GemmParams gp) {
+  int moe_row0 = 0;
+  if constexpr (MOE) {
+    moe_row0 = moe_enter(gp.p, gp.moe, blockIdx.y);
+    if (gp.p.M <= 0) return;
+  }
+  constexpr int MT = BM / 32;                      // MFMA row tiles per wave
+  constexpr int A_LOADS = BM * (kBK / 8) / 256;    // 16-byte activation loads per thread per tile
+  constexpr int A_TILE_BYTES = BM * kAUnitsPerRow * 16;
+  extern __shared__ __align__(16) unsigned char smem[];  // two activation tiles
+  const Problem& p = gp.p;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int j = lane & 31;
+  const int kq = lane >> 5;
+  const int N = p.N, K = p.K, M = p.M;
+
+  // XCD-aware tile order.  Workgroup ids are dealt round-robin to the 8 XCDs (id % 8), each
+  // with its own L2.  Every XCD is given its own slice of M tiles and walks all column
+  // blocks of it: the activation rows of the slice (BM x K, a few MB) stay resident in that
+  // XCD's L2 and are re-read from there by every column block, while the packed weights are
+  // the streamed operand (each column block is read once per XCD, prefetched ahead).
+  // (A grid of a single round, at most one workgroup per CU, measured faster the other way
+  // round: each XCD takes a few column blocks and all M tiles of them.)
+  const int tiles_m = (M + BM - 1) / BM;
+  constexpr int BN = 4 * 32 * NW;
+  const int tiles_n = N / BN;
+  int tm, tn;
+  const int total_tiles = tiles_m * tiles_n;
+  if constexpr (MOE) {
+    if ((int)blockIdx.x >= total_tiles * gp.splits) return;
+  }
+  const int split = blockIdx.x / total_tiles;  // workgroups of one split are neighbours in id
+  {
+    const int bid = blockIdx.x - split * total_tiles;
+    const int total = total_tiles;
+    if (tiles_m % 8 == 0 && total > 256) {
+      const int mpx = tiles_m >> 3;  // M tiles per XCD
+      const int xcd = bid & 7;
+      const int local = bid >> 3;
+      tm = xcd * mpx + local % mpx;
+      tn = local / mpx;
+    } else if (total % 8 == 0) {
+      const int lin = (bid & 7) * (total >> 3) + (bid >> 3);
+      tm = lin % tiles_m;
+      tn = lin / tiles_m;
+    } else {
+      tm = bid % tiles_m;
+      tn = bid / tiles_m;
+    }
+  }
+  const int m0 = tm * BM;
+  const int n0 = tn * BN;
+  const int nw = n0 + wave * 32 * NW;  // first column of this wave
+  const int ncol = nw + NW * j;        // first of this lane's NW columns
+
+  const SpliceK splice = gemm_splice_consts();
+  const int KT_all = K / kBK;
+  // this workgroup's K tiles [kt_begin, KT)
+  const int kt_begin = (int)((long)split * KT_all / gp.splits);
+  const int KT = (int)((long)(split + 1) * KT_all / gp.splits);
+
+  // ---- packed-weight stream: words [K/8 + kq][ncol, ncol+1], two K tiles ahead
+  const char* wbase = (const char*)p.qweight;
+  const uint32_t w_lane = ((uint32_t)kq * (uint32_t)N + (uint32_t)ncol) * 4u;
+  const size_t kstep_bytes = (size_t)N * 8;  // two packed rows per MFMA K step
+  struct BWords { uint32_t v[NW]; };
+  BWords bq[2][kKSteps];
+  auto load_b = [&](int kt, BWords (&dst)[kKSteps]) {
+#pragma unroll
+    for (int s = 0; s < kKSteps; ++s)
+    {
+      const char* addr = wbase + (size_t)(kt * kKSteps + s) * kstep_bytes + w_lane;
+      if constexpr (NW == 2) {
+        const uint2_t t = *(const uint2_t*)addr;
+        dst[s].v[0] = t.x; dst[s].v[1] = t.y;
+      } else {
+        dst[s].v[0] = *(const uint32_t*)addr;
+      }
+    }
+  };
+
+  // ---- group constants for this lane's two columns.  They are rebuilt for every tile
+  // from two tiny (cached) loads, which keeps the steady-state loop free of branches.
+  ColConsts cc[GPT][NW], cc_next[GPT][NW];
+  uint32_t sraw[GPT], zraw[GPT];
+  const int zshift = (ncol & 7) * 4;
+  auto load_group_raw = [&](int kt) {
+#pragma unroll
+    for (int g = 0; g < GPT; ++g) {
+      int gi = (kt * kBK + g * (kBK / GPT)) / p.groupsize;
+      gi = min(gi, p.num_groups - 1);
+      if constexpr (NW == 2) sraw[g] = *(const uint32_t*)(p.scales + (size_t)gi * N + ncol);
+      else sraw[g] = *(const uint16_t*)(p.scales + (size_t)gi * N + ncol);
+      zraw[g] = p.qzeros[(size_t)gi * (N >> 3) + (ncol >> 3)];
+    }
+  };
+  auto make_group = [&](ColConsts (&dst)[GPT][NW]) {
+#pragma unroll
+    for (int g = 0; g < GPT; ++g) {
+      const uint32_t z2 = gptq_zero_plus_one(zraw[g]) >> zshift;
+      const half2_t s01 = as_half2(sraw[g]);
+      dst[g][0] = make_col_consts(z2 & 0xFu, s01.x);
+      if constexpr (NW == 2) dst[g][1] = make_col_consts((z2 >> 4) & 0xFu, s01.y);
+    }
+  };
+
+  // ---- activation tile: global -> registers -> (permuted) LDS
+  const uint16_t* xs = (const uint16_t*)p.x;
+  // Register staging sets: with two sets (128-row tiles) a tile's loads are issued two
+  // tiles before they are written to LDS; the 256-row tile has registers for one set only.
+  constexpr int ASETS = BM == 128 ? 2 : 1;
+  uint4_t areg[ASETS][A_LOADS];
+  int moe_xrow[MOE ? A_LOADS : 1];  // grouped launch with a row map: x row of each staged row
+  if constexpr (MOE) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int row = min(m0 + ((tid + 256 * i) >> 3), M - 1);
+      moe_xrow[i] = gp.moe.x_rows != nullptr ? gp.moe.x_rows[moe_row0 + row] : row;
+    }
+  }
+  auto load_a = [&](int kt, auto set_c) {
+    constexpr int set = decltype(set_c)::value % ASETS;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int u = tid + 256 * i;
+      const int m = u >> 3, kb = u & 7;
+      // rows past M re-read the last row: their results are never stored
+      const int row = MOE ? moe_xrow[i] : min(m0 + m, M - 1);
+      areg[set][i] = *(const uint4_t*)(xs + (size_t)row * K + kt * kBK + kb * 8);
+    }
+  };
+  auto store_a = [&](int buf, auto set_c) {
+    constexpr int set = decltype(set_c)::value % ASETS;
+    unsigned char* base = smem + buf * A_TILE_BYTES;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int u = tid + 256 * i;
+      const int m = u >> 3, kb = u & 7;
+      const uint4_t v = areg[set][i];
+      uint4_t o;
+      o.x = (v.x & 0xFFFFu) | (v.z << 16);
+      o.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
+      o.z = (v.y & 0xFFFFu) | (v.w << 16);
+      o.w = (v.y >> 16) | (v.w & 0xFFFF0000u);
+      *(uint4_t*)(base + (m * kAUnitsPerRow + kb) * 16) = o;
+    }
+  };
+
+  float16_t acc[MT][NW];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int f = 0; f < NW; ++f)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mt][f][r] = 0.f;
+
+  const int a_lane_off = (j * kAUnitsPerRow + kq) * 16;
+  uint4_t afrag[2][MT];  // A fragments of the current / next MFMA K step
+  uint4_t bfrag[2][NW];  // unpacked B fragments of the current / next step
+  auto read_a = [&](int buf, int s, uint4_t (&dst)[MT]) {
+    const unsigned char* abase = smem + buf * A_TILE_BYTES + a_lane_off;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      dst[mt] = *(const uint4_t*)(abase + (mt * 32 * kAUnitsPerRow + 2 * s) * 16);
+  };
+  auto group_of_step = [](int s) { return GPT == 1 ? 0 : (s * 16) / (kBK / GPT); };
+
+  // ---- prologue: tile 0 staged, tile 1 in flight, first fragments ready
+  const int last_tile = KT - 1;
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  load_a(kt_begin, I0{});
+  load_b(kt_begin, bq[0]);
+  load_b(min(kt_begin + 1, last_tile), bq[1]);
+  load_group_raw(kt_begin);
+  if constexpr (ASETS == 2) load_a(min(kt_begin + 1, last_tile), I1{});
+  store_a(0, I0{});
+  if constexpr (ASETS == 2) load_a(min(kt_begin + 2, last_tile), I0{});
+  else load_a(min(kt_begin + 1, last_tile), I0{});
+  make_group(cc);
+  __syncthreads();
+  read_a(0, 0, afrag[0]);
+#pragma unroll
+  for (int f = 0; f < NW; ++f) bfrag[0][f] = dequant_word<DTYPE>(bq[0][0].v[f], cc[0][f], splice);
+
+  // One K tile, software pipelined: while the MFMAs of step s run, the VALU unpacks the
+  // weights of step s+1 and the LDS returns its A fragments; the global loads of tile
+  // kt+2 and the LDS writes of tile kt+1 are spread over the steps.  Tile indices past the
+  // end are clamped (the last tile is fetched again and ignored) so the body has no
+  // branches and the scheduler sees one region per step.  `cur` selects the LDS buffer and
+  // the weight-register set at compile time; the loop is unrolled by two.
+  auto tile_step = [&](int kt, auto cur_c) {
+    constexpr int cur = decltype(cur_c)::value;
+    const int kt1 = min(kt + 1, last_tile);
+    const int kt2 = min(kt + 2, last_tile);
+#pragma unroll
+    for (int s = 0; s < kKSteps; ++s) {
+      const int sb = s & 1;
+      // (1) LDS reads of the next step's A fragments go first so that they get the early
+      // LDS slots of this step.  The last step reads the first fragments of tile kt+1 from
+      // the other buffer, which the barrier below (between steps 2 and 3) has published.
+      if (s + 1 < kKSteps) read_a(cur, s + 1, afrag[sb ^ 1]);
+      else read_a(cur ^ 1, 0, afrag[sb ^ 1]);
+      // (2) unpack the next step's weights
+      if (s + 1 < kKSteps) {
+        const int g = group_of_step(s + 1);
+#pragma unroll
+        for (int f = 0; f < NW; ++f)
+          bfrag[sb ^ 1][f] = dequant_word<DTYPE>(bq[cur][s + 1].v[f], cc[g][f], splice);
+      } else {
+#pragma unroll
+        for (int f = 0; f < NW; ++f)
+          bfrag[sb ^ 1][f] = dequant_word<DTYPE>(bq[cur ^ 1][0].v[f], cc_next[0][f], splice);
+      }
+      // (3) side work of this step
+      if (s == 0) {
+        // tile kt+1 (staged in register set (kt+1) % ASETS) -> the other LDS buffer
+        store_a(cur ^ 1, std::integral_constant<int, cur ^ 1>{});
+        load_group_raw(kt1);    // scales / zero points the next tile starts with
+      }
+      if (s == 1) {
+        // refill the set that was just written out: tile kt+3 with two sets, kt+2 with one
+        if constexpr (ASETS == 2) load_a(min(kt + 3, last_tile), std::integral_constant<int, cur ^ 1>{});
+        else load_a(kt2, I0{});
+      }
+      if (s == 2) make_group(cc_next);
+      // (4) the MFMAs of this step
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int f = 0; f < NW; ++f) acc[mt][f] = mfma32<DTYPE>(afrag[sb][mt], bfrag[sb][f], acc[mt][f]);
+      }
+      if (s == kKSteps - 1) load_b(kt2, bq[cur]);
+      // interleave: after every MFMA a few VALU ops, one LDS op and one global load
+#pragma unroll
+      for (int i = 0; i < NW * MT; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+        __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+      if (s == kKSteps - 2) {
+        // One barrier per tile.  Here every wave has finished reading this tile's buffer
+        // (the step-3 fragments were read above) and has written its share of the next
+        // tile into the other buffer (step 0), so after the barrier the other buffer may
+        // be read (step 3) and this one overwritten (step 0 of the next tile).
+        __syncthreads();
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < GPT; ++g) {
+#pragma unroll
+      for (int f = 0; f < NW; ++f) cc[g][f] = cc_next[g][f];
+    }
+  };
+  {
+    int kt = kt_begin;
+    for (; kt + 1 < KT; kt += 2) {
+      tile_step(kt, std::integral_constant<int, 0>{});
+      tile_step(kt + 1, std::integral_constant<int, 1>{});
+    }
+    if (kt < KT) tile_step(kt, std::integral_constant<int, 0>{});
+  }
+
+  // ---- epilogue: C layout of the 32x32 MFMA: register r of lane (j, kq) is row
+  // 8*(r/4) + 4*kq + r%4, column j.  Fragments 0/1 are adjacent columns -> one 32-bit store.
+  if (gp.splits > 1) {
+    // fp32 partial tile; bias, rounding and the store to y happen in the reduction kernel
+    float* part = gp.partials + (size_t)split * M * N;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
+        if (m < M) {
+          if constexpr (NW == 2) *(float2_t*)(part + (size_t)m * N + ncol) = float2_t{acc[mt][0][r], acc[mt][1][r]};
+          else part[(size_t)m * N + ncol] = acc[mt][0][r];
+        }
+      }
+    }
+    return;
+  }
+  uint16_t* y = (uint16_t*)p.y;
+  float bias_f[NW] = {};
+  const bool has_bias = p.bias != nullptr;
+  if (has_bias) {
+#pragma unroll
+    for (int f = 0; f < NW; ++f) bias_f[f] = load_act<DTYPE>(p.bias, ncol + f);
+  }
+  // The sum is rounded to the activation dtype first and the bias added in that dtype
+  // (one more rounding), like `out + bias` on a half tensor.
+  auto finish = [&](float v, float b) -> uint32_t {
+    uint16_t o = store_act<DTYPE>(v);
+    if (has_bias) {
+      float ob;
+      if constexpr (DTYPE == Q4_DTYPE_F16) ob = (float)__builtin_bit_cast(half_t, o);
+      else ob = bf16_bits_to_f32(o);
+      o = store_act<DTYPE>(ob + b);
+    }
+    return o;
+  };
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
+      if (m < M) {
+        const uint32_t lo = finish(acc[mt][0][r], bias_f[0]);
+        if constexpr (NW == 2) {
+          const uint32_t hi = finish(acc[mt][1][r], bias_f[1]);
+          *(uint32_t*)(y + (size_t)m * N + ncol) = lo | (hi << 16);
+        } else {
+          y[(size_t)m * N + ncol] = (uint16_t)lo;
+        }
+      }
+    }
+  }
+}
+
+// y[m][n] = round(sum over splits of partials[s][m][n]) (+ bias), four columns per thread.
+template <int DTYPE>
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restrict__ partials,
+                                                          const void* __restrict__ bias, uint16_t* __restrict__ y,
+                                                          int M, int N, int splits) {
+  const long quads = (long)M * (N >> 2);
+  const size_t stride = (size_t)M * N;
+  for (long q = (long)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (long)gridDim.x * blockDim.x) {
+    const size_t e = (size_t)q * 4;
+    const int n = (int)(e % (size_t)N);
+    float4_t sum = *(const float4_t*)(partials + e);
+    for (int sp = 1; sp < splits; ++sp) {
+      const float4_t v = *(const float4_t*)(partials + (size_t)sp * stride + e);
+      sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+    }
+    uint2_t o;
+    o.x = (uint32_t)finish_output<DTYPE>(sum.x, bias, n) | ((uint32_t)finish_output<DTYPE>(sum.y, bias, n + 1) << 16);
+    o.y = (uint32_t)finish_output<DTYPE>(sum.z, bias, n + 2) | ((uint32_t)finish_output<DTYPE>(sum.w, bias, n + 3) << 16);
+    *(uint2_t*)(y + e) = o;
+  }
+}
+
+}  // namespace q4
+

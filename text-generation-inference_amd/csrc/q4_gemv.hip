@@ -225,6 +225,8 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.cells = cfg.splits > 1 ? (unsigned long long*)((char*)workspace + Q4_WORKSPACE_TICKET_BYTES) : nullptr;
   gp.slab_stride = slab_stride;
   gp.slab_bytes = (int)slab_bytes;
+  gp.partial_rows = M;
+  gp.moe = q4::MoeView{};
   dim3 grid((unsigned)(ntiles * cfg.splits), (unsigned)mchunks);
   dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
   if (gate_up_act != 0) {

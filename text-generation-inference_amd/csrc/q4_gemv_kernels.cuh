@@ -51,6 +51,8 @@ struct GemvParams {
   int fixed_point_split;  // fp16 outputs: combine the splits with one 64-bit atomic per element
   int slab_stride;  // bytes between activation rows in LDS
   int slab_bytes;   // size of the activation slab region
+  int partial_rows;  // rows of one split's slice of `partials` (M; grouped launches: all pairs)
+  MoeView moe;       // grouped launches only (MOE kernels): blockIdx.z is the expert
 };
 
 // Constants of the nibble splice, hidden from constant folding (empty asm, no instruction
@@ -148,15 +150,18 @@ struct SlabStager {
   static constexpr int kLoads = 2;  // 16-byte activation loads per thread kept in flight
   uint4_t xv[kLoads];
   const uint16_t* xs;
+  const int32_t* rows;  // grouped launches: row of x behind every staged row, else nullptr
   int kb_per_row, items;
 
   __device__ __forceinline__ uint4_t fetch(const GemvParams& gp, int idx) const {
     const int m = idx / kb_per_row;
     const int kb = idx - m * kb_per_row;
-    return *(const uint4_t*)(xs + (size_t)m * gp.p.K + kb * 8);
+    const int mr = rows != nullptr ? rows[m] : m;
+    return *(const uint4_t*)(xs + (size_t)mr * gp.p.K + kb * 8);
   }
-  __device__ __forceinline__ void issue(const GemvParams& gp, const Decomp& d) {
-    xs = (const uint16_t*)gp.p.x + (size_t)d.mb * gp.p.K + d.kwg0;
+  __device__ __forceinline__ void issue(const GemvParams& gp, const Decomp& d, const int32_t* row_map = nullptr) {
+    rows = row_map;
+    xs = (const uint16_t*)gp.p.x + (row_map != nullptr ? 0 : (size_t)d.mb * gp.p.K) + d.kwg0;
     kb_per_row = d.KR >> 3;
     items = d.mloc * kb_per_row;
 #pragma unroll
@@ -336,7 +341,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
     for (int r = 0; r < RMAX; ++r) {
       const int m = 4 * d.kq + r;
       if (m < d.mloc) {
-        float* dst = gp.partials + ((size_t)d.split * p.M + d.mb + m) * N + col0;
+        float* dst = gp.partials + ((size_t)d.split * gp.partial_rows + d.mb + m) * N + col0;
 #pragma unroll
         for (int t = 0; t < NT; ++t)
           __hip_atomic_store(dst + (FUSE && t >= NT / 2 ? half_n + t - NT / 2 : t), out[t][r], __ATOMIC_RELAXED,
@@ -347,14 +352,14 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   __shared__ uint32_t ticket_s;
-  uint32_t* ticket = gp.tickets + blockIdx.y * d.ntiles + d.tile;
+  uint32_t* ticket = gp.tickets + (blockIdx.z * gridDim.y + blockIdx.y) * d.ntiles + d.tile;
   if (d.tid == 0) {
     ticket_s = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
   if (ticket_s != (uint32_t)(gp.splits - 1)) return;
   {
-    const size_t sstride = (size_t)p.M * N;
+    const size_t sstride = (size_t)gp.partial_rows * N;
     // sum of the partials of one output element, in split order
     auto total = [&](int m, int n) {
       const float* src = gp.partials + (size_t)(d.mb + m) * N + n;
@@ -409,10 +414,19 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
 // four neighbouring gate columns and the four up columns N/2 further (two 128-bit loads per
 // packed row); a wave covers 64 gate and 64 up columns, and the activation and the product
 // happen in the lane that owns both sums.
-template <int DTYPE, int RMAX, int GSTEPS, bool STATIC128, int WORDS, bool FUSE = false>
+// MOE: grouped launch, blockIdx.z is the expert; its rows (at most 16 per row block) and its
+// tensors are found through gp.moe, workgroups of experts without rows leave at once.
+template <int DTYPE, int RMAX, int GSTEPS, bool STATIC128, int WORDS, bool FUSE = false, bool MOE = false>
 __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   static_assert(FUSE == (WORDS == 8), "eight words per lane = four gate + four up columns (fused only)");
   extern __shared__ __align__(16) unsigned char smem[];
+  const int32_t* moe_rows = nullptr;
+  if constexpr (MOE) {
+    const int row0 = moe_enter(gp.p, gp.moe, blockIdx.z);
+    if (gp.p.M <= (int)blockIdx.y * kRowsPerBlock) return;
+    gp.partials += (size_t)row0 * gp.p.N;
+    if (gp.moe.x_rows != nullptr) moe_rows = gp.moe.x_rows + row0 + blockIdx.y * kRowsPerBlock;
+  }
   const Problem& p = gp.p;
   const Decomp d = make_decomp(gp, 16 * WORDS);
   const int N = p.N;
@@ -425,7 +439,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   constexpr int PF = kPrefetch * 4 / WORDS;  // chunks in flight: same bytes for every WORDS
 
   SlabStager<true> slab;
-  slab.issue(gp, d);
+  slab.issue(gp, d, moe_rows);
 
   // ---- issue the first PF chunks of weight loads.  Addresses are a wave-uniform 64-bit
   // base plus a per-lane 32-bit byte offset.

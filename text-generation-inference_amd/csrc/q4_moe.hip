@@ -1,0 +1,451 @@
+// Mixture of experts: routing, the grouped (per-expert) linear layer and the weighted sum.
+//
+// The rows of the grouped problem are the (token, expert) pairs sorted by expert.  Nothing
+// on this path needs the host to know how many rows an expert received:
+//   * moe_route_kernel (one workgroup) computes softmax -> top-k -> renormalisation per token
+//     and counting-sorts the pairs by expert with LDS atomics;
+//   * the grouped linear layer launches the ordinary decode or prefill kernel once more per
+//     expert (a grid dimension); every workgroup reads its expert's row range from device
+//     memory, narrows the problem to it and leaves at once when the range is empty or ends
+//     before its tile.  The decode kernel therefore streams the packed weights of exactly
+//     the experts that were chosen, once each, whatever the number of tokens (<= 16);
+//   * moe_combine_kernel adds the topk rows of every token, weighted, in fp32.
+#include "q4_gemm_kernels.cuh"
+#include "q4_gemv_kernels.cuh"
+
+namespace q4 {
+
+constexpr int kMoeMaxExperts = 256;
+constexpr int kMoeMaxTopk = 8;
+
+template <int GDT>
+__device__ __forceinline__ float load_logit(const void* g, size_t i) {
+  if constexpr (GDT == Q4_DTYPE_F16) return (float)((const half_t*)g)[i];
+  else if constexpr (GDT == Q4_DTYPE_BF16) return bf16_bits_to_f32(((const uint16_t*)g)[i]);
+  else return ((const float*)g)[i];
+}
+
+template <int GDT>
+__global__ __launch_bounds__(1024) void moe_route_kernel(const void* __restrict__ gating, int T, int E, int topk,
+                                                         int renormalize, float* __restrict__ topk_weights,
+                                                         int32_t* __restrict__ topk_ids,
+                                                         int32_t* __restrict__ sorted_tokens,
+                                                         int32_t* __restrict__ pair_slot,
+                                                         int32_t* __restrict__ expert_offsets) {
+  __shared__ int count[kMoeMaxExperts];
+  __shared__ int cursor[kMoeMaxExperts];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+
+  // ---- per token: softmax over the experts in fp32, the topk largest (ties: lowest index)
+  for (int t = tid; t < T; t += blockDim.x) {
+    const size_t row = (size_t)t * E;
+    float mx = load_logit<GDT>(gating, row);
+    for (int e = 1; e < E; ++e) mx = fmaxf(mx, load_logit<GDT>(gating, row + e));
+    float sum = 0.f;
+    for (int e = 0; e < E; ++e) sum += expf(load_logit<GDT>(gating, row + e) - mx);
+    int chosen[kMoeMaxTopk];
+    float weight[kMoeMaxTopk];
+    float wsum = 0.f;
+    for (int j = 0; j < topk; ++j) {
+      int best = -1;
+      float bv = 0.f;
+      for (int e = 0; e < E; ++e) {
+        bool taken = false;
+        for (int i = 0; i < j; ++i) taken |= chosen[i] == e;
+        if (taken) continue;
+        const float v = load_logit<GDT>(gating, row + e);
+        if (best < 0 || v > bv) {
+          best = e;
+          bv = v;
+        }
+      }
+      chosen[j] = best;
+      weight[j] = expf(bv - mx) / sum;
+      wsum += weight[j];
+    }
+    for (int j = 0; j < topk; ++j) {
+      topk_ids[(size_t)t * topk + j] = chosen[j];
+      topk_weights[(size_t)t * topk + j] = renormalize ? weight[j] / wsum : weight[j];
+      atomicAdd(&count[chosen[j]], 1);
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      expert_offsets[e] = run;
+      cursor[e] = run;
+      run += count[e];
+    }
+    expert_offsets[E] = run;
+  }
+  __syncthreads();
+  // ---- scatter: every pair takes the next free row of its expert
+  for (int t = tid; t < T; t += blockDim.x) {
+    for (int j = 0; j < topk; ++j) {
+      const int e = topk_ids[(size_t)t * topk + j];  // written above by this same thread
+      const int slot = atomicAdd(&cursor[e], 1);
+      sorted_tokens[slot] = t;
+      pair_slot[(size_t)t * topk + j] = slot;
+    }
+  }
+}
+
+// out[t, n..n+7] = sum_j w[t, j] * y[slot(t, j), n..n+7]
+template <int DTYPE>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t* __restrict__ y,
+                                                          const float* __restrict__ topk_weights,
+                                                          const int32_t* __restrict__ pair_slot,
+                                                          uint16_t* __restrict__ out, int topk, int N) {
+  const int t = blockIdx.y;
+  const int n = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (n >= N) return;
+  float acc[8] = {};
+  for (int j = 0; j < topk; ++j) {
+    const float w = topk_weights[(size_t)t * topk + j];
+    const int slot = pair_slot[(size_t)t * topk + j];
+    const uint4_t v = *(const uint4_t*)(y + (size_t)slot * N + n);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float lo, hi;
+      if constexpr (DTYPE == Q4_DTYPE_F16) {
+        const half2_t h = as_half2(u[i]);
+        lo = (float)h.x;
+        hi = (float)h.y;
+      } else {
+        lo = bf16_bits_to_f32((uint16_t)(u[i] & 0xFFFFu));
+        hi = bf16_bits_to_f32((uint16_t)(u[i] >> 16));
+      }
+      acc[2 * i] = fmaf(w, lo, acc[2 * i]);
+      acc[2 * i + 1] = fmaf(w, hi, acc[2 * i + 1]);
+    }
+  }
+  uint4_t o;
+  o.x = (uint32_t)store_act<DTYPE>(acc[0]) | ((uint32_t)store_act<DTYPE>(acc[1]) << 16);
+  o.y = (uint32_t)store_act<DTYPE>(acc[2]) | ((uint32_t)store_act<DTYPE>(acc[3]) << 16);
+  o.z = (uint32_t)store_act<DTYPE>(acc[4]) | ((uint32_t)store_act<DTYPE>(acc[5]) << 16);
+  o.w = (uint32_t)store_act<DTYPE>(acc[6]) | ((uint32_t)store_act<DTYPE>(acc[7]) << 16);
+  *(uint4_t*)(out + (size_t)t * N + n) = o;
+}
+
+}  // namespace q4
+
+namespace q4host {
+
+using q4::GemmParams;
+using q4::GemvParams;
+using q4::MoeView;
+using q4::Problem;
+
+namespace {
+
+int validate_moe_weight(const q4_moe_weight* w, const char* who) {
+  if (w == nullptr) {
+    set_error("%s: null q4_moe_weight", who);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  const q4_weight& e0 = w->expert0;
+  if (w->num_experts < 1 || w->num_experts > q4::kMoeMaxExperts) {
+    set_error("%s: num_experts=%d must be in 1..%d", who, w->num_experts, q4::kMoeMaxExperts);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (e0.qweight == nullptr || e0.qzeros == nullptr || e0.scales == nullptr) {
+    set_error("%s: null qweight/qzeros/scales", who);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (e0.K < 8 || e0.N < 8 || e0.K % 8 != 0 || e0.N % 8 != 0 || e0.groupsize < 1 || e0.num_groups < 1 ||
+      (long)e0.num_groups * e0.groupsize < e0.K) {
+    set_error("%s: bad geometry K=%d N=%d groupsize=%d num_groups=%d", who, e0.K, e0.N, e0.groupsize,
+              e0.num_groups);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (e0.layout != Q4_LAYOUT_GPTQ || e0.g_idx != nullptr) {
+    set_error("%s: the grouped kernels take the GPTQ layout without g_idx (layout=%d g_idx=%p)", who, e0.layout,
+              (const void*)e0.g_idx);
+    return Q4_ERR_UNSUPPORTED;
+  }
+  const long qw = (long)(e0.K / 8) * e0.N, qz = (long)e0.num_groups * (e0.N / 8), sc = (long)e0.num_groups * e0.N;
+  if (w->qweight_stride < qw || w->qzeros_stride < qz || w->scales_stride < sc) {
+    set_error("%s: expert strides (%lld, %lld, %lld) smaller than one expert (%ld, %ld, %ld)", who,
+              (long long)w->qweight_stride, (long long)w->qzeros_stride, (long long)w->scales_stride, qw, qz, sc);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  return Q4_OK;
+}
+
+// Decode plan of a grouped launch: the single-matrix configuration for the same row count,
+// with the cross-workgroup K split divided by the number of experts expected to be active
+// (their workgroups fill the chip together).
+struct MoeGemvPlan {
+  bool ok;
+  GemvConfig cfg;
+  int ntiles;
+  size_t smem;
+};
+
+MoeGemvPlan moe_gemv_plan(const q4_moe_weight* w, int tokens, int topk, int dtype) {
+  using namespace q4;
+  MoeGemvPlan pl{};
+  const q4_weight* e0 = &w->expert0;
+  const int rows = tokens < kRowsPerBlock ? tokens : kRowsPerBlock;
+  if (tokens > kRowsPerBlock || !gemv_supported(e0, rows, dtype)) return pl;
+  GemvConfig cfg = gemv_pick_config(e0, rows);
+  cfg.words = 4;
+  if (e0->N % (64 * cfg.wcol) != 0) cfg.wcol = 1;
+  if (cfg.wcol * cfg.wk > 8 || e0->K % (cfg.wk * 128) != 0) return pl;
+  long active = (long)tokens * topk;
+  if (active > w->num_experts) active = w->num_experts;
+  int splits = (int)(cfg.splits / active);
+  if (splits < 1) splits = 1;
+  while (splits > 1 && e0->K % (splits * cfg.wk * 128) != 0) --splits;
+  const int ntiles = e0->N / (64 * cfg.wcol);
+  if ((long)ntiles * w->num_experts > Q4_WORKSPACE_TICKET_BYTES / 4) splits = 1;
+  // the activation slab of 16 rows x K / splits must fit LDS: split further if it does not
+  const size_t smem_limit = 160 * 1024 - 1024;
+  auto smem_of = [&](int sp) {
+    const size_t slab = ((size_t)rows * ((size_t)e0->K / sp * 2 + 16) + 15) & ~(size_t)15;
+    const size_t red = (size_t)(cfg.wk - 1) * cfg.wcol * 4 * 4 * 64 * sizeof(float);
+    return slab > red ? slab : red;
+  };
+  while (smem_of(splits) > smem_limit) {
+    int next = splits + 1;
+    while (next <= e0->K / (cfg.wk * 128) && e0->K % (next * cfg.wk * 128) != 0) ++next;
+    if (next > e0->K / (cfg.wk * 128) || (long)ntiles * w->num_experts > Q4_WORKSPACE_TICKET_BYTES / 4) return pl;
+    splits = next;
+  }
+  cfg.splits = splits;
+  pl.ok = true;
+  pl.cfg = cfg;
+  pl.ntiles = ntiles;
+  pl.smem = smem_of(splits);
+  return pl;
+}
+
+template <typename Kernel>
+void launch_with_smem(Kernel k, dim3 grid, dim3 block, size_t smem, hipStream_t stream, const GemvParams& gp) {
+  if (smem > 64 * 1024)
+    (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  hipLaunchKernelGGL(k, grid, block, smem, stream, gp);
+}
+
+template <int DTYPE>
+void launch_moe_gemv_dtype(int gs, dim3 grid, dim3 block, size_t smem, hipStream_t stream, const GemvParams& gp) {
+  using namespace q4;
+  if (gs == 128) launch_with_smem(gemv_gptq_kernel<DTYPE, 4, 4, true, 4, false, true>, grid, block, smem, stream, gp);
+  else if (gs > 128) launch_with_smem(gemv_gptq_kernel<DTYPE, 4, 4, false, 4, false, true>, grid, block, smem, stream, gp);
+  else if (gs == 64) launch_with_smem(gemv_gptq_kernel<DTYPE, 4, 2, false, 4, false, true>, grid, block, smem, stream, gp);
+  else launch_with_smem(gemv_gptq_kernel<DTYPE, 4, 1, false, 4, false, true>, grid, block, smem, stream, gp);
+}
+
+template <int DTYPE, int NW>
+void launch_moe_gemm_tile(int gs, dim3 grid, size_t smem, hipStream_t stream, const GemmParams& gp) {
+  using namespace q4;
+  if (gs == 32) hipLaunchKernelGGL((gemm_gptq_kernel<DTYPE, 128, 2, NW, true>), grid, dim3(256), smem, stream, gp);
+  else hipLaunchKernelGGL((gemm_gptq_kernel<DTYPE, 128, 1, NW, true>), grid, dim3(256), smem, stream, gp);
+}
+
+MoeView make_view(const q4_moe_weight* w, const int32_t* x_rows, const int32_t* offsets) {
+  MoeView mv;
+  mv.offsets = offsets;
+  mv.x_rows = x_rows;
+  mv.qweight_stride = (long)w->qweight_stride;
+  mv.qzeros_stride = (long)w->qzeros_stride;
+  mv.scales_stride = (long)w->scales_stride;
+  return mv;
+}
+
+}  // namespace
+
+size_t moe_workspace_bytes(const q4_moe_weight* w, int tokens, int topk) {
+  const MoeGemvPlan pl = moe_gemv_plan(w, tokens, topk, Q4_DTYPE_F16);
+  size_t bytes = Q4_WORKSPACE_COUNTER_BYTES;
+  if (pl.ok && pl.cfg.splits > 1) bytes += (size_t)pl.cfg.splits * tokens * topk * w->expert0.N * sizeof(float);
+  return bytes;
+}
+
+int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_rows, const int32_t* offsets, void* y,
+                      int tokens, int topk, int dtype, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  using namespace q4;
+  const q4_weight* e0 = &w->expert0;
+  const int pairs = tokens * topk;
+  const MoeView mv = make_view(w, x_rows, offsets);
+  const MoeGemvPlan pl = moe_gemv_plan(w, tokens, topk, dtype);
+  if (pl.ok) {
+    const GemvConfig& cfg = pl.cfg;
+    float* partials = nullptr;
+    uint32_t* tickets = nullptr;
+    if (cfg.splits > 1) {
+      const size_t need = Q4_WORKSPACE_COUNTER_BYTES + (size_t)cfg.splits * pairs * e0->N * sizeof(float);
+      if (workspace == nullptr || workspace_bytes < need) {
+        set_error("q4_moe_linear: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+        return Q4_ERR_WORKSPACE;
+      }
+      tickets = (uint32_t*)workspace;
+      partials = (float*)((char*)workspace + Q4_WORKSPACE_COUNTER_BYTES);
+    }
+    GemvParams gp;
+    gp.p = Problem{e0->qweight, e0->qzeros, (const half_t*)e0->scales, nullptr, x, nullptr, y,
+                   0,           e0->K,      e0->N,                     e0->groupsize, e0->num_groups};
+    gp.p.gate_up_act = 0;
+    gp.partials = partials;
+    gp.tickets = tickets;
+    gp.wcol = cfg.wcol;
+    gp.wk = cfg.wk;
+    gp.splits = cfg.splits;
+    gp.cells = nullptr;
+    gp.fixed_point_split = 0;
+    gp.slab_stride = e0->K / cfg.splits * 2 + 16;
+    gp.slab_bytes = (int)pl.smem;
+    gp.partial_rows = pairs;
+    gp.moe = mv;
+    const dim3 grid((unsigned)(pl.ntiles * cfg.splits), 1, (unsigned)w->num_experts);
+    const dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
+    if (dtype == Q4_DTYPE_F16) launch_moe_gemv_dtype<Q4_DTYPE_F16>(e0->groupsize, grid, block, pl.smem, stream, gp);
+    else launch_moe_gemv_dtype<Q4_DTYPE_BF16>(e0->groupsize, grid, block, pl.smem, stream, gp);
+  } else if (gemm_supported(e0, tokens, dtype)) {
+    GemmParams gp;
+    gp.p = Problem{e0->qweight, e0->qzeros, (const half_t*)e0->scales, nullptr, x, nullptr, y,
+                   0,           e0->K,      e0->N,                     e0->groupsize, e0->num_groups};
+    gp.p.gate_up_act = 0;
+    gp.partials = nullptr;
+    gp.splits = 1;
+    gp.moe = mv;
+    // an expert can receive every token: the grid covers `tokens` rows per expert
+    const int nw = e0->N % 256 == 0 ? 2 : 1;
+    const long tiles = (long)((tokens + 127) / 128) * (e0->N / (128 * nw));
+    if (tiles > 0x7fffffffL || w->num_experts > 65535) {
+      set_error("q4_moe_linear: grid too large");
+      return Q4_ERR_UNSUPPORTED;
+    }
+    const dim3 grid((unsigned)tiles, (unsigned)w->num_experts);
+    const size_t smem = 2 * (size_t)128 * kAUnitsPerRow * 16;
+    if (dtype == Q4_DTYPE_F16) {
+      if (nw == 2) launch_moe_gemm_tile<Q4_DTYPE_F16, 2>(e0->groupsize, grid, smem, stream, gp);
+      else launch_moe_gemm_tile<Q4_DTYPE_F16, 1>(e0->groupsize, grid, smem, stream, gp);
+    } else {
+      if (nw == 2) launch_moe_gemm_tile<Q4_DTYPE_BF16, 2>(e0->groupsize, grid, smem, stream, gp);
+      else launch_moe_gemm_tile<Q4_DTYPE_BF16, 1>(e0->groupsize, grid, smem, stream, gp);
+    }
+  } else {
+    set_error("q4_moe_linear: no grouped kernel for tokens=%d K=%d N=%d groupsize=%d", tokens, e0->K, e0->N,
+              e0->groupsize);
+    return Q4_ERR_UNSUPPORTED;
+  }
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    set_error("q4_moe_linear: launch failed: %s", hipGetErrorString(err));
+    return Q4_ERR_LAUNCH;
+  }
+  return Q4_OK;
+}
+
+}  // namespace q4host
+
+using namespace q4host;
+
+extern "C" {
+
+int q4_moe_route(const void* gating, int gating_dtype, int tokens, int experts, int topk, int renormalize,
+                 float* topk_weights, int32_t* topk_ids, int32_t* sorted_tokens, int32_t* pair_slot,
+                 int32_t* expert_offsets, void* stream) {
+  if (tokens < 0 || experts < 1 || experts > q4::kMoeMaxExperts || topk < 1 || topk > q4::kMoeMaxTopk ||
+      topk > experts) {
+    set_error("q4_moe_route: tokens=%d experts=%d (1..%d) topk=%d (1..%d, <= experts)", tokens, experts,
+              q4::kMoeMaxExperts, topk, q4::kMoeMaxTopk);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (expert_offsets == nullptr ||
+      (tokens > 0 && (gating == nullptr || topk_weights == nullptr || topk_ids == nullptr ||
+                      sorted_tokens == nullptr || pair_slot == nullptr))) {
+    set_error("q4_moe_route: null pointer");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(1), block(1024);
+  if (gating_dtype == Q4_DTYPE_F16)
+    hipLaunchKernelGGL(q4::moe_route_kernel<Q4_DTYPE_F16>, grid, block, 0, s, gating, tokens, experts, topk,
+                       renormalize, topk_weights, topk_ids, sorted_tokens, pair_slot, expert_offsets);
+  else if (gating_dtype == Q4_DTYPE_BF16)
+    hipLaunchKernelGGL(q4::moe_route_kernel<Q4_DTYPE_BF16>, grid, block, 0, s, gating, tokens, experts, topk,
+                       renormalize, topk_weights, topk_ids, sorted_tokens, pair_slot, expert_offsets);
+  else if (gating_dtype == Q4_DTYPE_F32)
+    hipLaunchKernelGGL(q4::moe_route_kernel<Q4_DTYPE_F32>, grid, block, 0, s, gating, tokens, experts, topk,
+                       renormalize, topk_weights, topk_ids, sorted_tokens, pair_slot, expert_offsets);
+  else {
+    set_error("q4_moe_route: unknown gating dtype %d", gating_dtype);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    set_error("q4_moe_route: launch failed: %s", hipGetErrorString(err));
+    return Q4_ERR_LAUNCH;
+  }
+  return Q4_OK;
+}
+
+int q4_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_rows, const int32_t* expert_offsets,
+                  void* y, int tokens, int topk, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = validate_moe_weight(w, "q4_moe_linear");
+  if (rc != Q4_OK) return rc;
+  if (dtype != Q4_DTYPE_F16 && dtype != Q4_DTYPE_BF16) {
+    set_error("q4_moe_linear: unknown dtype %d", dtype);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (tokens < 0 || topk < 1 || topk > q4::kMoeMaxTopk || (long)tokens * topk > 0x7fffffffL) {
+    set_error("q4_moe_linear: tokens=%d topk=%d", tokens, topk);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (tokens == 0) return Q4_OK;
+  if (x == nullptr || y == nullptr || expert_offsets == nullptr) {
+    set_error("q4_moe_linear: null x / y / expert_offsets");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  return launch_moe_linear(w, x, x_rows, expert_offsets, y, tokens, topk, dtype, workspace, workspace_bytes,
+                           (hipStream_t)stream);
+}
+
+int q4_moe_combine(const void* y_sorted, const float* topk_weights, const int32_t* pair_slot, void* out, int tokens,
+                   int topk, int N, int dtype, void* stream) {
+  if (tokens < 0 || tokens > 65535 * 16 || topk < 1 || topk > q4::kMoeMaxTopk || N < 8 || N % 8 != 0 ||
+      (dtype != Q4_DTYPE_F16 && dtype != Q4_DTYPE_BF16)) {
+    set_error("q4_moe_combine: tokens=%d topk=%d N=%d (multiple of 8) dtype=%d", tokens, topk, N, dtype);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (tokens == 0) return Q4_OK;
+  if (y_sorted == nullptr || topk_weights == nullptr || pair_slot == nullptr || out == nullptr) {
+    set_error("q4_moe_combine: null pointer");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  const int per_block = 256 * 8;
+  // rows beyond the grid's y limit are taken in slices
+  for (int t0 = 0; t0 < tokens; t0 += 65535) {
+    const int nt = tokens - t0 < 65535 ? tokens - t0 : 65535;
+    const dim3 grid((unsigned)((N + per_block - 1) / per_block), (unsigned)nt);
+    const float* tw = topk_weights + (size_t)t0 * topk;
+    const int32_t* ps = pair_slot + (size_t)t0 * topk;
+    uint16_t* o = (uint16_t*)out + (size_t)t0 * N;
+    if (dtype == Q4_DTYPE_F16)
+      hipLaunchKernelGGL(q4::moe_combine_kernel<Q4_DTYPE_F16>, grid, dim3(256), 0, s, (const uint16_t*)y_sorted, tw, ps,
+                         o, topk, N);
+    else
+      hipLaunchKernelGGL(q4::moe_combine_kernel<Q4_DTYPE_BF16>, grid, dim3(256), 0, s, (const uint16_t*)y_sorted, tw,
+                         ps, o, topk, N);
+  }
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    set_error("q4_moe_combine: launch failed: %s", hipGetErrorString(err));
+    return Q4_ERR_LAUNCH;
+  }
+  return Q4_OK;
+}
+
+size_t q4_moe_workspace_bytes(const q4_moe_weight* w, int tokens, int topk) {
+  if (validate_moe_weight(w, "q4_moe_workspace_bytes") != Q4_OK || tokens < 0 || topk < 1) return 0;
+  return moe_workspace_bytes(w, tokens, topk);
+}
+
+}  // extern "C"

@@ -1,0 +1,140 @@
+"""Sparse mixture-of-experts layer on GPTQ int4 experts.
+
+Mirrors the constructor and forward of the reference's `GPTQMarlinSparseMoELayer`
+(server/text_generation_server/layers/moe/gptq_marlin.py:54-146): the experts' gate/up and
+down projections are loaded through the same `Weights` calls (`get_multi_weights_col`,
+`get_weights_row`, :149-183) and stacked along a leading expert dimension (:186-229), and
+`forward(x, gating_output=...)` routes every token to its top-k experts.  Differences: the
+tensors stay in checkpoint layout (no Marlin repack, hence no perm / is_full_k fields) and
+the grouped int4 kernels of this package do the work that the reference takes from the
+`kernels-community/moe` package, which only exists for CUDA.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+import torch.nn as nn
+
+from ... import ops
+from ..gptq import GPTQWeight
+from ..gptq.quant_linear import is_trivial_g_idx
+
+
+@dataclass
+class GPTQMoEWeight:
+    """Stacked experts of one projection: qweight [E, K/8, N], qzeros [E, G, N/8], scales [E, G, N]."""
+
+    qweight: torch.Tensor
+    qzeros: torch.Tensor
+    scales: torch.Tensor
+    groupsize: int
+
+    def packed(self) -> ops.PackedMoeWeight:
+        return ops.make_packed_moe(self.qweight, self.qzeros, self.scales, self.groupsize)
+
+
+def _check_expert(weight, name: str) -> GPTQWeight:
+    if not isinstance(weight, GPTQWeight):
+        raise ValueError(f"{name}: expected GPTQ weights, got {type(weight).__name__}")
+    if weight.bits != 4:
+        raise NotImplementedError(f"{name}: only 4-bit experts are supported, got {weight.bits}")
+    if weight.use_awq_kernel:
+        raise NotImplementedError(
+            f"{name}: experts in the AWQ layout are not covered by the grouped kernels; load the checkpoint "
+            "with quantize='gptq' so that the loader converts it (fast_awq_to_gptq)"
+        )
+    if weight.g_idx is not None and not is_trivial_g_idx(weight.g_idx, weight.groupsize):
+        raise NotImplementedError(f"{name}: act-order (desc_act) experts are not covered by the grouped kernels")
+    return weight
+
+
+def _pack_weight(*, n_experts: int, expert: int, moe_weight: Optional[GPTQMoEWeight], weight: GPTQWeight) -> GPTQMoEWeight:
+    """gptq_marlin.py:186-229: allocate on the first expert, copy every expert into its slice."""
+    if moe_weight is None:
+        moe_weight = GPTQMoEWeight(
+            qweight=torch.empty((n_experts,) + weight.qweight.shape, dtype=weight.qweight.dtype, device=weight.qweight.device),
+            qzeros=torch.empty((n_experts,) + weight.qzeros.shape, dtype=weight.qzeros.dtype, device=weight.qzeros.device),
+            scales=torch.empty((n_experts,) + weight.scales.shape, dtype=weight.scales.dtype, device=weight.scales.device),
+            groupsize=weight.groupsize,
+        )
+    if weight.groupsize != moe_weight.groupsize:
+        raise ValueError(f"expert {expert} has groupsize {weight.groupsize}, expert 0 {moe_weight.groupsize}")
+    moe_weight.qweight[expert] = weight.qweight
+    moe_weight.qzeros[expert] = weight.qzeros
+    moe_weight.scales[expert] = weight.scales
+    return moe_weight
+
+
+def _load_expert_multi_weights_col(*, prefix: str, n_experts: int, names: List[str], weights) -> GPTQMoEWeight:
+    moe_weight = None
+    for i in range(n_experts):
+        weight = weights.get_multi_weights_col([f"{prefix}.{i}.{name}" for name in names], 0)
+        moe_weight = _pack_weight(n_experts=n_experts, expert=i, moe_weight=moe_weight,
+                                  weight=_check_expert(weight, f"{prefix}.{i}"))
+    assert moe_weight is not None
+    return moe_weight
+
+
+def _load_expert_weights_row(*, prefix: str, n_experts: int, name: str, weights) -> GPTQMoEWeight:
+    moe_weight = None
+    for i in range(n_experts):
+        weight = weights.get_weights_row(f"{prefix}.{i}.{name}")
+        moe_weight = _pack_weight(n_experts=n_experts, expert=i, moe_weight=moe_weight,
+                                  weight=_check_expert(weight, f"{prefix}.{i}.{name}"))
+    assert moe_weight is not None
+    return moe_weight
+
+
+class GPTQSparseMoELayer(nn.Module):
+    """MoE layer on the grouped int4 kernels; same keyword constructor as the reference's."""
+
+    def __init__(
+        self,
+        *,
+        n_expert_group: Optional[int],
+        n_experts: int,
+        prefix: str,
+        renormalize: bool,
+        topk: int,
+        topk_group: Optional[int],
+        weights,
+        gate_proj_name: str = "gate_proj",
+        up_proj_name: str = "up_proj",
+        down_proj_name: str = "down_proj",
+        scoring_func: Optional[str] = "softmax",
+        e_score_correction_bias: Optional[float] = None,
+        hidden_act: str = "silu",
+    ):
+        super().__init__()
+        assert (n_expert_group is None) == (
+            topk_group is None
+        ), "n_expert_group and topk_group must both be None or have some value"
+        if n_expert_group is not None:
+            raise NotImplementedError("grouped top-k routing (n_expert_group / topk_group) is not implemented")
+        if scoring_func not in (None, "softmax"):
+            raise NotImplementedError(f"scoring func {scoring_func} is not handled")
+        if e_score_correction_bias is not None:
+            raise NotImplementedError("e_score_correction_bias is not implemented")
+        self.n_experts = n_experts
+        self.topk = topk
+        self.renormalize = renormalize
+        self.hidden_act = hidden_act
+        self.gate_up_proj = _load_expert_multi_weights_col(
+            prefix=prefix, n_experts=n_experts, names=[gate_proj_name, up_proj_name], weights=weights
+        )
+        self.down_proj = _load_expert_weights_row(prefix=prefix, n_experts=n_experts, name=down_proj_name, weights=weights)
+        self.bits = 4
+        self._gate_up = self.gate_up_proj.packed()
+        self._down = self.down_proj.packed()
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor, *, gating_output: torch.Tensor) -> torch.Tensor:
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        assert x2.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
+        assert gating_output.shape[1] == self.n_experts, "Number of experts mismatch"
+        out = ops.moe_forward(self._gate_up, self._down, x2, gating_output, self.topk, self.renormalize, self.hidden_act)
+        return out.reshape(shape)

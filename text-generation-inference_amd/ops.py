@@ -296,3 +296,136 @@ def select_path(w: PackedWeight, M: int, dtype: torch.dtype = torch.float16) -> 
     rc = _lib.load().q4_select_path(ctypes.byref(st), int(M), _DTYPES[dtype])
     _lib.check(rc)
     return _lib.PATH_NAMES[rc]
+
+
+# --------------------------------------------------------------------------- mixture of experts
+
+
+@dataclass
+class PackedMoeWeight:
+    """The experts of one projection, stacked along a leading expert dimension in checkpoint
+    layout: qweight [E, K/8, N], qzeros [E, G, N/8], scales [E, G, N] (GPTQ, no g_idx)."""
+
+    qweight: torch.Tensor
+    qzeros: torch.Tensor
+    scales: torch.Tensor
+    K: int
+    N: int
+    groupsize: int
+    num_groups: int
+    num_experts: int
+
+    def struct(self) -> _lib.Q4MoeWeight:
+        e0 = _lib.Q4Weight(
+            self.qweight.data_ptr(), self.qzeros.data_ptr(), self.scales.data_ptr(), None,
+            self.K, self.N, self.groupsize, self.num_groups, LAYOUT_GPTQ,
+        )
+        return _lib.Q4MoeWeight(e0, self.num_experts, self.qweight.stride(0), self.qzeros.stride(0), self.scales.stride(0))
+
+
+def make_packed_moe(qweight, qzeros, scales, groupsize: int) -> PackedMoeWeight:
+    """Validate stacked expert tensors and wrap them for the grouped kernels."""
+    if qweight.dim() != 3 or qzeros.dim() != 3 or scales.dim() != 3:
+        raise ValueError("stacked expert tensors must be [E, ...] with three dimensions")
+    E = qweight.shape[0]
+    one = make_packed(qweight[0], qzeros[0], scales[0], None, groupsize, LAYOUT_GPTQ)
+    if qzeros.shape[0] != E or scales.shape[0] != E:
+        raise ValueError(f"expert counts differ: {E}, {qzeros.shape[0]}, {scales.shape[0]}")
+    for name, t in (("qweight", qweight), ("qzeros", qzeros), ("scales", scales)):
+        if not t[0].is_contiguous():
+            raise ValueError(f"{name}: every expert's slice must be contiguous")
+    return PackedMoeWeight(qweight, qzeros, scales, one.K, one.N, one.groupsize, one.num_groups, E)
+
+
+@dataclass
+class MoeRouting:
+    """Result of `moe_route`; every tensor lives on the device."""
+
+    topk_weights: torch.Tensor   # f32 [T, k]
+    topk_ids: torch.Tensor       # i32 [T, k]
+    sorted_tokens: torch.Tensor  # i32 [T*k]: token of every row of the expert-sorted order
+    pair_slot: torch.Tensor      # i32 [T*k]: sorted row of pair (t, j)
+    expert_offsets: torch.Tensor  # i32 [E+1]
+
+
+_GATING_DTYPES = {torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16, torch.float32: _lib.DTYPE_F32}
+
+
+def moe_route(gating_output: torch.Tensor, topk: int, renormalize: bool = True) -> MoeRouting:
+    """softmax -> top-k (-> renormalise) per token and the sort of the pairs by expert."""
+    _require_cuda(gating_output, "gating_output")
+    if gating_output.dim() != 2 or gating_output.dtype not in _GATING_DTYPES:
+        raise ValueError("gating_output must be a [tokens, experts] float16/bfloat16/float32 tensor")
+    g = gating_output.contiguous()
+    T, E = g.shape
+    dev = g.device
+    r = MoeRouting(
+        torch.empty((T, topk), dtype=torch.float32, device=dev),
+        torch.empty((T, topk), dtype=torch.int32, device=dev),
+        torch.empty((T * topk,), dtype=torch.int32, device=dev),
+        torch.empty((T * topk,), dtype=torch.int32, device=dev),
+        torch.empty((E + 1,), dtype=torch.int32, device=dev),
+    )
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().q4_moe_route(
+            g.data_ptr(), _GATING_DTYPES[g.dtype], T, E, int(topk), int(bool(renormalize)),
+            r.topk_weights.data_ptr(), r.topk_ids.data_ptr(), r.sorted_tokens.data_ptr(), r.pair_slot.data_ptr(),
+            r.expert_offsets.data_ptr(), _stream_handle(dev),
+        ))
+    return r
+
+
+def moe_linear(w: PackedMoeWeight, x: torch.Tensor, routing: MoeRouting, gather: bool) -> torch.Tensor:
+    """Grouped linear layer: sorted row r becomes x_row(r) @ W[expert of r].
+
+    gather=True: x is [tokens, K] and row r reads its token's row (first projection);
+    gather=False: x is [tokens*k, K] already in sorted order (second projection).
+    Returns y [tokens*k, N] in sorted order.
+    """
+    _require_cuda(x, "x")
+    if x.dtype not in _DTYPES:
+        raise TypeError(f"x must be float16 or bfloat16, got {x.dtype}")
+    T, k = routing.topk_ids.shape
+    rows = T if gather else T * k
+    if x.dim() != 2 or tuple(x.shape) != (rows, w.K):
+        raise ValueError(f"x must be [{rows}, {w.K}], got {tuple(x.shape)}")
+    x = x.contiguous()
+    y = torch.empty((T * k, w.N), dtype=x.dtype, device=x.device)
+    if T == 0:
+        return y
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        stream = _stream_handle(x.device)
+        st = w.struct()
+        ws = reserve_workspace(x.device, int(lib.q4_moe_workspace_bytes(ctypes.byref(st), T, k)), stream)
+        _lib.check(lib.q4_moe_linear(
+            ctypes.byref(st), x.data_ptr(), routing.sorted_tokens.data_ptr() if gather else None,
+            routing.expert_offsets.data_ptr(), y.data_ptr(), T, k, _DTYPES[x.dtype], ws.data_ptr(), ws.numel(), stream,
+        ))
+    return y
+
+
+def moe_combine(y_sorted: torch.Tensor, routing: MoeRouting) -> torch.Tensor:
+    """out[t] = sum_j topk_weights[t, j] * y_sorted[slot(t, j)] (fp32 sum, one rounding)."""
+    _require_cuda(y_sorted, "y_sorted")
+    T, k = routing.topk_ids.shape
+    y_sorted = y_sorted.contiguous()
+    N = y_sorted.shape[1]
+    out = torch.empty((T, N), dtype=y_sorted.dtype, device=y_sorted.device)
+    if T == 0:
+        return out
+    with torch.cuda.device(y_sorted.device):
+        _lib.check(_lib.load().q4_moe_combine(
+            y_sorted.data_ptr(), routing.topk_weights.data_ptr(), routing.pair_slot.data_ptr(), out.data_ptr(),
+            T, k, N, _DTYPES[y_sorted.dtype], _stream_handle(y_sorted.device),
+        ))
+    return out
+
+
+def moe_forward(gate_up: PackedMoeWeight, down: PackedMoeWeight, x: torch.Tensor, gating_output: torch.Tensor,
+                topk: int, renormalize: bool = True, act: str = "silu") -> torch.Tensor:
+    """The sparse MoE block: route, [gate | up] projection, act(gate) * up, down projection,
+    weighted sum over the chosen experts."""
+    routing = moe_route(gating_output, topk, renormalize)
+    h = act_mul(moe_linear(gate_up, x, routing, gather=True), act)
+    return moe_combine(moe_linear(down, h, routing, gather=False), routing)
