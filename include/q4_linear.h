@@ -176,8 +176,8 @@ int q4_moe_route(const void* gating, int gating_dtype, int tokens, int experts, 
                  int32_t* expert_offsets, void* stream);
 
 /* y[r, :] = x[x_rows ? x_rows[r] : r, :] @ W_e for every sorted row r of every expert e.
- * y is [tokens*topk, N] in sorted order.  Up to 16 tokens the decode kernel runs once per
- * expert that has rows; above, the MFMA kernel.  Workspace as for q4_linear, sized by
+ * y is [tokens*topk, N] in sorted order.  Up to 16 tokens (64 when K <= 8192) the decode
+ * kernel runs once per expert and 16 rows it received; above, the MFMA kernel.  Workspace as for q4_linear, sized by
  * q4_moe_workspace_bytes, zero-initialised once. */
 int q4_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_rows, const int32_t* expert_offsets,
                   void* y, int tokens, int topk, int dtype, void* workspace, size_t workspace_bytes, void* stream);

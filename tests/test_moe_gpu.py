@@ -91,7 +91,11 @@ def _experts(oracle, gpu, E, K, N, gs, dtype, seed, sym=False):
     (7, 4, 4, 1024, 256, 64),       # every token on every expert
     (5, 8, 2, 512, 256, 32),
     (3, 8, 2, 1024, 512, -1),       # one group
-    (17, 8, 2, 1024, 512, 128),     # first size of the MFMA kernel
+    (17, 8, 2, 1024, 512, 128),
+    (40, 2, 2, 1024, 512, 128),     # decode kernel, 40 rows per expert: three row blocks each
+    (64, 8, 2, 2048, 512, 128),     # last size of the decode kernel
+    (65, 8, 2, 1024, 512, 128),     # first size of the MFMA kernel (split-K: few tiles)
+    (100, 8, 2, 4096, 256, 128),    # MFMA kernel, deeper split-K
     (200, 8, 2, 1024, 768, 128),    # 128-column tiles (N not a multiple of 256)
     (300, 4, 1, 512, 512, 64),
     (130, 8, 2, 512, 256, 32),

@@ -126,6 +126,7 @@ int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, nullptr, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
   gp.moe = q4::MoeView{};
+  gp.partial_rows = M;
   GemmPlan g = gemm_plan(M, w->K, w->N);
   // without room for the partial tiles every workgroup owns a whole tile (slower, same result
   // up to fp32 summation order)

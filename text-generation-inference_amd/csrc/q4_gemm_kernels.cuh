@@ -41,6 +41,7 @@ struct GemmParams {
   // the output is written directly.
   float* __restrict__ partials;
   int splits;
+  int partial_rows;  // rows of one split's slice of `partials` (M; grouped launches: all pairs)
   MoeView moe;  // grouped launches only (MOE kernels): blockIdx.y is the expert
 };
 
@@ -390,7 +391,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm
   // 8*(r/4) + 4*kq + r%4, column j.  Fragments 0/1 are adjacent columns -> one 32-bit store.
   if (gp.splits > 1) {
     // fp32 partial tile; bias, rounding and the store to y happen in the reduction kernel
-    float* part = gp.partials + (size_t)split * M * N;
+    float* part = gp.partials + ((size_t)split * gp.partial_rows + moe_row0) * N;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll

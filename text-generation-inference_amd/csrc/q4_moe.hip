@@ -8,7 +8,7 @@
 //     expert (a grid dimension); every workgroup reads its expert's row range from device
 //     memory, narrows the problem to it and leaves at once when the range is empty or ends
 //     before its tile.  The decode kernel therefore streams the packed weights of exactly
-//     the experts that were chosen, once each, whatever the number of tokens (<= 16);
+//     the experts that were chosen, once per 16 rows they received;
 //   * moe_combine_kernel adds the topk rows of every token, weighted, in fp32.
 #include "q4_gemm_kernels.cuh"
 #include "q4_gemv_kernels.cuh"
@@ -182,16 +182,28 @@ int validate_moe_weight(const q4_moe_weight* w, const char* who) {
 struct MoeGemvPlan {
   bool ok;
   GemvConfig cfg;
-  int ntiles;
+  int ntiles, mchunks;
   size_t smem;
 };
+
+// The decode kernel takes 16 rows of an expert per workgroup; an expert can receive every
+// token, so the grid has ceil(tokens / 16) row blocks per expert, of which those past the
+// expert's count leave at once.  Each further block of an expert re-reads its weights (from
+// L2 where it can).  Measured on Mixtral shapes (8 experts, top-2), decode against MFMA
+// kernel: 4096 x 28672 113 / 268 us at 17 tokens, 163 / 240 us at 64; 14336 x 4096 (few
+// column tiles, long K: the MFMA kernel splits K) 106 / 110 us at 17 tokens, 194 / 108 us
+// at 64.  So the decode kernel is kept up to 64 tokens for K <= 8192 and up to 16 beyond.
+constexpr int kMoeDecodeMaxTokens = 64;
+constexpr int kMoeDecodeMaxTokensLongK = 16;
 
 MoeGemvPlan moe_gemv_plan(const q4_moe_weight* w, int tokens, int topk, int dtype) {
   using namespace q4;
   MoeGemvPlan pl{};
   const q4_weight* e0 = &w->expert0;
   const int rows = tokens < kRowsPerBlock ? tokens : kRowsPerBlock;
-  if (tokens > kRowsPerBlock || !gemv_supported(e0, rows, dtype)) return pl;
+  if (tokens > (e0->K <= 8192 ? kMoeDecodeMaxTokens : kMoeDecodeMaxTokensLongK) || !gemv_supported(e0, rows, dtype))
+    return pl;
+  const int mchunks = (tokens + kRowsPerBlock - 1) / kRowsPerBlock;
   GemvConfig cfg = gemv_pick_config(e0, rows);
   cfg.words = 4;
   if (e0->N % (64 * cfg.wcol) != 0) cfg.wcol = 1;
@@ -202,7 +214,8 @@ MoeGemvPlan moe_gemv_plan(const q4_moe_weight* w, int tokens, int topk, int dtyp
   if (splits < 1) splits = 1;
   while (splits > 1 && e0->K % (splits * cfg.wk * 128) != 0) --splits;
   const int ntiles = e0->N / (64 * cfg.wcol);
-  if ((long)ntiles * w->num_experts > Q4_WORKSPACE_TICKET_BYTES / 4) splits = 1;
+  const bool tickets_fit = (long)ntiles * mchunks * w->num_experts <= Q4_WORKSPACE_TICKET_BYTES / 4;
+  if (!tickets_fit) splits = 1;
   // the activation slab of 16 rows x K / splits must fit LDS: split further if it does not
   const size_t smem_limit = 160 * 1024 - 1024;
   auto smem_of = [&](int sp) {
@@ -213,13 +226,14 @@ MoeGemvPlan moe_gemv_plan(const q4_moe_weight* w, int tokens, int topk, int dtyp
   while (smem_of(splits) > smem_limit) {
     int next = splits + 1;
     while (next <= e0->K / (cfg.wk * 128) && e0->K % (next * cfg.wk * 128) != 0) ++next;
-    if (next > e0->K / (cfg.wk * 128) || (long)ntiles * w->num_experts > Q4_WORKSPACE_TICKET_BYTES / 4) return pl;
+    if (next > e0->K / (cfg.wk * 128) || !tickets_fit) return pl;
     splits = next;
   }
   cfg.splits = splits;
   pl.ok = true;
   pl.cfg = cfg;
   pl.ntiles = ntiles;
+  pl.mchunks = mchunks;
   pl.smem = smem_of(splits);
   return pl;
 }
@@ -247,6 +261,20 @@ void launch_moe_gemm_tile(int gs, dim3 grid, size_t smem, hipStream_t stream, co
   else hipLaunchKernelGGL((gemm_gptq_kernel<DTYPE, 128, 1, NW, true>), grid, dim3(256), smem, stream, gp);
 }
 
+// Split-K factor of the grouped MFMA launch.  The host does not know the experts' row counts:
+// it plans for an even spread (tokens * topk / experts rows each) and splits K when those
+// tiles alone would leave CUs idle (Mixtral down projection at 64 tokens: 8 experts x 16
+// column tiles, 224 K tiles each).
+int moe_gemm_splits(const q4_moe_weight* w, int tokens, int topk) {
+  const q4_weight* e0 = &w->expert0;
+  const long pairs = (long)tokens * topk;
+  const long avg_rows = (pairs + w->num_experts - 1) / w->num_experts;
+  const int nw = e0->N % 256 == 0 ? 2 : 1;
+  const long tiles = (long)w->num_experts * ((avg_rows + 127) / 128) * (e0->N / (128 * nw));
+  if (tiles >= 256 || pairs > 0x7fffffffL) return 1;
+  return gemm_pick_splits(tiles, e0->K / q4::kBK, (int)pairs, e0->N, 0.9, 1.3);
+}
+
 MoeView make_view(const q4_moe_weight* w, const int32_t* x_rows, const int32_t* offsets) {
   MoeView mv;
   mv.offsets = offsets;
@@ -262,7 +290,10 @@ MoeView make_view(const q4_moe_weight* w, const int32_t* x_rows, const int32_t* 
 size_t moe_workspace_bytes(const q4_moe_weight* w, int tokens, int topk) {
   const MoeGemvPlan pl = moe_gemv_plan(w, tokens, topk, Q4_DTYPE_F16);
   size_t bytes = Q4_WORKSPACE_COUNTER_BYTES;
-  if (pl.ok && pl.cfg.splits > 1) bytes += (size_t)pl.cfg.splits * tokens * topk * w->expert0.N * sizeof(float);
+  int splits = 1;
+  if (pl.ok) splits = pl.cfg.splits;
+  else if (gemm_supported(&w->expert0, tokens, Q4_DTYPE_F16)) splits = moe_gemm_splits(w, tokens, topk);
+  if (splits > 1) bytes += (size_t)splits * tokens * topk * w->expert0.N * sizeof(float);
   return bytes;
 }
 
@@ -301,7 +332,7 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
     gp.slab_bytes = (int)pl.smem;
     gp.partial_rows = pairs;
     gp.moe = mv;
-    const dim3 grid((unsigned)(pl.ntiles * cfg.splits), 1, (unsigned)w->num_experts);
+    const dim3 grid((unsigned)(pl.ntiles * cfg.splits), (unsigned)pl.mchunks, (unsigned)w->num_experts);
     const dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
     if (dtype == Q4_DTYPE_F16) launch_moe_gemv_dtype<Q4_DTYPE_F16>(e0->groupsize, grid, block, pl.smem, stream, gp);
     else launch_moe_gemv_dtype<Q4_DTYPE_BF16>(e0->groupsize, grid, block, pl.smem, stream, gp);
@@ -310,12 +341,17 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
     gp.p = Problem{e0->qweight, e0->qzeros, (const half_t*)e0->scales, nullptr, x, nullptr, y,
                    0,           e0->K,      e0->N,                     e0->groupsize, e0->num_groups};
     gp.p.gate_up_act = 0;
-    gp.partials = nullptr;
-    gp.splits = 1;
+    int splits = moe_gemm_splits(w, tokens, topk);
+    if (splits > 1 && (workspace == nullptr || workspace_bytes < Q4_WORKSPACE_COUNTER_BYTES +
+                                                                     (size_t)splits * pairs * e0->N * sizeof(float)))
+      splits = 1;  // no room for partial tiles
+    gp.partials = splits > 1 ? (float*)((char*)workspace + Q4_WORKSPACE_COUNTER_BYTES) : nullptr;
+    gp.splits = splits;
+    gp.partial_rows = pairs;
     gp.moe = mv;
     // an expert can receive every token: the grid covers `tokens` rows per expert
     const int nw = e0->N % 256 == 0 ? 2 : 1;
-    const long tiles = (long)((tokens + 127) / 128) * (e0->N / (128 * nw));
+    const long tiles = (long)((tokens + 127) / 128) * (e0->N / (128 * nw)) * splits;
     if (tiles > 0x7fffffffL || w->num_experts > 65535) {
       set_error("q4_moe_linear: grid too large");
       return Q4_ERR_UNSUPPORTED;
@@ -329,6 +365,7 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
       if (nw == 2) launch_moe_gemm_tile<Q4_DTYPE_BF16, 2>(e0->groupsize, grid, smem, stream, gp);
       else launch_moe_gemm_tile<Q4_DTYPE_BF16, 1>(e0->groupsize, grid, smem, stream, gp);
     }
+    if (splits > 1) launch_gemm_reduce(gp.partials, nullptr, y, pairs, e0->N, splits, dtype, stream);
   } else {
     set_error("q4_moe_linear: no grouped kernel for tokens=%d K=%d N=%d groupsize=%d", tokens, e0->K, e0->N,
               e0->groupsize);
