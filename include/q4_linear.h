@@ -144,11 +144,11 @@ size_t q4_workspace_bytes(int M, int K, int N);
 /*
  * ---- Mixture of experts: the same linear layer, grouped over experts -----------------
  *
- * Replaces, for GPTQ checkpoints, what the reference's sparse MoE layer
+ * Replaces, for GPTQ and AWQ checkpoints, what the reference's sparse MoE layer
  * (server/text_generation_server/layers/moe/gptq_marlin.py:116-146 -> fused_marlin_moe,
  * :232-351) gets from the un-vendored `kernels-community/moe` package (fused_topk +
  * fused_marlin_moe): routing, the two grouped projections and the weighted sum.  The
- * expert tensors stay in checkpoint layout, stacked along a leading expert dimension
+ * expert tensors stay in checkpoint layout (GPTQ with or without act-order, or AWQ), stacked along a leading expert dimension
  * (what _pack_weight, gptq_marlin.py:186-229, builds) -- there is no Marlin repack.
  *
  * Rows are (token, expert) pairs sorted by expert.  q4_moe_route writes, all on the
@@ -160,11 +160,12 @@ size_t q4_workspace_bytes(int M, int K, int N);
  * The order of the rows of one expert is not specified (no output depends on it).
  */
 typedef struct q4_moe_weight {
-  q4_weight expert0;      /* geometry and the tensors of expert 0: GPTQ layout, g_idx NULL */
+  q4_weight expert0;      /* geometry and the tensors of expert 0 (either layout, g_idx optional) */
   int32_t num_experts;
-  int64_t qweight_stride; /* elements between consecutive experts' qweight / qzeros / scales */
+  int64_t qweight_stride; /* elements between consecutive experts' qweight / qzeros / scales / g_idx */
   int64_t qzeros_stride;
   int64_t scales_stride;
+  int64_t g_idx_stride;   /* ignored when expert0.g_idx is NULL */
 } q4_moe_weight;
 
 #define Q4_DTYPE_F32 2 /* gating logits only */

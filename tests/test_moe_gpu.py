@@ -3,8 +3,6 @@ kernels), the weighted sum and the whole block, against the oracle."""
 
 from __future__ import annotations
 
-import json
-
 import numpy as np
 import pytest
 import torch
@@ -83,6 +81,25 @@ def _experts(oracle, gpu, E, K, N, gs, dtype, seed, sym=False):
     return stack(qws), stack(qzs), stack(scs), dense
 
 
+def _packed_experts(pkg, oracle, gpu, kind, E, K, N, gs, dtype, seed):
+    """PackedMoeWeight + dense matrices for kind in {"gptq", "act", "awq"}."""
+    qws, qzs, scs, gis, dense = [], [], [], [], []
+    for e in range(E):
+        if kind == "awq":
+            qw, qz, sc = oracle.make_awq(K, N, gs, seed=seed + e)
+            dense.append(oracle.dequant_awq(qw, qz, sc, gs, dtype))
+        else:
+            qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=seed + e, sym=False, act_order=(kind == "act"))
+            dense.append(oracle.dequant_gptq(qw, qz, sc, gi, gs, dtype))
+            if gi is not None:
+                gis.append(gi)
+        qws.append(qw); qzs.append(qz); scs.append(sc)
+    stack = lambda a: to_dev(np.stack(a), gpu)
+    w = pkg.ops.make_packed_moe(stack(qws), stack(qzs), stack(scs), gs, stack(gis) if gis else None,
+                                1 if kind == "awq" else 0)
+    return w, dense
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("T,E,k,K,N,gs", [
     (1, 8, 2, 1024, 512, 128),      # decode, most experts without rows
@@ -123,6 +140,45 @@ def test_moe_linear_gather(pkg, oracle, gpu, T, E, k, K, N, gs, dtype):
             ref[slot[rows * k + js]] = y32
     err = max_rel_err(y, ref)
     assert err <= (TOL_BF16 if bf else TOL), f"max rel err {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("kind", ["act", "awq"])
+@pytest.mark.parametrize("T,E,k,K,N,gs", [
+    (1, 8, 2, 1024, 512, 128),      # decode kernels (act-order: fp16 only, bf16 takes the MFMA kernel)
+    (9, 4, 2, 2048, 512, 128),
+    (16, 4, 4, 1024, 256, 64),      # 16 rows on every expert
+    (17, 8, 2, 1024, 512, 128),     # MFMA kernel (LDS unpack), split-K
+    (150, 4, 2, 1024, 256, 128),    # two row tiles on some experts
+    (40, 8, 2, 8192, 128, 32),      # act-order: 256 groups, parameters gathered from global memory
+])
+def test_moe_linear_act_order_and_awq(pkg, oracle, gpu, kind, T, E, k, K, N, gs, dtype):
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(T + K + len(kind))
+    w, dense = _packed_experts(pkg, oracle, gpu, kind, E, K, N, gs, dtype, seed=T + 3)
+    g, _ = _gating(rng, T, E, "f32")
+    r = pkg.ops.moe_route(g.to(gpu), k, True)
+    x = oracle.make_x(T, K, seed=T, dtype=dtype)
+    y = to_f32(pkg.ops.moe_linear(w, to_dev(x, gpu, bf16=bf), r, gather=True))
+    assert np.isfinite(y).all()
+    ids = r.topk_ids.cpu().numpy()
+    slot = r.pair_slot.cpu().numpy()
+    ref = np.zeros_like(y)
+    for e in range(E):
+        rows, js = np.nonzero(ids == e)
+        if rows.size:
+            ref[slot[rows * k + js]], _ = oracle.linear_forward(x[rows], dense[e], None, dtype)
+    err = max_rel_err(y, ref)
+    assert err <= (TOL_BF16 if bf else TOL), f"max rel err {err:.3e}"
+    # second projection form: x already sorted
+    xs = oracle.make_x(T * k, K, seed=T + 1, dtype=dtype)
+    y2 = to_f32(pkg.ops.moe_linear(w, to_dev(xs, gpu, bf16=bf), r, gather=False))
+    off = r.expert_offsets.cpu().numpy()
+    ref2 = np.zeros_like(y2)
+    for e in range(E):
+        if off[e + 1] > off[e]:
+            ref2[off[e]:off[e + 1]], _ = oracle.linear_forward(xs[off[e]:off[e + 1]], dense[e], None, dtype)
+    assert max_rel_err(y2, ref2) <= (TOL_BF16 if bf else TOL)
 
 
 @pytest.mark.parametrize("T", [2, 16, 40])
@@ -215,33 +271,41 @@ def test_moe_block_mixtral_shape_decode(pkg, oracle, gpu):
     assert max_rel_err(to_f32(out), ref32) <= 2 * TOL
 
 
-def test_sparse_moe_layer_from_safetensors(pkg, oracle, gpu, tmp_path):
+@pytest.mark.parametrize("desc_act", [False, True])
+def test_sparse_moe_layer_from_safetensors(pkg, oracle, gpu, tmp_path, desc_act):
     """The layer class loads per-expert checkpoint tensors through the package's Weights and
-    matches the oracle; leading dimensions of x are kept."""
+    matches the oracle; leading dimensions of x are kept.  desc_act: every projection has a
+    permuted g_idx (gate and up of an expert share theirs, as a checkpoint's do)."""
     E, k, H, I, gs = 4, 2, 256, 512, 64
     tensors, gu, dn = {}, [], []
     for e in range(E):
         parts = []
+        perm_rng = np.random.default_rng(1000 + e)
+        g_in = (np.arange(H) // gs).astype(np.int32)
+        g_mid = (np.arange(I) // gs).astype(np.int32)
+        if desc_act:
+            g_in, g_mid = g_in[perm_rng.permutation(H)], g_mid[perm_rng.permutation(I)]
         for name, (K, N), seed in (("gate_proj", (H, I), 1), ("up_proj", (H, I), 2), ("down_proj", (I, H), 3)):
             qw, qz, sc, _ = oracle.make_gptq(K, N, gs, seed=10 * e + seed, sym=False)
+            gi = g_in if K == H else g_mid
             pre = f"moe.experts.{e}.{name}"
             tensors[f"{pre}.qweight"] = torch.from_numpy(qw.view(np.int32).copy())
             tensors[f"{pre}.qzeros"] = torch.from_numpy(qz.view(np.int32).copy())
             tensors[f"{pre}.scales"] = torch.from_numpy(sc.copy())
-            tensors[f"{pre}.g_idx"] = torch.arange(K, dtype=torch.int32) // gs
-            parts.append(oracle.dequant_gptq(qw, qz, sc, None, gs, "f16"))
+            tensors[f"{pre}.g_idx"] = torch.from_numpy(gi.copy())
+            parts.append(oracle.dequant_gptq(qw, qz, sc, gi, gs, "f16"))
         gu.append(np.concatenate(parts[:2], axis=1))
         dn.append(parts[2])
     path = tmp_path / "model.safetensors"
     save_file(tensors, str(path))
-    (tmp_path / "config.json").write_text(json.dumps({"quantization_config": {"bits": 4, "group_size": gs, "quant_method": "gptq", "desc_act": False, "sym": False}}))
     from types import SimpleNamespace
 
-    loader = pkg.GPTQWeightsLoader(bits=4, groupsize=gs, desc_act=False, quant_method="gptq", quantize="gptq", sym=False,
-                                   modules_to_not_convert=[])
+    loader = pkg.GPTQWeightsLoader(bits=4, groupsize=gs, desc_act=desc_act, quant_method="gptq", quantize="gptq",
+                                   sym=False, modules_to_not_convert=[])
     weights = pkg.Weights([path], gpu, torch.float16, SimpleNamespace(rank=lambda: 0, size=lambda: 1), loader)
     layer = pkg.GPTQSparseMoELayer(n_expert_group=None, n_experts=E, prefix="moe.experts", renormalize=True, topk=k,
                                    topk_group=None, weights=weights)
+    assert (layer._gate_up.g_idx is not None) == desc_act and (layer._down.g_idx is not None) == desc_act
     rng = np.random.default_rng(5)
     x = oracle.make_x(6, H, seed=2)
     g = rng.standard_normal((6, E)).astype(np.float32)

@@ -60,6 +60,7 @@ class Q4MoeWeight(Structure):
         ("qweight_stride", c_int64),
         ("qzeros_stride", c_int64),
         ("scales_stride", c_int64),
+        ("g_idx_stride", c_int64),
     ]
 
 

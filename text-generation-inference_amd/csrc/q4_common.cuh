@@ -157,7 +157,7 @@ struct Problem {
 struct MoeView {
   const int32_t* __restrict__ offsets;  // [experts + 1], device memory
   const int32_t* __restrict__ x_rows;   // [pairs] or nullptr
-  long qweight_stride, qzeros_stride, scales_stride;
+  long qweight_stride, qzeros_stride, scales_stride, g_idx_stride;
 };
 
 // Narrows `p` to expert e.  Returns the expert's first sorted row; p.M becomes its row count
@@ -168,6 +168,7 @@ __device__ __forceinline__ int moe_enter(Problem& p, const MoeView& mv, int e) {
   p.qweight += (size_t)e * mv.qweight_stride;
   p.qzeros += (size_t)e * mv.qzeros_stride;
   p.scales += (size_t)e * mv.scales_stride;
+  if (p.g_idx != nullptr) p.g_idx += (size_t)e * mv.g_idx_stride;
   p.y = (uint16_t*)p.y + (size_t)row0 * p.N;
   if (mv.x_rows == nullptr) p.x = (const uint16_t*)p.x + (size_t)row0 * p.K;
   return row0;
@@ -196,8 +197,17 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
 bool gemv_gate_up_supported(const q4_weight* w, int M, int dtype);
 int launch_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, hipStream_t stream);
 bool gemm_awq_supported(const q4_weight* w, int M, int dtype);
+// Host description of a grouped (mixture-of-experts) launch.
+struct MoeLaunch {
+  q4::MoeView view;
+  int num_experts;
+  int tokens;  // an expert can receive at most this many rows
+  int pairs;   // tokens * topk: rows of the sorted order
+};
+// moe != nullptr: grouped launch, M = moe->tokens, y and the partial tiles have moe->pairs rows
 int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
-                    void* workspace, size_t workspace_bytes, hipStream_t stream);
+                    void* workspace, size_t workspace_bytes, hipStream_t stream, const MoeLaunch* moe = nullptr);
+size_t gemm_awq_moe_workspace_bytes(const q4_weight* w, const MoeLaunch* moe);
 bool gemm_supported(const q4_weight* w, int M, int dtype);
 int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                 void* workspace, size_t workspace_bytes, hipStream_t stream);

@@ -42,7 +42,9 @@ struct AwqGemmParams {
   // partials[split][M][N], combined by gemm_reduce_kernel
   float* __restrict__ partials;
   int splits;
+  int partial_rows;  // rows of one split's slice of `partials` (M; grouped launches: all pairs)
   Problem p;
+  MoeView moe;  // grouped launches only (MOE kernels): blockIdx.y is the expert
 };
 
 struct AwqSplice {
@@ -71,9 +73,16 @@ constexpr int kModeActNarrow = 3;  // GPTQ layout with g_idx, LDS table of fp16 
 constexpr int kActWideGroupBytes = kABN * 4;
 constexpr int kActNarrowGroupBytes = kABN * 3;  // 128 fp16 scales, then 128 zero-point bytes
 
-template <int DTYPE, int MODE>
+// MOE: grouped launch, blockIdx.y is the expert; its row count is read from device memory, so
+// the grid covers the largest possible count and surplus workgroups leave at once.
+template <int DTYPE, int MODE, bool MOE = false>
 __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   constexpr bool ACT = MODE != kModeAwq;
+  int moe_row0 = 0;
+  if constexpr (MOE) {
+    moe_row0 = moe_enter(gp.p, gp.moe, blockIdx.y);
+    if (gp.p.M <= 0) return;
+  }
   constexpr bool TABLE = MODE == kModeActWide || MODE == kModeActNarrow;
   constexpr int GROUP_BYTES = MODE == kModeActWide ? kActWideGroupBytes : kActNarrowGroupBytes;
   constexpr int A_TILE = kABM * kAUnits * 16;   // bytes
@@ -91,6 +100,9 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   const int NC = N >> 3;
   const int tiles_m = (M + kABM - 1) / kABM;
   const int tiles_all = tiles_m * (N / kABN);
+  if constexpr (MOE) {
+    if ((int)blockIdx.x >= tiles_all * gp.splits) return;
+  }
   const int split = blockIdx.x / tiles_all;
   const int tile_id = blockIdx.x - split * tiles_all;
   const int tm = tile_id % tiles_m;
@@ -262,12 +274,21 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   // ---- activation tile: global -> registers -> LDS (natural K order)
   const uint16_t* xs = (const uint16_t*)p.x;
   uint4_t areg[A_LOADS];
+  int moe_xrow[MOE ? A_LOADS : 1];  // grouped launch with a row map: x row of each staged row
+  if constexpr (MOE) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int row = min(m0 + ((tid + 256 * i) >> 3), M - 1);
+      moe_xrow[i] = gp.moe.x_rows != nullptr ? gp.moe.x_rows[moe_row0 + row] : row;
+    }
+  }
   auto load_a = [&](int kt) {
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
       const int u = tid + 256 * i;
       const int m = u >> 3, kb = u & 7;
-      const int row = min(m0 + m, M - 1);  // rows past M re-read the last row, never stored
+      // rows past M re-read the last row, never stored
+      const int row = MOE ? moe_xrow[i] : min(m0 + m, M - 1);
       areg[i] = *(const uint4_t*)(xs + (size_t)row * K + kt * kABK + kb * 8);
     }
   };
@@ -404,7 +425,7 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
 
   // ---- epilogue: register r of lane (j, kq) is row 8*(r/4) + 4*kq + r%4, column j
   if (gp.splits > 1) {
-    float* part = gp.partials + (size_t)split * M * N;
+    float* part = gp.partials + ((size_t)split * gp.partial_rows + moe_row0) * N;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
       const int n = n0 + wn * 64 + nt * 32 + j;
@@ -482,9 +503,24 @@ int gemm_awq_splits(int M, int K, int N, bool one_per_cu) {
   return tiles < 256 ? gemm_pick_splits(tiles, K / q4::kABK, M, N, 1.0, 1.9) : 1;
 }
 
+// Split-K factor of a grouped launch.  The host does not know the experts' row counts: it
+// plans for an even spread (pairs / experts rows each).
+static int moe_awq_splits(const q4_weight* w, const MoeLaunch* moe) {
+  const long avg_rows = ((long)moe->pairs + moe->num_experts - 1) / moe->num_experts;
+  const long tiles = (long)moe->num_experts * ((avg_rows + q4::kABM - 1) / q4::kABM) * (w->N / q4::kABN);
+  if (gemm_act_order_table(w)) return tiles < 1024 ? gemm_pick_splits(tiles, w->K / q4::kABK, moe->pairs, w->N, 1.0, 1.0, 1) : 1;
+  return tiles < 256 ? gemm_pick_splits(tiles, w->K / q4::kABK, moe->pairs, w->N, 1.0, 1.9) : 1;
+}
+
+size_t gemm_awq_moe_workspace_bytes(const q4_weight* w, const MoeLaunch* moe) {
+  const int splits = moe_awq_splits(w, moe);
+  return splits > 1 ? (size_t)splits * moe->pairs * w->N * sizeof(float) : 0;
+}
+
 int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
-                    void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                    void* workspace, size_t workspace_bytes, hipStream_t stream, const MoeLaunch* moe) {
   using namespace q4;
+  // grouped launch: M is the largest row count an expert can have (the number of tokens)
   if (!gemm_awq_supported(w, M, dtype)) {
     set_error("q4_linear(gemm/awq): unsupported problem (M=%d K=%d N=%d groupsize=%d)", M, w->K, w->N,
               w->groupsize);
@@ -493,38 +529,51 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
   AwqGemmParams gp;
   gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, w->g_idx, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
-  int splits = gemm_awq_splits(M, w->K, w->N, gemm_act_order_table(w));
+  const int out_rows = moe != nullptr ? moe->pairs : M;  // rows of y (and of one split's partials)
+  int splits = moe != nullptr ? moe_awq_splits(w, moe) : gemm_awq_splits(M, w->K, w->N, gemm_act_order_table(w));
   if (splits > 1 && (workspace == nullptr ||
-                     workspace_bytes < Q4_WORKSPACE_COUNTER_BYTES + (size_t)splits * M * w->N * sizeof(float)))
+                     workspace_bytes < Q4_WORKSPACE_COUNTER_BYTES + (size_t)splits * out_rows * w->N * sizeof(float)))
     splits = 1;  // no room for partial tiles: one workgroup per whole tile
   gp.splits = splits;
+  gp.partial_rows = out_rows;
   gp.partials = splits > 1 ? (float*)((char*)workspace + Q4_WORKSPACE_COUNTER_BYTES) : nullptr;
+  gp.moe = moe != nullptr ? moe->view : MoeView{};
   const long total = (long)((M + kABM - 1) / kABM) * (w->N / kABN) * splits;
-  if (total > 0x7fffffffL) {
+  const long experts = moe != nullptr ? moe->num_experts : 1;
+  if (total > 0x7fffffffL || experts > 65535) {
     set_error("q4_linear(gemm/awq): grid too large");
     return Q4_ERR_UNSUPPORTED;
   }
   const size_t tiles_smem = kAwqTilesLdsBytes;
-  const int mode = gemm_awq_mode(w, total);
+  const int mode = gemm_awq_mode(w, total * experts);
   const size_t smem = tiles_smem + (mode == kModeActWide     ? (size_t)w->num_groups * kActWideGroupBytes
                                     : mode == kModeActNarrow ? (size_t)w->num_groups * kActNarrowGroupBytes
                                                              : 0);
+  const dim3 grid((unsigned)total, (unsigned)experts);
   auto launch = [&](auto k) {
     (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipLaunchKernelGGL(k, dim3((unsigned)total), dim3(256), smem, stream, gp);
+    hipLaunchKernelGGL(k, grid, dim3(256), smem, stream, gp);
   };
-  auto launch_dtype = [&](auto dt) {
+  auto launch_mode = [&](auto dt, auto grouped) {
     constexpr int DT = decltype(dt)::value;
+    constexpr bool G = decltype(grouped)::value;
     switch (mode) {
-      case kModeAwq: launch(gemm_awq_kernel<DT, kModeAwq>); break;
-      case kModeActWide: launch(gemm_awq_kernel<DT, kModeActWide>); break;
-      case kModeActNarrow: launch(gemm_awq_kernel<DT, kModeActNarrow>); break;
-      default: launch(gemm_awq_kernel<DT, kModeActGather>); break;
+      case kModeAwq: launch(gemm_awq_kernel<DT, kModeAwq, G>); break;
+      case kModeActWide: launch(gemm_awq_kernel<DT, kModeActWide, G>); break;
+      case kModeActNarrow: launch(gemm_awq_kernel<DT, kModeActNarrow, G>); break;
+      default: launch(gemm_awq_kernel<DT, kModeActGather, G>); break;
     }
   };
-  if (dtype == Q4_DTYPE_F16) launch_dtype(std::integral_constant<int, Q4_DTYPE_F16>{});
-  else launch_dtype(std::integral_constant<int, Q4_DTYPE_BF16>{});
-  if (splits > 1) launch_gemm_reduce(gp.partials, bias, y, M, w->N, splits, dtype, stream);
+  using F16 = std::integral_constant<int, Q4_DTYPE_F16>;
+  using BF16 = std::integral_constant<int, Q4_DTYPE_BF16>;
+  if (moe != nullptr) {
+    if (dtype == Q4_DTYPE_F16) launch_mode(F16{}, std::true_type{});
+    else launch_mode(BF16{}, std::true_type{});
+  } else {
+    if (dtype == Q4_DTYPE_F16) launch_mode(F16{}, std::false_type{});
+    else launch_mode(BF16{}, std::false_type{});
+  }
+  if (splits > 1) launch_gemm_reduce(gp.partials, bias, y, out_rows, w->N, splits, dtype, stream);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {
     set_error("q4_linear(gemm/awq): launch failed: %s", hipGetErrorString(err));

@@ -141,6 +141,17 @@ __device__ __forceinline__ Decomp make_decomp(const GemvParams& gp, int wave_col
   return d;
 }
 
+// Entry of a grouped (MOE) decode launch: narrows gp to the expert blockIdx.z.  Returns false
+// when this workgroup's row block lies beyond the expert's rows (the whole workgroup leaves).
+// `rows` receives the activation-row map of the block, or nullptr when x is in sorted order.
+__device__ __forceinline__ bool moe_enter_decode(GemvParams& gp, const int32_t*& rows) {
+  const int row0 = moe_enter(gp.p, gp.moe, blockIdx.z);
+  if (gp.p.M <= (int)blockIdx.y * kRowsPerBlock) return false;
+  gp.partials += (size_t)row0 * gp.p.N;
+  rows = gp.moe.x_rows != nullptr ? gp.moe.x_rows + row0 + blockIdx.y * kRowsPerBlock : nullptr;
+  return true;
+}
+
 // Activation slab [mloc][KR] -> LDS.  The global loads are issued before the weight loads
 // (memory returns in issue order, so L2 hits must not queue behind the HBM stream they are
 // needed to consume) and stored after them.  PERMUTE stores every 8-block in the K order
@@ -422,10 +433,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int32_t* moe_rows = nullptr;
   if constexpr (MOE) {
-    const int row0 = moe_enter(gp.p, gp.moe, blockIdx.z);
-    if (gp.p.M <= (int)blockIdx.y * kRowsPerBlock) return;
-    gp.partials += (size_t)row0 * gp.p.N;
-    if (gp.moe.x_rows != nullptr) moe_rows = gp.moe.x_rows + row0 + blockIdx.y * kRowsPerBlock;
+    if (!moe_enter_decode(gp, moe_rows)) return;
   }
   const Problem& p = gp.p;
   const Decomp d = make_decomp(gp, 16 * WORDS);
@@ -592,9 +600,13 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
 // ---------------------------------------------------------------------------------------
 // GPTQ with g_idx (act-order), fp16.  LDS: [slab][g_idx slice as uint16][table G x tile_cols].
 // Table entry (g, column) = fp16 scale | fp16 -(1024 + zero) << 16.
-template <int RMAX>
+template <int RMAX, bool MOE = false>
 __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
   extern __shared__ __align__(16) unsigned char smem[];
+  const int32_t* moe_rows = nullptr;
+  if constexpr (MOE) {
+    if (!moe_enter_decode(gp, moe_rows)) return;
+  }
   const Problem& p = gp.p;
   const Decomp d = make_decomp(gp, 64);
   const int N = p.N;
@@ -603,7 +615,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
   constexpr int PF = 2;  // 32-row steps of weight loads in flight per wave
 
   SlabStager<true> slab;
-  slab.issue(gp, d);
+  slab.issue(gp, d, moe_rows);
 
   const char* wbase = (const char*)(p.qweight + (size_t)(d.kw0 / 8) * N);
   const uint32_t w_lane = ((uint32_t)d.kq * (uint32_t)N + (uint32_t)nl) * 4u;
@@ -716,9 +728,13 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
 // AWQ layout.  Wave tile: 256 columns (32 packed words) x 32 rows per step; lane (j, kq)
 // loads words [8 rows of K block kq][2 adjacent words] and owns the 16 adjacent columns
 // starting at 8 * (first word of the wave + 2 j).
-template <int DTYPE, int RMAX>
+template <int DTYPE, int RMAX, bool MOE = false>
 __global__ __launch_bounds__(512) void gemv_awq_kernel(GemvParams gp) {
   extern __shared__ __align__(16) unsigned char smem[];
+  const int32_t* moe_rows = nullptr;
+  if constexpr (MOE) {
+    if (!moe_enter_decode(gp, moe_rows)) return;
+  }
   const Problem& p = gp.p;
   const Decomp d = make_decomp(gp, 256);
   const int N = p.N;
@@ -729,7 +745,7 @@ __global__ __launch_bounds__(512) void gemv_awq_kernel(GemvParams gp) {
   constexpr int PF = 3;  // 32-row steps (8 x 64-bit loads each) in flight per wave
 
   SlabStager<false> slab;
-  slab.issue(gp, d);
+  slab.issue(gp, d, moe_rows);
 
   const char* wbase = (const char*)(p.qweight + (size_t)d.kw0 * NC);
   const uint32_t w_lane = ((uint32_t)(d.kq * 8) * (uint32_t)NC + (uint32_t)cw) * 4u;

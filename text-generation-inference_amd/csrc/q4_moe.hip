@@ -156,19 +156,26 @@ int validate_moe_weight(const q4_moe_weight* w, const char* who) {
     set_error("%s: null qweight/qzeros/scales", who);
     return Q4_ERR_INVALID_ARGUMENT;
   }
-  if (e0.K < 8 || e0.N < 8 || e0.K % 8 != 0 || e0.N % 8 != 0 || e0.groupsize < 1 || e0.num_groups < 1 ||
-      (long)e0.num_groups * e0.groupsize < e0.K) {
+  if (e0.K < 8 || e0.N < 8 || e0.K % 8 != 0 || e0.N % 8 != 0 || e0.groupsize < 1 || e0.num_groups < 1) {
     set_error("%s: bad geometry K=%d N=%d groupsize=%d num_groups=%d", who, e0.K, e0.N, e0.groupsize,
               e0.num_groups);
     return Q4_ERR_INVALID_ARGUMENT;
   }
-  if (e0.layout != Q4_LAYOUT_GPTQ || e0.g_idx != nullptr) {
-    set_error("%s: the grouped kernels take the GPTQ layout without g_idx (layout=%d g_idx=%p)", who, e0.layout,
-              (const void*)e0.g_idx);
-    return Q4_ERR_UNSUPPORTED;
+  if (e0.layout != Q4_LAYOUT_GPTQ && e0.layout != Q4_LAYOUT_AWQ) {
+    set_error("%s: unknown layout %d", who, e0.layout);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (e0.layout == Q4_LAYOUT_AWQ && e0.g_idx != nullptr) {
+    set_error("%s: g_idx is not defined for the AWQ layout", who);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (e0.g_idx == nullptr && (long)e0.num_groups * e0.groupsize < e0.K) {
+    set_error("%s: %d groups of %d rows do not cover K=%d", who, e0.num_groups, e0.groupsize, e0.K);
+    return Q4_ERR_INVALID_ARGUMENT;
   }
   const long qw = (long)(e0.K / 8) * e0.N, qz = (long)e0.num_groups * (e0.N / 8), sc = (long)e0.num_groups * e0.N;
-  if (w->qweight_stride < qw || w->qzeros_stride < qz || w->scales_stride < sc) {
+  if (w->qweight_stride < qw || w->qzeros_stride < qz || w->scales_stride < sc ||
+      (e0.g_idx != nullptr && w->g_idx_stride < e0.K)) {
     set_error("%s: expert strides (%lld, %lld, %lld) smaller than one expert (%ld, %ld, %ld)", who,
               (long long)w->qweight_stride, (long long)w->qzeros_stride, (long long)w->scales_stride, qw, qz, sc);
     return Q4_ERR_INVALID_ARGUMENT;
@@ -182,8 +189,8 @@ int validate_moe_weight(const q4_moe_weight* w, const char* who) {
 struct MoeGemvPlan {
   bool ok;
   GemvConfig cfg;
-  int ntiles, mchunks;
-  size_t smem;
+  int ntiles, mchunks, rows;
+  size_t slab_bytes, smem;
 };
 
 // The decode kernel takes 16 rows of an expert per workgroup; an expert can receive every
@@ -192,7 +199,8 @@ struct MoeGemvPlan {
 // L2 where it can).  Measured on Mixtral shapes (8 experts, top-2), decode against MFMA
 // kernel: 4096 x 28672 113 / 268 us at 17 tokens, 163 / 240 us at 64; 14336 x 4096 (few
 // column tiles, long K: the MFMA kernel splits K) 106 / 110 us at 17 tokens, 194 / 108 us
-// at 64.  So the decode kernel is kept up to 64 tokens for K <= 8192 and up to 16 beyond.
+// at 64.  So the contiguous-group decode kernel is kept up to 64 tokens for K <= 8192 and up
+// to 16 beyond; the act-order and AWQ decode kernels, whose cost per row is higher, up to 16.
 constexpr int kMoeDecodeMaxTokens = 64;
 constexpr int kMoeDecodeMaxTokensLongK = 16;
 
@@ -200,28 +208,35 @@ MoeGemvPlan moe_gemv_plan(const q4_moe_weight* w, int tokens, int topk, int dtyp
   using namespace q4;
   MoeGemvPlan pl{};
   const q4_weight* e0 = &w->expert0;
+  const bool awq = e0->layout == Q4_LAYOUT_AWQ;
+  const bool act = !awq && e0->g_idx != nullptr;
   const int rows = tokens < kRowsPerBlock ? tokens : kRowsPerBlock;
-  if (tokens > (e0->K <= 8192 ? kMoeDecodeMaxTokens : kMoeDecodeMaxTokensLongK) || !gemv_supported(e0, rows, dtype))
-    return pl;
+  const int max_tokens = (awq || act || e0->K > 8192) ? kMoeDecodeMaxTokensLongK : kMoeDecodeMaxTokens;
+  if (tokens > max_tokens || !gemv_supported(e0, rows, dtype)) return pl;
   const int mchunks = (tokens + kRowsPerBlock - 1) / kRowsPerBlock;
   GemvConfig cfg = gemv_pick_config(e0, rows);
   cfg.words = 4;
-  if (e0->N % (64 * cfg.wcol) != 0) cfg.wcol = 1;
-  if (cfg.wcol * cfg.wk > 8 || e0->K % (cfg.wk * 128) != 0) return pl;
+  const int wave_cols = awq ? 256 : 64;
+  if (e0->N % (wave_cols * cfg.wcol) != 0) cfg.wcol = 1;
+  if (e0->N % wave_cols != 0 || cfg.wcol * cfg.wk > 8 || e0->K % (cfg.wk * 128) != 0) return pl;
   long active = (long)tokens * topk;
   if (active > w->num_experts) active = w->num_experts;
   int splits = (int)(cfg.splits / active);
   if (splits < 1) splits = 1;
   while (splits > 1 && e0->K % (splits * cfg.wk * 128) != 0) --splits;
-  const int ntiles = e0->N / (64 * cfg.wcol);
+  const int ntiles = e0->N / (wave_cols * cfg.wcol);
   const bool tickets_fit = (long)ntiles * mchunks * w->num_experts <= Q4_WORKSPACE_TICKET_BYTES / 4;
   if (!tickets_fit) splits = 1;
-  // the activation slab of 16 rows x K / splits must fit LDS: split further if it does not
+  // LDS: the activation slab of `rows` x K / splits, for act-order also the g_idx slice and
+  // the parameter table; the wk waves' partial sums reuse it.  Split further if it does not fit.
   const size_t smem_limit = 160 * 1024 - 1024;
+  const int nt = awq ? 16 : 4;
+  auto slab_of = [&](int sp) { return ((size_t)rows * ((size_t)e0->K / sp * 2 + 16) + 15) & ~(size_t)15; };
   auto smem_of = [&](int sp) {
-    const size_t slab = ((size_t)rows * ((size_t)e0->K / sp * 2 + 16) + 15) & ~(size_t)15;
-    const size_t red = (size_t)(cfg.wk - 1) * cfg.wcol * 4 * 4 * 64 * sizeof(float);
-    return slab > red ? slab : red;
+    size_t bytes = slab_of(sp);
+    if (act) bytes += (((size_t)e0->K / sp * 2 + 15) & ~(size_t)15) + (size_t)e0->num_groups * 64 * cfg.wcol * 4;
+    const size_t red = (size_t)(cfg.wk - 1) * cfg.wcol * nt * 4 * 64 * sizeof(float);
+    return bytes > red ? bytes : red;
   };
   while (smem_of(splits) > smem_limit) {
     int next = splits + 1;
@@ -234,6 +249,8 @@ MoeGemvPlan moe_gemv_plan(const q4_moe_weight* w, int tokens, int topk, int dtyp
   pl.cfg = cfg;
   pl.ntiles = ntiles;
   pl.mchunks = mchunks;
+  pl.rows = rows;
+  pl.slab_bytes = slab_of(splits);
   pl.smem = smem_of(splits);
   return pl;
 }
@@ -246,8 +263,19 @@ void launch_with_smem(Kernel k, dim3 grid, dim3 block, size_t smem, hipStream_t 
 }
 
 template <int DTYPE>
-void launch_moe_gemv_dtype(int gs, dim3 grid, dim3 block, size_t smem, hipStream_t stream, const GemvParams& gp) {
+void launch_moe_gemv_dtype(const q4_weight* e0, dim3 grid, dim3 block, size_t smem, hipStream_t stream,
+                           const GemvParams& gp) {
   using namespace q4;
+  const int gs = e0->groupsize;
+  if (e0->layout == Q4_LAYOUT_AWQ) {
+    launch_with_smem(gemv_awq_kernel<DTYPE, 4, true>, grid, block, smem, stream, gp);
+    return;
+  }
+  if (e0->g_idx != nullptr) {
+    // fp16 only (checked by the plan through gemv_supported)
+    launch_with_smem(gemv_gptq_act_kernel<4, true>, grid, block, smem, stream, gp);
+    return;
+  }
   if (gs == 128) launch_with_smem(gemv_gptq_kernel<DTYPE, 4, 4, true, 4, false, true>, grid, block, smem, stream, gp);
   else if (gs > 128) launch_with_smem(gemv_gptq_kernel<DTYPE, 4, 4, false, 4, false, true>, grid, block, smem, stream, gp);
   else if (gs == 64) launch_with_smem(gemv_gptq_kernel<DTYPE, 4, 2, false, 4, false, true>, grid, block, smem, stream, gp);
@@ -282,6 +310,7 @@ MoeView make_view(const q4_moe_weight* w, const int32_t* x_rows, const int32_t* 
   mv.qweight_stride = (long)w->qweight_stride;
   mv.qzeros_stride = (long)w->qzeros_stride;
   mv.scales_stride = (long)w->scales_stride;
+  mv.g_idx_stride = (long)w->g_idx_stride;
   return mv;
 }
 
@@ -293,6 +322,10 @@ size_t moe_workspace_bytes(const q4_moe_weight* w, int tokens, int topk) {
   int splits = 1;
   if (pl.ok) splits = pl.cfg.splits;
   else if (gemm_supported(&w->expert0, tokens, Q4_DTYPE_F16)) splits = moe_gemm_splits(w, tokens, topk);
+  else if (gemm_awq_supported(&w->expert0, tokens, Q4_DTYPE_F16)) {
+    const MoeLaunch ml{MoeView{}, w->num_experts, tokens, tokens * topk};
+    return bytes + gemm_awq_moe_workspace_bytes(&w->expert0, &ml);
+  }
   if (splits > 1) bytes += (size_t)splits * tokens * topk * w->expert0.N * sizeof(float);
   return bytes;
 }
@@ -318,7 +351,7 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
       partials = (float*)((char*)workspace + Q4_WORKSPACE_COUNTER_BYTES);
     }
     GemvParams gp;
-    gp.p = Problem{e0->qweight, e0->qzeros, (const half_t*)e0->scales, nullptr, x, nullptr, y,
+    gp.p = Problem{e0->qweight, e0->qzeros, (const half_t*)e0->scales, e0->g_idx, x, nullptr, y,
                    0,           e0->K,      e0->N,                     e0->groupsize, e0->num_groups};
     gp.p.gate_up_act = 0;
     gp.partials = partials;
@@ -329,13 +362,13 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
     gp.cells = nullptr;
     gp.fixed_point_split = 0;
     gp.slab_stride = e0->K / cfg.splits * 2 + 16;
-    gp.slab_bytes = (int)pl.smem;
+    gp.slab_bytes = (int)pl.slab_bytes;
     gp.partial_rows = pairs;
     gp.moe = mv;
     const dim3 grid((unsigned)(pl.ntiles * cfg.splits), (unsigned)pl.mchunks, (unsigned)w->num_experts);
     const dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
-    if (dtype == Q4_DTYPE_F16) launch_moe_gemv_dtype<Q4_DTYPE_F16>(e0->groupsize, grid, block, pl.smem, stream, gp);
-    else launch_moe_gemv_dtype<Q4_DTYPE_BF16>(e0->groupsize, grid, block, pl.smem, stream, gp);
+    if (dtype == Q4_DTYPE_F16) launch_moe_gemv_dtype<Q4_DTYPE_F16>(e0, grid, block, pl.smem, stream, gp);
+    else launch_moe_gemv_dtype<Q4_DTYPE_BF16>(e0, grid, block, pl.smem, stream, gp);
   } else if (gemm_supported(e0, tokens, dtype)) {
     GemmParams gp;
     gp.p = Problem{e0->qweight, e0->qzeros, (const half_t*)e0->scales, nullptr, x, nullptr, y,
@@ -366,6 +399,10 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
       else launch_moe_gemm_tile<Q4_DTYPE_BF16, 1>(e0->groupsize, grid, smem, stream, gp);
     }
     if (splits > 1) launch_gemm_reduce(gp.partials, nullptr, y, pairs, e0->N, splits, dtype, stream);
+  } else if (gemm_awq_supported(e0, tokens, dtype)) {
+    // AWQ layout and act-order: the MFMA kernel that unpacks the weights into LDS
+    const MoeLaunch ml{mv, w->num_experts, tokens, pairs};
+    return launch_gemm_awq(e0, x, nullptr, y, tokens, dtype, workspace, workspace_bytes, stream, &ml);
   } else {
     set_error("q4_moe_linear: no grouped kernel for tokens=%d K=%d N=%d groupsize=%d", tokens, e0->K, e0->N,
               e0->groupsize);

@@ -5,7 +5,8 @@ Mirrors the constructor and forward of the reference's `GPTQMarlinSparseMoELayer
 down projections are loaded through the same `Weights` calls (`get_multi_weights_col`,
 `get_weights_row`, :149-183) and stacked along a leading expert dimension (:186-229), and
 `forward(x, gating_output=...)` routes every token to its top-k experts.  Differences: the
-tensors stay in checkpoint layout (no Marlin repack, hence no perm / is_full_k fields) and
+tensors stay in checkpoint layout -- GPTQ with or without act-order, or AWQ (no Marlin repack,
+hence no perm / is_full_k fields) -- and
 the grouped int4 kernels of this package do the work that the reference takes from the
 `kernels-community/moe` package, which only exists for CUDA.
 """
@@ -19,21 +20,29 @@ import torch
 import torch.nn as nn
 
 from ... import ops
+from ..._lib import LAYOUT_AWQ, LAYOUT_GPTQ
 from ..gptq import GPTQWeight
 from ..gptq.quant_linear import is_trivial_g_idx
 
 
 @dataclass
 class GPTQMoEWeight:
-    """Stacked experts of one projection: qweight [E, K/8, N], qzeros [E, G, N/8], scales [E, G, N]."""
+    """Stacked experts of one projection: qweight [E, K/8, N] (AWQ: [E, K, N/8]), qzeros
+    [E, G, N/8], scales [E, G, N], g_idx [E, K] or None."""
 
     qweight: torch.Tensor
     qzeros: torch.Tensor
     scales: torch.Tensor
+    g_idx: Optional[torch.Tensor]
     groupsize: int
+    use_awq_kernel: bool
 
     def packed(self) -> ops.PackedMoeWeight:
-        return ops.make_packed_moe(self.qweight, self.qzeros, self.scales, self.groupsize)
+        g_idx = self.g_idx
+        if g_idx is not None and all(is_trivial_g_idx(g, self.groupsize) for g in g_idx):
+            g_idx = None  # sequential groups in every expert: the kernels index by k // groupsize
+        return ops.make_packed_moe(self.qweight, self.qzeros, self.scales, self.groupsize, g_idx,
+                                   LAYOUT_AWQ if self.use_awq_kernel else LAYOUT_GPTQ)
 
 
 def _check_expert(weight, name: str) -> GPTQWeight:
@@ -41,13 +50,6 @@ def _check_expert(weight, name: str) -> GPTQWeight:
         raise ValueError(f"{name}: expected GPTQ weights, got {type(weight).__name__}")
     if weight.bits != 4:
         raise NotImplementedError(f"{name}: only 4-bit experts are supported, got {weight.bits}")
-    if weight.use_awq_kernel:
-        raise NotImplementedError(
-            f"{name}: experts in the AWQ layout are not covered by the grouped kernels; load the checkpoint "
-            "with quantize='gptq' so that the loader converts it (fast_awq_to_gptq)"
-        )
-    if weight.g_idx is not None and not is_trivial_g_idx(weight.g_idx, weight.groupsize):
-        raise NotImplementedError(f"{name}: act-order (desc_act) experts are not covered by the grouped kernels")
     return weight
 
 
@@ -58,13 +60,20 @@ def _pack_weight(*, n_experts: int, expert: int, moe_weight: Optional[GPTQMoEWei
             qweight=torch.empty((n_experts,) + weight.qweight.shape, dtype=weight.qweight.dtype, device=weight.qweight.device),
             qzeros=torch.empty((n_experts,) + weight.qzeros.shape, dtype=weight.qzeros.dtype, device=weight.qzeros.device),
             scales=torch.empty((n_experts,) + weight.scales.shape, dtype=weight.scales.dtype, device=weight.scales.device),
+            g_idx=None if weight.g_idx is None else torch.empty(
+                (n_experts,) + weight.g_idx.shape, dtype=weight.g_idx.dtype, device=weight.g_idx.device),
             groupsize=weight.groupsize,
+            use_awq_kernel=weight.use_awq_kernel,
         )
-    if weight.groupsize != moe_weight.groupsize:
-        raise ValueError(f"expert {expert} has groupsize {weight.groupsize}, expert 0 {moe_weight.groupsize}")
+    if weight.groupsize != moe_weight.groupsize or weight.use_awq_kernel != moe_weight.use_awq_kernel:
+        raise ValueError(f"expert {expert} differs from expert 0 in groupsize or layout")
+    if (weight.g_idx is None) != (moe_weight.g_idx is None):
+        raise ValueError(f"expert {expert} differs from expert 0 in having a g_idx")
     moe_weight.qweight[expert] = weight.qweight
     moe_weight.qzeros[expert] = weight.qzeros
     moe_weight.scales[expert] = weight.scales
+    if weight.g_idx is not None:
+        moe_weight.g_idx[expert] = weight.g_idx
     return moe_weight
 
 

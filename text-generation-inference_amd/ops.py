@@ -304,37 +304,48 @@ def select_path(w: PackedWeight, M: int, dtype: torch.dtype = torch.float16) -> 
 @dataclass
 class PackedMoeWeight:
     """The experts of one projection, stacked along a leading expert dimension in checkpoint
-    layout: qweight [E, K/8, N], qzeros [E, G, N/8], scales [E, G, N] (GPTQ, no g_idx)."""
+    layout: GPTQ qweight [E, K/8, N] (AWQ [E, K, N/8]), qzeros [E, G, N/8], scales [E, G, N],
+    optional g_idx [E, K] (GPTQ act-order)."""
 
     qweight: torch.Tensor
     qzeros: torch.Tensor
     scales: torch.Tensor
+    g_idx: Optional[torch.Tensor]
     K: int
     N: int
     groupsize: int
     num_groups: int
     num_experts: int
+    layout: int
 
     def struct(self) -> _lib.Q4MoeWeight:
         e0 = _lib.Q4Weight(
-            self.qweight.data_ptr(), self.qzeros.data_ptr(), self.scales.data_ptr(), None,
-            self.K, self.N, self.groupsize, self.num_groups, LAYOUT_GPTQ,
+            self.qweight.data_ptr(), self.qzeros.data_ptr(), self.scales.data_ptr(),
+            self.g_idx.data_ptr() if self.g_idx is not None else None,
+            self.K, self.N, self.groupsize, self.num_groups, self.layout,
         )
-        return _lib.Q4MoeWeight(e0, self.num_experts, self.qweight.stride(0), self.qzeros.stride(0), self.scales.stride(0))
+        return _lib.Q4MoeWeight(
+            e0, self.num_experts, self.qweight.stride(0), self.qzeros.stride(0), self.scales.stride(0),
+            self.g_idx.stride(0) if self.g_idx is not None else 0,
+        )
 
 
-def make_packed_moe(qweight, qzeros, scales, groupsize: int) -> PackedMoeWeight:
+def make_packed_moe(qweight, qzeros, scales, groupsize: int, g_idx=None, layout: int = LAYOUT_GPTQ) -> PackedMoeWeight:
     """Validate stacked expert tensors and wrap them for the grouped kernels."""
     if qweight.dim() != 3 or qzeros.dim() != 3 or scales.dim() != 3:
         raise ValueError("stacked expert tensors must be [E, ...] with three dimensions")
     E = qweight.shape[0]
-    one = make_packed(qweight[0], qzeros[0], scales[0], None, groupsize, LAYOUT_GPTQ)
+    if g_idx is not None and (g_idx.dim() != 2 or g_idx.shape[0] != E):
+        raise ValueError(f"g_idx must be [{E}, K], got {tuple(g_idx.shape)}")
+    one = make_packed(qweight[0], qzeros[0], scales[0], g_idx[0] if g_idx is not None else None, groupsize, layout)
     if qzeros.shape[0] != E or scales.shape[0] != E:
         raise ValueError(f"expert counts differ: {E}, {qzeros.shape[0]}, {scales.shape[0]}")
+    if g_idx is not None:
+        g_idx = g_idx.to(torch.int32).contiguous()
     for name, t in (("qweight", qweight), ("qzeros", qzeros), ("scales", scales)):
         if not t[0].is_contiguous():
             raise ValueError(f"{name}: every expert's slice must be contiguous")
-    return PackedMoeWeight(qweight, qzeros, scales, one.K, one.N, one.groupsize, one.num_groups, E)
+    return PackedMoeWeight(qweight, qzeros, scales, g_idx, one.K, one.N, one.groupsize, one.num_groups, E, layout)
 
 
 @dataclass
