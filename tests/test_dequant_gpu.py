@@ -13,7 +13,7 @@ GPTQ_CASES = [
     (128, 64, 128, True, False),
     (256, 128, 32, False, False),
     (512, 256, 64, False, True),
-    (4096, 4096, 128, True, False),   # cfg1 shape
+    (4096, 4096, 128, True, False),   # BASELINE.json configs[0] shape
     (1024, 264, 128, False, False),   # N multiple of 8 only
     (1000, 64, 40, False, False),     # K multiple of 8 only, odd groupsize
     (2048, 512, -1, False, False),    # one group

@@ -54,7 +54,7 @@ GEMV_SHAPES = [(4096, 4096), (4096, 6144), (4096, 28672), (14336, 4096)]
 
 
 def test_cfg1_gptq_m16(pkg, oracle, gpu):
-    """BASELINE configs[0]: K=N=4096, groupsize 128, sym, M=16."""
+    """BASELINE.json configs[0]: K=N=4096, groupsize 128, sym, M=16."""
     _run(pkg, oracle, gpu, 4096, 4096, 128, 16, seed=1)
 
 
@@ -161,7 +161,7 @@ def test_gemm_llama3_8b_fp16(pkg, oracle, gpu, K, N, M):
 
 
 def test_gemm_gate_up_bf16(pkg, oracle, gpu):
-    """cfg3: bf16 activations, widest projection."""
+    """BASELINE.json configs[2]: bf16 activations, widest projection."""
     _run(pkg, oracle, gpu, 4096, 28672, 128, 512, dtype="bf16", path=2, seed=77)
 
 
@@ -248,13 +248,13 @@ def test_auto_dispatch(pkg, oracle, gpu):
 @pytest.mark.parametrize("K,N", [(4096, 14336), (14336, 4096)])
 @pytest.mark.parametrize("M", [1, 2, 4, 16])
 def test_awq_decode_mistral(pkg, oracle, gpu, K, N, M):
-    """cfg5: AWQ GEMM layout, asymmetric zeros, Mistral-7B shapes, decode kernel."""
+    """BASELINE.json configs[4]: AWQ GEMM layout, asymmetric zeros, Mistral-7B shapes, decode kernel."""
     _run(pkg, oracle, gpu, K, N, 128, M, layout="awq", path=1, seed=K // 256 + M)
 
 
 @pytest.mark.parametrize("M", [3, 7, 16, 17, 40, 64, 256])
 def test_awq_m_sweep_chunked(pkg, oracle, gpu, M):
-    """The AWQ decode kernel takes any M in row chunks of 16 (cfg5 sweeps M up to 256)."""
+    """The AWQ decode kernel takes any M in row chunks of 16 (BASELINE.json configs[4] sweeps M up to 256)."""
     _run(pkg, oracle, gpu, 1024, 512, 128, M, layout="awq", bias=(M % 2 == 1), seed=M)
 
 
@@ -288,7 +288,7 @@ def test_awq_auto_path_is_native(pkg, oracle, gpu):
 @pytest.mark.parametrize("K,N", [(8192, 10240), (28672, 8192)])
 @pytest.mark.parametrize("M", [1, 16])
 def test_act_order_decode_llama70b(pkg, oracle, gpu, K, N, M):
-    """cfg4: desc_act=True with a random row permutation, Llama-3-70B per-layer shapes."""
+    """BASELINE.json configs[3]: desc_act=True with a random row permutation, Llama-3-70B per-layer shapes."""
     _run(pkg, oracle, gpu, K, N, 128, M, act=True, path=1, seed=K // 1024 + M)
 
 
@@ -379,7 +379,7 @@ def test_gemm_n_multiple_of_128_only(pkg, oracle, gpu):
 
 @pytest.mark.parametrize("K,N,M", [(8192, 10240, 1024), (1024, 256, 200), (2048, 128, 64)])
 def test_act_order_gemm(pkg, oracle, gpu, K, N, M):
-    """cfg4 prefill: desc_act through the MFMA kernel (per-row scale/zero gathered by g_idx)."""
+    """BASELINE.json configs[3], prefill: desc_act through the MFMA kernel (per-row scale/zero gathered by g_idx)."""
     _run(pkg, oracle, gpu, K, N, 128, M, sym=(K == 8192), act=True, path=2, bias=(M == 200), seed=K // 512 + M)
 
 
