@@ -60,6 +60,7 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--gemm-m", type=int, default=2048)
+    ap.add_argument("--no-moe", action="store_true", help="skip the mixture-of-experts block leg")
     ap.add_argument("--copies", type=int, default=0, help="weight copies to rotate over (0 = auto)")
     ap.add_argument("--no-dense-ref", action="store_true",
                     help="skip timing torch's dense fp16 matmul (hipBLASLt) on the GEMM shapes")
@@ -336,6 +337,34 @@ def main():
                              "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                              "frac": round(tot_f / tot_t / 1e12 / MFMA_PEAK_TFLOPS, 4), "traffic": None},
             }
+
+    # ---- mixture-of-experts block (Mixtral-8x7B shapes: 8 experts, top-2, 4096 -> 2 x 14336 -> 4096):
+    # routing, both grouped projections, activation and weighted sum, per block call
+    if not args.no_moe:
+        del weights
+        torch.cuda.empty_cache()
+        E, topk, H, I = 8, 2, 4096, 14336
+        gen = torch.Generator(device=dev).manual_seed(7)
+
+        def experts(K, N):
+            qw = torch.randint(-2**31, 2**31 - 1, (E, K // 8, N), dtype=torch.int32, device=dev, generator=gen)
+            qz = torch.full((E, K // GROUPSIZE, N // 8), 0x77777777, dtype=torch.int32, device=dev)
+            sc = (torch.rand((E, K // GROUPSIZE, N), device=dev, generator=gen) * 0.019 + 0.001).half()
+            return pkg.ops.make_packed_moe(qw, qz, sc, GROUPSIZE)
+
+        gate_up, down = experts(H, 2 * I), experts(I, H)
+        moe = {}
+        for T in (1, 16, 1024):
+            xm = torch.randn((T, H), device=dev, dtype=torch.float16)
+            logits = torch.randn((T, E), device=dev, dtype=torch.float32, generator=gen)
+            active = int(torch.unique(torch.topk(logits, topk, dim=1).indices).numel())
+            fn = lambda: pkg.ops.moe_forward(gate_up, down, xm, logits, topk, True, "silu")
+            avg, _ = time_kernel_launches(torch, [fn], 10)
+            wbytes = active * 3 * H * I / 2
+            fl = 2.0 * T * topk * 3 * H * I
+            moe[f"tokens_{T}"] = {"us_avg": round(avg * 1e6, 1), "experts_active": active,
+                                  "weight_GBps": round(wbytes / avg / 1e9, 1), "TFLOPs": round(fl / avg / 1e12, 1)}
+        out["moe_block"] = {"experts": E, "topk": topk, "hidden": H, "intermediate": I, "per_tokens": moe}
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(M)
