@@ -67,7 +67,7 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   // (and at any M once the tiles alone are well over the CU count: 4096 x 28672 at M = 1
   // measured 16.7 against 17.0-17.8 us)
   if (w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && w->N % 128 == 0 &&
-      ((M >= 8 && w->N / 64 >= 256) || w->N / 64 >= 384))
+      ((M >= 8 && w->N / 64 >= 256) || (M >= 12 && w->N / 64 >= 128) || w->N / 64 >= 384))
     c.wcol = 2;
   const bool act = w->layout == Q4_LAYOUT_GPTQ && w->g_idx != nullptr;
   if (act && chunks % 8 == 0) c.wk = 8;  // the group table is built once per workgroup
@@ -87,11 +87,20 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   const bool cheap_combine = M == 1 && w->layout == Q4_LAYOUT_GPTQ && !gate_up;
   if (cheap_combine) target_wgs = 768;
   if (gate_up) target_wgs = 256;        // 512-thread workgroups: one per CU
-  int want = (target_wgs + ntiles / 2) / ntiles;
+  // the targets count four-wave workgroups: one with two column tiles (eight waves) counts twice
+  // (4096 x 14336 at M = 16, two tiles per workgroup: 16.6 us with two splits, 18.9 us with four)
+  const int tile_units = ntiles * (gate_up ? 1 : c.wcol);
+  int want = (target_wgs + tile_units / 2) / tile_units;
   // tiles that fill the chip on their own are not split (4096 x 28672: 18.5 us with two
   // splits against 16.7 us with one)
   if (want < 1 || ntiles * c.wcol >= 256) want = 1;
-  long lds_budget = 60000 - 16L * rows;
+  // The slab of a workgroup is rows x K / splits activations.  Normally it is held to ~68 KB so
+  // that two workgroups share a CU (16 rows x 2048: 4096 x 14336 at M = 16 takes 16.6 us with two
+  // splits against 20 us with four); when the column tiles alone fill the chip, splitting K only
+  // to make the slab smaller costs more (partial sums of every row through memory) than the
+  // lost co-residency: 4096 x 28672 at M = 16 takes 19.7 us unsplit with a 128 KB slab against
+  // 30.8 us with four splits.
+  long lds_budget = (want == 1 && ntiles * c.wcol >= 256 ? 150000 : 70000) - 16L * rows;
   if (act) lds_budget = 150000 - (long)w->num_groups * 64 * 4 - 16L * rows;
   // bytes per K row in LDS: activations, plus the uint16 g_idx slice for act-order
   const long per_row = (long)rows * 2 + (act ? 2 : 0);
