@@ -68,6 +68,12 @@ def test_decode_small_shapes_split_k(pkg, oracle, gpu, K, N, gs, M):
           seed=K // 64 + N + M)
 
 
+@pytest.mark.parametrize("M", [1, 2])
+def test_decode_fused_ragged_k_partition(pkg, oracle, gpu, M):
+    """43 chunks of 128 rows do not divide over the wave slots of the fused kernel."""
+    _case(pkg, oracle, gpu, 43 * 128, 512, 128, M, fused=True, seed=M + 5)
+
+
 @pytest.mark.parametrize("act", ["silu", "gelu_tanh", "gelu", "gelu_fast", "gelu_pytorch_tanh"])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_activations_decode_and_prefill(pkg, oracle, gpu, act, dtype):

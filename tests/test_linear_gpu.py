@@ -234,8 +234,8 @@ def test_auto_dispatch(pkg, oracle, gpu):
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
     assert pkg.ops.select_path(pk, 1) == "gemv"
     assert pkg.ops.select_path(pk, 16) == "gemv"
-    assert pkg.ops.select_path(pk, 48) == "gemv"   # small matrix: row-chunked decode up to 48 rows
-    assert pkg.ops.select_path(pk, 49) == "gemm"
+    assert pkg.ops.select_path(pk, 64) == "gemv"   # small matrix: row-blocked decode up to 64 rows
+    assert pkg.ops.select_path(pk, 65) == "gemm"
     qw, qz, sc, _ = oracle.make_gptq(1000, 264, 40, seed=3)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 40, 0)
     assert pkg.ops.select_path(pk, 1) == "generic"
@@ -372,6 +372,34 @@ def test_awq_dispatch_large_m(pkg, oracle, gpu):
 def test_gemm_n_multiple_of_128_only(pkg, oracle, gpu):
     """N = 384 is not a multiple of 256: the GEMM takes its 128-column tile."""
     _run(pkg, oracle, gpu, 1024, 384, 128, 3000, sym=False, bias=True, path=2, seed=384)
+
+
+# --------------------------------------------------------------------------- K that does not divide evenly
+
+
+@pytest.mark.parametrize("layout,act", [("gptq", False), ("gptq", True), ("awq", False)])
+@pytest.mark.parametrize("M", [1, 3, 16, 20])
+def test_gemv_ragged_k_partition(pkg, oracle, gpu, layout, act, M):
+    """K = 43 chunks of 128 rows (prime): the wave slots get two or three chunks each
+    (Llama-2-7B's down projection has K = 11008 = 86 chunks)."""
+    _run(pkg, oracle, gpu, 43 * 128, 512, 128, M, layout=layout, act=act, sym=False, bias=(M == 3), path=1, seed=M + 43)
+
+
+@pytest.mark.parametrize("cfg", [(1, 4, 3), (1, 4, 5), (2, 2, 7), (1, 8, 2), (1, 3, 5), (1, 1, 43)])
+def test_gemv_ragged_k_explicit_decompositions(pkg, oracle, gpu, cfg):
+    """43 chunks over wk x splits slots that do not divide them."""
+    _run(pkg, oracle, gpu, 43 * 128, 256, 128, 5, sym=False, cfg=cfg, seed=sum(cfg))
+    _run(pkg, oracle, gpu, 43 * 128, 256, 64, 2, sym=False, cfg=cfg, seed=sum(cfg) + 1)
+
+
+def test_gemv_llama2_7b_down_shape(pkg, oracle, gpu):
+    _run(pkg, oracle, gpu, 11008, 4096, 128, 1, path=1, seed=11)
+    _run(pkg, oracle, gpu, 11008, 4096, 128, 16, path=1, seed=12)
+
+
+def test_gemv_rejects_more_wave_slots_than_chunks(pkg, oracle, gpu):
+    with pytest.raises(pkg._lib.Q4Error):
+        _run(pkg, oracle, gpu, 512, 256, 128, 2, cfg=(1, 4, 2))  # 4 chunks, 8 slots
 
 
 # --------------------------------------------------------------------------- act-order prefill GEMM

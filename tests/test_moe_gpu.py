@@ -106,6 +106,7 @@ def _packed_experts(pkg, oracle, gpu, kind, E, K, N, gs, dtype, seed):
     (4, 8, 2, 1024, 512, 128),
     (16, 8, 2, 2048, 1024, 128),    # decode, 16 rows possible per expert
     (7, 4, 4, 1024, 256, 64),       # every token on every expert
+    (3, 8, 2, 43 * 128, 256, 128),  # 43 chunks of 128 rows: uneven K ranges
     (5, 8, 2, 512, 256, 32),
     (3, 8, 2, 1024, 512, -1),       # one group
     (17, 8, 2, 1024, 512, 128),

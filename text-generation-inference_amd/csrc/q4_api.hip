@@ -85,12 +85,16 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   const bool contiguous_gptq = w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr;
   const long weights = (long)w->K * w->N;
   if (contiguous_gptq) {
-    // Measured crossover on MI355X (Llama-3-8B shapes).  The decode kernel's cost grows with
-    // every 16-row chunk, the split-K GEMM's is nearly flat up to a few hundred rows:
-    // 4096 x 4096 (2^24 weights) decode 15.2 / 17.1 / 22.7 us against GEMM 17.3 / 18.6 / 19.1 us
-    // at M = 32 / 48 / 64; 4096 x 6144 decode 17.1 / 20.3 against 18.6 / 19.5 us at M = 32 / 40;
-    // 14336 x 4096 and 4096 x 28672 are faster through the GEMM from M = 17 on.
-    const bool small = M <= 16 || (M <= 32 && weights <= (1L << 25)) || (M <= 48 && weights <= (1L << 24));
+    // Measured crossover on MI355X.  The decode kernel works in blocks of 16 rows that run side
+    // by side (a second block costs little: the weights are shared through L2), the split-K
+    // GEMM is nearly flat in M up to a few hundred rows.  Decode / GEMM in us at M = 32:
+    // 4096 x 4096 11.6 / 17.3, 4096 x 6144 12.7 / 18.8, 4096 x 14336 17.6 / 27.5, 4096 x 28672
+    // 34.5 / 40.7, 8192 x 8192 22.1 / 28.5, but 8192 x 10240 38.4 / 32.6, 5120 x 13824 32.9 / 28.9,
+    // 14336 x 4096 30.5 / 26.0 (at M = 17: 25.7 / 25.3).  From the third block on (M = 48) the
+    // GEMM wins except on the smallest matrices (4096 x 4096: 12.6 / 19.2 at M = 64, 24.4 / 20.8
+    // at M = 96; 2048 x 8192: 10.8 / 15.2 at M = 64).
+    const bool small = M <= 16 || (M <= 32 && (w->K <= 4096 || (w->K <= 8192 && weights <= (1L << 26)))) ||
+                       (M <= 64 && weights <= (1L << 24));
     if (small && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
     if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;
     if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;

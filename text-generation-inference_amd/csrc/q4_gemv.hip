@@ -62,7 +62,7 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   const int mchunks = (M + q4::kRowsPerBlock - 1) / q4::kRowsPerBlock;
   const int chunks = w->K / 128;
   c.wcol = 1;
-  c.wk = chunks % 4 == 0 ? 4 : (chunks % 2 == 0 ? 2 : 1);
+  c.wk = chunks >= 4 ? 4 : (chunks >= 2 ? 2 : 1);
   // wide layers with many rows: two column tiles per workgroup halve the slab staging
   // (and at any M once the tiles alone are well over the CU count: 4096 x 28672 at M = 1
   // measured 16.7 against 17.0-17.8 us)
@@ -70,18 +70,22 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
       ((M >= 8 && w->N / 64 >= 256) || (M >= 12 && w->N / 64 >= 128) || w->N / 64 >= 384))
     c.wcol = 2;
   const bool act = w->layout == Q4_LAYOUT_GPTQ && w->g_idx != nullptr;
-  if (act && chunks % 8 == 0) c.wk = 8;  // the group table is built once per workgroup
+  if (act && (chunks % 8 == 0 || chunks >= 32)) c.wk = 8;  // the group table is built once per workgroup
+  // many rows, one column tile per workgroup: eight waves along K share one activation slab
+  // (M = 16: 4096 x 6144 12.1 against 14.9 us, 14336 x 4096 18.8 against 22.4 us)
+  const bool contiguous = w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr;
+  if (contiguous && !gate_up && M >= 12 && c.wcol == 1 && (chunks % 8 == 0 || chunks >= 32)) c.wk = 8;
   if (gate_up) {
     // a wave owns 64 gate and 64 up columns (twice the bytes of a plain wave): eight waves
     // along K keep the wave count, and with it the bytes in flight, of the plain kernel
     c.wcol = 1;
     c.words = 8;
-    if (chunks % 8 == 0) c.wk = 8;
+    if (chunks % 8 == 0 || chunks >= 32) c.wk = 8;
   }
-  const int per_wg = chunks / c.wk;      // chunks left to distribute over splits x per-wave work
+  const int per_wg = chunks / c.wk;      // most splits: one chunk per wave
   const int wave_cols = w->layout == Q4_LAYOUT_AWQ ? 256 : (gate_up ? 128 : 64);
   const int ntiles = (w->N / (wave_cols * c.wcol)) * mchunks;
-  int target_wgs = M <= 4 ? 512 : 384;  // partial-sum traffic grows with M
+  int target_wgs = M <= 8 ? 512 : 384;  // partial-sum traffic grows with M
   // a single fp16 row combines its splits with one atomic per element: more, shorter
   // workgroups pay (4096 x 6144: 7.7 us with 8 splits against 8.4 us with 4)
   const bool cheap_combine = M == 1 && w->layout == Q4_LAYOUT_GPTQ && !gate_up;
@@ -89,29 +93,41 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   if (gate_up) target_wgs = 256;        // 512-thread workgroups: one per CU
   // the targets count four-wave workgroups: one with two column tiles (eight waves) counts twice
   // (4096 x 14336 at M = 16, two tiles per workgroup: 16.6 us with two splits, 18.9 us with four)
-  const int tile_units = ntiles * (gate_up ? 1 : c.wcol);
+  const int tile_units = ntiles * (gate_up ? 1 : c.wcol) * (contiguous && !gate_up && c.wk == 8 ? 2 : 1);
   int want = (target_wgs + tile_units / 2) / tile_units;
   // tiles that fill the chip on their own are not split (4096 x 28672: 18.5 us with two
   // splits against 16.7 us with one)
   if (want < 1 || ntiles * c.wcol >= 256) want = 1;
-  // The slab of a workgroup is rows x K / splits activations.  Normally it is held to ~68 KB so
-  // that two workgroups share a CU (16 rows x 2048: 4096 x 14336 at M = 16 takes 16.6 us with two
-  // splits against 20 us with four); when the column tiles alone fill the chip, splitting K only
-  // to make the slab smaller costs more (partial sums of every row through memory) than the
-  // lost co-residency: 4096 x 28672 at M = 16 takes 19.7 us unsplit with a 128 KB slab against
-  // 30.8 us with four splits.
-  long lds_budget = (want == 1 && ntiles * c.wcol >= 256 ? 150000 : 70000) - 16L * rows;
+  // long K: no wave walks more than ~1024 rows when the tiles leave room for more workgroups
+  // (28672 x 8192 at M = 8: 41.7 us with seven splits, 46.2 us with four)
+  else if (contiguous && !gate_up && want < w->K / (c.wk * 1024)) want = w->K / (c.wk * 1024);
+  // The slab of a workgroup is rows x K / splits activations and may take most of the LDS (one
+  // workgroup per CU then): splitting K only to make the slab smaller costs more -- partial
+  // sums of every row through memory -- than the lost co-residency.  4096 x 28672 at M = 16:
+  // 19.7 us unsplit with a 128 KB slab against 30.8 us with four splits; 5120 x 13824 at M = 16:
+  // 16 us with two splits (80 KB) against 26.8 us with five.
+  long lds_budget = 150000 - 16L * rows;
   if (act) lds_budget = 150000 - (long)w->num_groups * 64 * 4 - 16L * rows;
   // bytes per K row in LDS: activations, plus the uint16 g_idx slice for act-order
   const long per_row = (long)rows * 2 + (act ? 2 : 0);
-  int min_splits = lds_budget > 0 ? (int)(((long)w->K * per_row + lds_budget - 1) / lds_budget) : per_wg;
+  const int max_splits = per_wg;  // every wave gets at least one 128-row chunk
+  int min_splits = lds_budget > 0 ? (int)(((long)w->K * per_row + lds_budget - 1) / lds_budget) : max_splits;
   if (min_splits < 1) min_splits = 1;
-  int best = per_wg;  // always legal: one chunk per wave
-  long best_cost = -1;
-  for (int dv = 1; dv <= per_wg; ++dv) {
-    if (per_wg % dv != 0 || dv < min_splits) continue;
-    const long cost = dv > want ? (long)dv * 1000 / want : (long)want * 1000 / dv;
-    if (best_cost < 0 || cost < best_cost) {
+  if (min_splits > max_splits) min_splits = max_splits;
+  // K is dealt out in 128-row chunks over splits x wk wave slots.  A count that divides the
+  // chunks evenly is preferred; when none is near the wanted one (K = 11008: 86 chunks) the
+  // slots differ by one chunk and the cost carries the imbalance.
+  int best = max_splits;
+  double best_cost = -1.0;
+  for (int dv = min_splits; dv <= max_splits; ++dv) {
+    const long slots = (long)dv * c.wk;
+    const double balance = (double)((chunks + slots - 1) / slots) * slots / chunks;  // >= 1
+    // too few workgroups cost more than too many (13824 x 5120 at M = 16 wants five splits:
+    // nine take 19.4 us, three 24 us)
+    double cost = dv > want ? (double)dv / want : 1.5 * want / dv;
+    cost *= balance;
+    if (chunks % slots != 0) cost *= 1.25;
+    if (best_cost < 0.0 || cost < best_cost) {
       best_cost = cost;
       best = dv;
     }
@@ -178,14 +194,20 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   }
   const int wave_cols = awq ? 256 : 16 * cfg.words;
   if (cfg.wcol < 1 || cfg.wk < 1 || cfg.splits < 1 || cfg.wcol * cfg.wk > 8 ||
-      w->N % (wave_cols * cfg.wcol) != 0 || w->K % (cfg.splits * cfg.wk * 128) != 0) {
+      w->N % (wave_cols * cfg.wcol) != 0 || w->K % 128 != 0 || (long)cfg.splits * cfg.wk > w->K / 128) {
     set_error("q4_linear(gemv): bad config wcol=%d wk=%d splits=%d for K=%d N=%d", cfg.wcol, cfg.wk,
               cfg.splits, w->K, w->N);
     return Q4_ERR_INVALID_ARGUMENT;
   }
   const int rows = M < kRowsPerBlock ? M : kRowsPerBlock;
   const int mchunks = (M + kRowsPerBlock - 1) / kRowsPerBlock;
-  const int KR = w->K / cfg.splits;
+  // largest K range of a workgroup: K goes out in 128-row chunks over splits x wk wave slots
+  const long kchunks = w->K / 128, kslots = (long)cfg.splits * cfg.wk;
+  int KR = 0;
+  for (int sp = 0; sp < cfg.splits; ++sp) {
+    const int r = (int)(((long)(sp + 1) * cfg.wk * kchunks / kslots - (long)sp * cfg.wk * kchunks / kslots) * 128);
+    if (r > KR) KR = r;
+  }
   const int slab_stride = KR * 2 + 16;
   const int rmax = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
   const int nt = awq ? 16 : cfg.words;
@@ -234,6 +256,7 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.cells = cfg.splits > 1 ? (unsigned long long*)((char*)workspace + Q4_WORKSPACE_TICKET_BYTES) : nullptr;
   gp.slab_stride = slab_stride;
   gp.slab_bytes = (int)slab_bytes;
+  gp.kr_max = KR;
   gp.partial_rows = M;
   gp.moe = q4::MoeView{};
   dim3 grid((unsigned)(ntiles * cfg.splits), (unsigned)mchunks);

@@ -51,6 +51,7 @@ struct GemvParams {
   int fixed_point_split;  // fp16 outputs: combine the splits with one 64-bit atomic per element
   int slab_stride;  // bytes between activation rows in LDS
   int slab_bytes;   // size of the activation slab region
+  int kr_max;        // largest K range of a workgroup (K is dealt out in 128-row chunks)
   int partial_rows;  // rows of one split's slice of `partials` (M; grouped launches: all pairs)
   MoeView moe;       // grouped launches only (MOE kernels): blockIdx.z is the expert
 };
@@ -114,7 +115,8 @@ __device__ __forceinline__ float4_t mfma16(const uint4_t a, const half2_t b[4], 
 struct Decomp {
   int tid, lane, wave, wc, wkk, j, kq, nthreads;
   int tile_cols, ntiles, tile, split;
-  int KR, KW, kwg0, kw0;
+  int KR, KW, kwg0, kw0;  // K range of the workgroup [kwg0, kwg0 + KR) and of the wave [kw0, kw0 + KW)
+  int kwo;                // kw0 - kwg0: the wave's offset inside the workgroup's slab
   int mb, mloc;  // first activation row of this workgroup and number of live rows (<= 16)
 };
 
@@ -132,10 +134,18 @@ __device__ __forceinline__ Decomp make_decomp(const GemvParams& gp, int wave_col
   d.ntiles = gp.p.N / d.tile_cols;
   d.tile = blockIdx.x % d.ntiles;
   d.split = blockIdx.x / d.ntiles;
-  d.KR = gp.p.K / gp.splits;
-  d.KW = d.KR / gp.wk;
-  d.kwg0 = d.split * d.KR;
-  d.kw0 = d.kwg0 + d.wkk * d.KW;
+  // K is dealt out in chunks of 128 rows over splits x wk wave slots, as evenly as the chunk
+  // count allows (ranges differ by at most one chunk when it is not a multiple of the slots)
+  const long chunks = gp.p.K / kChunkRows;
+  const long slots = (long)gp.splits * gp.wk;
+  const long slot0 = (long)d.split * gp.wk;
+  const int g0 = (int)(slot0 * chunks / slots), g1 = (int)((slot0 + gp.wk) * chunks / slots);
+  const int c0 = (int)((slot0 + d.wkk) * chunks / slots), c1 = (int)((slot0 + d.wkk + 1) * chunks / slots);
+  d.kwg0 = g0 * kChunkRows;
+  d.KR = (g1 - g0) * kChunkRows;
+  d.kw0 = c0 * kChunkRows;
+  d.KW = (c1 - c0) * kChunkRows;
+  d.kwo = d.kw0 - d.kwg0;
   d.mb = blockIdx.y * kRowsPerBlock;
   d.mloc = min(kRowsPerBlock, gp.p.M - d.mb);
   return d;
@@ -516,7 +526,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
 
   const bool row_live = d.j < d.mloc;  // A-operand row of this lane
   const unsigned char* a_base =
-      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.wkk * d.KW + d.kq * 8) * 2;
+      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.kwo + d.kq * 8) * 2;
 
   const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   float4_t tot[WORDS], acc[WORDS];
@@ -638,7 +648,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
     gidx_s[i] = (uint16_t)g;
   }
   // ---- scale / zero table of the workgroup's columns, all groups
-  uint32_t* table = (uint32_t*)(smem + gp.slab_bytes + ((d.KR * 2 + 15) & ~15));
+  uint32_t* table = (uint32_t*)(smem + gp.slab_bytes + ((gp.kr_max * 2 + 15) & ~15));
   const int tc = d.tile_cols;
   {
     const int nbase = d.tile * tc;
@@ -665,8 +675,8 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
 
   const bool row_live = d.j < d.mloc;
   const unsigned char* a_base =
-      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.wkk * d.KW + d.kq * 8) * 2;
-  const uint16_t* g_base = gidx_s + d.wkk * d.KW + d.kq * 8;
+      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.kwo + d.kq * 8) * 2;
+  const uint16_t* g_base = gidx_s + d.kwo + d.kq * 8;
   const uint32_t* t_lane = table + d.wc * 64 + 4 * d.j;
 
   const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -766,7 +776,7 @@ __global__ __launch_bounds__(512) void gemv_awq_kernel(GemvParams gp) {
 
   const bool row_live = d.j < d.mloc;
   const unsigned char* a_base =
-      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.wkk * d.KW + d.kq * 8) * 2;
+      smem + (size_t)d.j * gp.slab_stride + (size_t)(d.kwo + d.kq * 8) * 2;
 
   const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   float4_t acc[16];

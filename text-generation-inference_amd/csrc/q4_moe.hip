@@ -189,7 +189,7 @@ int validate_moe_weight(const q4_moe_weight* w, const char* who) {
 struct MoeGemvPlan {
   bool ok;
   GemvConfig cfg;
-  int ntiles, mchunks, rows;
+  int ntiles, mchunks, rows, kr_max;
   size_t slab_bytes, smem;
 };
 
@@ -218,32 +218,39 @@ MoeGemvPlan moe_gemv_plan(const q4_moe_weight* w, int tokens, int topk, int dtyp
   cfg.words = 4;
   const int wave_cols = awq ? 256 : 64;
   if (e0->N % (wave_cols * cfg.wcol) != 0) cfg.wcol = 1;
-  if (e0->N % wave_cols != 0 || cfg.wcol * cfg.wk > 8 || e0->K % (cfg.wk * 128) != 0) return pl;
+  const int kchunks = e0->K / 128;
+  if (e0->N % wave_cols != 0 || cfg.wcol * cfg.wk > 8 || cfg.wk > kchunks) return pl;
   long active = (long)tokens * topk;
   if (active > w->num_experts) active = w->num_experts;
+  const int max_splits = kchunks / cfg.wk;
   int splits = (int)(cfg.splits / active);
   if (splits < 1) splits = 1;
-  while (splits > 1 && e0->K % (splits * cfg.wk * 128) != 0) --splits;
+  // prefer a count that deals the 128-row chunks out evenly
+  while (splits > 1 && kchunks % (splits * cfg.wk) != 0) --splits;
   const int ntiles = e0->N / (wave_cols * cfg.wcol);
   const bool tickets_fit = (long)ntiles * mchunks * w->num_experts <= Q4_WORKSPACE_TICKET_BYTES / 4;
   if (!tickets_fit) splits = 1;
-  // LDS: the activation slab of `rows` x K / splits, for act-order also the g_idx slice and
-  // the parameter table; the wk waves' partial sums reuse it.  Split further if it does not fit.
+  // LDS: the activation slab of `rows` x (largest K range of a workgroup), for act-order also
+  // the g_idx slice and the parameter table; the wk waves' partial sums reuse it.  Split
+  // further if it does not fit.
   const size_t smem_limit = 160 * 1024 - 1024;
   const int nt = awq ? 16 : 4;
-  auto slab_of = [&](int sp) { return ((size_t)rows * ((size_t)e0->K / sp * 2 + 16) + 15) & ~(size_t)15; };
+  auto kr_of = [&](int sp) {
+    const long slots = (long)sp * cfg.wk;
+    return (size_t)((kchunks * cfg.wk + slots - 1) / slots) * 128;  // upper bound of a workgroup's range
+  };
+  auto slab_of = [&](int sp) { return ((size_t)rows * (kr_of(sp) * 2 + 16) + 15) & ~(size_t)15; };
   auto smem_of = [&](int sp) {
     size_t bytes = slab_of(sp);
-    if (act) bytes += (((size_t)e0->K / sp * 2 + 15) & ~(size_t)15) + (size_t)e0->num_groups * 64 * cfg.wcol * 4;
+    if (act) bytes += ((kr_of(sp) * 2 + 15) & ~(size_t)15) + (size_t)e0->num_groups * 64 * cfg.wcol * 4;
     const size_t red = (size_t)(cfg.wk - 1) * cfg.wcol * nt * 4 * 64 * sizeof(float);
     return bytes > red ? bytes : red;
   };
   while (smem_of(splits) > smem_limit) {
-    int next = splits + 1;
-    while (next <= e0->K / (cfg.wk * 128) && e0->K % (next * cfg.wk * 128) != 0) ++next;
-    if (next > e0->K / (cfg.wk * 128) || !tickets_fit) return pl;
-    splits = next;
+    if (splits >= max_splits || !tickets_fit) return pl;
+    ++splits;
   }
+  pl.kr_max = (int)kr_of(splits);
   cfg.splits = splits;
   pl.ok = true;
   pl.cfg = cfg;
@@ -361,7 +368,8 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
     gp.splits = cfg.splits;
     gp.cells = nullptr;
     gp.fixed_point_split = 0;
-    gp.slab_stride = e0->K / cfg.splits * 2 + 16;
+    gp.slab_stride = pl.kr_max * 2 + 16;
+    gp.kr_max = pl.kr_max;
     gp.slab_bytes = (int)pl.slab_bytes;
     gp.partial_rows = pairs;
     gp.moe = mv;
