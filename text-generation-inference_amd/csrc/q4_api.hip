@@ -87,13 +87,13 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   if (contiguous_gptq) {
     // Measured crossover on MI355X.  The decode kernel works in blocks of 16 rows that run side
     // by side (a second block costs little: the weights are shared through L2), the split-K
-    // GEMM is nearly flat in M up to a few hundred rows.  Decode / GEMM in us at M = 32:
-    // 4096 x 4096 11.6 / 17.3, 4096 x 6144 12.7 / 18.8, 4096 x 14336 17.6 / 27.5, 4096 x 28672
-    // 34.5 / 40.7, 8192 x 8192 22.1 / 28.5, but 8192 x 10240 38.4 / 32.6, 5120 x 13824 32.9 / 28.9,
-    // 14336 x 4096 30.5 / 26.0 (at M = 17: 25.7 / 25.3).  From the third block on (M = 48) the
-    // GEMM wins except on the smallest matrices (4096 x 4096: 12.6 / 19.2 at M = 64, 24.4 / 20.8
+    // GEMM (64-row tiles up to M = 64) is nearly flat in M.  Decode / GEMM in us at M = 32:
+    // 4096 x 4096 11.6 / 15.8, 4096 x 6144 12.7 / 17.3, 4096 x 14336 17.6 / 21.1, 8192 x 8192
+    // 22.1 / 23.4, but 4096 x 28672 34.5 / 30.6, 8192 x 10240 38.4 / 32.6, 5120 x 13824 32.9 / 28.9,
+    // 14336 x 4096 30.5 / 23.5 (at M = 17: 25.7 / 22.9).  From the third block on (M = 48) the
+    // GEMM wins except on the smallest matrices (4096 x 4096: 12.6 / 17.9 at M = 64, 24.4 / 20.8
     // at M = 96; 2048 x 8192: 10.8 / 15.2 at M = 64).
-    const bool small = M <= 16 || (M <= 32 && (w->K <= 4096 || (w->K <= 8192 && weights <= (1L << 26)))) ||
+    const bool small = M <= 16 || (M <= 32 && w->K <= 8192 && weights <= (1L << 26)) ||
                        (M <= 64 && weights <= (1L << 24));
     if (small && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
     if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;

@@ -116,12 +116,12 @@ __device__ __forceinline__ float16_t mfma32(const uint4_t a, const uint4_t b, fl
   }
 }
 
-// BM: rows per workgroup (128 or 256).  GPT: quantisation groups per K tile (1 or 2).
+// BM: rows per workgroup (64, 128 or 256).  GPT: quantisation groups per K tile (1 or 2).
 // NW: packed words (columns) per lane and K step: 2 -> 256-column workgroup tile, 1 -> 128.
 // MOE: grouped launch, blockIdx.y is the expert; its row count is read from device memory, so
 // the grid covers the largest possible count and surplus workgroups leave at once.
 template <int DTYPE, int BM, int GPT, int NW, bool MOE = false>
-__global__ __launch_bounds__(256, (BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm_gptq_kernel(GemmParams gp) {
+__global__ __launch_bounds__(256, (BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm_gptq_kernel(GemmParams gp) {
   int moe_row0 = 0;
   if constexpr (MOE) {
     moe_row0 = moe_enter(gp.p, gp.moe, blockIdx.y);
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm
   const uint16_t* xs = (const uint16_t*)p.x;
   // Register staging sets: with two sets (128-row tiles) a tile's loads are issued two
   // tiles before they are written to LDS; the 256-row tile has registers for one set only.
-  constexpr int ASETS = BM == 128 ? 2 : 1;
+  constexpr int ASETS = BM <= 128 ? 2 : 1;
   uint4_t areg[ASETS][A_LOADS];
   int moe_xrow[MOE ? A_LOADS : 1];  // grouped launch with a row map: x row of each staged row
   if constexpr (MOE) {
