@@ -289,11 +289,18 @@ void launch_moe_gemv_dtype(const q4_weight* e0, dim3 grid, dim3 block, size_t sm
   else launch_with_smem(gemv_gptq_kernel<DTYPE, 4, 1, false, 4, false, true>, grid, block, smem, stream, gp);
 }
 
-template <int DTYPE, int NW>
+template <int DTYPE, int BM, int NW>
 void launch_moe_gemm_tile(int gs, dim3 grid, size_t smem, hipStream_t stream, const GemmParams& gp) {
   using namespace q4;
-  if (gs == 32) hipLaunchKernelGGL((gemm_gptq_kernel<DTYPE, 128, 2, NW, true>), grid, dim3(256), smem, stream, gp);
-  else hipLaunchKernelGGL((gemm_gptq_kernel<DTYPE, 128, 1, NW, true>), grid, dim3(256), smem, stream, gp);
+  if (gs == 32) hipLaunchKernelGGL((gemm_gptq_kernel<DTYPE, BM, 2, NW, true>), grid, dim3(256), smem, stream, gp);
+  else hipLaunchKernelGGL((gemm_gptq_kernel<DTYPE, BM, 1, NW, true>), grid, dim3(256), smem, stream, gp);
+}
+
+// Row tile of the grouped MFMA launch: 64 rows while the experts receive at most 64 rows on
+// average (three workgroups per CU keep more weight loads in flight), else 128.
+int moe_gemm_bm(const q4_moe_weight* w, int tokens, int topk) {
+  const long avg_rows = ((long)tokens * topk + w->num_experts - 1) / w->num_experts;
+  return avg_rows <= 64 && w->expert0.N % 256 == 0 ? 64 : 128;
 }
 
 // Split-K factor of the grouped MFMA launch.  The host does not know the experts' row counts:
@@ -305,7 +312,8 @@ int moe_gemm_splits(const q4_moe_weight* w, int tokens, int topk) {
   const long pairs = (long)tokens * topk;
   const long avg_rows = (pairs + w->num_experts - 1) / w->num_experts;
   const int nw = e0->N % 256 == 0 ? 2 : 1;
-  const long tiles = (long)w->num_experts * ((avg_rows + 127) / 128) * (e0->N / (128 * nw));
+  const int bm = moe_gemm_bm(w, tokens, topk);
+  const long tiles = (long)w->num_experts * ((avg_rows + bm - 1) / bm) * (e0->N / (128 * nw));
   if (tiles >= 256 || pairs > 0x7fffffffL) return 1;
   return gemm_pick_splits(tiles, e0->K / q4::kBK, (int)pairs, e0->N, 0.9, 1.3);
 }
@@ -392,19 +400,22 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
     gp.moe = mv;
     // an expert can receive every token: the grid covers `tokens` rows per expert
     const int nw = e0->N % 256 == 0 ? 2 : 1;
-    const long tiles = (long)((tokens + 127) / 128) * (e0->N / (128 * nw)) * splits;
+    const int bm = moe_gemm_bm(w, tokens, topk);
+    const long tiles = (long)((tokens + bm - 1) / bm) * (e0->N / (128 * nw)) * splits;
     if (tiles > 0x7fffffffL || w->num_experts > 65535) {
       set_error("q4_moe_linear: grid too large");
       return Q4_ERR_UNSUPPORTED;
     }
     const dim3 grid((unsigned)tiles, (unsigned)w->num_experts);
-    const size_t smem = 2 * (size_t)128 * kAUnitsPerRow * 16;
+    const size_t smem = 2 * (size_t)bm * kAUnitsPerRow * 16;
     if (dtype == Q4_DTYPE_F16) {
-      if (nw == 2) launch_moe_gemm_tile<Q4_DTYPE_F16, 2>(e0->groupsize, grid, smem, stream, gp);
-      else launch_moe_gemm_tile<Q4_DTYPE_F16, 1>(e0->groupsize, grid, smem, stream, gp);
+      if (bm == 64) launch_moe_gemm_tile<Q4_DTYPE_F16, 64, 2>(e0->groupsize, grid, smem, stream, gp);
+      else if (nw == 2) launch_moe_gemm_tile<Q4_DTYPE_F16, 128, 2>(e0->groupsize, grid, smem, stream, gp);
+      else launch_moe_gemm_tile<Q4_DTYPE_F16, 128, 1>(e0->groupsize, grid, smem, stream, gp);
     } else {
-      if (nw == 2) launch_moe_gemm_tile<Q4_DTYPE_BF16, 2>(e0->groupsize, grid, smem, stream, gp);
-      else launch_moe_gemm_tile<Q4_DTYPE_BF16, 1>(e0->groupsize, grid, smem, stream, gp);
+      if (bm == 64) launch_moe_gemm_tile<Q4_DTYPE_BF16, 64, 2>(e0->groupsize, grid, smem, stream, gp);
+      else if (nw == 2) launch_moe_gemm_tile<Q4_DTYPE_BF16, 128, 2>(e0->groupsize, grid, smem, stream, gp);
+      else launch_moe_gemm_tile<Q4_DTYPE_BF16, 128, 1>(e0->groupsize, grid, smem, stream, gp);
     }
     if (splits > 1) launch_gemm_reduce(gp.partials, nullptr, y, pairs, e0->N, splits, dtype, stream);
   } else if (gemm_awq_supported(e0, tokens, dtype)) {
