@@ -84,6 +84,55 @@ def test_argument_validation_without_gpu(pkg):
     assert lib.q4_linear(ctypes.byref(w), None, None, None, 0, 0, None, 0, None) == 0
 
 
+def test_moe_argument_validation_without_gpu(pkg):
+    """The grouped entry points reject bad arguments before anything is launched."""
+    import ctypes
+
+    lib = pkg._lib.load()
+    L = pkg._lib
+
+    def moe(K, N, gs, experts=8, layout=0, g_idx=False, strides=None):
+        e0 = _weight(pkg, K, N, gs, layout, g_idx)
+        G = max(1, K // gs)
+        st = strides or ((K // 8) * N, G * (N // 8), G * N, K)
+        return L.Q4MoeWeight(e0, experts, *st)
+
+    assert int(L.DTYPE_F32) == 2
+    # routing: experts and topk limits, null outputs
+    assert lib.q4_moe_route(0x10, 2, 4, 300, 2, 1, 0x20, 0x30, 0x40, 0x50, 0x60, None) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_moe_route(0x10, 2, 4, 8, 9, 1, 0x20, 0x30, 0x40, 0x50, 0x60, None) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_moe_route(0x10, 2, 4, 8, 2, 1, None, 0x30, 0x40, 0x50, 0x60, None) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_moe_route(0x10, 7, 4, 8, 2, 1, 0x20, 0x30, 0x40, 0x50, 0x60, None) == L.ERR_INVALID_ARGUMENT
+    assert b"gating dtype" in lib.q4_last_error()
+    # grouped linear: null weight, bad geometry, strides smaller than an expert, AWQ with g_idx
+    assert lib.q4_moe_linear(None, 0x10, None, 0x20, 0x30, 4, 2, 0, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    w = moe(4096, 4100, 128)
+    assert lib.q4_moe_linear(ctypes.byref(w), 0x10, None, 0x20, 0x30, 4, 2, 0, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    w = moe(4096, 4096, 128, strides=(100, 100, 100, 100))
+    assert lib.q4_moe_linear(ctypes.byref(w), 0x10, None, 0x20, 0x30, 4, 2, 0, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    assert b"strides" in lib.q4_last_error()
+    w = moe(4096, 4096, 128, layout=1, g_idx=True)
+    assert lib.q4_moe_linear(ctypes.byref(w), 0x10, None, 0x20, 0x30, 4, 2, 0, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    w = moe(4096, 4096, 128, experts=0)
+    assert lib.q4_moe_linear(ctypes.byref(w), 0x10, None, 0x20, 0x30, 4, 2, 0, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    w = moe(4096, 4096, 128)
+    assert lib.q4_moe_linear(ctypes.byref(w), 0x10, None, 0x20, 0x30, 4, 2, 5, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_moe_linear(ctypes.byref(w), None, None, 0x20, 0x30, 4, 2, 0, None, 0, None) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_moe_linear(ctypes.byref(w), None, None, None, None, 0, 2, 0, None, 0, None) == 0  # no tokens
+    # a shape no grouped kernel takes (K not a multiple of 64)
+    w = moe(4104, 4096, 8)
+    assert lib.q4_moe_linear(ctypes.byref(w), 0x10, None, 0x20, 0x30, 4, 2, 0, None, 0, None) == L.ERR_UNSUPPORTED
+    # weighted sum
+    assert lib.q4_moe_combine(0x10, 0x20, 0x30, 0x40, 4, 2, 4100, 0, None) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_moe_combine(0x10, 0x20, 0x30, None, 4, 2, 4096, 0, None) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_moe_combine(None, None, None, None, 0, 2, 4096, 0, None) == 0
+    # workspace: at least the counters; more when the decode plan splits K over workgroups
+    w = moe(4096, 4096, 128)
+    assert lib.q4_moe_workspace_bytes(ctypes.byref(w), 1, 2) >= L.WORKSPACE_COUNTER_BYTES
+    assert lib.q4_moe_workspace_bytes(ctypes.byref(w), 1024, 2) >= L.WORKSPACE_COUNTER_BYTES
+    assert lib.q4_moe_workspace_bytes(None, 1, 2) == 0
+
+
 def test_path_selection_and_workspace(pkg):
     lib = pkg._lib.load()
     L = pkg._lib
