@@ -114,6 +114,25 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   int min_splits = lds_budget > 0 ? (int)(((long)w->K * per_row + lds_budget - 1) / lds_budget) : max_splits;
   if (min_splits < 1) min_splits = 1;
   if (min_splits > max_splits) min_splits = max_splits;
+  // Act-order with many rows: the kernel does per-weight table lookups and needs two
+  // workgroups per CU to hide them, so slab + g_idx slice + table are held to half the LDS
+  // where an even split allows it (8192 x 10240 at M = 16: 27.9 us with eight splits against
+  // 42.9 us with four; 14336 x 4096: 29.6 us with fourteen against 33.5 us with seven).
+  bool even_only = false;
+  if (act && M >= 12) {
+    const long half_lds = 80896 - (long)w->num_groups * 64 * 4 - 16L * rows;
+    if (half_lds > 0) {
+      // sized for a full block of 16 rows: 12 rows measured better with the same split
+      const int need = (int)(((long)w->K * (q4::kRowsPerBlock * 2 + 2) + half_lds - 1) / half_lds);
+      for (int dv = need > min_splits ? need : min_splits; dv <= max_splits; ++dv) {
+        if (chunks % (dv * c.wk) == 0) {
+          min_splits = dv;
+          even_only = true;
+          break;
+        }
+      }
+    }
+  }
   // K is dealt out in 128-row chunks over splits x wk wave slots.  A count that divides the
   // chunks evenly is preferred; when none is near the wanted one (K = 11008: 86 chunks) the
   // slots differ by one chunk and the cost carries the imbalance.
@@ -126,7 +145,10 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
     // nine take 19.4 us, three 24 us)
     double cost = dv > want ? (double)dv / want : 1.5 * want / dv;
     cost *= balance;
-    if (chunks % slots != 0) cost *= 1.25;
+    if (chunks % slots != 0) {
+      if (even_only) continue;
+      cost *= 1.25;
+    }
     if (best_cost < 0.0 || cost < best_cost) {
       best_cost = cost;
       best = dv;

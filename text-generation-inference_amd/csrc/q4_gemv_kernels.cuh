@@ -703,9 +703,10 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
         // rows pr and pr + 4 of the K block share one splice (nibbles 16 bits apart)
+        // one byte permute each: the low halves (scales) and the high halves (-(1024 + z))
         const uint32_t ea = e[pr][t], eb = e[pr + 4][t];
-        const uint32_t s2 = (ea & 0xFFFFu) | (eb << 16);
-        const uint32_t c2 = (ea >> 16) | (eb & 0xFFFF0000u);
+        const uint32_t s2 = __builtin_amdgcn_perm(eb, ea, 0x05040100u);
+        const uint32_t c2 = __builtin_amdgcn_perm(eb, ea, 0x07060302u);
         const uint32_t q2 = ((words[t] >> (4 * pr)) & splice.mask_lo) | splice.magic;
         const half2_t dq = as_half2(q2) + as_half2(c2);  // exact q - z
         b[pr] = dq * as_half2(s2);                       // one fp16 rounding, as the reference
