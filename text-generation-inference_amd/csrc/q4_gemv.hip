@@ -75,6 +75,11 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   // (M = 16: 4096 x 6144 12.1 against 14.9 us, 14336 x 4096 18.8 against 22.4 us)
   const bool contiguous = w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr;
   if (contiguous && !gate_up && M >= 12 && c.wcol == 1 && (chunks % 8 == 0 || chunks >= 32)) c.wk = 8;
+  // AWQ from 4 rows on, long enough K: eight waves along K share one activation slab
+  // (4096 x 14336 at M = 8: 25.3 against 28.2 us; 14336 x 4096 at M = 4: 23.6 against 28.4 us;
+  // 4096 x 4096 keeps four waves and eight splits: 15.4 against 18.2 us)
+  const bool awq8 = w->layout == Q4_LAYOUT_AWQ && M >= 4 && chunks % 8 == 0 && (long)chunks * w->N >= 32L * 8192;
+  if (awq8) c.wk = 8;
   if (gate_up) {
     // a wave owns 64 gate and 64 up columns (twice the bytes of a plain wave): eight waves
     // along K keep the wave count, and with it the bytes in flight, of the plain kernel
@@ -93,7 +98,7 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   if (gate_up) target_wgs = 256;        // 512-thread workgroups: one per CU
   // the targets count four-wave workgroups: one with two column tiles (eight waves) counts twice
   // (4096 x 14336 at M = 16, two tiles per workgroup: 16.6 us with two splits, 18.9 us with four)
-  const int tile_units = ntiles * (gate_up ? 1 : c.wcol) * (contiguous && !gate_up && c.wk == 8 ? 2 : 1);
+  const int tile_units = ntiles * (gate_up ? 1 : c.wcol) * (((contiguous && !gate_up) || awq8) && c.wk == 8 ? 2 : 1);
   int want = (target_wgs + tile_units / 2) / tile_units;
   // tiles that fill the chip on their own are not split (4096 x 28672: 18.5 us with two
   // splits against 16.7 us with one)
