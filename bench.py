@@ -321,6 +321,13 @@ def main():
                         "frac_of_mfma_peak": round(fl / avg / 1e12 / MFMA_PEAK_TFLOPS, 4)}
             tot_f += fl
             tot_t += avg
+            # the same kernel on bf16 activations (bf16 weights rounded once from the fp32 product)
+            xb = torch.randn((Mg, K), device=dev, dtype=torch.bfloat16)
+            yb = torch.empty((Mg, N), device=dev, dtype=torch.bfloat16)
+            bfns = [(lambda c=c, i=i: pkg.ops.linear(weights[c][i], xb, None, out=yb)) for c in range(copies)]
+            bavg, _ = time_kernel_launches(torch, bfns, 20)
+            gm[name]["bf16_TFLOPs"] = round(fl / bavg / 1e12, 1)
+            del xb, yb
             if not args.no_dense_ref:
                 # context, not the product: the vendor library's dense fp16 GEMM on the same
                 # shape and box (weights already dequantized, 4x the weight bytes), timed the same way

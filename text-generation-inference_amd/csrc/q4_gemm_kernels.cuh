@@ -46,6 +46,8 @@ struct GemmParams {
 };
 
 typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef float gemm_float2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 gemm_bf16x2_t __attribute__((ext_vector_type(2)));
 
 struct SpliceK {
   uint32_t mask_lo, mask_hi, magic;
@@ -92,13 +94,12 @@ __device__ __forceinline__ uint4_t dequant_word(uint32_t w, const ColConsts& c, 
     out.z = as_u32(d[2] * c.s2);
     out.w = as_u32(d[3] * c.s2);
   } else {
-    // bf16: exact fp32 product, rounded once
+    // bf16: exact fp32 product, rounded once to nearest even by the packed convert
     uint32_t o[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float lo = (float)d[i].x * c.sf;
-      const float hi = (float)d[i].y * c.sf;
-      o[i] = (uint32_t)f32_to_bf16_rne(lo) | ((uint32_t)f32_to_bf16_rne(hi) << 16);
+      const gemm_float2_t f = {(float)d[i].x * c.sf, (float)d[i].y * c.sf};
+      o[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, gemm_bf16x2_t));
     }
     out.x = o[0]; out.y = o[1]; out.z = o[2]; out.w = o[3];
   }
