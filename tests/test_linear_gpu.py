@@ -392,6 +392,20 @@ def test_gemv_ragged_k_explicit_decompositions(pkg, oracle, gpu, cfg):
     _run(pkg, oracle, gpu, 43 * 128, 256, 64, 2, sym=False, cfg=cfg, seed=sum(cfg) + 1)
 
 
+@pytest.mark.parametrize("layout,act", [("gptq", False), ("gptq", True), ("awq", False)])
+def test_decode_picker_sweep(pkg, oracle, gpu, layout, act):
+    """Whatever decomposition the picker chooses must be launchable and right: chunk counts
+    with awkward divisors, narrow and wide N, every row count of a block and beyond."""
+    rng = np.random.default_rng(7)
+    cases = []
+    for chunks in (1, 2, 3, 5, 7, 9, 11, 13, 24, 43):
+        for N in ((256, 512) if layout == "awq" else (64, 192, 512)):
+            cases.append((chunks * 128, N, int(rng.integers(1, 21))))
+    cases += [(86 * 128, 1024, 16), (40 * 128, 2048, 12), (108 * 128, 768 if layout != "awq" else 1024, 5)]
+    for K, N, M in cases:
+        _run(pkg, oracle, gpu, K, N, 128, M, layout=layout, act=act, sym=False, path=1, seed=K // 128 + N + M)
+
+
 def test_gemv_llama2_7b_down_shape(pkg, oracle, gpu):
     _run(pkg, oracle, gpu, 11008, 4096, 128, 1, path=1, seed=11)
     _run(pkg, oracle, gpu, 11008, 4096, 128, 16, path=1, seed=12)
