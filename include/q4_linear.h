@@ -176,6 +176,14 @@ int q4_moe_route(const void* gating, int gating_dtype, int tokens, int experts, 
                  float* topk_weights, int32_t* topk_ids, int32_t* sorted_tokens, int32_t* pair_slot,
                  int32_t* expert_offsets, void* stream);
 
+/* Grouped top-k (the in-tree definition: server/text_generation_server/layers/moe/
+ * fused_moe_ipex.py:21-50): the experts form num_expert_group equal groups, a token keeps the
+ * topk_group groups whose best expert scores highest and chooses its topk experts among those.
+ * num_expert_group = 0: plain top-k.  At most 32 groups. */
+int q4_moe_route_grouped(const void* gating, int gating_dtype, int tokens, int experts, int topk, int renormalize,
+                         int num_expert_group, int topk_group, float* topk_weights, int32_t* topk_ids,
+                         int32_t* sorted_tokens, int32_t* pair_slot, int32_t* expert_offsets, void* stream);
+
 /* y[r, :] = x[x_rows ? x_rows[r] : r, :] @ W_e for every sorted row r of every expert e.
  * y is [tokens*topk, N] in sorted order.  Up to 16 tokens (64 when K <= 8192) the decode
  * kernel runs once per expert and 16 rows it received; above, the MFMA kernel.  Workspace as for q4_linear, sized by

@@ -29,6 +29,9 @@ Pinning status (what proves each function right, other than itself):
   moe_fused_topk
         pinned: scipy.special.softmax + argsort brute force, hand-computed two-expert case,
         weights sum to 1 after renormalisation; follows the in-tree pure-PyTorch routine.
+  moe_grouped_topk
+        pinned: brute force from the definition (group maxima, kept groups, masked top-k) and
+        the special cases one group (== moe_fused_topk) and all groups kept (== moe_fused_topk).
   moe_forward
         structure pinned by the in-tree dense formulation it follows (every expert applied
         to every token, weighted by the scattered top-k weights) through its already pinned
@@ -310,6 +313,26 @@ def moe_fused_topk(gating: np.ndarray, topk: int, renormalize: bool):
     prob = (e / e.sum(axis=1, keepdims=True, dtype=np.float32)).astype(np.float32)
     ids = np.argsort(-prob, axis=1, kind="stable")[:, :topk]
     w = np.take_along_axis(prob, ids, axis=1)
+    if renormalize:
+        w = w / w.sum(axis=1, keepdims=True, dtype=np.float32)
+    return w.astype(np.float32), ids.astype(np.int32)
+
+
+def moe_grouped_topk(gating: np.ndarray, topk: int, renormalize: bool, num_expert_group: int, topk_group: int):
+    """Grouped routing (layers/moe/fused_moe_ipex.py:21-50): softmax over all experts, the
+    score of a group is its largest member, the `topk_group` best groups stay, every expert
+    outside them is masked to 0, then top-k and the optional renormalisation as above."""
+    g = np.asarray(gating).astype(np.float32)
+    T, E = g.shape
+    e = np.exp(g - g.max(axis=1, keepdims=True), dtype=np.float32)
+    prob = (e / e.sum(axis=1, keepdims=True, dtype=np.float32)).astype(np.float32)
+    group_scores = prob.reshape(T, num_expert_group, -1).max(axis=2)
+    keep = np.argsort(-group_scores, axis=1, kind="stable")[:, :topk_group]
+    mask = np.zeros((T, num_expert_group), dtype=bool)
+    np.put_along_axis(mask, keep, True, axis=1)
+    masked = np.where(np.repeat(mask, E // num_expert_group, axis=1), prob, np.float32(0.0))
+    ids = np.argsort(-masked, axis=1, kind="stable")[:, :topk]
+    w = np.take_along_axis(masked, ids, axis=1)
     if renormalize:
         w = w / w.sum(axis=1, keepdims=True, dtype=np.float32)
     return w.astype(np.float32), ids.astype(np.int32)

@@ -34,6 +34,30 @@ def test_fused_topk_hand_case_and_ties(oracle):
     assert ids.tolist() == [[0, 1]] and np.allclose(w, [[0.5, 0.5]])
 
 
+def test_grouped_topk_brute_force_and_special_cases(oracle):
+    rng = np.random.default_rng(4)
+    for T, E, groups, keep, k in [(9, 16, 4, 2, 3), (5, 160, 8, 3, 6), (3, 8, 8, 4, 2), (4, 12, 3, 1, 4)]:
+        g = (rng.standard_normal((T, E)) * 2).astype(np.float32)
+        for renorm in (False, True):
+            w, ids = oracle.moe_grouped_topk(g, k, renorm, groups, keep)
+            p = softmax(g.astype(np.float64), axis=1)
+            per = E // groups
+            for t in range(T):
+                gmax = [p[t, a * per:(a + 1) * per].max() for a in range(groups)]
+                kept = sorted(range(groups), key=lambda a: (-gmax[a], a))[:keep]
+                cand = [e for e in range(E) if e // per in kept]
+                order = sorted(cand, key=lambda e: (-p[t, e], e))[:k]
+                assert ids[t].tolist() == order
+                want = p[t, order] / (p[t, order].sum() if renorm else 1.0)
+                assert np.allclose(w[t], want, rtol=2e-6, atol=1e-9)
+    # one group, or every group kept: plain top-k
+    g = rng.standard_normal((6, 12)).astype(np.float32)
+    for groups, keep in ((1, 1), (4, 4)):
+        w, ids = oracle.moe_grouped_topk(g, 3, True, groups, keep)
+        w0, ids0 = oracle.moe_fused_topk(g, 3, True)
+        assert np.array_equal(ids, ids0) and np.allclose(w, w0)
+
+
 def test_moe_forward_equals_the_dense_sum_over_all_experts(oracle):
     """Applying every expert to every token with zero weight for the ones not chosen (the
     reference's dense formulation) gives the same block output."""

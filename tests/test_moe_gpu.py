@@ -57,6 +57,26 @@ def test_route(pkg, oracle, gpu, T, E, k, dtype):
         _check_routing_structure(r, T, E, k)
 
 
+@pytest.mark.parametrize("T,E,groups,keep,k", [(1, 16, 4, 2, 3), (33, 160, 8, 3, 6), (300, 64, 8, 4, 8), (7, 8, 8, 2, 2),
+                                              (5, 12, 3, 1, 4), (4, 64, 32, 5, 5)])
+def test_route_grouped(pkg, oracle, gpu, T, E, groups, keep, k):
+    rng = np.random.default_rng(T + E)
+    g, g32 = _gating(rng, T, E, "f32")
+    for renorm in (True, False):
+        r = pkg.ops.moe_route(g.to(gpu), k, renorm, groups, keep)
+        w, ids = oracle.moe_grouped_topk(g32, k, renorm, groups, keep)
+        assert np.array_equal(r.topk_ids.cpu().numpy(), ids)
+        assert np.allclose(r.topk_weights.cpu().numpy(), w, rtol=1e-5, atol=1e-7)
+        _check_routing_structure(r, T, E, k)
+
+
+def test_route_grouped_rejects_bad_groups(pkg, gpu):
+    z = torch.zeros((2, 16), device=gpu)
+    for groups, keep, k in ((3, 1, 2), (4, 5, 2), (4, 1, 5), (64, 2, 2)):
+        with pytest.raises(pkg._lib.Q4Error):
+            pkg.ops.moe_route(z, k, True, groups, keep)
+
+
 def test_route_ties_take_the_lowest_expert(pkg, gpu):
     r = pkg.ops.moe_route(torch.zeros((2, 8), device=gpu), 2, True)
     assert r.topk_ids.cpu().tolist() == [[0, 1], [0, 1]]

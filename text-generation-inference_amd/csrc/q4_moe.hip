@@ -25,9 +25,12 @@ __device__ __forceinline__ float load_logit(const void* g, size_t i) {
   else return ((const float*)g)[i];
 }
 
+// groups > 0: grouped top-k -- the experts form `groups` equal groups, a token keeps the
+// `topk_group` groups with the largest member and chooses its experts among those only.
 template <int GDT>
 __global__ __launch_bounds__(1024) void moe_route_kernel(const void* __restrict__ gating, int T, int E, int topk,
-                                                         int renormalize, float* __restrict__ topk_weights,
+                                                         int renormalize, int groups, int topk_group,
+                                                         float* __restrict__ topk_weights,
                                                          int32_t* __restrict__ topk_ids,
                                                          int32_t* __restrict__ sorted_tokens,
                                                          int32_t* __restrict__ pair_slot,
@@ -45,6 +48,26 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const void* __restrict_
     for (int e = 1; e < E; ++e) mx = fmaxf(mx, load_logit<GDT>(gating, row + e));
     float sum = 0.f;
     for (int e = 0; e < E; ++e) sum += expf(load_logit<GDT>(gating, row + e) - mx);
+    // groups a token may choose from, as a bit mask (softmax is monotonic: logits decide)
+    uint32_t allowed = 0xFFFFFFFFu;
+    const int per_group = groups > 0 ? E / groups : E;
+    if (groups > 0) {
+      allowed = 0u;
+      for (int j = 0; j < topk_group; ++j) {
+        int best = -1;
+        float bv = 0.f;
+        for (int g = 0; g < groups; ++g) {
+          if ((allowed >> g) & 1u) continue;
+          float gm = load_logit<GDT>(gating, row + (size_t)g * per_group);
+          for (int e = 1; e < per_group; ++e) gm = fmaxf(gm, load_logit<GDT>(gating, row + (size_t)g * per_group + e));
+          if (best < 0 || gm > bv) {
+            best = g;
+            bv = gm;
+          }
+        }
+        allowed |= 1u << best;
+      }
+    }
     int chosen[kMoeMaxTopk];
     float weight[kMoeMaxTopk];
     float wsum = 0.f;
@@ -52,6 +75,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const void* __restrict_
       int best = -1;
       float bv = 0.f;
       for (int e = 0; e < E; ++e) {
+        if (groups > 0 && !((allowed >> (e / per_group)) & 1u)) continue;
         bool taken = false;
         for (int i = 0; i < j; ++i) taken |= chosen[i] == e;
         if (taken) continue;
@@ -441,13 +465,20 @@ using namespace q4host;
 
 extern "C" {
 
-int q4_moe_route(const void* gating, int gating_dtype, int tokens, int experts, int topk, int renormalize,
-                 float* topk_weights, int32_t* topk_ids, int32_t* sorted_tokens, int32_t* pair_slot,
-                 int32_t* expert_offsets, void* stream) {
+int q4_moe_route_grouped(const void* gating, int gating_dtype, int tokens, int experts, int topk, int renormalize,
+                         int num_expert_group, int topk_group, float* topk_weights, int32_t* topk_ids,
+                         int32_t* sorted_tokens, int32_t* pair_slot, int32_t* expert_offsets, void* stream) {
   if (tokens < 0 || experts < 1 || experts > q4::kMoeMaxExperts || topk < 1 || topk > q4::kMoeMaxTopk ||
       topk > experts) {
     set_error("q4_moe_route: tokens=%d experts=%d (1..%d) topk=%d (1..%d, <= experts)", tokens, experts,
               q4::kMoeMaxExperts, topk, q4::kMoeMaxTopk);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (num_expert_group != 0 &&
+      (num_expert_group < 1 || num_expert_group > 32 || experts % num_expert_group != 0 || topk_group < 1 ||
+       topk_group > num_expert_group || topk > topk_group * (experts / num_expert_group))) {
+    set_error("q4_moe_route: %d groups (1..32, dividing %d experts), %d of them kept, topk=%d must fit in them",
+              num_expert_group, experts, topk_group, topk);
     return Q4_ERR_INVALID_ARGUMENT;
   }
   if (expert_offsets == nullptr ||
@@ -460,13 +491,16 @@ int q4_moe_route(const void* gating, int gating_dtype, int tokens, int experts, 
   const dim3 grid(1), block(1024);
   if (gating_dtype == Q4_DTYPE_F16)
     hipLaunchKernelGGL(q4::moe_route_kernel<Q4_DTYPE_F16>, grid, block, 0, s, gating, tokens, experts, topk,
-                       renormalize, topk_weights, topk_ids, sorted_tokens, pair_slot, expert_offsets);
+                       renormalize, num_expert_group, topk_group, topk_weights, topk_ids, sorted_tokens, pair_slot,
+                       expert_offsets);
   else if (gating_dtype == Q4_DTYPE_BF16)
     hipLaunchKernelGGL(q4::moe_route_kernel<Q4_DTYPE_BF16>, grid, block, 0, s, gating, tokens, experts, topk,
-                       renormalize, topk_weights, topk_ids, sorted_tokens, pair_slot, expert_offsets);
+                       renormalize, num_expert_group, topk_group, topk_weights, topk_ids, sorted_tokens, pair_slot,
+                       expert_offsets);
   else if (gating_dtype == Q4_DTYPE_F32)
     hipLaunchKernelGGL(q4::moe_route_kernel<Q4_DTYPE_F32>, grid, block, 0, s, gating, tokens, experts, topk,
-                       renormalize, topk_weights, topk_ids, sorted_tokens, pair_slot, expert_offsets);
+                       renormalize, num_expert_group, topk_group, topk_weights, topk_ids, sorted_tokens, pair_slot,
+                       expert_offsets);
   else {
     set_error("q4_moe_route: unknown gating dtype %d", gating_dtype);
     return Q4_ERR_INVALID_ARGUMENT;
@@ -477,6 +511,13 @@ int q4_moe_route(const void* gating, int gating_dtype, int tokens, int experts, 
     return Q4_ERR_LAUNCH;
   }
   return Q4_OK;
+}
+
+int q4_moe_route(const void* gating, int gating_dtype, int tokens, int experts, int topk, int renormalize,
+                 float* topk_weights, int32_t* topk_ids, int32_t* sorted_tokens, int32_t* pair_slot,
+                 int32_t* expert_offsets, void* stream) {
+  return q4_moe_route_grouped(gating, gating_dtype, tokens, experts, topk, renormalize, 0, 0, topk_weights, topk_ids,
+                              sorted_tokens, pair_slot, expert_offsets, stream);
 }
 
 int q4_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_rows, const int32_t* expert_offsets,

@@ -121,13 +121,13 @@ class GPTQSparseMoELayer(nn.Module):
         assert (n_expert_group is None) == (
             topk_group is None
         ), "n_expert_group and topk_group must both be None or have some value"
-        if n_expert_group is not None:
-            raise NotImplementedError("grouped top-k routing (n_expert_group / topk_group) is not implemented")
         if scoring_func not in (None, "softmax"):
             raise NotImplementedError(f"scoring func {scoring_func} is not handled")
         if e_score_correction_bias is not None:
             raise NotImplementedError("e_score_correction_bias is not implemented")
         self.n_experts = n_experts
+        self.n_expert_group = n_expert_group
+        self.topk_group = topk_group
         self.topk = topk
         self.renormalize = renormalize
         self.hidden_act = hidden_act
@@ -145,5 +145,6 @@ class GPTQSparseMoELayer(nn.Module):
         x2 = x.reshape(-1, shape[-1])
         assert x2.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
         assert gating_output.shape[1] == self.n_experts, "Number of experts mismatch"
-        out = ops.moe_forward(self._gate_up, self._down, x2, gating_output, self.topk, self.renormalize, self.hidden_act)
+        out = ops.moe_forward(self._gate_up, self._down, x2, gating_output, self.topk, self.renormalize, self.hidden_act,
+                              self.n_expert_group or 0, self.topk_group or 0)
         return out.reshape(shape)

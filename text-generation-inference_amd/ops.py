@@ -362,8 +362,10 @@ class MoeRouting:
 _GATING_DTYPES = {torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16, torch.float32: _lib.DTYPE_F32}
 
 
-def moe_route(gating_output: torch.Tensor, topk: int, renormalize: bool = True) -> MoeRouting:
-    """softmax -> top-k (-> renormalise) per token and the sort of the pairs by expert."""
+def moe_route(gating_output: torch.Tensor, topk: int, renormalize: bool = True,
+              num_expert_group: int = 0, topk_group: int = 0) -> MoeRouting:
+    """softmax -> top-k (-> renormalise) per token and the sort of the pairs by expert.
+    num_expert_group > 0: grouped top-k (experts are chosen inside the topk_group best groups)."""
     _require_cuda(gating_output, "gating_output")
     if gating_output.dim() != 2 or gating_output.dtype not in _GATING_DTYPES:
         raise ValueError("gating_output must be a [tokens, experts] float16/bfloat16/float32 tensor")
@@ -378,9 +380,9 @@ def moe_route(gating_output: torch.Tensor, topk: int, renormalize: bool = True) 
         torch.empty((E + 1,), dtype=torch.int32, device=dev),
     )
     with torch.cuda.device(dev):
-        _lib.check(_lib.load().q4_moe_route(
+        _lib.check(_lib.load().q4_moe_route_grouped(
             g.data_ptr(), _GATING_DTYPES[g.dtype], T, E, int(topk), int(bool(renormalize)),
-            r.topk_weights.data_ptr(), r.topk_ids.data_ptr(), r.sorted_tokens.data_ptr(), r.pair_slot.data_ptr(),
+            int(num_expert_group or 0), int(topk_group or 0), r.topk_weights.data_ptr(), r.topk_ids.data_ptr(), r.sorted_tokens.data_ptr(), r.pair_slot.data_ptr(),
             r.expert_offsets.data_ptr(), _stream_handle(dev),
         ))
     return r
@@ -434,9 +436,10 @@ def moe_combine(y_sorted: torch.Tensor, routing: MoeRouting) -> torch.Tensor:
 
 
 def moe_forward(gate_up: PackedMoeWeight, down: PackedMoeWeight, x: torch.Tensor, gating_output: torch.Tensor,
-                topk: int, renormalize: bool = True, act: str = "silu") -> torch.Tensor:
+                topk: int, renormalize: bool = True, act: str = "silu",
+                num_expert_group: int = 0, topk_group: int = 0) -> torch.Tensor:
     """The sparse MoE block: route, [gate | up] projection, act(gate) * up, down projection,
     weighted sum over the chosen experts."""
-    routing = moe_route(gating_output, topk, renormalize)
+    routing = moe_route(gating_output, topk, renormalize, num_expert_group, topk_group)
     h = act_mul(moe_linear(gate_up, x, routing, gather=True), act)
     return moe_combine(moe_linear(down, h, routing, gather=False), routing)
