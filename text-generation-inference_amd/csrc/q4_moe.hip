@@ -37,63 +37,76 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const void* __restrict_
                                                          int32_t* __restrict__ expert_offsets) {
   __shared__ int count[kMoeMaxExperts];
   __shared__ int cursor[kMoeMaxExperts];
+  // logits of a batch of tokens, staged with coalesced loads: a thread that walks its token's
+  // row in global memory pays a memory round trip per expert
+  constexpr int kStage = 8192;
+  __shared__ float logits[kStage];
   const int tid = threadIdx.x;
   for (int e = tid; e < E; e += blockDim.x) count[e] = 0;
   __syncthreads();
 
-  // ---- per token: softmax over the experts in fp32, the topk largest (ties: lowest index)
-  for (int t = tid; t < T; t += blockDim.x) {
-    const size_t row = (size_t)t * E;
-    float mx = load_logit<GDT>(gating, row);
-    for (int e = 1; e < E; ++e) mx = fmaxf(mx, load_logit<GDT>(gating, row + e));
-    float sum = 0.f;
-    for (int e = 0; e < E; ++e) sum += expf(load_logit<GDT>(gating, row + e) - mx);
-    // groups a token may choose from, as a bit mask (softmax is monotonic: logits decide)
-    uint32_t allowed = 0xFFFFFFFFu;
-    const int per_group = groups > 0 ? E / groups : E;
-    if (groups > 0) {
-      allowed = 0u;
-      for (int j = 0; j < topk_group; ++j) {
+  const int batch = kStage / E;  // tokens per staged batch (E <= 256)
+  for (int t0 = 0; t0 < T; t0 += batch) {
+    const int nt = min(batch, T - t0);
+    for (int i = tid; i < nt * E; i += blockDim.x) logits[i] = load_logit<GDT>(gating, (size_t)t0 * E + i);
+    __syncthreads();
+    // ---- per token: softmax over the experts in fp32, the topk largest (ties: lowest index)
+    for (int tl = tid; tl < nt; tl += blockDim.x) {
+      const int t = t0 + tl;
+      const float* lg = logits + tl * E;
+      float mx = lg[0];
+      for (int e = 1; e < E; ++e) mx = fmaxf(mx, lg[e]);
+      float sum = 0.f;
+      for (int e = 0; e < E; ++e) sum += expf(lg[e] - mx);
+      // groups a token may choose from, as a bit mask (softmax is monotonic: logits decide)
+      uint32_t allowed = 0xFFFFFFFFu;
+      const int per_group = groups > 0 ? E / groups : E;
+      if (groups > 0) {
+        allowed = 0u;
+        for (int j = 0; j < topk_group; ++j) {
+          int best = -1;
+          float bv = 0.f;
+          for (int g = 0; g < groups; ++g) {
+            if ((allowed >> g) & 1u) continue;
+            float gm = lg[g * per_group];
+            for (int e = 1; e < per_group; ++e) gm = fmaxf(gm, lg[g * per_group + e]);
+            if (best < 0 || gm > bv) {
+              best = g;
+              bv = gm;
+            }
+          }
+          allowed |= 1u << best;
+        }
+      }
+      // no per-thread arrays (they would live in scratch memory): a chosen expert is struck
+      // from the staged row, ids and weights go straight to their output
+      float* row_lg = logits + tl * E;
+      float wsum = 0.f;
+      for (int j = 0; j < topk; ++j) {
         int best = -1;
         float bv = 0.f;
-        for (int g = 0; g < groups; ++g) {
-          if ((allowed >> g) & 1u) continue;
-          float gm = load_logit<GDT>(gating, row + (size_t)g * per_group);
-          for (int e = 1; e < per_group; ++e) gm = fmaxf(gm, load_logit<GDT>(gating, row + (size_t)g * per_group + e));
-          if (best < 0 || gm > bv) {
-            best = g;
-            bv = gm;
+        for (int e = 0; e < E; ++e) {
+          if (groups > 0 && !((allowed >> (e / per_group)) & 1u)) continue;
+          const float v = row_lg[e];
+          if (v == -INFINITY) continue;  // taken (or never eligible)
+          if (best < 0 || v > bv) {
+            best = e;
+            bv = v;
           }
         }
-        allowed |= 1u << best;
+        if (best < 0) best = 0;  // every logit -inf: keep the indices in range
+        const float pw = expf(bv - mx) / sum;
+        wsum += pw;
+        topk_ids[(size_t)t * topk + j] = best;
+        topk_weights[(size_t)t * topk + j] = pw;
+        row_lg[best] = -INFINITY;
+        atomicAdd(&count[best], 1);
+      }
+      if (renormalize) {
+        for (int j = 0; j < topk; ++j) topk_weights[(size_t)t * topk + j] /= wsum;
       }
     }
-    int chosen[kMoeMaxTopk];
-    float weight[kMoeMaxTopk];
-    float wsum = 0.f;
-    for (int j = 0; j < topk; ++j) {
-      int best = -1;
-      float bv = 0.f;
-      for (int e = 0; e < E; ++e) {
-        if (groups > 0 && !((allowed >> (e / per_group)) & 1u)) continue;
-        bool taken = false;
-        for (int i = 0; i < j; ++i) taken |= chosen[i] == e;
-        if (taken) continue;
-        const float v = load_logit<GDT>(gating, row + e);
-        if (best < 0 || v > bv) {
-          best = e;
-          bv = v;
-        }
-      }
-      chosen[j] = best;
-      weight[j] = expf(bv - mx) / sum;
-      wsum += weight[j];
-    }
-    for (int j = 0; j < topk; ++j) {
-      topk_ids[(size_t)t * topk + j] = chosen[j];
-      topk_weights[(size_t)t * topk + j] = renormalize ? weight[j] / wsum : weight[j];
-      atomicAdd(&count[chosen[j]], 1);
-    }
+    __syncthreads();  // the batch is consumed before the next one overwrites it
   }
   __syncthreads();
   if (tid == 0) {
@@ -488,7 +501,9 @@ int q4_moe_route_grouped(const void* gating, int gating_dtype, int tokens, int e
     return Q4_ERR_INVALID_ARGUMENT;
   }
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid(1), block(1024);
+  // one thread per token, one workgroup: a few tokens need a single wave
+  const int threads = tokens >= 1024 ? 1024 : (tokens <= 64 ? 64 : ((tokens + 63) / 64) * 64);
+  const dim3 grid(1), block((unsigned)threads);
   if (gating_dtype == Q4_DTYPE_F16)
     hipLaunchKernelGGL(q4::moe_route_kernel<Q4_DTYPE_F16>, grid, block, 0, s, gating, tokens, experts, topk,
                        renormalize, num_expert_group, topk_group, topk_weights, topk_ids, sorted_tokens, pair_slot,
