@@ -191,6 +191,14 @@ int q4_moe_route_grouped(const void* gating, int gating_dtype, int tokens, int e
 int q4_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_rows, const int32_t* expert_offsets,
                   void* y, int tokens, int topk, int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* First projection with the gated-MLP epilogue: every expert's W packs [gate | up] along N and
+ * y[r, :] = act(x_r @ gate_e) * (x_r @ up_e), [tokens*topk, N/2] in sorted order.  One launch
+ * where the fused decode kernel applies (one token, GPTQ layout with contiguous groups
+ * of at least 128 rows); Q4_ERR_UNSUPPORTED otherwise -- then q4_moe_linear + q4_act_mul. */
+int q4_moe_linear_gate_up(const q4_moe_weight* w, const void* x, const int32_t* x_rows, const int32_t* expert_offsets,
+                          void* y, int tokens, int topk, int dtype, int act, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
 /* out[t, :] = sum_j topk_weights[t, j] * y_sorted[pair_slot[t*topk + j], :], summed in fp32
  * in the order j = 0, 1, ..., rounded once. */
 int q4_moe_combine(const void* y_sorted, const float* topk_weights, const int32_t* pair_slot, void* out,

@@ -133,6 +133,30 @@ def test_moe_argument_validation_without_gpu(pkg):
     assert lib.q4_moe_workspace_bytes(None, 1, 2) == 0
 
 
+def test_workspace_sizing_covers_every_launch(pkg):
+    """A workspace of the advertised size is never reported as too small, whatever kernel the
+    dispatch takes (the launch itself fails here for want of a GPU, after the size check)."""
+    import ctypes
+
+    lib = pkg._lib.load()
+    L = pkg._lib
+    for layout, g_idx in ((0, False), (0, True), (1, False)):
+        for K, N in [(14336, 4096), (4096, 28672), (4096, 4096), (11008, 4096), (8192, 1024), (5504, 512)]:
+            for M in (1, 2, 3, 4, 8, 12, 16, 17, 32, 40, 64, 65, 200, 1000, 2048):
+                for dt in (0, 1):
+                    w = _weight(pkg, K, N, 128, layout, g_idx)
+                    ws = lib.q4_workspace_bytes(M, K, N)
+                    rc = lib.q4_linear(ctypes.byref(w), 0x10, None, 0x20, M, dt, 0x40, ws, None)
+                    assert rc != L.ERR_WORKSPACE, (layout, g_idx, K, N, M, dt, lib.q4_last_error())
+                    G = K // 128
+                    mw = L.Q4MoeWeight(w, 8, (K // 8) * N, G * (N // 8), G * N, K)
+                    ws = lib.q4_moe_workspace_bytes(ctypes.byref(mw), M, 2)
+                    rc = lib.q4_moe_linear(ctypes.byref(mw), 0x10, None, 0x20, 0x30, M, 2, dt, 0x40, ws, None)
+                    assert rc != L.ERR_WORKSPACE, ("moe", layout, g_idx, K, N, M, dt, lib.q4_last_error())
+                    rc = lib.q4_moe_linear_gate_up(ctypes.byref(mw), 0x10, None, 0x20, 0x30, M, 2, dt, 0, 0x40, ws, None)
+                    assert rc != L.ERR_WORKSPACE, ("moe fused", layout, g_idx, K, N, M, dt, lib.q4_last_error())
+
+
 def test_path_selection_and_workspace(pkg):
     lib = pkg._lib.load()
     L = pkg._lib

@@ -202,6 +202,39 @@ def test_moe_linear_act_order_and_awq(pkg, oracle, gpu, kind, T, E, k, K, N, gs,
     assert max_rel_err(y2, ref2) <= (TOL_BF16 if bf else TOL)
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("T,E,k,K,I,gs,act", [
+    (1, 8, 2, 1024, 512, 128, "silu"),       # fused decode kernel
+    (1, 8, 2, 2048, 1024, 128, "gelu_tanh"),
+    (1, 4, 4, 43 * 128, 256, 256, "silu"),   # uneven K ranges, every expert chosen
+    (2, 8, 2, 2048, 1024, 128, "silu"),      # two tokens: two-kernel route
+    (1, 8, 2, 1024, 512, 64, "silu"),        # groups of 64 rows: grouped linear + act_mul
+    (3, 8, 2, 1024, 512, 128, "silu"),       # three tokens: two-kernel route
+])
+def test_moe_linear_gate_up(pkg, oracle, gpu, T, E, k, K, I, gs, act, dtype):
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(T + K + I)
+    qw, qz, sc, dense = _experts(oracle, gpu, E, K, 2 * I, gs, dtype, seed=T + I)
+    w = pkg.ops.make_packed_moe(qw, qz, sc, gs)
+    g, _ = _gating(rng, T, E, "f32")
+    r = pkg.ops.moe_route(g.to(gpu), k, True)
+    x = oracle.make_x(T, K, seed=T + 2, dtype=dtype)
+    y = pkg.ops.moe_linear_gate_up(w, to_dev(x, gpu, bf16=bf), r, act)
+    torch.cuda.synchronize()
+    assert y.shape == (T * k, I)
+    y = to_f32(y)
+    ids = r.topk_ids.cpu().numpy()
+    slot = r.pair_slot.cpu().numpy()
+    ref = np.zeros_like(y)
+    oracle_act = {"gelu_tanh": "gelu_tanh"}.get(act, act)
+    for e in range(E):
+        rows, js = np.nonzero(ids == e)
+        if rows.size:
+            ref[slot[rows * k + js]], _ = oracle.gate_up_forward(x[rows], dense[e], oracle_act, None, dtype)
+    err = max_rel_err(y, ref)
+    assert err <= 2 * (TOL_BF16 if bf else TOL), f"max rel err {err:.3e}"
+
+
 @pytest.mark.parametrize("T", [2, 16, 40])
 def test_moe_linear_sorted_input(pkg, oracle, gpu, T):
     """Second projection: x is already in sorted order."""

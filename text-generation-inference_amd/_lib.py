@@ -100,6 +100,10 @@ SIGNATURES = {
         c_int,
         [POINTER(Q4MoeWeight), c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),
+    "q4_moe_linear_gate_up": (
+        c_int,
+        [POINTER(Q4MoeWeight), c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
+    ),
     "q4_moe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "q4_moe_workspace_bytes": (c_size_t, [POINTER(Q4MoeWeight), c_int, c_int]),
 }

@@ -9,7 +9,7 @@ using q4::Problem;
 
 // fused gated-MLP instantiations live in their own translation unit (q4_gemv_gate_up.hip)
 void launch_gemv_gate_up(const GemvParams& gp, int dtype, int rmax, bool static128, dim3 grid, dim3 block,
-                         size_t smem, hipStream_t stream);
+                         size_t smem, hipStream_t stream, bool grouped);
 
 static bool groupsize_ok_contiguous(int gs) {
   return gs == 32 || gs == 64 || (gs >= 128 && gs % 128 == 0);
@@ -289,7 +289,7 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   dim3 grid((unsigned)(ntiles * cfg.splits), (unsigned)mchunks);
   dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
   if (gate_up_act != 0) {
-    launch_gemv_gate_up(gp, dtype, rmax, w->groupsize == 128, grid, block, smem, stream);
+    launch_gemv_gate_up(gp, dtype, rmax, w->groupsize == 128, grid, block, smem, stream, false);
   } else if (dtype == Q4_DTYPE_F16) {
     if (rmax == 1) launch_rmax<Q4_DTYPE_F16, 1>(w, gp, cfg.words, grid, block, smem, stream);
     else if (rmax == 2) launch_rmax<Q4_DTYPE_F16, 2>(w, gp, cfg.words, grid, block, smem, stream);

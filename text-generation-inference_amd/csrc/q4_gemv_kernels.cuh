@@ -154,8 +154,10 @@ __device__ __forceinline__ Decomp make_decomp(const GemvParams& gp, int wave_col
 // Entry of a grouped (MOE) decode launch: narrows gp to the expert blockIdx.z.  Returns false
 // when this workgroup's row block lies beyond the expert's rows (the whole workgroup leaves).
 // `rows` receives the activation-row map of the block, or nullptr when x is in sorted order.
-__device__ __forceinline__ bool moe_enter_decode(GemvParams& gp, const int32_t*& rows) {
+__device__ __forceinline__ bool moe_enter_decode(GemvParams& gp, const int32_t*& rows, bool half_width_output = false) {
   const int row0 = moe_enter(gp.p, gp.moe, blockIdx.z);
+  // the gated-MLP epilogue writes N / 2 columns per row
+  if (half_width_output) gp.p.y = (uint16_t*)gp.p.y - (size_t)row0 * (gp.p.N >> 1);
   if (gp.p.M <= (int)blockIdx.y * kRowsPerBlock) return false;
   gp.partials += (size_t)row0 * gp.p.N;
   rows = gp.moe.x_rows != nullptr ? gp.moe.x_rows + row0 + blockIdx.y * kRowsPerBlock : nullptr;
@@ -443,7 +445,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int32_t* moe_rows = nullptr;
   if constexpr (MOE) {
-    if (!moe_enter_decode(gp, moe_rows)) return;
+    if (!moe_enter_decode(gp, moe_rows, FUSE)) return;
   }
   const Problem& p = gp.p;
   const Decomp d = make_decomp(gp, 16 * WORDS);

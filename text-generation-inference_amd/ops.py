@@ -418,6 +418,36 @@ def moe_linear(w: PackedMoeWeight, x: torch.Tensor, routing: MoeRouting, gather:
     return y
 
 
+def moe_linear_gate_up(w: PackedMoeWeight, x: torch.Tensor, routing: MoeRouting, act: str = "silu") -> torch.Tensor:
+    """First projection of the experts with the gated-MLP tail: sorted row r becomes
+    act(x[token(r)] @ gate_e) * (x[token(r)] @ up_e), [tokens*k, N/2].  One fused launch where
+    the decode kernel offers it (one token), else grouped linear + act_mul."""
+    _require_cuda(x, "x")
+    if x.dtype not in _DTYPES:
+        raise TypeError(f"x must be float16 or bfloat16, got {x.dtype}")
+    if act not in _lib.ACTIVATIONS:
+        raise ValueError(f"unknown activation {act!r}; known: {sorted(_lib.ACTIVATIONS)}")
+    T, k = routing.topk_ids.shape
+    if x.dim() != 2 or tuple(x.shape) != (T, w.K):
+        raise ValueError(f"x must be [{T}, {w.K}], got {tuple(x.shape)}")
+    x = x.contiguous()
+    if T > 0:
+        lib = _lib.load()
+        y = torch.empty((T * k, w.N // 2), dtype=x.dtype, device=x.device)
+        with torch.cuda.device(x.device):
+            stream = _stream_handle(x.device)
+            st = w.struct()
+            ws = reserve_workspace(x.device, int(lib.q4_moe_workspace_bytes(ctypes.byref(st), T, k)), stream)
+            rc = lib.q4_moe_linear_gate_up(
+                ctypes.byref(st), x.data_ptr(), routing.sorted_tokens.data_ptr(), routing.expert_offsets.data_ptr(),
+                y.data_ptr(), T, k, _DTYPES[x.dtype], _lib.ACTIVATIONS[act], ws.data_ptr(), ws.numel(), stream,
+            )
+        if rc != _lib.ERR_UNSUPPORTED:
+            _lib.check(rc)
+            return y
+    return act_mul(moe_linear(w, x, routing, gather=True), act)
+
+
 def moe_combine(y_sorted: torch.Tensor, routing: MoeRouting) -> torch.Tensor:
     """out[t] = sum_j topk_weights[t, j] * y_sorted[slot(t, j)] (fp32 sum, one rounding)."""
     _require_cuda(y_sorted, "y_sorted")
@@ -441,5 +471,5 @@ def moe_forward(gate_up: PackedMoeWeight, down: PackedMoeWeight, x: torch.Tensor
     """The sparse MoE block: route, [gate | up] projection, act(gate) * up, down projection,
     weighted sum over the chosen experts."""
     routing = moe_route(gating_output, topk, renormalize, num_expert_group, topk_group)
-    h = act_mul(moe_linear(gate_up, x, routing, gather=True), act)
+    h = moe_linear_gate_up(gate_up, x, routing, act)
     return moe_combine(moe_linear(down, h, routing, gather=False), routing)
