@@ -78,7 +78,9 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   // AWQ from 4 rows on, long enough K: eight waves along K share one activation slab
   // (4096 x 14336 at M = 8: 25.3 against 28.2 us; 14336 x 4096 at M = 4: 23.6 against 28.4 us;
   // 4096 x 4096 keeps four waves and eight splits: 15.4 against 18.2 us)
-  const bool awq8 = w->layout == Q4_LAYOUT_AWQ && M >= 4 && chunks % 8 == 0 && (long)chunks * w->N >= 32L * 8192;
+  // (and at any M once K is long: 14336 x 4096 at M = 1: 13.2 against 17.5 us)
+  const bool awq8 = w->layout == Q4_LAYOUT_AWQ && (M >= 4 || chunks >= 64) && chunks % 8 == 0 &&
+                    (long)chunks * w->N >= 32L * 8192;
   if (awq8) c.wk = 8;
   if (gate_up) {
     // a wave owns 64 gate and 64 up columns (twice the bytes of a plain wave): eight waves
@@ -276,10 +278,12 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   // fp16, one row, plain epilogue, four columns per lane: one atomic per element beats the
   // ticket (measured on MI355X at M = 1: 12.3 against 13.6 us for 14336 x 4096, 8.3 / 9.0 us
   // for 4096 x 6144, 7.1 / 7.8 us for 4096 x 4096).  Every further row doubles the atomics,
-  // which execute at the memory side: already slower at M = 2 (9.3 against 8.0 us) and for the
-  // AWQ kernel's 16 columns per lane (16.5 against 13.8 us).
+  // which execute at the memory side: already slower at M = 2 (9.3 against 8.0 us).  The AWQ
+  // kernel (16 columns per lane) first transposes its sums through LDS so that an atomic
+  // instruction covers 64 consecutive cells (4096 x 14336: 13.3 against 14.8 us with tickets;
+  // issued straight from the 16 lanes that hold the row it measured 16.5 us).
   gp.fixed_point_split = cfg.splits > 1 && cfg.splits <= 14 && dtype == Q4_DTYPE_F16 && gate_up_act == 0 &&
-                         !awq && M == 1 && (size_t)w->N * 8 <= Q4_WORKSPACE_CELL_BYTES;
+                         (!awq || cfg.wcol == 1) && M == 1 && (size_t)w->N * 8 <= Q4_WORKSPACE_CELL_BYTES;
   gp.cells = cfg.splits > 1 ? (unsigned long long*)((char*)workspace + Q4_WORKSPACE_TICKET_BYTES) : nullptr;
   gp.slab_stride = slab_stride;
   gp.slab_bytes = (int)slab_bytes;

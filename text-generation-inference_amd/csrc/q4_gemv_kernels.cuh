@@ -319,9 +319,44 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
   // before the first call; they are left zero.
   if constexpr (DTYPE == Q4_DTYPE_F16 && !FUSE) {
     if (gp.fixed_point_split) {
+      constexpr unsigned long long kOne = 1ull << 56, kHalf = 1ull << 55;
+      if constexpr (NT == 16) {
+        // Sixteen columns per lane (AWQ): issued from the 16 lanes that hold row 0, every
+        // atomic instruction would touch 16 cache lines.  The wave's 256 sums go through LDS
+        // so that a lane owns columns lane, lane + 64, ..: each instruction then covers 64
+        // consecutive cells.  Single row, one column tile per workgroup (the host checks).
+        if (d.wkk == 0) {
+          float* tile = (float*)smem;  // the K waves' partials were consumed above by this same wave
+          if (d.kq == 0) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) tile[d.j * NT + t] = out[t][0];
+          }
+          const int nbase = d.tile * d.tile_cols;
+          unsigned long long* cell = gp.cells + (size_t)d.mb * N + nbase;
+          unsigned long long before[4], inc[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const float v = tile[d.lane + 64 * u];
+            long long q = 1ll << 51;  // non-finite
+            if (fabsf(v) <= 3.0e38f) q = __float2ll_rn(fminf(fmaxf(v, -131072.f), 131072.f) * 268435456.f);
+            inc[u] = kOne + (unsigned long long)q;
+            before[u] = __hip_atomic_fetch_add(cell + d.lane + 64 * u, inc[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const unsigned long long now = before[u] + inc[u];
+            if ((long long)(now + kHalf) >> 56 == (long long)gp.splits) {
+              const long long sum = (long long)(now - ((unsigned long long)gp.splits << 56));
+              const int n = nbase + d.lane + 64 * u;
+              y[(size_t)d.mb * N + n] = finish_output<DTYPE>((float)sum * (1.0f / 268435456.f), p.bias, n);
+              __hip_atomic_store(cell + d.lane + 64 * u, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+          }
+        }
+        return;
+      }
       if (d.wkk == 0) {
         unsigned long long* cells = gp.cells;
-        constexpr unsigned long long kOne = 1ull << 56, kHalf = 1ull << 55;
 #pragma unroll
         for (int r = 0; r < RMAX; ++r) {
           const int m = 4 * d.kq + r;
