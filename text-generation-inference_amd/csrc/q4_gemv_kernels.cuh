@@ -320,11 +320,13 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
   if constexpr (DTYPE == Q4_DTYPE_F16 && !FUSE) {
     if (gp.fixed_point_split) {
       constexpr unsigned long long kOne = 1ull << 56, kHalf = 1ull << 55;
-      if constexpr (NT == 16) {
-        // Sixteen columns per lane (AWQ): issued from the 16 lanes that hold row 0, every
-        // atomic instruction would touch 16 cache lines.  The wave's 256 sums go through LDS
-        // so that a lane owns columns lane, lane + 64, ..: each instruction then covers 64
-        // consecutive cells.  Single row, one column tile per workgroup (the host checks).
+      if constexpr (NT >= 4) if (gp.wcol == 1) {
+        // The sums of row 0 sit in the 16 lanes of K block 0, NT adjacent columns each: issued
+        // from there, an atomic instruction touches 16 separate groups of cells (with the AWQ
+        // kernel's 16 columns per lane: 16 cache lines).  The wave's 16 * NT sums go through
+        // LDS so that a lane owns columns lane, lane + 64, ..: every instruction then covers 64
+        // consecutive cells with all lanes active.  Single row, one column tile per workgroup.
+        constexpr int PER_LANE = NT >= 4 ? NT / 4 : 1;  // 16 * NT sums over 64 lanes
         if (d.wkk == 0) {
           float* tile = (float*)smem;  // the K waves' partials were consumed above by this same wave
           if (d.kq == 0) {
@@ -333,9 +335,9 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
           }
           const int nbase = d.tile * d.tile_cols;
           unsigned long long* cell = gp.cells + (size_t)d.mb * N + nbase;
-          unsigned long long before[4], inc[4];
+          unsigned long long before[PER_LANE], inc[PER_LANE];
 #pragma unroll
-          for (int u = 0; u < 4; ++u) {
+          for (int u = 0; u < PER_LANE; ++u) {
             const float v = tile[d.lane + 64 * u];
             long long q = 1ll << 51;  // non-finite
             if (fabsf(v) <= 3.0e38f) q = __float2ll_rn(fminf(fmaxf(v, -131072.f), 131072.f) * 268435456.f);
@@ -343,7 +345,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
             before[u] = __hip_atomic_fetch_add(cell + d.lane + 64 * u, inc[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
 #pragma unroll
-          for (int u = 0; u < 4; ++u) {
+          for (int u = 0; u < PER_LANE; ++u) {
             const unsigned long long now = before[u] + inc[u];
             if ((long long)(now + kHalf) >> 56 == (long long)gp.splits) {
               const long long sum = (long long)(now - ((unsigned long long)gp.splits << 56));
