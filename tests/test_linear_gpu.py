@@ -106,13 +106,13 @@ def test_gemv_deterministic_and_tickets_reset(pkg, oracle, gpu):
 def test_gemv_single_row_fixed_point_combine(pkg, oracle, gpu, K, N):
     """M = 1, fp16: the K splits meet in 64-bit fixed-point cells (integer adds, so the sum does
     not depend on arrival order).  Bit-reproducible, cells back at zero, and the same row
-    computed through the ticket path (the row duplicated to M = 2) agrees to fp16 rounding."""
+    computed through the ticket path (the row repeated to M = 4) agrees to fp16 rounding."""
     qw, qz, sc, _ = oracle.make_gptq(K, N, 128, seed=K + N, sym=False)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
     x = to_dev(oracle.make_x(1, K, seed=5), gpu)
     a = pkg.ops.linear(pk, x, None, path=1)
     b = pkg.ops.linear(pk, x, None, path=1)
-    two = pkg.ops.linear(pk, torch.cat([x, x]), None, path=1)
+    two = pkg.ops.linear(pk, torch.cat([x, x, x, x]), None, path=1)
     torch.cuda.synchronize()
     assert torch.equal(a, b)
     for ws in pkg.ops._workspaces.values():
@@ -122,6 +122,39 @@ def test_gemv_single_row_fixed_point_combine(pkg, oracle, gpu, K, N):
     assert max_rel_err(to_f32(a), y32) <= TOL
     assert max_rel_err(to_f32(a), to_f32(two[:1])) <= 1e-3
     assert float((a == two[:1]).float().mean()) > 0.9
+
+
+@pytest.mark.parametrize("layout,act", [("gptq", False), ("gptq", True), ("awq", False)])
+@pytest.mark.parametrize("M", [2, 3])
+def test_gemv_few_rows_fixed_point_combine(pkg, oracle, gpu, layout, act, M):
+    """Two and three fp16 rows also meet in the cells, a row at a time, each wave's sums
+    transposed so that one atomic instruction covers 64 consecutive cells.  Same checks as for
+    one row; the ticket path (the rows padded to M = 4) is the second opinion."""
+    K, N = 4096, 4096
+    if layout == "awq":
+        qw, qz, sc = oracle.make_awq(K, N, 128, seed=M)
+        gi = None
+        w = oracle.dequant_awq(qw, qz, sc, 128, "f16")
+    else:
+        qw, qz, sc, gi = oracle.make_gptq(K, N, 128, seed=M, sym=False, act_order=act)
+        w = oracle.dequant_gptq(qw, qz, sc, gi, 128, "f16")
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), 128,
+                             1 if layout == "awq" else 0)
+    xh = oracle.make_x(M, K, seed=7 + M)
+    x = to_dev(xh, gpu)
+    bias = to_dev(np.random.default_rng(M).standard_normal(N).astype(np.float16), gpu)
+    a = pkg.ops.linear(pk, x, bias, path=1).clone()
+    b = pkg.ops.linear(pk, x, bias, path=1).clone()
+    pad = torch.cat([x, x[: 4 - M]])
+    four = pkg.ops.linear(pk, pad, bias, path=1)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    for ws in pkg.ops._workspaces.values():
+        assert int(ws[: pkg._lib.WORKSPACE_COUNTER_BYTES].sum().item()) == 0
+    y32, _ = oracle.linear_forward(xh, w, bias.cpu().numpy(), "f16")
+    assert max_rel_err(to_f32(a), y32) <= TOL
+    assert max_rel_err(to_f32(a), to_f32(four[:M])) <= 1e-3
+    assert float((a == four[:M]).float().mean()) > 0.9
 
 
 def test_gemv_single_row_non_finite_input_leaves_the_cells_clean(pkg, oracle, gpu):
@@ -272,9 +305,9 @@ def test_awq_decompositions(pkg, oracle, gpu, cfg):
 def test_awq_auto_path_is_native(pkg, oracle, gpu):
     qw, qz, sc = oracle.make_awq(1024, 512, 128, seed=0)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 1)
-    for M in (1, 6):
+    for M in (1, 8):
         assert pkg.ops.select_path(pk, M) == "gemv"
-    for M in (7, 17, 100, 256):
+    for M in (9, 17, 100, 256):
         assert pkg.ops.select_path(pk, M) == "gemm"  # the LDS-unpack MFMA kernel, split-K on small grids
     qw, qz, sc, gi = oracle.make_gptq(1024, 512, 128, seed=0, act_order=True)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), 128, 0)
@@ -359,11 +392,12 @@ def test_awq_gemm_bit_exact_weights_through_identity(pkg, oracle, gpu):
 def test_awq_dispatch_large_m(pkg, oracle, gpu):
     qw, qz, sc = oracle.make_awq(1024, 14336, 128, seed=0)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 1)
-    assert pkg.ops.select_path(pk, 6) == "gemv"
-    assert pkg.ops.select_path(pk, 7) == "gemm"
+    assert pkg.ops.select_path(pk, 8) == "gemv"
+    assert pkg.ops.select_path(pk, 9) == "gemm"
     assert pkg.ops.select_path(pk, 64) == "gemm"
     # the first row count that goes to the GEMM moves with the shape (measured crossovers)
-    for K, N, first in [(14336, 4096, 6), (4096, 14336, 12), (8192, 10240, 10), (8192, 28672, 17), (28672, 8192, 17)]:
+    for K, N, first in [(4096, 4096, 9), (4096, 6144, 14), (11008, 4096, 10), (14336, 4096, 17), (4096, 14336, 17),
+                        (8192, 10240, 17), (8192, 28672, 33), (28672, 8192, 33)]:
         w = pkg.ops.PackedWeight(pk.qweight, pk.qzeros, pk.scales, None, K, N, 128, K // 128, 1)  # geometry only
         assert pkg.ops.select_path(w, first - 1) == "gemv", (K, N)
         assert pkg.ops.select_path(w, first) == "gemm", (K, N)

@@ -108,17 +108,20 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   // rows), from about M = 48 on when it has to gather scales and zero points from global
   // memory (~2x slower per tile).
   // AWQ: the decode kernel's time grows with every row (16 accumulator sets, ~250 VGPRs)
-  // while the split-K GEMM is flat in M (17.7 us for 4096 x 4096, 30 us for 4096 x 14336,
-  // 40 us for 8192 x 10240, 88 / 103 us for 28672 x 8192 / 8192 x 28672).  First M at which
-  // the GEMM was faster: 4096 x 4096 7, 4096 x 14336 13, 8192 x 8192 15, 5120 x 13824 5,
-  // 8192 x 10240 9, 14336 x 4096 9, 13824 x 5120 4, 28672 x 8192 and 8192 x 28672 above 16.
+  // while the split-K GEMM is flat in M (17.2 us for 4096 x 4096, 20.4 us for 4096 x 6144,
+  // 27 us for 11008 x 4096, 30 us for 4096 x 14336, 40 us for 8192 x 10240, 92 / 108 us for
+  // 28672 x 8192 / 8192 x 28672: it unpacks every weight through LDS once per 128 rows).
+  // First M at which the GEMM was faster: 4096 x 4096 9, 4096 x 6144 14, 5120 x 5120 16,
+  // 11008 x 4096 10; above 16 for 4096 x 11008, 4096 x 14336, 14336 x 4096, 8192 x 8192,
+  // 8192 x 10240, 5120 x 13824, 13824 x 5120; 28672 x 8192 and 8192 x 28672 in two row
+  // chunks up to 32 rows (96 against 95 / 131 us at M = 32).
   bool small = M <= 16 || (w->layout == Q4_LAYOUT_GPTQ && M <= 48 && !gemm_act_order_table(w));
   if (w->layout == Q4_LAYOUT_AWQ) {
-    int first_gemm_m = 12;
-    if (weights >= (1L << 27)) first_gemm_m = 17;
-    else if (w->K > 8192) first_gemm_m = 6;
-    else if (w->K >= 8192 && weights > (1L << 26)) first_gemm_m = 10;
-    else if (weights <= (1L << 25)) first_gemm_m = 7;
+    int first_gemm_m = 17;
+    if (weights >= (1L << 27)) first_gemm_m = 33;
+    else if (weights <= (1L << 24)) first_gemm_m = 9;
+    else if (weights <= (1L << 25)) first_gemm_m = 14;
+    else if ((w->K / 128) % 8 != 0 && weights <= (1L << 26)) first_gemm_m = 10;
     small = M < first_gemm_m;
   }
   if (!small && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;

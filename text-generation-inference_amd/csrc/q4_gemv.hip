@@ -75,12 +75,13 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   // (M = 16: 4096 x 6144 12.1 against 14.9 us, 14336 x 4096 18.8 against 22.4 us)
   const bool contiguous = w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr;
   if (contiguous && !gate_up && M >= 12 && c.wcol == 1 && (chunks % 8 == 0 || chunks >= 32)) c.wk = 8;
-  // AWQ from 4 rows on, long enough K: eight waves along K share one activation slab
-  // (4096 x 14336 at M = 8: 25.3 against 28.2 us; 14336 x 4096 at M = 4: 23.6 against 28.4 us;
-  // 4096 x 4096 keeps four waves and eight splits: 15.4 against 18.2 us)
-  // (and at any M once K is long: 14336 x 4096 at M = 1: 13.2 against 17.5 us)
-  const bool awq8 = w->layout == Q4_LAYOUT_AWQ && (M >= 4 || chunks >= 64) && chunks % 8 == 0 &&
-                    (long)chunks * w->N >= 32L * 8192;
+  // AWQ: eight waves along K share one activation slab from 8 rows on, from 4 rows on large
+  // layers and at any M once K is long (14336 x 4096 at M = 1: 13.2 against 17.5 us;
+  // 4096 x 14336 at M = 8: 25.3 against 28.2 us; 4096 x 4096 up to 4 rows keeps four waves and
+  // eight splits: 13.9 against 15.8 us).  A K that does not deal out evenly over eight waves
+  // stays with four at small M (11008 x 4096 at M = 1: 14.9 against 17.1 us).
+  const bool awq8 = w->layout == Q4_LAYOUT_AWQ && chunks >= 8 &&
+                    (M >= 8 || (M >= 4 && (long)chunks * w->N >= 32L * 8192) || (chunks >= 64 && chunks % 8 == 0));
   if (awq8) c.wk = 8;
   if (gate_up) {
     // a wave owns 64 gate and 64 up columns (twice the bytes of a plain wave): eight waves
@@ -140,12 +141,38 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
       }
     }
   }
+  if (awq8) {
+    // 512-thread workgroups, one resident per CU for most slab sizes: the grid is held to one
+    // round of 256 and aims at all of it for up to 8 rows, at three quarters beyond (the
+    // partial sums grow with M).  Fitted on a sweep of 13 layer shapes x M = 1..16 on MI355X:
+    // within 1.3 % of the best measured configuration on average (28672 x 8192 at M = 8: 42
+    // against 62 us with ten ragged splits; 8192 x 10240 at M = 1: 18.6 against 24.7 us).
+    const double target = M <= 8 ? 256.0 : 192.0;
+    int best_dv = min_splits;
+    double best = -1.0;
+    for (int dv = min_splits; dv <= max_splits; ++dv) {
+      const double wgs = (double)ntiles * dv;
+      if (wgs > 256.0 && dv > min_splits) break;
+      double cost = wgs > target ? wgs / target : target / wgs;
+      if (chunks % (dv * c.wk) != 0) cost *= 1.2;
+      if (best < 0.0 || cost < best) {
+        best = cost;
+        best_dv = dv;
+      }
+    }
+    c.splits = best_dv;
+    return c;
+  }
+  // four AWQ waves: at most 448 workgroups (13824 x 5120 at M = 1: 18.4 us with 14 splits
+  // against 22.8 us with 27)
+  const int max_wgs = w->layout == Q4_LAYOUT_AWQ ? 448 : 1 << 30;
   // K is dealt out in 128-row chunks over splits x wk wave slots.  A count that divides the
   // chunks evenly is preferred; when none is near the wanted one (K = 11008: 86 chunks) the
   // slots differ by one chunk and the cost carries the imbalance.
-  int best = max_splits;
+  int best = -1;
   double best_cost = -1.0;
   for (int dv = min_splits; dv <= max_splits; ++dv) {
+    if ((long)ntiles * dv > max_wgs && dv > min_splits) break;
     const long slots = (long)dv * c.wk;
     const double balance = (double)((chunks + slots - 1) / slots) * slots / chunks;  // >= 1
     // too few workgroups cost more than too many (13824 x 5120 at M = 16 wants five splits:
@@ -161,7 +188,7 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
       best = dv;
     }
   }
-  c.splits = best;
+  c.splits = best > 0 ? best : max_splits;
   return c;
 }
 
@@ -245,11 +272,6 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   if (act) smem += (((size_t)KR * 2 + 15) & ~(size_t)15) + (size_t)w->num_groups * 64 * cfg.wcol * 4;
   const size_t red = (size_t)(cfg.wk - 1) * cfg.wcol * nt * rmax * 64 * sizeof(float);
   if (red > smem) smem = red;
-  const size_t smem_limit = 160 * 1024 - 1024;  // gfx950: 160 KB of LDS per workgroup
-  if (smem > smem_limit) {
-    set_error("q4_linear(gemv): config needs %zu bytes of LDS (> %zu)", smem, smem_limit);
-    return Q4_ERR_INVALID_ARGUMENT;
-  }
   const int ntiles = w->N / (wave_cols * cfg.wcol);
   if ((long)ntiles * mchunks > Q4_WORKSPACE_TICKET_BYTES / 4) {
     set_error("q4_linear(gemv): too many tiles (%d x %d)", ntiles, mchunks);
@@ -275,15 +297,26 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.wcol = cfg.wcol;
   gp.wk = cfg.wk;
   gp.splits = cfg.splits;
-  // fp16, one row, plain epilogue, four columns per lane: one atomic per element beats the
-  // ticket (measured on MI355X at M = 1: 12.3 against 13.6 us for 14336 x 4096, 8.3 / 9.0 us
-  // for 4096 x 6144, 7.1 / 7.8 us for 4096 x 4096).  Every further row doubles the atomics,
-  // which execute at the memory side: already slower at M = 2 (9.3 against 8.0 us).  The AWQ
-  // kernel (16 columns per lane) first transposes its sums through LDS so that an atomic
-  // instruction covers 64 consecutive cells (4096 x 14336: 13.3 against 14.8 us with tickets;
-  // issued straight from the 16 lanes that hold the row it measured 16.5 us).
+  // fp16, few rows, plain epilogue, at least four columns per lane: one atomic per element beats
+  // the ticket.  The kernel first transposes a wave's sums through LDS (behind the K-wave
+  // partials) so that an atomic instruction covers 64 consecutive cells of one row: issued
+  // straight from the 16 lanes that hold a row, the four instructions of a GPTQ row cost 1 us
+  // more than the one (4096 x 4096, M = 1: 7.05 against 5.97 us; tickets 7.8 us).  The adds
+  // execute at the memory side, about 0.8 us per row of 4096 cells x 8 splits: up to three rows
+  // they beat the tickets (GPTQ 4096 x 4096, M = 2: 6.8 against 8.1 us, M = 3: 7.5 / 8.3; AWQ
+  // 14336 x 4096, M = 3: 18.1 / 22.4), from four rows on they do not.
+  constexpr int kCellRowsMax = 3;
   gp.fixed_point_split = cfg.splits > 1 && cfg.splits <= 14 && dtype == Q4_DTYPE_F16 && gate_up_act == 0 &&
-                         (!awq || cfg.wcol == 1) && M == 1 && (size_t)w->N * 8 <= Q4_WORKSPACE_CELL_BYTES;
+                         (nt >= 4 ? M <= kCellRowsMax : M == 1) && (size_t)M * w->N * 8 <= Q4_WORKSPACE_CELL_BYTES;
+  if (gp.fixed_point_split && nt >= 4) {
+    const size_t tile = red + (size_t)cfg.wcol * (rmax < 4 ? rmax : kRowsPerBlock) * 16 * nt * sizeof(float);
+    if (tile > smem) smem = tile;
+  }
+  const size_t smem_limit = 160 * 1024 - 1024;  // gfx950: 160 KB of LDS per workgroup
+  if (smem > smem_limit) {
+    set_error("q4_linear(gemv): config needs %zu bytes of LDS (> %zu)", smem, smem_limit);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
   gp.cells = cfg.splits > 1 ? (unsigned long long*)((char*)workspace + Q4_WORKSPACE_TICKET_BYTES) : nullptr;
   gp.slab_stride = slab_stride;
   gp.slab_bytes = (int)slab_bytes;
