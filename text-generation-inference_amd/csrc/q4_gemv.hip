@@ -67,7 +67,10 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   // (and at any M once the tiles alone are well over the CU count: 4096 x 28672 at M = 1
   // measured 16.7 against 17.0-17.8 us)
   if (w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && w->N % 128 == 0 &&
-      ((M >= 8 && w->N / 64 >= 256) || (M >= 12 && w->N / 64 >= 128) || w->N / 64 >= 384))
+      ((M >= 8 && w->N / 64 >= 256) || (M >= 12 && w->N / 64 >= 128) || w->N / 64 >= 384 ||
+       // long K: the slab staging of a workgroup is long, two tiles share it (28672 x 8192:
+       // 23.3 against 25.2 us at M = 1, 28.6 against 36.3 us at M = 8)
+       (w->K >= 16384 && w->N / 64 >= 128)))
     c.wcol = 2;
   const bool act = w->layout == Q4_LAYOUT_GPTQ && w->g_idx != nullptr;
   if (act && (chunks % 8 == 0 || chunks >= 32)) c.wk = 8;  // the group table is built once per workgroup
@@ -75,6 +78,15 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   // (M = 16: 4096 x 6144 12.1 against 14.9 us, 14336 x 4096 18.8 against 22.4 us)
   const bool contiguous = w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr;
   if (contiguous && !gate_up && M >= 12 && c.wcol == 1 && (chunks % 8 == 0 || chunks >= 32)) c.wk = 8;
+  // 192..256 column tiles, 2..11 rows: one round of eight-wave workgroups over the whole K,
+  // nothing to combine (4096 x 14336: 10.9 against 11.1 us at M = 2, 12.7 against 14.1 us at
+  // M = 8; 5120 x 13824: 11.9 / 12.6 and 14.2 / 15.4 us; with 172 tiles it does not pay)
+  if (contiguous && !gate_up && M >= 2 && M < 12 && c.wcol == 1 && w->N / 64 >= 192 && w->N / 64 <= 256 &&
+      chunks >= 8 && (long)w->K * (rows * 2) <= 150000 - 16L * rows) {
+    c.wk = 8;
+    c.splits = 1;
+    return c;
+  }
   // AWQ: eight waves along K share one activation slab from 8 rows on, from 4 rows on large
   // layers and at any M once K is long (14336 x 4096 at M = 1: 13.2 against 17.5 us;
   // 4096 x 14336 at M = 8: 25.3 against 28.2 us; 4096 x 4096 up to 4 rows keeps four waves and
