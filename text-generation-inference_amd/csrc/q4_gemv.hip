@@ -73,7 +73,52 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
        (w->K >= 16384 && w->N / 64 >= 128)))
     c.wcol = 2;
   const bool act = w->layout == Q4_LAYOUT_GPTQ && w->g_idx != nullptr;
-  if (act && (chunks % 8 == 0 || chunks >= 32)) c.wk = 8;  // the group table is built once per workgroup
+  if (act) {
+    // Act-order: the kernel is bound by its per-weight table lookups (VALU + LDS), wants two
+    // 512-thread workgroups per CU and builds the table of all groups once per workgroup.
+    // Eight waves along K share table and slab; from 192 column tiles on (128 from 12 rows on)
+    // two column tiles of four waves do.  The split count aims at 448 workgroups within the
+    // LDS budget; with 12 rows or more, when the slab leaves room for one workgroup per CU
+    // only, a single round of at most 256 is taken instead if K splits that way.  Fitted on a
+    // sweep of 14 layer shapes x M = 1..16 on MI355X: 3.4 % above the best measured
+    // configuration on average (the rule before: 10 %; 11008 x 4096 at M = 4: 24.0 -> 19.2 us,
+    // 8192 x 28672 at M = 4: 64.7 -> 47.7 us, 4096 x 28672 at M = 8: 37.8 -> 28.7 us).
+    const int n64 = w->N / 64;
+    const long table1 = (long)w->num_groups * 64 * 4;
+    c.wcol = (w->N % 128 == 0 && (n64 >= 192 || (M >= 12 && n64 >= 128)) && 2 * table1 <= 64 * 1024) ? 2 : 1;
+    c.wk = c.wcol == 2 ? 4 : (chunks >= 8 ? 8 : c.wk);
+    const int tiles = (w->N / (64 * c.wcol)) * mchunks;
+    const int max_dv = chunks / c.wk;
+    auto lds_bytes = [&](int dv) {
+      const long kr = (long)((chunks + dv - 1) / dv) * 128;
+      return (long)rows * (kr * 2 + 16) + kr * 2 + table1 * c.wcol + 32;
+    };
+    const long lds_limit = 160 * 1024 - 1024;
+    int best_dv = max_dv;
+    double best = -1.0;
+    for (int dv = 1; dv <= max_dv; ++dv) {
+      if (lds_bytes(dv) > 150000) continue;
+      const double wgs = (double)tiles * dv;
+      double cost = wgs >= 448.0 ? wgs / 448.0 : 448.0 / wgs;
+      if (chunks % (dv * c.wk) != 0) cost *= 1.15;
+      if (lds_bytes(dv) > 80 * 1024) cost *= 1.5;  // one workgroup per CU: half the waves to hide the lookups
+      if (best < 0.0 || cost < best) {
+        best = cost;
+        best_dv = dv;
+      }
+    }
+    if (M >= 12 && lds_bytes(best_dv) > 80 * 1024) {
+      for (int dv = best_dv - 1; dv >= 1; --dv) {
+        const long wgs = (long)tiles * dv;
+        if (wgs > 256) continue;
+        if (wgs < 224 || lds_bytes(dv) > lds_limit) break;
+        best_dv = dv;
+        break;
+      }
+    }
+    c.splits = best_dv;
+    return c;
+  }
   // many rows, one column tile per workgroup: eight waves along K share one activation slab
   // (M = 16: 4096 x 6144 12.1 against 14.9 us, 14336 x 4096 18.8 against 22.4 us)
   const bool contiguous = w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr;
@@ -127,32 +172,11 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   // 19.7 us unsplit with a 128 KB slab against 30.8 us with four splits; 5120 x 13824 at M = 16:
   // 16 us with two splits (80 KB) against 26.8 us with five.
   long lds_budget = 150000 - 16L * rows;
-  if (act) lds_budget = 150000 - (long)w->num_groups * 64 * 4 - 16L * rows;
-  // bytes per K row in LDS: activations, plus the uint16 g_idx slice for act-order
-  const long per_row = (long)rows * 2 + (act ? 2 : 0);
+  const long per_row = (long)rows * 2;  // bytes per K row in LDS
   const int max_splits = per_wg;  // every wave gets at least one 128-row chunk
   int min_splits = lds_budget > 0 ? (int)(((long)w->K * per_row + lds_budget - 1) / lds_budget) : max_splits;
   if (min_splits < 1) min_splits = 1;
   if (min_splits > max_splits) min_splits = max_splits;
-  // Act-order with many rows: the kernel does per-weight table lookups and needs two
-  // workgroups per CU to hide them, so slab + g_idx slice + table are held to half the LDS
-  // where an even split allows it (8192 x 10240 at M = 16: 27.9 us with eight splits against
-  // 42.9 us with four; 14336 x 4096: 29.6 us with fourteen against 33.5 us with seven).
-  bool even_only = false;
-  if (act && M >= 12) {
-    const long half_lds = 80896 - (long)w->num_groups * 64 * 4 - 16L * rows;
-    if (half_lds > 0) {
-      // sized for a full block of 16 rows: 12 rows measured better with the same split
-      const int need = (int)(((long)w->K * (q4::kRowsPerBlock * 2 + 2) + half_lds - 1) / half_lds);
-      for (int dv = need > min_splits ? need : min_splits; dv <= max_splits; ++dv) {
-        if (chunks % (dv * c.wk) == 0) {
-          min_splits = dv;
-          even_only = true;
-          break;
-        }
-      }
-    }
-  }
   if (awq8) {
     // 512-thread workgroups, one resident per CU for most slab sizes: the grid is held to one
     // round of 256 and aims at all of it for up to 8 rows, at three quarters beyond (the
@@ -191,10 +215,7 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
     // nine take 19.4 us, three 24 us)
     double cost = dv > want ? (double)dv / want : 1.5 * want / dv;
     cost *= balance;
-    if (chunks % slots != 0) {
-      if (even_only) continue;
-      cost *= 1.25;
-    }
+    if (chunks % slots != 0) cost *= 1.25;
     if (best_cost < 0.0 || cost < best_cost) {
       best_cost = cost;
       best = dv;
