@@ -33,8 +33,8 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E peak
 MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16/bf16 MFMA peak
 
-# FETCH_SIZE 14334.3 KiB x 2.000 (copy-kernel calibration) + WRITE_SIZE 369.3 KiB x 1.000
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 30268677
+# FETCH_SIZE 14182.1 KiB x 2.000 (copy-kernel calibration) + WRITE_SIZE 321.0 KiB x 1.000
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 29373594
 
 SHAPES = [  # name, K, N
     ("qkv_proj", 4096, 6144),
