@@ -157,6 +157,23 @@ def test_gemv_few_rows_fixed_point_combine(pkg, oracle, gpu, layout, act, M):
     assert float((a == four[:M]).float().mean()) > 0.9
 
 
+@pytest.mark.parametrize("gs", [32, 64, 128, -1])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M", [17, 20])
+def test_gemv_two_row_blocks(pkg, oracle, gpu, M, dtype, gs):
+    """17..20 rows on the contiguous-group decode kernel: one workgroup runs two MFMA row blocks
+    per unpacked word (rows 16.. are the second block; its dead rows stay out of the output)."""
+    _run(pkg, oracle, gpu, 2048, 512, gs, M, dtype=dtype, sym=False, bias=(M == 20), path=1, seed=M + 3)
+
+
+@pytest.mark.parametrize("K,N", [(4096, 4096), (14336, 4096), (4096, 14336)])
+def test_gemv_two_row_blocks_llama_shapes(pkg, oracle, gpu, K, N):
+    qw, qz, sc, _ = oracle.make_gptq(K, N, 128, seed=1)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
+    assert pkg.ops.select_path(pk, 18) == "gemv"
+    _run(pkg, oracle, gpu, K, N, 128, 18, sym=False, seed=K // 128 + 18)
+
+
 def test_gemv_single_row_non_finite_input_leaves_the_cells_clean(pkg, oracle, gpu):
     """inf / NaN activations in different K splits make every output non-finite (as in the
     reference; opposite infinities must not cancel) and must not leave anything behind in the

@@ -93,7 +93,7 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
     // 14336 x 4096 30.5 / 23.5 (at M = 17: 25.7 / 22.9).  From the third block on (M = 48) the
     // GEMM wins except on the smallest matrices (4096 x 4096: 12.6 / 17.9 at M = 64, 24.4 / 20.8
     // at M = 96; 2048 x 8192: 10.8 / 15.2 at M = 64).
-    const bool small = M <= 16 || (M <= 32 && w->K <= 8192 && weights <= (1L << 26)) ||
+    const bool small = M <= 16 || gemv_rows32_supported(w, M) || (M <= 32 && w->K <= 8192 && weights <= (1L << 26)) ||
                        (M <= 64 && weights <= (1L << 24));
     if (small && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
     if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;
@@ -258,6 +258,7 @@ int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, 
     return Q4_ERR_INVALID_ARGUMENT;
   }
   GemvConfig cfg{wcol, wk, splits, words};
+  if (words == 4 && gemv_rows32_supported(w, M)) cfg.rows_per_block = 32;  // as q4_linear would
   return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, &cfg, (hipStream_t)stream);
 }
 

@@ -187,8 +187,10 @@ struct GemvConfig {
   int wk;      // waves across K in a workgroup
   int splits;  // workgroups across K (cross-workgroup reduction through the workspace)
   int words;   // GPTQ contiguous-group kernel: packed words per lane (4, 2, 1 -> 64/32/16-column tiles)
+  int rows_per_block = 16;  // 32: GPTQ contiguous-group kernel with two MFMA row blocks (17..32 rows)
 };
 bool gemv_supported(const q4_weight* w, int M, int dtype);
+bool gemv_rows32_supported(const q4_weight* w, int M);
 GemvConfig gemv_pick_config(const q4_weight* w, int M);
 GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up);
 int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,

@@ -49,6 +49,22 @@ bool gemv_gate_up_supported(const q4_weight* w, int M, int dtype) {
          M <= 2 && gemv_supported(w, M, dtype);
 }
 
+// 17..20 rows on the contiguous-group kernel: one workgroup takes all of them (two MFMA row
+// blocks per unpacked word) with the configuration of 16 rows, when its slab still fits.
+// Measured against the GEMM / two 16-row workgroups at M = 17: 14336 x 4096 18.0 against
+// 22.8 us, 4096 x 28672 21.8 / 29.0, 8192 x 8192 18.2 / 20.9, 8192 x 28672 45.6 / 49.8.  The
+// slab, its staging and the partial sums grow with every row: once the slab forces more K
+// splits than 16 rows take (4096 x 28672 from 19 rows, 14336 x 4096 from 21) the kernel
+// loses (M = 24: 33.5 against 29.6 us, 29.5 against 23.2 us).
+bool gemv_rows32_supported(const q4_weight* w, int M) {
+  if (!(w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && M > 16 && M <= 20 && w->groupsize >= 32)) return false;
+  if (!gemv_supported(w, 16, Q4_DTYPE_F16)) return false;
+  const GemvConfig c = gemv_pick_config(w, 16, false);
+  const long chunks = w->K / 128;
+  const long kr = (chunks + c.splits - 1) / c.splits * 128;
+  return (long)M * (kr * 2 + 16) <= 150000;
+}
+
 GemvConfig gemv_pick_config(const q4_weight* w, int M) { return gemv_pick_config(w, M, false); }
 
 GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
@@ -58,8 +74,13 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   // activation slab (rows x K/splits) must fit its share of LDS.
   GemvConfig c;
   c.words = 4;
-  const int rows = M < q4::kRowsPerBlock ? M : q4::kRowsPerBlock;
-  const int mchunks = (M + q4::kRowsPerBlock - 1) / q4::kRowsPerBlock;
+  if (!gate_up && gemv_rows32_supported(w, M)) {
+    c = gemv_pick_config(w, 16, false);
+    c.rows_per_block = 32;
+    return c;
+  }
+  const int rows = M < c.rows_per_block ? M : c.rows_per_block;
+  const int mchunks = (M + c.rows_per_block - 1) / c.rows_per_block;
   const int chunks = w->K / 128;
   c.wcol = 1;
   c.wk = chunks >= 4 ? 4 : (chunks >= 2 ? 2 : 1);
@@ -257,6 +278,18 @@ static void launch_rmax(const q4_weight* w, const GemvParams& gp, int words, dim
   }
 }
 
+// 32 rows per workgroup: contiguous-group kernel, 64-column waves
+template <int DTYPE>
+static void launch_rows32(const q4_weight* w, const GemvParams& gp, dim3 grid, dim3 block, size_t smem,
+                          hipStream_t stream) {
+  using namespace q4;
+  const int gs = w->groupsize;
+  if (gs == 128) launch_kernel(gemv_gptq_kernel<DTYPE, 8, 4, true, 4>, gp, grid, block, smem, stream);
+  else if (gs > 128) launch_kernel(gemv_gptq_kernel<DTYPE, 8, 4, false, 4>, gp, grid, block, smem, stream);
+  else if (gs == 64) launch_kernel(gemv_gptq_kernel<DTYPE, 8, 2, false, 4>, gp, grid, block, smem, stream);
+  else launch_kernel(gemv_gptq_kernel<DTYPE, 8, 1, false, 4>, gp, grid, block, smem, stream);
+}
+
 int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                 void* workspace, size_t workspace_bytes, const GemvConfig* cfg_in,
                 hipStream_t stream, int gate_up_act) {
@@ -288,8 +321,14 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
               cfg.splits, w->K, w->N);
     return Q4_ERR_INVALID_ARGUMENT;
   }
-  const int rows = M < kRowsPerBlock ? M : kRowsPerBlock;
-  const int mchunks = (M + kRowsPerBlock - 1) / kRowsPerBlock;
+  if (cfg.rows_per_block != 16 && !(cfg.rows_per_block == 32 && contiguous && gate_up_act == 0 && cfg.words == 4)) {
+    set_error("q4_linear(gemv): %d rows per workgroup need the contiguous-group kernel with 64-column waves",
+              cfg.rows_per_block);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  const int rpb = cfg.rows_per_block;
+  const int rows = M < rpb ? M : rpb;
+  const int mchunks = (M + rpb - 1) / rpb;
   // largest K range of a workgroup: K goes out in 128-row chunks over splits x wk wave slots
   const long kchunks = w->K / 128, kslots = (long)cfg.splits * cfg.wk;
   int KR = 0;
@@ -298,7 +337,7 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
     if (r > KR) KR = r;
   }
   const int slab_stride = KR * 2 + 16;
-  const int rmax = M <= 1 ? 1 : (M <= 2 ? 2 : 4);
+  const int rmax = rpb == 32 ? 8 : (M <= 1 ? 1 : (M <= 2 ? 2 : 4));
   const int nt = awq ? 16 : cfg.words;
   const size_t slab_bytes = ((size_t)rows * slab_stride + 15) & ~(size_t)15;
   size_t smem = slab_bytes;
@@ -355,11 +394,15 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.slab_bytes = (int)slab_bytes;
   gp.kr_max = KR;
   gp.partial_rows = M;
+  gp.rows_per_block = rpb;
   gp.moe = q4::MoeView{};
   dim3 grid((unsigned)(ntiles * cfg.splits), (unsigned)mchunks);
   dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
   if (gate_up_act != 0) {
     launch_gemv_gate_up(gp, dtype, rmax, w->groupsize == 128, grid, block, smem, stream, false);
+  } else if (rmax == 8) {
+    if (dtype == Q4_DTYPE_F16) launch_rows32<Q4_DTYPE_F16>(w, gp, grid, block, smem, stream);
+    else launch_rows32<Q4_DTYPE_BF16>(w, gp, grid, block, smem, stream);
   } else if (dtype == Q4_DTYPE_F16) {
     if (rmax == 1) launch_rmax<Q4_DTYPE_F16, 1>(w, gp, cfg.words, grid, block, smem, stream);
     else if (rmax == 2) launch_rmax<Q4_DTYPE_F16, 2>(w, gp, cfg.words, grid, block, smem, stream);

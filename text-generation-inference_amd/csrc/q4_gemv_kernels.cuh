@@ -54,6 +54,7 @@ struct GemvParams {
   int slab_bytes;   // size of the activation slab region
   int kr_max;        // largest K range of a workgroup (K is dealt out in 128-row chunks)
   int partial_rows;  // rows of one split's slice of `partials` (M; grouped launches: all pairs)
+  int rows_per_block;  // activation rows per workgroup: 16, or 32 (two MFMA row blocks per unpacked word)
   MoeView moe;       // grouped launches only (MOE kernels): blockIdx.z is the expert
 };
 
@@ -147,8 +148,8 @@ __device__ __forceinline__ Decomp make_decomp(const GemvParams& gp, int wave_col
   d.kw0 = c0 * kChunkRows;
   d.KW = (c1 - c0) * kChunkRows;
   d.kwo = d.kw0 - d.kwg0;
-  d.mb = blockIdx.y * kRowsPerBlock;
-  d.mloc = min(kRowsPerBlock, gp.p.M - d.mb);
+  d.mb = blockIdx.y * gp.rows_per_block;
+  d.mloc = min(gp.rows_per_block, gp.p.M - d.mb);
   return d;
 }
 
@@ -159,9 +160,9 @@ __device__ __forceinline__ bool moe_enter_decode(GemvParams& gp, const int32_t*&
   const int row0 = moe_enter(gp.p, gp.moe, blockIdx.z);
   // the gated-MLP epilogue writes N / 2 columns per row
   if (half_width_output) gp.p.y = (uint16_t*)gp.p.y - (size_t)row0 * (gp.p.N >> 1);
-  if (gp.p.M <= (int)blockIdx.y * kRowsPerBlock) return false;
+  if (gp.p.M <= (int)blockIdx.y * gp.rows_per_block) return false;
   gp.partials += (size_t)row0 * gp.p.N;
-  rows = gp.moe.x_rows != nullptr ? gp.moe.x_rows + row0 + blockIdx.y * kRowsPerBlock : nullptr;
+  rows = gp.moe.x_rows != nullptr ? gp.moe.x_rows + row0 + blockIdx.y * gp.rows_per_block : nullptr;
   return true;
 }
 
@@ -219,7 +220,11 @@ struct SlabStager {
   }
 };
 
-// Everything after the K loop.  out[t][r] is the fp32 sum of output row 4*kq + r (relative
+// Row (relative to the workgroup's first) of accumulator slot r of a lane: an MFMA row block
+// gives a lane rows 4*kq .. 4*kq + 3; slots 4..7 are the second block of 16 rows.
+__device__ __forceinline__ int out_row(const Decomp& d, int r) { return 4 * d.kq + (r & 3) + ((r >> 2) << 4); }
+
+// Everything after the K loop.  out[t][r] is the fp32 sum of output row out_row(r) (relative
 // to the workgroup's first row) and column col0 + t: every lane owns NT adjacent columns.
 // FUSE (NT = 8): gated-MLP epilogue.  out[0..3] are four gate columns col0 .. col0 + 3 and
 // out[4..7] the matching up columns N/2 + col0 ..; the output is act(gate) * up, [M, N/2].
@@ -259,7 +264,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
       if (d.wkk == 0) {
 #pragma unroll
         for (int r = 0; r < RMAX; ++r) {
-          const int m = 4 * d.kq + r;
+          const int m = out_row(d, r);
           if (m < d.mloc) {
             uint32_t o[NT / 2];
 #pragma unroll
@@ -282,7 +287,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
     if (d.wkk == 0) {
 #pragma unroll
       for (int r = 0; r < RMAX; ++r) {
-        const int m = 4 * d.kq + r;
+        const int m = out_row(d, r);
         if (m < d.mloc) {
           uint16_t* dst = y + (size_t)(d.mb + m) * N + col0;
           uint16_t o[NT];
@@ -335,7 +340,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
           float* tile = (float*)smem + (size_t)(gp.wk - 1) * gp.wcol * NT * RMAX * 64 + (size_t)d.wc * TILE_ROWS * TW;
 #pragma unroll
           for (int r = 0; r < RMAX; ++r) {
-            const int m = 4 * d.kq + r;
+            const int m = out_row(d, r);
             if (m < d.mloc) {
 #pragma unroll
               for (int t = 0; t < NT; ++t) tile[m * TW + d.j * NT + t] = out[t][r];
@@ -373,7 +378,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
         unsigned long long* cells = gp.cells;
 #pragma unroll
         for (int r = 0; r < RMAX; ++r) {
-          const int m = 4 * d.kq + r;
+          const int m = out_row(d, r);
           if (m < d.mloc) {
             unsigned long long* cell = cells + (size_t)(d.mb + m) * N + col0;
             unsigned long long before[NT], inc[NT];
@@ -411,7 +416,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
   if (d.wkk == 0) {
 #pragma unroll
     for (int r = 0; r < RMAX; ++r) {
-      const int m = 4 * d.kq + r;
+      const int m = out_row(d, r);
       if (m < d.mloc) {
         float* dst = gp.partials + ((size_t)d.split * gp.partial_rows + d.mb + m) * N + col0;
 #pragma unroll
@@ -619,13 +624,22 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   __syncthreads();
 
   const bool row_live = d.j < d.mloc;  // A-operand row of this lane
+  // RMAX = 8: a second block of 16 activation rows takes the same unpacked weights
+  constexpr bool ROWS32 = RMAX == 8;
+  constexpr int R1 = RMAX < 4 ? RMAX : 4;  // live accumulator slots of the first block
+  const bool row_live2 = ROWS32 && 16 + d.j < d.mloc;
   const unsigned char* a_base =
       smem + (size_t)d.j * gp.slab_stride + (size_t)(d.kwo + d.kq * 8) * 2;
 
   const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   float4_t tot[WORDS], acc[WORDS];
+  float4_t tot2[ROWS32 ? WORDS : 1], acc2[ROWS32 ? WORDS : 1];
 #pragma unroll
   for (int t = 0; t < WORDS; ++t) tot[t] = acc[t] = zero4;
+  if constexpr (ROWS32) {
+#pragma unroll
+    for (int t = 0; t < WORDS; ++t) tot2[t] = acc2[t] = zero4;
+  }
   half2_t czlo[WORDS], czhi[WORDS];
   const SpliceConsts splice = splice_consts();
 
@@ -658,15 +672,24 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
       }
       uint4_t a = {0u, 0u, 0u, 0u};
       if (row_live) a = *(const uint4_t*)(a_base + (size_t)(c * kChunkRows + st * 32) * 2);
+      uint4_t a2 = {0u, 0u, 0u, 0u};
+      if constexpr (ROWS32) {
+        if (row_live2) a2 = *(const uint4_t*)(a_base + (size_t)16 * gp.slab_stride + (size_t)(c * kChunkRows + st * 32) * 2);
+      }
 #pragma unroll
       for (int t = 0; t < WORDS; ++t) {
         half2_t b[4];
         unpack_word_f16(w[st].v[t], czlo[t], czhi[t], splice, b);
         if (first && kStaticGroups) {
           acc[t] = mfma16<DTYPE>(a, b, zero4);
+          if constexpr (ROWS32) acc2[t] = mfma16<DTYPE>(a2, b, zero4);
         } else {
           if (first && group_start) acc[t] = zero4;
           acc[t] = mfma16<DTYPE>(a, b, acc[t]);
+          if constexpr (ROWS32) {
+            if (first && group_start) acc2[t] = zero4;
+            acc2[t] = mfma16<DTYPE>(a2, b, acc2[t]);
+          }
         }
       }
       if (last && (kStaticGroups || group_end)) {
@@ -675,7 +698,11 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
           const half2_t pr = as_half2(s[gi].v[t >> 1]);
           const float sf = (float)((t & 1) ? pr.y : pr.x);
 #pragma unroll
-          for (int r = 0; r < RMAX; ++r) tot[t][r] = fmaf(sf, acc[t][r], tot[t][r]);
+          for (int r = 0; r < R1; ++r) tot[t][r] = fmaf(sf, acc[t][r], tot[t][r]);
+          if constexpr (ROWS32) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) tot2[t][r] = fmaf(sf, acc2[t][r], tot2[t][r]);
+          }
         }
       }
     }
@@ -697,7 +724,10 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
 #pragma unroll
   for (int t = 0; t < WORDS; ++t)
 #pragma unroll
-    for (int r = 0; r < RMAX; ++r) out[t][r] = tot[t][r];
+    for (int r = 0; r < RMAX; ++r) {
+      if constexpr (ROWS32) out[t][r] = r < 4 ? tot[t][r & 3] : tot2[t][r & 3];
+      else out[t][r] = tot[t][r];
+    }
   gemv_finish<DTYPE, WORDS, RMAX, FUSE>(gp, d, out, nl, smem);
 }
 

@@ -441,6 +441,7 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
     gp.splits = cfg.splits;
     gp.cells = nullptr;
     gp.fixed_point_split = 0;
+    gp.rows_per_block = kRowsPerBlock;
     gp.slab_stride = pl.kr_max * 2 + 16;
     gp.kr_max = pl.kr_max;
     gp.slab_bytes = (int)pl.slab_bytes;
