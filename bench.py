@@ -61,6 +61,8 @@ def parse_args():
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--gemm-m", type=int, default=2048)
     ap.add_argument("--no-moe", action="store_true", help="skip the mixture-of-experts block leg")
+    ap.add_argument("--no-batch", action="store_true",
+                    help="skip the batched-decode leg (GPTQ at 4..64 rows, AWQ and act-order at 1 and 16 rows)")
     ap.add_argument("--copies", type=int, default=0, help="weight copies to rotate over (0 = auto)")
     ap.add_argument("--no-dense-ref", action="store_true",
                     help="skip timing torch's dense fp16 matmul (hipBLASLt) on the GEMM shapes")
@@ -80,6 +82,22 @@ def make_weights(pkg, torch, device, K, N, seed):
     qzeros = torch.full((G, N // 8), 0x77777777, dtype=torch.int32, device=device)
     scales = (torch.rand((G, N), device=device, generator=g) * (2e-2 - 1e-3) + 1e-3).to(torch.float16)
     return pkg.ops.make_packed(qweight, qzeros, scales, None, GROUPSIZE, 0)
+
+
+def make_weights_variant(pkg, torch, device, K, N, seed, kind):
+    """The same synthetic tensors in the AWQ layout ("awq": qweight [K, N/8]) or as GPTQ with a
+    shuffled g_idx ("act_order")."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    G = K // GROUPSIZE
+    scales = (torch.rand((G, N), device=device, generator=g) * (2e-2 - 1e-3) + 1e-3).to(torch.float16)
+    qzeros = torch.full((G, N // 8), 0x77777777, dtype=torch.int32, device=device)
+    if kind == "awq":
+        qweight = torch.randint(-(2**31), 2**31 - 1, (K, N // 8), dtype=torch.int64, device=device, generator=g).to(torch.int32)
+        return pkg.ops.make_packed(qweight, qzeros, scales, None, GROUPSIZE, 1)
+    qweight = torch.randint(-(2**31), 2**31 - 1, (K // 8, N), dtype=torch.int64, device=device, generator=g).to(torch.int32)
+    g_idx = (torch.randperm(K, device=device, generator=g) // GROUPSIZE).to(torch.int32)
+    return pkg.ops.make_packed(qweight, qzeros, scales, g_idx, GROUPSIZE, 0)
 
 
 def time_kernel_launches(torch, fn_list, reps):
@@ -344,6 +362,36 @@ def main():
                              "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                              "frac": round(tot_f / tot_t / 1e12 / MFMA_PEAK_TFLOPS, 4), "traffic": None},
             }
+
+    # ---- batched decode: the same four projections with more activation rows (the serving
+    # batch), and the other two weight formats; us per step = sum over the four projections
+    if not args.no_batch:
+        batch = {}
+
+        def step_us(wlist, Mb):
+            tot = 0.0
+            paths = []
+            for i, (name, K, N) in enumerate(SHAPES):
+                xb = torch.randn((Mb, K), device=dev, dtype=torch.float16)
+                yb = torch.empty((Mb, N), device=dev, dtype=torch.float16)
+                fns = [(lambda c=c, i=i: pkg.ops.linear(wlist[c][i], xb, None, out=yb)) for c in range(len(wlist))]
+                avg, _ = time_kernel_launches(torch, fns, 48)
+                tot += avg
+                paths.append(pkg.ops.select_path(wlist[0][i], Mb))
+                del xb, yb
+            return {"us_per_step": round(tot * 1e6, 1), "weight_GBps": round(step_weight_bytes / tot / 1e9, 1),
+                    "paths": "/".join(paths)}
+
+        for Mb in (4, 16, 18, 32, 64):
+            batch[f"gptq_m{Mb}"] = step_us(weights, Mb)
+        for kind in ("awq", "act_order"):
+            wl = [[make_weights_variant(pkg, torch, dev, K, N, 31 * c + i, kind) for i, (_, K, N) in enumerate(SHAPES)]
+                  for c in range(min(copies, 3))]
+            for Mb in (1, 16):
+                batch[f"{kind}_m{Mb}"] = step_us(wl, Mb)
+            del wl
+            torch.cuda.empty_cache()
+        out["batched_decode"] = batch
 
     # ---- mixture-of-experts block (Mixtral-8x7B shapes: 8 experts, top-2, 4096 -> 2 x 14336 -> 4096):
     # routing, both grouped projections, activation and weighted sum, per block call
