@@ -258,7 +258,7 @@ int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, 
     return Q4_ERR_INVALID_ARGUMENT;
   }
   GemvConfig cfg{wcol, wk, splits, words};
-  if (words == 4 && gemv_rows32_supported(w, M)) cfg.rows_per_block = 32;  // as q4_linear would
+  if (words == 4 && gemv_rows32_kernel(w, M)) cfg.rows_per_block = 32;  // one workgroup for all rows
   return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, &cfg, (hipStream_t)stream);
 }
 

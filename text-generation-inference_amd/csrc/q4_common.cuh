@@ -191,6 +191,7 @@ struct GemvConfig {
 };
 bool gemv_supported(const q4_weight* w, int M, int dtype);
 bool gemv_rows32_supported(const q4_weight* w, int M);
+bool gemv_rows32_kernel(const q4_weight* w, int M);
 GemvConfig gemv_pick_config(const q4_weight* w, int M);
 GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up);
 int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,

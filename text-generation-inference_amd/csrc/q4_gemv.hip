@@ -56,8 +56,12 @@ bool gemv_gate_up_supported(const q4_weight* w, int M, int dtype) {
 // slab, its staging and the partial sums grow with every row: once the slab forces more K
 // splits than 16 rows take (4096 x 28672 from 19 rows, 14336 x 4096 from 21) the kernel
 // loses (M = 24: 33.5 against 29.6 us, 29.5 against 23.2 us).
+bool gemv_rows32_kernel(const q4_weight* w, int M) {
+  return w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && M > 16 && M <= 32 && w->groupsize >= 32;
+}
+
 bool gemv_rows32_supported(const q4_weight* w, int M) {
-  if (!(w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && M > 16 && M <= 20 && w->groupsize >= 32)) return false;
+  if (!gemv_rows32_kernel(w, M) || M > 20) return false;
   if (!gemv_supported(w, 16, Q4_DTYPE_F16)) return false;
   const GemvConfig c = gemv_pick_config(w, 16, false);
   const long chunks = w->K / 128;
