@@ -113,6 +113,22 @@ int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, i
 int q4_linear_gate_up(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                       int act, void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * Act-order by row order instead of per-weight lookups, as the reference's exllamav2 path does
+ * (QMatrix::make_sequential and make_sequential_kernel,
+ * server/exllamav2_kernels/exllamav2_kernels/cuda/q_matrix.cu:524-640; activations read
+ * through b_q_perm, cuda/q_gemm_kernel_gptq.cuh:116).  With perm = a stable argsort of g_idx,
+ * q4_gptq_make_sequential writes qweight_out whose packed row i holds checkpoint row perm[i]
+ * (GPTQ layout, [K/8, N], once at load time; qzeros and scales are unchanged).  When every group
+ * has exactly `groupsize` rows the result is a contiguous-group matrix: pass it with g_idx = NULL
+ * and feed q4_linear the activations in the same order, x_seq[m][i] = x[m][perm[i]], which
+ * q4_gather_columns produces (16-bit elements, [M, K], K a multiple of 8).  Indices outside
+ * 0..K-1 are clamped.
+ */
+int q4_gptq_make_sequential(const uint32_t* qweight, const int32_t* perm, uint32_t* qweight_out, int K, int N,
+                            void* stream);
+int q4_gather_columns(const void* x, const int32_t* perm, void* out, int M, int K, void* stream);
+
 /* y[M, inter] = act(gate_up[:, :inter]) * gate_up[:, inter:] for gate_up [M, 2 * inter]. */
 int q4_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, void* stream);
 

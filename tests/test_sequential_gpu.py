@@ -1,0 +1,125 @@
+"""Act-order by row order: q4_gptq_make_sequential + q4_gather_columns (exllamav2's
+make_sequential / q_perm, q_matrix.cu:524-640) against the oracle.
+
+The repacked matrix is pinned by what the layout fixes: unpacking its rows with the oracle's
+independent unpacker must give exactly the checkpoint rows in perm order, the dequantized matrix
+handed back in checkpoint order must equal the oracle's act-order dequantization bit for bit,
+and the forward must agree with the oracle like every other path (and with the table-lookup
+kernels, which take the same weights in checkpoint order)."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-3
+
+
+def to_dev(a, gpu):
+    if a is None:
+        return None
+    if a.dtype == np.uint32:
+        a = a.view(np.int32)
+    return torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+
+
+def max_rel_err(got, ref):
+    return float(np.abs(got - ref).max() / max(1e-6, np.abs(ref).max()))
+
+
+def build(pkg, oracle, gpu, K, N, gs, seed):
+    qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=seed, sym=False, act_order=True)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), gs, 0)
+    return qw, qz, sc, gi, pk
+
+
+@pytest.mark.parametrize("K,N,gs", [(256, 64, 32), (1024, 512, 128), (4096, 1024, 128), (512, 264, 64)])
+def test_rows_are_the_checkpoint_rows_in_group_order(pkg, oracle, gpu, K, N, gs):
+    qw, qz, sc, gi, pk = build(pkg, oracle, gpu, K, N, gs, seed=K + N)
+    seq = pkg.ops.make_sequential(pk)
+    assert seq is not None and seq.g_idx is None and seq.perm.dtype == torch.int32
+    perm = seq.perm.cpu().numpy()
+    assert sorted(perm.tolist()) == list(range(K))
+    assert np.array_equal(gi[perm], np.arange(K) // gs)          # group order
+    assert all(np.all(np.diff(perm[g * gs:(g + 1) * gs]) > 0) for g in range(K // gs))  # stable
+    rows = oracle.unpack_rows(qw)
+    got = oracle.unpack_rows(seq.qweight.cpu().numpy())
+    assert np.array_equal(got, rows[perm])
+    # dequantized and handed back in checkpoint order: the act-order matrix, bit for bit
+    want = oracle.dequant_gptq(qw, qz, sc, gi, gs, "f16")
+    w = pkg.ops.dequantize(seq)
+    assert np.array_equal(w.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 40, 300])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_forward_matches_oracle_and_table_kernels(pkg, oracle, gpu, M, dtype):
+    K, N, gs = 2048, 1024, 128
+    qw, qz, sc, gi, pk = build(pkg, oracle, gpu, K, N, gs, seed=M)
+    seq = pkg.ops.make_sequential(pk)
+    bf = dtype == "bf16"
+    w = oracle.dequant_gptq(qw, qz, sc, gi, gs, dtype)
+    xh = oracle.make_x(M, K, seed=M + 1, dtype=dtype)
+    x = torch.from_numpy(xh.view(np.int16)).to(gpu).view(torch.bfloat16) if bf else to_dev(xh, gpu)
+    y32, _ = oracle.linear_forward(xh, w, None, dtype)
+    got = pkg.ops.linear(seq, x)
+    g = got.float().cpu().numpy()
+    assert max_rel_err(g, y32) <= (8e-3 if bf else TOL)
+    if not bf:  # the table-lookup decode kernel is fp16 only
+        ref = pkg.ops.linear(pk, x).float().cpu().numpy()
+        assert max_rel_err(g, ref) <= TOL
+
+
+def test_gather_columns_is_exact(pkg, gpu):
+    g = torch.Generator(device=gpu).manual_seed(3)
+    x = torch.randn((37, 1024), device=gpu, dtype=torch.float16, generator=g)
+    perm = torch.randperm(1024, device=gpu, generator=g).to(torch.int32)
+    assert torch.equal(pkg.ops.gather_columns(x, perm), x[:, perm.long()])
+    xb = x.to(torch.bfloat16)
+    assert torch.equal(pkg.ops.gather_columns(xb, perm), xb[:, perm.long()])
+
+
+def test_groups_of_unequal_size_are_left_alone(pkg, oracle, gpu):
+    """A g_idx whose groups do not all hold `groupsize` rows cannot become contiguous."""
+    K, N, gs = 512, 64, 128
+    qw, qz, sc, gi, _ = build(pkg, oracle, gpu, K, N, gs, seed=1)
+    gi = gi.copy()
+    gi[np.flatnonzero(gi == 1)[0]] = 0  # group 0 gets 129 rows
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), gs, 0)
+    assert pkg.ops.make_sequential(pk) is None
+
+
+def test_argument_validation(pkg, gpu):
+    lib = pkg._lib.load()
+    L = pkg._lib
+    t = torch.zeros(64, dtype=torch.int32, device=gpu)
+    assert lib.q4_gptq_make_sequential(None, t.data_ptr(), t.data_ptr(), 64, 8, None) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_gptq_make_sequential(t.data_ptr(), t.data_ptr(), t.data_ptr(), 64, 8, None) == L.ERR_INVALID_ARGUMENT
+    o = torch.zeros(64, dtype=torch.int32, device=gpu)
+    assert lib.q4_gptq_make_sequential(t.data_ptr(), t.data_ptr(), o.data_ptr(), 60, 8, None) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_gather_columns(t.data_ptr(), t.data_ptr(), o.data_ptr(), 1, 12, None) == L.ERR_UNSUPPORTED
+    assert lib.q4_gather_columns(t.data_ptr(), t.data_ptr(), o.data_ptr(), 0, 12, None) == 0
+
+
+def test_quant_linear_repacks_once_and_keeps_memory_flat(pkg, oracle, gpu):
+    K, N, gs = 1024, 256, 128
+    qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=5, sym=False, act_order=True)
+    layer = pkg.QuantLinear(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), None, 4, gs)
+    xh = oracle.make_x(4, K, seed=9)
+    x = to_dev(xh, gpu)
+    y1 = layer(x)
+    assert layer.q_perm is not None and layer.packed().g_idx is None
+    first = layer.qweight.data_ptr()
+    y2 = layer(x)
+    assert layer.qweight.data_ptr() == first and torch.equal(y1, y2)
+    w = oracle.dequant_gptq(qw, qz, sc, gi, gs, "f16")
+    y32, _ = oracle.linear_forward(xh, w, None, "f16")
+    assert max_rel_err(y1.float().cpu().numpy(), y32) <= TOL
+    assert np.array_equal(layer.dequantize().cpu().numpy().view(np.uint16), w.view(np.uint16))
+    # a copy of the module (new storage) keeps working: the permutation travels as a buffer
+    import copy
+    twin = copy.deepcopy(layer)
+    assert torch.equal(twin(x), y1)

@@ -86,6 +86,8 @@ SIGNATURES = {
         [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),
     "q4_act_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "q4_gptq_make_sequential": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "q4_gather_columns": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "q4_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "q4_select_path": (c_int, [POINTER(Q4Weight), c_int, c_int]),
     "q4_moe_route": (

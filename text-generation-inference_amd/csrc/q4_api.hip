@@ -242,6 +242,40 @@ int q4_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int ac
   return launch_act_mul(gate_up, y, M, inter, dtype, act, (hipStream_t)stream);
 }
 
+int q4_gptq_make_sequential(const uint32_t* qweight, const int32_t* perm, uint32_t* qweight_out, int K, int N,
+                            void* stream) {
+  if (qweight == nullptr || perm == nullptr || qweight_out == nullptr || qweight == qweight_out) {
+    set_error("q4_gptq_make_sequential: null pointer, or output aliasing the input");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (K < 8 || K % 8 != 0 || N < 1) {
+    set_error("q4_gptq_make_sequential: K=%d must be a positive multiple of 8, N=%d positive", K, N);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (K / 8 > 65535) {
+    set_error("q4_gptq_make_sequential: K=%d has more than 65535 packed rows", K);
+    return Q4_ERR_UNSUPPORTED;
+  }
+  return launch_make_sequential(qweight, perm, qweight_out, K, N, (hipStream_t)stream);
+}
+
+int q4_gather_columns(const void* x, const int32_t* perm, void* out, int M, int K, void* stream) {
+  if (M < 0 || K < 0) {
+    set_error("q4_gather_columns: negative M=%d or K=%d", M, K);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M == 0 || K == 0) return Q4_OK;
+  if (x == nullptr || perm == nullptr || out == nullptr || x == out) {
+    set_error("q4_gather_columns: null pointer, or output aliasing the input");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (K % 8 != 0) {
+    set_error("q4_gather_columns: K=%d must be a multiple of 8", K);
+    return Q4_ERR_UNSUPPORTED;
+  }
+  return launch_gather_columns(x, perm, out, M, K, (hipStream_t)stream);
+}
+
 int q4_linear(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
               void* workspace, size_t workspace_bytes, void* stream) {
   return q4_linear_ex(w, x, bias, y, M, dtype, workspace, workspace_bytes, Q4_PATH_AUTO, stream);

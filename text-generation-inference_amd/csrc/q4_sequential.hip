@@ -1,0 +1,85 @@
+// Act-order without per-weight lookups: the rows of a GPTQ matrix are put into group order
+// once at load time and the activation columns follow the same order at run time, after which
+// the contiguous-group kernels apply.  The reference's exllamav2 path does the same
+// (QMatrix::make_sequential + make_sequential_kernel, cuda/q_matrix.cu:524-640, and the
+// b_q_perm gather of the activations in its GEMM, cuda/q_gemm_kernel_gptq.cuh:116).
+#include "q4_common.cuh"
+
+namespace q4 {
+
+// out word (r, n) = nibbles of source rows perm[8r .. 8r+7] of column n.  One thread per
+// column and packed row: the eight source words are coalesced along n.
+__global__ __launch_bounds__(256) void make_sequential_kernel(const uint32_t* __restrict__ qweight,
+                                                              const int32_t* __restrict__ perm,
+                                                              uint32_t* __restrict__ out, int K, int N) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  const int r = blockIdx.y;
+  if (n >= N) return;
+  uint32_t word = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int src = min(max(perm[8 * r + i], 0), K - 1);  // a bad index reads a wrong row, never outside
+    const uint32_t w = qweight[(size_t)(src >> 3) * N + n];
+    word |= ((w >> ((src & 7) * 4)) & 0xFu) << (4 * i);
+  }
+  out[(size_t)r * N + n] = word;
+}
+
+// out[m][i] = x[m][perm[i]] for 16-bit elements.  A thread gathers eight neighbours of the output
+// row (one 16-byte store); the reads hit a row of x that stays in L2.
+__global__ __launch_bounds__(256) void gather_columns_kernel(const uint16_t* __restrict__ x,
+                                                             const int32_t* __restrict__ perm,
+                                                             uint16_t* __restrict__ out, int M, int K) {
+  const int vec_per_row = K >> 3;
+  const long total = (long)M * vec_per_row;
+  for (long v = (long)blockIdx.x * blockDim.x + threadIdx.x; v < total; v += (long)gridDim.x * blockDim.x) {
+    const long m = v / vec_per_row;
+    const int c = (int)(v - m * vec_per_row) * 8;
+    const uint16_t* row = x + (size_t)m * K;
+    const uint4_t p0 = *(const uint4_t*)(perm + c);
+    const uint4_t p1 = *(const uint4_t*)(perm + c + 4);
+    const uint32_t idx[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+    uint32_t h[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = row[min(idx[i], (uint32_t)(K - 1))];
+    uint4_t o;
+    o.x = h[0] | (h[1] << 16);
+    o.y = h[2] | (h[3] << 16);
+    o.z = h[4] | (h[5] << 16);
+    o.w = h[6] | (h[7] << 16);
+    *(uint4_t*)(out + (size_t)m * K + c) = o;
+  }
+}
+
+}  // namespace q4
+
+namespace q4host {
+
+int launch_make_sequential(const uint32_t* qweight, const int32_t* perm, uint32_t* out, int K, int N,
+                           hipStream_t stream) {
+  dim3 grid((unsigned)((N + 255) / 256), (unsigned)(K / 8));
+  hipLaunchKernelGGL(q4::make_sequential_kernel, grid, dim3(256), 0, stream, qweight, perm, out, K, N);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    set_error("q4_gptq_make_sequential: launch failed: %s", hipGetErrorString(err));
+    return Q4_ERR_LAUNCH;
+  }
+  return Q4_OK;
+}
+
+int launch_gather_columns(const void* x, const int32_t* perm, void* out, int M, int K, hipStream_t stream) {
+  const long total = (long)M * (K / 8);
+  long blocks = (total + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(q4::gather_columns_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t*)x, perm,
+                     (uint16_t*)out, M, K);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    set_error("q4_gather_columns: launch failed: %s", hipGetErrorString(err));
+    return Q4_ERR_LAUNCH;
+  }
+  return Q4_OK;
+}
+
+}  // namespace q4host

@@ -10,6 +10,7 @@ the HIP library's q4_linear instead of the Triton kernel.
 from __future__ import annotations
 
 import math
+import os
 from typing import Optional
 
 import numpy as np
@@ -18,6 +19,12 @@ import torch.nn as nn
 
 from ... import ops
 from ..._lib import LAYOUT_GPTQ
+
+
+# Act-order layers: "repack" puts the rows of qweight into group order once (what the
+# reference's exllama matrices do) so that the contiguous-group kernels apply; "table" keeps
+# the checkpoint order and uses the kernels that look up every weight's group.
+ACT_ORDER_MODE = os.environ.get("Q4_ACT_ORDER", "repack")
 
 
 def is_trivial_g_idx(g_idx: torch.Tensor, groupsize: int) -> bool:
@@ -54,6 +61,9 @@ class QuantLinear(nn.Module):
 
         self.outfeatures = qweight.shape[1]
         self.infeatures = qweight.shape[0] * 32 // self.bits
+        # set once the rows of qweight have been put into group order: row i is checkpoint row
+        # q_perm[i] and g_idx describes the stored (sequential) rows
+        self.register_buffer("q_perm", None)
         self._packed: Optional[ops.PackedWeight] = None
 
     @classmethod
@@ -84,6 +94,7 @@ class QuantLinear(nn.Module):
         """
         if g_idx is not None:
             self.g_idx = g_idx.clone()
+        self.q_perm = None  # the rows written below are in checkpoint order
         gi = self.g_idx.to(torch.int64).cpu()
         scales = scales.detach().cpu().t().contiguous()
         zeros = zeros.detach().cpu().t().contiguous()
@@ -114,6 +125,18 @@ class QuantLinear(nn.Module):
             if g_idx is not None and is_trivial_g_idx(g_idx, self.groupsize):
                 g_idx = None  # sequential groups: the kernels index by k // groupsize
             pk = ops.make_packed(self.qweight, self.qzeros, self.scales, g_idx, self.groupsize, LAYOUT_GPTQ)
+            if self.q_perm is not None:
+                pk.perm = self.q_perm.to(torch.int32).contiguous()
+            elif pk.g_idx is not None and ACT_ORDER_MODE != "table" and self.qweight.is_cuda:
+                seq = ops.make_sequential(pk)
+                if seq is not None:
+                    # like the reference's exllama matrix, the module now holds the reordered
+                    # rows (the checkpoint-order tensor is dropped: memory stays flat)
+                    K = self.infeatures
+                    self.qweight = seq.qweight
+                    self.g_idx = (torch.arange(K, device=seq.qweight.device, dtype=torch.int64) // pk.groupsize).to(torch.int32)
+                    self.q_perm = seq.perm
+                    pk = seq
             self._packed = pk
         return pk
 

@@ -49,6 +49,9 @@ class PackedWeight:
     groupsize: int
     num_groups: int
     layout: int
+    # Rows in group order (make_sequential): packed row i holds checkpoint row perm[i] and the
+    # kernels take the activation columns in that order; None for checkpoint order.
+    perm: Optional[torch.Tensor] = None
 
     def struct(self) -> Q4Weight:
         return Q4Weight(
@@ -111,6 +114,47 @@ def make_packed(qweight, qzeros, scales, g_idx, groupsize: int, layout: int) -> 
     )
 
 
+def make_sequential(w: PackedWeight) -> Optional[PackedWeight]:
+    """Act-order weight with its rows put into group order, or None when that is not possible.
+
+    What the reference's exllamav2 matrix does at load time (QMatrix::make_sequential,
+    exllamav2_kernels/cuda/q_matrix.cu:566-640): perm is the stable argsort of g_idx, packed row
+    i of the new qweight is checkpoint row perm[i], and the activations are read through perm.
+    The contiguous-group kernels then apply (decode 1.5-2x, prefill 2x faster than the kernels
+    that look every weight's group up).  Needs every group to hold exactly `groupsize` rows,
+    which a GPTQ act-order g_idx (a permutation of arange(K) // groupsize) does.  The new
+    qweight is a second [K/8, N] tensor; the caller drops the old one to keep memory flat.
+    Runs once per layer at load time (one device->host sync for the check).
+    """
+    if w.g_idx is None or w.layout != LAYOUT_GPTQ or w.perm is not None:
+        return None
+    _require_cuda(w.qweight, "qweight")
+    K = w.K
+    if K % 8 or w.num_groups * w.groupsize != K:
+        return None
+    g = w.g_idx.to(torch.int64)
+    perm = torch.argsort(g, stable=True)
+    expect = torch.arange(K, device=g.device, dtype=torch.int64) // w.groupsize
+    if not bool(torch.equal(g[perm], expect)):
+        return None
+    perm32 = perm.to(torch.int32).contiguous()
+    out = torch.empty_like(w.qweight)
+    with torch.cuda.device(w.qweight.device):
+        _lib.check(_lib.load().q4_gptq_make_sequential(
+            w.qweight.data_ptr(), perm32.data_ptr(), out.data_ptr(), K, w.N, _stream_handle(out.device)))
+    return PackedWeight(out, w.qzeros, w.scales, None, K, w.N, w.groupsize, w.num_groups, w.layout, perm32)
+
+
+def gather_columns(x: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:
+    """x[:, perm] for a contiguous fp16/bf16 [M, K] tensor, through the HIP gather kernel."""
+    out = torch.empty_like(x)
+    if x.numel():
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.load().q4_gather_columns(
+                x.data_ptr(), perm.data_ptr(), out.data_ptr(), x.shape[0], x.shape[1], _stream_handle(x.device)))
+    return out
+
+
 def _stream_handle(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
@@ -146,6 +190,10 @@ def dequantize(w: PackedWeight, dtype: torch.dtype = torch.float16) -> torch.Ten
         _lib.check(
             _lib.load().q4_dequant(ctypes.byref(st), out.data_ptr(), _DTYPES[dtype], _stream_handle(out.device))
         )
+    if w.perm is not None:  # rows are in group order: hand them back in checkpoint order
+        ordered = torch.empty_like(out)
+        ordered.index_copy_(0, w.perm.to(torch.int64), out)
+        return ordered
     return out
 
 
@@ -172,6 +220,8 @@ def linear(
     if x.dim() != 2 or x.shape[1] != w.K:
         raise ValueError(f"x must be [M, {w.K}], got {tuple(x.shape)}")
     x = x.contiguous()
+    if w.perm is not None:
+        x = gather_columns(x, w.perm)
     M = x.shape[0]
     if out is not None:
         if tuple(out.shape) != (M, w.N) or out.dtype != x.dtype or out.device != x.device or not out.is_contiguous():
@@ -266,6 +316,9 @@ def linear_gate_up(
     if act not in _lib.ACTIVATIONS:
         raise ValueError(f"unknown activation {act!r}; known: {sorted(_lib.ACTIVATIONS)}")
     x = x.contiguous()
+    if w.perm is not None:
+        x = gather_columns(x, w.perm)
+        w = PackedWeight(w.qweight, w.qzeros, w.scales, None, w.K, w.N, w.groupsize, w.num_groups, w.layout)
     M, inter = x.shape[0], w.N // 2
     y = out if out is not None else torch.empty((M, inter), dtype=x.dtype, device=x.device)
     if tuple(y.shape) != (M, inter) or y.dtype != x.dtype or y.device != x.device or not y.is_contiguous():
