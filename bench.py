@@ -384,9 +384,14 @@ def main():
 
         for Mb in (4, 16, 18, 32, 64):
             batch[f"gptq_m{Mb}"] = step_us(weights, Mb)
-        for kind in ("awq", "act_order"):
-            wl = [[make_weights_variant(pkg, torch, dev, K, N, 31 * c + i, kind) for i, (_, K, N) in enumerate(SHAPES)]
-                  for c in range(min(copies, 3))]
+        # act_order: rows put into group order at load time (what the layers do by default),
+        # x read through the permutation; act_order_lookup: checkpoint order, g_idx in the kernel
+        for kind in ("awq", "act_order", "act_order_lookup"):
+            wl = [[make_weights_variant(pkg, torch, dev, K, N, 31 * c + i, "awq" if kind == "awq" else "act_order")
+                   for i, (_, K, N) in enumerate(SHAPES)] for c in range(min(copies, 3))]
+            if kind == "act_order":
+                wl = [[pkg.ops.make_sequential(w) for w in row] for row in wl]
+                torch.cuda.empty_cache()
             for Mb in (1, 16):
                 batch[f"{kind}_m{Mb}"] = step_us(wl, Mb)
             del wl

@@ -128,6 +128,17 @@ int q4_linear_gate_up(const q4_weight* w, const void* x, const void* bias, void*
 int q4_gptq_make_sequential(const uint32_t* qweight, const int32_t* perm, uint32_t* qweight_out, int K, int N,
                             void* stream);
 int q4_gather_columns(const void* x, const int32_t* perm, void* out, int M, int K, void* stream);
+/*
+ * q4_linear for a weight in group order, x in checkpoint order: y = x[:, perm] @ W (+ bias).
+ * With one or two rows and K <= 4096 the decode kernel reads x through perm while it stages it
+ * (no extra pass, as the reference's kernel does with b_q_perm); otherwise x is gathered once
+ * into the tail of the workspace, which therefore must hold q4_workspace_bytes_perm(M, K, N)
+ * bytes (its head is the zero-initialised area of q4_workspace_bytes).  `path` as for q4_linear_ex; perm NULL
+ * makes this q4_linear_ex.
+ */
+int q4_linear_perm(const q4_weight* w, const int32_t* perm, const void* x, const void* bias, void* y, int M,
+                   int dtype, void* workspace, size_t workspace_bytes, int path, void* stream);
+size_t q4_workspace_bytes_perm(int M, int K, int N);
 
 /* y[M, inter] = act(gate_up[:, :inter]) * gate_up[:, inter:] for gate_up [M, 2 * inter]. */
 int q4_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, void* stream);

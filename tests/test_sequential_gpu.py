@@ -73,6 +73,42 @@ def test_forward_matches_oracle_and_table_kernels(pkg, oracle, gpu, M, dtype):
         assert max_rel_err(g, ref) <= TOL
 
 
+@pytest.mark.parametrize("path,M", [(1, 2), (1, 18), (1, 40), (2, 40), (2, 700), (3, 5)])
+def test_forced_paths_read_x_through_perm(pkg, oracle, gpu, path, M):
+    """Decode kernels gather while staging (one, two and several row blocks), the prefill and
+    generic paths gather into the workspace tail first: same result as gathering by hand."""
+    K, N, gs = 4096, 512, 128
+    qw, qz, sc, gi, pk = build(pkg, oracle, gpu, K, N, gs, seed=path * 100 + M)
+    seq = pkg.ops.make_sequential(pk)
+    x = to_dev(oracle.make_x(M, K, seed=M), gpu)
+    bias = to_dev(np.random.default_rng(M).standard_normal(N).astype(np.float16), gpu)
+    got = pkg.ops.linear(seq, x, bias, path=path)
+    plain = pkg.ops.PackedWeight(seq.qweight, seq.qzeros, seq.scales, None, K, N, gs, K // gs, 0)
+    want = pkg.ops.linear(plain, x[:, seq.perm.long()].contiguous(), bias, path=path)
+    assert torch.equal(got, want)
+    w = oracle.dequant_gptq(qw, qz, sc, gi, gs, "f16")
+    y32, _ = oracle.linear_forward(x.cpu().numpy(), w, bias.cpu().numpy(), "f16")
+    assert max_rel_err(got.float().cpu().numpy(), y32) <= TOL
+
+
+def test_prefill_with_perm_needs_the_larger_workspace(pkg, oracle, gpu):
+    import ctypes
+    K, N, gs, M = 1024, 256, 128, 64
+    qw, qz, sc, gi, pk = build(pkg, oracle, gpu, K, N, gs, seed=2)
+    seq = pkg.ops.make_sequential(pk)
+    lib = pkg._lib.load()
+    small = int(lib.q4_workspace_bytes(M, K, N))
+    assert int(lib.q4_workspace_bytes_perm(M, K, N)) >= small + M * K * 2
+    ws = torch.zeros(small, dtype=torch.uint8, device=gpu)
+    x = torch.zeros((M, K), dtype=torch.float16, device=gpu)
+    y = torch.zeros((M, N), dtype=torch.float16, device=gpu)
+    st = seq.struct()
+    rc = lib.q4_linear_perm(ctypes.byref(st), seq.perm.data_ptr(), x.data_ptr(), None, y.data_ptr(), M, 0,
+                            ws.data_ptr(), ws.numel(), 2, None)
+    assert rc == pkg._lib.ERR_WORKSPACE
+    assert b"q4_workspace_bytes_perm" in lib.q4_last_error()
+
+
 def test_gather_columns_is_exact(pkg, gpu):
     g = torch.Generator(device=gpu).manual_seed(3)
     x = torch.randn((37, 1024), device=gpu, dtype=torch.float16, generator=g)

@@ -88,6 +88,9 @@ SIGNATURES = {
     "q4_act_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "q4_gptq_make_sequential": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "q4_gather_columns": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "q4_linear_perm": (c_int, [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                                c_size_t, c_int, c_void_p]),
+    "q4_workspace_bytes_perm": (c_size_t, [c_int, c_int, c_int]),
     "q4_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "q4_select_path": (c_int, [POINTER(Q4Weight), c_int, c_int]),
     "q4_moe_route": (

@@ -193,6 +193,60 @@ int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, i
   }
 }
 
+static size_t perm_gather_offset(int M, int K, int N) {
+  return (q4_workspace_bytes(M, K, N) + 255) & ~(size_t)255;
+}
+
+size_t q4_workspace_bytes_perm(int M, int K, int N) {
+  if (M < 1 || K < 1 || N < 1) return q4_workspace_bytes(M, K, N);
+  return perm_gather_offset(M, K, N) + (size_t)M * K * 2;
+}
+
+int q4_linear_perm(const q4_weight* w, const int32_t* perm, const void* x, const void* bias, void* y, int M,
+                   int dtype, void* workspace, size_t workspace_bytes, int path, void* stream) {
+  if (perm == nullptr) return q4_linear_ex(w, x, bias, y, M, dtype, workspace, workspace_bytes, path, stream);
+  int rc = validate_weight(w, "q4_linear_perm");
+  if (rc == Q4_OK) rc = validate_dtype(dtype, "q4_linear_perm");
+  if (rc != Q4_OK) return rc;
+  if (w->layout != Q4_LAYOUT_GPTQ || w->g_idx != nullptr) {
+    set_error("q4_linear_perm: the weight must be a GPTQ matrix whose rows are in group order (g_idx NULL)");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M < 0) {
+    set_error("q4_linear_perm: negative M=%d", M);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M == 0 || w->N == 0) return Q4_OK;
+  if (y == nullptr || x == nullptr) {
+    set_error("q4_linear_perm: null x or y");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (path == Q4_PATH_AUTO) path = q4_select_path(w, M, dtype);
+  // Decode of one or two rows with a short K: the kernel reads x through perm while it stages
+  // its activation slab.  Every workgroup gathers its own copy, so the saved launch (~2.5 us)
+  // is soon outweighed: measured against the separate pass at M = 1, 4096 x 4096 6.4 / 7.8 us,
+  // 4096 x 28672 15.8 / 17.3, but 14336 x 4096 13.4 / 12.3, 28672 x 8192 29.0 / 26.0, and at
+  // M = 16 4096 x 6144 18.1 / 14.3, 14336 x 4096 37.9 / 20.0.
+  if (path == Q4_PATH_GEMV && M <= 2 && w->K <= 4096)
+    return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, nullptr, (hipStream_t)stream, 0, perm);
+  // otherwise one gather pass into the tail of the workspace, then the kernel of the plain call
+  if (w->K % 8 != 0) {
+    set_error("q4_linear_perm: K=%d must be a multiple of 8", w->K);
+    return Q4_ERR_UNSUPPORTED;
+  }
+  const size_t offset = perm_gather_offset(M, w->K, w->N);
+  const size_t need = offset + (size_t)M * w->K * 2;
+  if (workspace == nullptr || workspace_bytes < need) {
+    set_error("q4_linear_perm: workspace of %zu bytes needed (q4_workspace_bytes_perm), %zu given", need,
+              workspace_bytes);
+    return Q4_ERR_WORKSPACE;
+  }
+  void* x_seq = (char*)workspace + offset;
+  rc = launch_gather_columns(x, perm, x_seq, M, w->K, (hipStream_t)stream);
+  if (rc != Q4_OK) return rc;
+  return q4_linear_ex(w, x_seq, bias, y, M, dtype, workspace, offset, path, stream);
+}
+
 int q4_linear_gate_up(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                       int act, void* workspace, size_t workspace_bytes, void* stream) {
   int rc = validate_weight(w, "q4_linear_gate_up");

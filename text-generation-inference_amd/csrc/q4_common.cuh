@@ -147,6 +147,9 @@ struct Problem {
   // and y[M, N/2] = act(x @ gate (+ bias)) * (x @ up (+ bias)); only kernels that say so
   // support it.
   int gate_up_act;
+  // Decode kernels only: column of x behind every K row (x_seq[m][k] = x[m][x_perm[k]], the
+  // row order of a weight whose act-order rows were put into group order), or nullptr.
+  const int32_t* __restrict__ x_perm;
 };
 
 // Grouped launch over the experts of a mixture-of-experts layer.  The rows of the problem are
@@ -196,7 +199,7 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M);
 GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up);
 int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                 void* workspace, size_t workspace_bytes, const GemvConfig* cfg, hipStream_t stream,
-                int gate_up_act = 0);
+                int gate_up_act = 0, const int32_t* x_perm = nullptr);
 bool gemv_gate_up_supported(const q4_weight* w, int M, int dtype);
 int launch_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, hipStream_t stream);
 int launch_make_sequential(const uint32_t* qweight, const int32_t* perm, uint32_t* out, int K, int N, hipStream_t stream);

@@ -296,7 +296,7 @@ static void launch_rows32(const q4_weight* w, const GemvParams& gp, dim3 grid, d
 
 int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                 void* workspace, size_t workspace_bytes, const GemvConfig* cfg_in,
-                hipStream_t stream, int gate_up_act) {
+                hipStream_t stream, int gate_up_act, const int32_t* x_perm) {
   using namespace q4;
   if (gate_up_act != 0 && !gemv_gate_up_supported(w, M, dtype)) {
     set_error("q4_linear_gate_up(gemv): no fused decode kernel for this weight (layout=%d g_idx=%p N=%d groupsize=%d)",
@@ -368,6 +368,7 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, w->g_idx, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
   gp.p.gate_up_act = gate_up_act;
+  gp.p.x_perm = x_perm;
   gp.partials = partials;
   gp.tickets = tickets;
   gp.wcol = cfg.wcol;

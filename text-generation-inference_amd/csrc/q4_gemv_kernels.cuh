@@ -176,17 +176,32 @@ struct SlabStager {
   uint4_t xv[kLoads];
   const uint16_t* xs;
   const int32_t* rows;  // grouped launches: row of x behind every staged row, else nullptr
+  const int32_t* cols;  // column of x behind every K row of the workgroup's range, else nullptr
   int kb_per_row, items;
 
   __device__ __forceinline__ uint4_t fetch(const GemvParams& gp, int idx) const {
     const int m = idx / kb_per_row;
     const int kb = idx - m * kb_per_row;
     const int mr = rows != nullptr ? rows[m] : m;
+    if (cols != nullptr) {
+      // eight scattered columns of the row (it stays in L2); a bad index is clamped
+      const uint16_t* row = xs + (size_t)mr * gp.p.K;
+      const uint4_t p0 = *(const uint4_t*)(cols + kb * 8);
+      const uint4_t p1 = *(const uint4_t*)(cols + kb * 8 + 4);
+      const uint32_t last = (uint32_t)(gp.p.K - 1);
+      uint4_t o;
+      o.x = (uint32_t)row[min(p0.x, last)] | ((uint32_t)row[min(p0.y, last)] << 16);
+      o.y = (uint32_t)row[min(p0.z, last)] | ((uint32_t)row[min(p0.w, last)] << 16);
+      o.z = (uint32_t)row[min(p1.x, last)] | ((uint32_t)row[min(p1.y, last)] << 16);
+      o.w = (uint32_t)row[min(p1.z, last)] | ((uint32_t)row[min(p1.w, last)] << 16);
+      return o;
+    }
     return *(const uint4_t*)(xs + (size_t)mr * gp.p.K + kb * 8);
   }
   __device__ __forceinline__ void issue(const GemvParams& gp, const Decomp& d, const int32_t* row_map = nullptr) {
     rows = row_map;
-    xs = (const uint16_t*)gp.p.x + (row_map != nullptr ? 0 : (size_t)d.mb * gp.p.K) + d.kwg0;
+    cols = gp.p.x_perm != nullptr ? gp.p.x_perm + d.kwg0 : nullptr;
+    xs = (const uint16_t*)gp.p.x + (row_map != nullptr ? 0 : (size_t)d.mb * gp.p.K) + (cols != nullptr ? 0 : d.kwg0);
     kb_per_row = d.KR >> 3;
     items = d.mloc * kb_per_row;
 #pragma unroll

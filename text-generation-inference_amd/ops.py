@@ -220,8 +220,8 @@ def linear(
     if x.dim() != 2 or x.shape[1] != w.K:
         raise ValueError(f"x must be [M, {w.K}], got {tuple(x.shape)}")
     x = x.contiguous()
-    if w.perm is not None:
-        x = gather_columns(x, w.perm)
+    if w.perm is not None and gemv_config is not None:
+        x = gather_columns(x, w.perm)  # explicit decode configurations take x in row order
     M = x.shape[0]
     if out is not None:
         if tuple(out.shape) != (M, w.N) or out.dtype != x.dtype or out.device != x.device or not out.is_contiguous():
@@ -245,6 +245,10 @@ def linear(
         need = _lib.WORKSPACE_COUNTER_BYTES
         if chosen in (_lib.PATH_GEMV, _lib.PATH_GEMM):
             need = workspace_bytes(M, w.K, w.N)
+        if w.perm is not None:
+            # weight in group order: x is gathered into the tail of the workspace (all but the
+            # shortest decode calls, which gather inside the kernel)
+            need = int(lib.q4_workspace_bytes_perm(M, w.K, w.N))
         ws = reserve_workspace(x.device, need, stream)
         st = w.struct()
         if gemv_config is not None:
@@ -256,6 +260,11 @@ def linear(
             rc = lib.q4_gemv_tuned(
                 ctypes.byref(st), x.data_ptr(), bias_ptr, y.data_ptr(), M, _DTYPES[x.dtype],
                 ws.data_ptr(), ws.numel(), wcol, wk, splits, words, stream,
+            )
+        elif w.perm is not None:
+            rc = lib.q4_linear_perm(
+                ctypes.byref(st), w.perm.data_ptr(), x.data_ptr(), bias_ptr, y.data_ptr(), M, _DTYPES[x.dtype],
+                ws.data_ptr(), ws.numel(), path, stream,
             )
         else:
             rc = lib.q4_linear_ex(
