@@ -159,3 +159,30 @@ def test_quant_linear_repacks_once_and_keeps_memory_flat(pkg, oracle, gpu):
     import copy
     twin = copy.deepcopy(layer)
     assert torch.equal(twin(x), y1)
+
+
+@pytest.mark.parametrize("M", [1, 16, 200])
+def test_wqlinear_converts_to_the_gptq_layout_bit_exactly(pkg, oracle, gpu, M, monkeypatch):
+    """The AWQ module serves its checkpoint through the GPTQ layout by default: same dense
+    matrix bit for bit (zero point 0 included: stored 15, read back as 0), same outputs as the
+    native AWQ kernels to rounding, AWQ-layout tensors dropped."""
+    K, N, gs = 1024, 512, 128
+    aq, az, sc = oracle.make_awq(K, N, gs, seed=M)
+    az = az.copy()
+    az[0, :4] = 0  # whole words of zero points 0
+    want = oracle.dequant_awq(aq, az, sc, gs, "f16")
+    import importlib
+    mod = importlib.import_module("text-generation-inference_amd.layers.awq.quantize")
+    conv = pkg.WQLinear(4, gs, to_dev(aq, gpu), to_dev(az, gpu), to_dev(sc, gpu), None)
+    xh = oracle.make_x(M, K, seed=M + 2)
+    x = to_dev(xh, gpu)
+    y = conv(x)
+    assert conv.gptq_layout and tuple(conv.qweight.shape) == (K // 8, N) and conv.packed().layout == 0
+    assert np.array_equal(conv.dequantize().cpu().numpy().view(np.uint16), want.view(np.uint16))
+    y32, _ = oracle.linear_forward(xh, want, None, "f16")
+    assert max_rel_err(y.float().cpu().numpy(), y32) <= TOL
+    monkeypatch.setattr(mod, "AWQ_MODE", "native")
+    native = pkg.WQLinear(4, gs, to_dev(aq, gpu), to_dev(az, gpu), to_dev(sc, gpu), None)
+    yn = native(x)
+    assert not native.gptq_layout and native.packed().layout == 1
+    assert max_rel_err(y.float().cpu().numpy(), yn.float().cpu().numpy()) <= TOL
