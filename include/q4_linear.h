@@ -139,6 +139,14 @@ int q4_gather_columns(const void* x, const int32_t* perm, void* out, int M, int 
 int q4_linear_perm(const q4_weight* w, const int32_t* perm, const void* x, const void* bias, void* y, int M,
                    int dtype, void* workspace, size_t workspace_bytes, int path, void* stream);
 size_t q4_workspace_bytes_perm(int M, int K, int N);
+/*
+ * Grouped form of q4_gather_columns for experts whose rows are in group order (perms [E, K],
+ * one q4_gptq_make_sequential per expert): out[r][i] = x[x_rows ? x_rows[r] : r][perms[e(r)][i]]
+ * for every sorted row r, e(r) its expert by expert_offsets.  out is [pairs, K] in sorted order
+ * and goes to q4_moe_linear with x_rows = NULL.
+ */
+int q4_moe_gather_columns(const void* x, const int32_t* x_rows, const int32_t* expert_offsets, const int32_t* perms,
+                          void* out, int num_experts, int pairs, int K, void* stream);
 
 /* y[M, inter] = act(gate_up[:, :inter]) * gate_up[:, inter:] for gate_up [M, 2 * inter]. */
 int q4_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, void* stream);

@@ -203,6 +203,51 @@ def test_moe_linear_act_order_and_awq(pkg, oracle, gpu, kind, T, E, k, K, N, gs,
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("T,E,k,K,N,gs", [(1, 8, 2, 1024, 512, 128), (9, 4, 2, 2048, 512, 128),
+                                          (100, 8, 2, 1024, 256, 64), (16, 4, 4, 43 * 128, 256, 128)])
+def test_moe_linear_act_order_rows_in_group_order(pkg, oracle, gpu, T, E, k, K, N, gs, dtype):
+    """Act-order experts repacked once (make_sequential_moe): every expert's rows are its
+    checkpoint rows in the order of a stable sort of its g_idx, activations are gathered per
+    sorted row with the row's expert's permutation, and both projection forms agree with the
+    oracle's act-order matrices."""
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(T + K)
+    w, dense = _packed_experts(pkg, oracle, gpu, "act", E, K, N, gs, dtype, seed=T + 5)
+    seq = pkg.ops.make_sequential_moe(w)
+    assert seq is not None and seq.g_idx is None and tuple(seq.perm.shape) == (E, K)
+    perm = seq.perm.cpu().numpy()
+    gi = w.g_idx.cpu().numpy()
+    for e in range(E):
+        assert np.array_equal(gi[e][perm[e]], np.arange(K) // (K if gs == -1 else gs))
+        rows = oracle.unpack_rows(w.qweight[e].cpu().numpy())
+        assert np.array_equal(oracle.unpack_rows(seq.qweight[e].cpu().numpy()), rows[perm[e]])
+    g, _ = _gating(rng, T, E, "f32")
+    r = pkg.ops.moe_route(g.to(gpu), k, True)
+    x = oracle.make_x(T, K, seed=T, dtype=dtype)
+    y = to_f32(pkg.ops.moe_linear(seq, to_dev(x, gpu, bf16=bf), r, gather=True))
+    ids = r.topk_ids.cpu().numpy()
+    slot = r.pair_slot.cpu().numpy()
+    ref = np.zeros_like(y)
+    for e in range(E):
+        rows, js = np.nonzero(ids == e)
+        if rows.size:
+            ref[slot[rows * k + js]], _ = oracle.linear_forward(x[rows], dense[e], None, dtype)
+    assert max_rel_err(y, ref) <= (TOL_BF16 if bf else TOL)
+    xs = oracle.make_x(T * k, K, seed=T + 1, dtype=dtype)
+    y2 = to_f32(pkg.ops.moe_linear(seq, to_dev(xs, gpu, bf16=bf), r, gather=False))
+    off = r.expert_offsets.cpu().numpy()
+    ref2 = np.zeros_like(y2)
+    for e in range(E):
+        if off[e + 1] > off[e]:
+            ref2[off[e]:off[e + 1]], _ = oracle.linear_forward(xs[off[e]:off[e + 1]], dense[e], None, dtype)
+    assert max_rel_err(y2, ref2) <= (TOL_BF16 if bf else TOL)
+    # the gated first projection takes the two-kernel route on such weights
+    if N % 2 == 0:
+        h = to_f32(pkg.ops.moe_linear_gate_up(seq, to_dev(x, gpu, bf16=bf), r, "silu"))
+        assert h.shape == (T * k, N // 2) and np.isfinite(h).all()
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("T,E,k,K,I,gs,act", [
     (1, 8, 2, 1024, 512, 128, "silu"),       # fused decode kernel
     (1, 8, 2, 2048, 1024, 128, "gelu_tanh"),
@@ -359,7 +404,9 @@ def test_sparse_moe_layer_from_safetensors(pkg, oracle, gpu, tmp_path, desc_act)
     weights = pkg.Weights([path], gpu, torch.float16, SimpleNamespace(rank=lambda: 0, size=lambda: 1), loader)
     layer = pkg.GPTQSparseMoELayer(n_expert_group=None, n_experts=E, prefix="moe.experts", renormalize=True, topk=k,
                                    topk_group=None, weights=weights)
-    assert (layer._gate_up.g_idx is not None) == desc_act and (layer._down.g_idx is not None) == desc_act
+    # act-order experts are put into group order once: no g_idx left, a permutation per expert
+    assert layer._gate_up.g_idx is None and layer._down.g_idx is None
+    assert (layer._gate_up.perm is not None) == desc_act and (layer._down.perm is not None) == desc_act
     rng = np.random.default_rng(5)
     x = oracle.make_x(6, H, seed=2)
     g = rng.standard_normal((6, E)).astype(np.float32)

@@ -193,6 +193,24 @@ int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, i
   }
 }
 
+int q4_moe_gather_columns(const void* x, const int32_t* x_rows, const int32_t* expert_offsets, const int32_t* perms,
+                          void* out, int num_experts, int pairs, int K, void* stream) {
+  if (num_experts < 1 || pairs < 0 || K < 0) {
+    set_error("q4_moe_gather_columns: bad num_experts=%d, pairs=%d or K=%d", num_experts, pairs, K);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (pairs == 0 || K == 0) return Q4_OK;
+  if (x == nullptr || expert_offsets == nullptr || perms == nullptr || out == nullptr || x == out) {
+    set_error("q4_moe_gather_columns: null pointer, or output aliasing the input");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (K % 8 != 0) {
+    set_error("q4_moe_gather_columns: K=%d must be a multiple of 8", K);
+    return Q4_ERR_UNSUPPORTED;
+  }
+  return launch_moe_gather_columns(x, x_rows, expert_offsets, perms, out, num_experts, pairs, K, (hipStream_t)stream);
+}
+
 static size_t perm_gather_offset(int M, int K, int N) {
   return (q4_workspace_bytes(M, K, N) + 255) & ~(size_t)255;
 }

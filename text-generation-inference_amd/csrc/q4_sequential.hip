@@ -51,9 +51,61 @@ __global__ __launch_bounds__(256) void gather_columns_kernel(const uint16_t* __r
   }
 }
 
+// Grouped form: sorted row r of expert e (offsets[e] <= r < offsets[e + 1]) becomes
+// x[x_rows ? x_rows[r] : r][perms[e][.]].  Output [pairs, K] in sorted order.
+__global__ __launch_bounds__(256) void moe_gather_columns_kernel(const uint16_t* __restrict__ x,
+                                                                 const int32_t* __restrict__ x_rows,
+                                                                 const int32_t* __restrict__ offsets,
+                                                                 const int32_t* __restrict__ perms,
+                                                                 uint16_t* __restrict__ out, int num_experts,
+                                                                 int pairs, int K) {
+  const int vec_per_row = K >> 3;
+  const long total = (long)pairs * vec_per_row;
+  for (long v = (long)blockIdx.x * blockDim.x + threadIdx.x; v < total; v += (long)gridDim.x * blockDim.x) {
+    const int r = (int)(v / vec_per_row);
+    const int c = (int)(v - (long)r * vec_per_row) * 8;
+    int lo = 0, hi = num_experts;  // expert of row r: the last e with offsets[e] <= r
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (offsets[mid] <= r) lo = mid; else hi = mid;
+    }
+    const uint16_t* row = x + (size_t)(x_rows != nullptr ? x_rows[r] : r) * K;
+    const int32_t* perm = perms + (size_t)lo * K;
+    const uint4_t p0 = *(const uint4_t*)(perm + c);
+    const uint4_t p1 = *(const uint4_t*)(perm + c + 4);
+    const uint32_t idx[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+    uint32_t h[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = row[min(idx[i], (uint32_t)(K - 1))];
+    uint4_t o;
+    o.x = h[0] | (h[1] << 16);
+    o.y = h[2] | (h[3] << 16);
+    o.z = h[4] | (h[5] << 16);
+    o.w = h[6] | (h[7] << 16);
+    *(uint4_t*)(out + (size_t)r * K + c) = o;
+  }
+}
+
 }  // namespace q4
 
 namespace q4host {
+
+int launch_moe_gather_columns(const void* x, const int32_t* x_rows, const int32_t* offsets, const int32_t* perms,
+                              void* out, int num_experts, int pairs, int K, hipStream_t stream) {
+  const long total = (long)pairs * (K / 8);
+  long blocks = (total + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(q4::moe_gather_columns_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t*)x,
+                     x_rows, offsets, perms, (uint16_t*)out, num_experts, pairs, K);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    set_error("q4_moe_gather_columns: launch failed: %s", hipGetErrorString(err));
+    return Q4_ERR_LAUNCH;
+  }
+  return Q4_OK;
+}
+
 
 int launch_make_sequential(const uint32_t* qweight, const int32_t* perm, uint32_t* out, int K, int N,
                            hipStream_t stream) {

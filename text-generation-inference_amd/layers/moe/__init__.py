@@ -22,7 +22,7 @@ import torch.nn as nn
 from ... import ops
 from ..._lib import LAYOUT_AWQ, LAYOUT_GPTQ
 from ..gptq import GPTQWeight
-from ..gptq.quant_linear import is_trivial_g_idx
+from ..gptq.quant_linear import ACT_ORDER_MODE, is_trivial_g_idx
 
 
 @dataclass
@@ -37,12 +37,26 @@ class GPTQMoEWeight:
     groupsize: int
     use_awq_kernel: bool
 
+    q_perm: Optional[torch.Tensor] = None  # set once the experts' rows are in group order
+
     def packed(self) -> ops.PackedMoeWeight:
         g_idx = self.g_idx
-        if g_idx is not None and all(is_trivial_g_idx(g, self.groupsize) for g in g_idx):
+        if self.q_perm is not None or (
+                g_idx is not None and all(is_trivial_g_idx(g, self.groupsize) for g in g_idx)):
             g_idx = None  # sequential groups in every expert: the kernels index by k // groupsize
-        return ops.make_packed_moe(self.qweight, self.qzeros, self.scales, self.groupsize, g_idx,
-                                   LAYOUT_AWQ if self.use_awq_kernel else LAYOUT_GPTQ)
+        pk = ops.make_packed_moe(self.qweight, self.qzeros, self.scales, self.groupsize, g_idx,
+                                 LAYOUT_AWQ if self.use_awq_kernel else LAYOUT_GPTQ)
+        if self.q_perm is not None:
+            pk.perm = self.q_perm
+        elif g_idx is not None and ACT_ORDER_MODE != "table" and self.qweight.is_cuda:
+            # act-order experts: rows into group order once, like the dense layers; the
+            # checkpoint-order tensor is dropped
+            seq = ops.make_sequential_moe(pk)
+            if seq is not None:
+                self.qweight = seq.qweight
+                self.q_perm = seq.perm
+                pk = seq
+        return pk
 
 
 def _check_expert(weight, name: str) -> GPTQWeight:

@@ -379,6 +379,9 @@ class PackedMoeWeight:
     num_groups: int
     num_experts: int
     layout: int
+    # Every expert's rows in group order (make_sequential_moe): perm [E, K] int32, packed row i of
+    # expert e holds its checkpoint row perm[e, i]; None for checkpoint order.
+    perm: Optional[torch.Tensor] = None
 
     def struct(self) -> _lib.Q4MoeWeight:
         e0 = _lib.Q4Weight(
@@ -408,6 +411,44 @@ def make_packed_moe(qweight, qzeros, scales, groupsize: int, g_idx=None, layout:
         if not t[0].is_contiguous():
             raise ValueError(f"{name}: every expert's slice must be contiguous")
     return PackedMoeWeight(qweight, qzeros, scales, g_idx, one.K, one.N, one.groupsize, one.num_groups, E, layout)
+
+
+def make_sequential_moe(w: PackedMoeWeight) -> Optional[PackedMoeWeight]:
+    """Stacked act-order experts with every expert's rows put into group order (see
+    make_sequential), or None when some expert's groups are not all `groupsize` rows.
+    The new qweight is a second [E, K/8, N] tensor; the caller drops the old one."""
+    if w.g_idx is None or w.layout != LAYOUT_GPTQ or w.perm is not None:
+        return None
+    _require_cuda(w.qweight, "qweight")
+    K, E = w.K, w.num_experts
+    if K % 8 or w.num_groups * w.groupsize != K:
+        return None
+    g = w.g_idx.to(torch.int64)
+    perm = torch.argsort(g, dim=1, stable=True)
+    expect = (torch.arange(K, device=g.device, dtype=torch.int64) // w.groupsize).expand(E, K)
+    if not bool(torch.equal(torch.gather(g, 1, perm), expect)):
+        return None
+    perm32 = perm.to(torch.int32).contiguous()
+    out = torch.empty_like(w.qweight)
+    lib = _lib.load()
+    with torch.cuda.device(w.qweight.device):
+        stream = _stream_handle(out.device)
+        for e in range(E):
+            _lib.check(lib.q4_gptq_make_sequential(
+                w.qweight[e].data_ptr(), perm32[e].data_ptr(), out[e].data_ptr(), K, w.N, stream))
+    return PackedMoeWeight(out, w.qzeros, w.scales, None, K, w.N, w.groupsize, w.num_groups, E, w.layout, perm32)
+
+
+def _moe_gather(w: PackedMoeWeight, x: torch.Tensor, routing: "MoeRouting", gather: bool) -> torch.Tensor:
+    """Activations of every sorted row in its expert's row order: [tokens*k, K]."""
+    T, k = routing.topk_ids.shape
+    out = torch.empty((T * k, w.K), dtype=x.dtype, device=x.device)
+    if out.numel():
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.load().q4_moe_gather_columns(
+                x.data_ptr(), routing.sorted_tokens.data_ptr() if gather else None, routing.expert_offsets.data_ptr(),
+                w.perm.data_ptr(), out.data_ptr(), w.num_experts, T * k, w.K, _stream_handle(x.device)))
+    return out
 
 
 @dataclass
@@ -465,6 +506,9 @@ def moe_linear(w: PackedMoeWeight, x: torch.Tensor, routing: MoeRouting, gather:
     if x.dim() != 2 or tuple(x.shape) != (rows, w.K):
         raise ValueError(f"x must be [{rows}, {w.K}], got {tuple(x.shape)}")
     x = x.contiguous()
+    if w.perm is not None and T > 0:
+        x = _moe_gather(w, x, routing, gather)  # sorted rows, columns in each expert's row order
+        gather = False
     y = torch.empty((T * k, w.N), dtype=x.dtype, device=x.device)
     if T == 0:
         return y
@@ -493,7 +537,7 @@ def moe_linear_gate_up(w: PackedMoeWeight, x: torch.Tensor, routing: MoeRouting,
     if x.dim() != 2 or tuple(x.shape) != (T, w.K):
         raise ValueError(f"x must be [{T}, {w.K}], got {tuple(x.shape)}")
     x = x.contiguous()
-    if T > 0:
+    if T > 0 and w.perm is None:
         lib = _lib.load()
         y = torch.empty((T * k, w.N // 2), dtype=x.dtype, device=x.device)
         with torch.cuda.device(x.device):
