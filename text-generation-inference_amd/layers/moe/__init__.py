@@ -22,6 +22,8 @@ import torch.nn as nn
 from ... import ops
 from ..._lib import LAYOUT_AWQ, LAYOUT_GPTQ
 from ..gptq import GPTQWeight
+from ..awq.conversion_utils import fast_awq_to_gptq
+from ..awq.quantize import AWQ_MODE
 from ..gptq.quant_linear import ACT_ORDER_MODE, is_trivial_g_idx
 
 
@@ -40,6 +42,13 @@ class GPTQMoEWeight:
     q_perm: Optional[torch.Tensor] = None  # set once the experts' rows are in group order
 
     def packed(self) -> ops.PackedMoeWeight:
+        if self.use_awq_kernel and AWQ_MODE != "native" and self.qweight.is_cuda:
+            # AWQ-layout experts: one conversion to the GPTQ layout (bit-exact, see WQLinear),
+            # expert by expert to bound the temporaries; the AWQ tensors are dropped
+            converted = [fast_awq_to_gptq(self.qweight[e], self.qzeros[e]) for e in range(self.qweight.shape[0])]
+            self.qweight = torch.stack([c[0] for c in converted]).contiguous()
+            self.qzeros = torch.stack([c[1] for c in converted]).contiguous()
+            self.use_awq_kernel = False
         g_idx = self.g_idx
         if self.q_perm is not None or (
                 g_idx is not None and all(is_trivial_g_idx(g, self.groupsize) for g in g_idx)):
