@@ -140,6 +140,22 @@ int q4_linear_perm(const q4_weight* w, const int32_t* perm, const void* x, const
                    int dtype, void* workspace, size_t workspace_bytes, int path, void* stream);
 size_t q4_workspace_bytes_perm(int M, int K, int N);
 /*
+ * One block of the GPTQ solver's column loop (GPTQ.fasterquant,
+ * server/text_generation_server/layers/gptq/quantize.py:294-331; the quantizer's range rule,
+ * Quantizer.find_params, :60-101 with mse off, and its rounding, :54-58).  W [rows, K] fp32
+ * holds the current weights (one row per output feature); U [K, K] is the upper Cholesky factor
+ * of the inverse damped Hessian.  For the columns i1 .. i1+count-1 (count <= 128) in turn:
+ * at a group start find scale and zero of the group from the current values, quantize the
+ * column to 4 bits, store scale*(q - zero) in Q, (w - q) / U_ii in err [rows, 128], add
+ * (w - q)^2 / U_ii^2 / 2 to loss [rows], and subtract err * U[i, c] from every later column c
+ * of the block.  W itself is not written; the caller follows with
+ * W[:, i1+count:] -= err @ U[i1:i1+count, i1+count:].  groupsize <= 0: scale / zero [rows]
+ * are given; else they are [rows, num_groups] and the groups starting in the block are written.
+ */
+int q4_gptq_solve_block(float* W, const float* U, float* Q, float* err, float* loss, float* scale, float* zero,
+                        int rows, int K, int i1, int count, int groupsize, int num_groups, int sym, void* stream);
+
+/*
  * Grouped form of q4_gather_columns for experts whose rows are in group order (perms [E, K],
  * one q4_gptq_make_sequential per expert): out[r][i] = x[x_rows ? x_rows[r] : r][perms[e(r)][i]]
  * for every sorted row r, e(r) its expert by expert_offsets.  out is [pairs, K] in sorted order

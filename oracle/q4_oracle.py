@@ -362,6 +362,85 @@ def moe_forward(x, gating, gate_up_w, down_w, topk, renormalize=True, act="silu"
 # --------------------------------------------------------------------------- synthetic inputs
 
 
+def gptq_find_params(x, sym):
+    """Range rule of the reference's quantizer with mse off (quantize.py:60-101): per row of x
+    (float64), the range always contains 0; sym mirrors it; an all-zero row gets [-1, 1].
+    Returns (scale, zero) per row, 4 bits."""
+    x = np.asarray(x, dtype=np.float64)
+    lo = np.minimum(x.min(axis=1), 0.0)
+    hi = np.maximum(x.max(axis=1), 0.0)
+    if sym:
+        hi = np.maximum(np.abs(lo), hi)
+        lo = np.where(lo < 0, -hi, lo)
+    dead = (lo == 0) & (hi == 0)
+    lo = np.where(dead, -1.0, lo)
+    hi = np.where(dead, 1.0, hi)
+    scale = (hi - lo) / 15.0
+    zero = np.full_like(scale, 8.0) if sym else np.rint(-lo / scale)
+    return scale, zero
+
+
+def gptq_fasterquant(W, H, blocksize=128, percdamp=0.01, groupsize=-1, act_order=False, sym=True):
+    """The GPTQ solver in float64, column by column (quantize.py:243-351).
+
+    W [rows, K] (one row per output feature), H [K, K] the accumulated Hessian 2/n X X^T.
+    Dead inputs (H_ii = 0) get H_ii = 1 and zero weights; act_order walks the columns by
+    decreasing H_ii; H is damped by percdamp * mean(diag); U is the upper Cholesky factor of
+    inv(H).  Every column is rounded with its group's (scale, zero) (found when the group starts,
+    from the values its columns had when the block started) and its error (w - q) / U_ii is subtracted, times U[i, c],
+    from every later column c.  Returns Q (dequantized values, checkpoint column order),
+    scale [rows, G], zero [rows, G], g_idx [K], error = sum of (w - q)^2 / U_ii^2 / 2, and the
+    damped (and, with act_order, permuted) H together with the column order used.
+    Plain loops: for small cases only."""
+    W = np.array(W, dtype=np.float64)
+    H = np.array(H, dtype=np.float64)
+    rows, K = W.shape
+    dead = np.diag(H) == 0
+    H[dead, dead] = 1.0
+    W[:, dead] = 0.0
+    perm = np.arange(K)
+    if act_order:
+        perm = np.argsort(-np.diag(H), kind="stable")
+        W = W[:, perm]
+        H = H[perm][:, perm]
+    H[np.arange(K), np.arange(K)] += percdamp * np.mean(np.diag(H))
+    Hinv = np.linalg.inv(H)
+    U = np.linalg.cholesky(Hinv).T  # upper factor: inv(H) = U^T U (torch.linalg.cholesky(upper=True))
+    Q = np.zeros_like(W)
+    error = 0.0
+    gs = K if groupsize == -1 else groupsize
+    G = (K + gs - 1) // gs
+    scale = np.zeros((rows, G))
+    zero = np.zeros((rows, G))
+    if groupsize == -1:
+        scale[:, 0], zero[:, 0] = gptq_find_params(W, sym)
+    for i1 in range(0, K, blocksize):
+        i2 = min(i1 + blocksize, K)
+        Err = np.zeros((rows, i2 - i1))
+        W1 = W[:, i1:i2].copy()  # the block's working copy; W keeps the values of block entry
+        for i in range(i1, i2):
+            g = i // gs
+            if groupsize != -1 and i % gs == 0:
+                # from W, which has the updates of finished blocks only (quantize.py:308-312)
+                scale[:, g], zero[:, g] = gptq_find_params(W[:, i:i + gs], sym)
+            w = W1[:, i - i1]
+            d = U[i, i]
+            q = scale[:, g] * (np.clip(np.rint(w / scale[:, g]) + zero[:, g], 0, 15) - zero[:, g])
+            Q[:, i] = q
+            error += float(np.sum((w - q) ** 2 / d ** 2)) / 2
+            err = (w - q) / d
+            W1[:, i - i1:] -= np.outer(err, U[i, i:i2])
+            Err[:, i - i1] = err
+        W[:, i2:] -= Err @ U[i1:i2, i2:]
+    g_idx = (np.arange(K) // gs).astype(np.int32)
+    Hd = H
+    if act_order:
+        inv = np.argsort(perm)
+        Q = Q[:, inv]
+        g_idx = g_idx[inv]
+    return Q, scale, zero, g_idx, error, Hd, perm
+
+
 def make_gptq(K, N, groupsize=128, seed=0, sym=True, act_order=False):
     """Seeded synthetic GPTQ tensors of the benchmark's shape.
 

@@ -19,12 +19,14 @@ from .layers.gptq import (  # noqa: F401
     set_device,
 )
 from .layers.awq.quantize import WQLinear  # noqa: F401
+from .layers.gptq.solver import GPTQ  # noqa: F401
 from .layers.moe import GPTQSparseMoELayer, GPTQMoEWeight  # noqa: F401
 from .layers.awq import conversion_utils  # noqa: F401
 from .utils.weights import Weights, WeightsLoader, DefaultWeightsLoader, UnquantizedWeight  # noqa: F401
 from .utils.quantization import get_loader, get_quantizer_config  # noqa: F401
 
 __all__ = [
+    "GPTQ",
     "GPTQWeight",
     "GPTQWeightsLoader",
     "Weights",

@@ -193,6 +193,26 @@ int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, i
   }
 }
 
+int q4_gptq_solve_block(float* W, const float* U, float* Q, float* err, float* loss, float* scale, float* zero,
+                        int rows, int K, int i1, int count, int groupsize, int num_groups, int sym, void* stream) {
+  if (W == nullptr || U == nullptr || Q == nullptr || err == nullptr || loss == nullptr || scale == nullptr ||
+      zero == nullptr) {
+    set_error("q4_gptq_solve_block: null pointer");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (rows < 1 || K < 1 || i1 < 0 || count < 1 || count > 128 || i1 + count > K) {
+    set_error("q4_gptq_solve_block: bad rows=%d, K=%d or block [%d, %d) (at most 128 columns)", rows, K, i1,
+              i1 + count);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (groupsize > 0 ? (long)num_groups * groupsize < K : num_groups != 1) {
+    set_error("q4_gptq_solve_block: %d groups of %d columns do not cover K=%d", num_groups, groupsize, K);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  return launch_gptq_solve_block(W, U, Q, err, loss, scale, zero, rows, K, i1, count, groupsize, num_groups, sym,
+                                 (hipStream_t)stream);
+}
+
 int q4_moe_gather_columns(const void* x, const int32_t* x_rows, const int32_t* expert_offsets, const int32_t* perms,
                           void* out, int num_experts, int pairs, int K, void* stream) {
   if (num_experts < 1 || pairs < 0 || K < 0) {

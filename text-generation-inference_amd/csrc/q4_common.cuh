@@ -204,6 +204,8 @@ bool gemv_gate_up_supported(const q4_weight* w, int M, int dtype);
 int launch_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, hipStream_t stream);
 int launch_make_sequential(const uint32_t* qweight, const int32_t* perm, uint32_t* out, int K, int N, hipStream_t stream);
 int launch_gather_columns(const void* x, const int32_t* perm, void* out, int M, int K, hipStream_t stream);
+int launch_gptq_solve_block(float* W, const float* U, float* Q, float* Err, float* loss, float* scale, float* zero,
+                            int rows, int K, int i1, int count, int groupsize, int G, int sym, hipStream_t stream);
 int launch_moe_gather_columns(const void* x, const int32_t* x_rows, const int32_t* offsets, const int32_t* perms,
                               void* out, int num_experts, int pairs, int K, hipStream_t stream);
 bool gemm_awq_supported(const q4_weight* w, int M, int dtype);

@@ -1,0 +1,119 @@
+"""GPTQ: the solver that chooses the 4-bit weights of one linear layer from calibration inputs.
+
+Mirrors the interface of the reference's `GPTQ` class
+(server/text_generation_server/layers/gptq/quantize.py:147-375): `add_batch(inp, out)`
+accumulates the Hessian 2/n * X X^T of the layer's inputs, `fasterquant(...)` returns
+(scale, zero, g_idx, error) and leaves the quantized weights in `layer.weight`, ready for
+`QuantLinear.pack`.  The Hessian products, the two Cholesky factorizations and the update of
+the columns behind a block are library linear algebra (torch on the GPU, as in the
+reference); the column loop inside a block -- 128 dependent steps that the reference runs as
+several small kernels each -- is one launch of the HIP kernel behind q4_gptq_solve_block.
+Linear layers only (the reference also unfolds Conv2d / transformers.Conv1D inputs); the
+quantizer's mse search is not offered.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn as nn
+
+from ... import _lib
+
+BLOCK = 128  # columns per kernel launch
+
+
+class GPTQ:
+    def __init__(self, layer: nn.Module, sym: bool = True):
+        if not isinstance(layer, nn.Linear):
+            raise NotImplementedError("the solver handles nn.Linear layers")
+        self.layer = layer
+        self.dev = layer.weight.device
+        self.rows, self.columns = layer.weight.shape
+        self.H = torch.zeros((self.columns, self.columns), device=self.dev, dtype=torch.float32)
+        self.nsamples = 0
+        self.sym = bool(sym)
+
+    def add_batch(self, inp: torch.Tensor, out: torch.Tensor = None):
+        """H <- running mean of 2 x x^T over all calibration rows (quantize.py:170-216)."""
+        if inp.dim() == 2:
+            inp = inp.unsqueeze(0)
+        batch = inp.shape[0]
+        x = inp.reshape(-1, inp.shape[-1]).t().float()  # [columns, tokens]
+        self.H *= self.nsamples / (self.nsamples + batch)
+        self.nsamples += batch
+        x = math.sqrt(2 / self.nsamples) * x
+        self.H += x.matmul(x.t())
+
+    @torch.no_grad()
+    def fasterquant(self, blocksize: int = BLOCK, percdamp: float = 0.01, groupsize: int = -1,
+                    act_order: bool = False, name: str = ""):
+        if not self.H.is_cuda:
+            raise RuntimeError("the GPTQ solver runs on the GPU only (no CPU fallback exists in this package)")
+        if blocksize < 1 or blocksize > BLOCK:
+            raise ValueError(f"blocksize must be 1..{BLOCK}, got {blocksize}")
+        K, rows = self.columns, self.rows
+        W = self.layer.weight.data.clone().float().contiguous()
+        H = self.H.clone()
+        dead = torch.diag(H) == 0
+        H[dead, dead] = 1
+        W[:, dead] = 0
+        perm = None
+        if act_order:
+            perm = torch.argsort(torch.diag(H), descending=True)
+            W = W[:, perm].contiguous()
+            H = H[perm][:, perm]
+        diag = torch.arange(K, device=self.dev)
+        H[diag, diag] += percdamp * torch.mean(torch.diag(H))
+        # upper factor U of inv(H): inv(H) = U^T U
+        L = torch.linalg.cholesky(H)
+        Hinv = torch.cholesky_inverse(L)
+        try:
+            U = torch.linalg.cholesky(Hinv, upper=True)
+        except Exception:  # the reference's fallback for a factorization that fails (quantize.py:282-286)
+            U = torch.linalg.cholesky(Hinv + 1e-5 * torch.eye(K, device=self.dev), upper=True)
+        U = U.contiguous()
+
+        gs = K if groupsize == -1 else int(groupsize)
+        G = (K + gs - 1) // gs
+        Q = torch.zeros_like(W)
+        scale = torch.zeros((rows, G), device=self.dev, dtype=torch.float32)
+        zero = torch.zeros((rows, G), device=self.dev, dtype=torch.float32)
+        loss = torch.zeros((rows,), device=self.dev, dtype=torch.float32)
+        err = torch.zeros((rows, BLOCK), device=self.dev, dtype=torch.float32)
+        if groupsize == -1:
+            # one range per row, from the weights as they are before any column is quantized
+            lo = torch.clamp(W.min(dim=1).values, max=0)
+            hi = torch.clamp(W.max(dim=1).values, min=0)
+            if self.sym:
+                hi = torch.maximum(lo.abs(), hi)
+                lo = torch.where(lo < 0, -hi, lo)
+            flat = (lo == 0) & (hi == 0)
+            lo = torch.where(flat, torch.full_like(lo, -1), lo)
+            hi = torch.where(flat, torch.full_like(hi, 1), hi)
+            scale[:, 0] = (hi - lo) / 15
+            zero[:, 0] = 8 if self.sym else torch.round(-lo / scale[:, 0])
+        lib = _lib.load()
+        with torch.cuda.device(self.dev):
+            stream = torch.cuda.current_stream(self.dev).cuda_stream
+            for i1 in range(0, K, blocksize):
+                count = min(blocksize, K - i1)
+                _lib.check(lib.q4_gptq_solve_block(
+                    W.data_ptr(), U.data_ptr(), Q.data_ptr(), err.data_ptr(), loss.data_ptr(), scale.data_ptr(),
+                    zero.data_ptr(), rows, K, i1, count, -1 if groupsize == -1 else gs, G, int(self.sym), stream))
+                i2 = i1 + count
+                if i2 < K:
+                    W[:, i2:] -= err[:, :count].matmul(U[i1:i2, i2:])
+        error = float(loss.sum().item())
+        g_idx = (torch.arange(K, device=self.dev) // gs).to(torch.int32)
+        if perm is not None:
+            invperm = torch.argsort(perm)
+            Q = Q[:, invperm]
+            g_idx = g_idx[invperm]
+        self.layer.weight.data = Q.reshape(self.layer.weight.shape).to(self.layer.weight.data.dtype)
+        return scale, zero, g_idx, error
+
+    def free(self):
+        self.H = None
+        torch.cuda.empty_cache()
