@@ -38,6 +38,14 @@ Pinning status (what proves each function right, other than itself):
         parts (linear_forward, gate_up_forward).  The reference's GPTQ MoE kernels
         (kernels-community/moe, fused_marlin_moe) are not in the tree: their internal
         roundings are parity unpinned; GPU results are compared within the GEMM tolerance.
+  gptq_find_params / gptq_fasterquant (the solver, float64)
+        pinned: with a diagonal Hessian the result is round-to-nearest with the group ranges
+        (closed form); for any Hessian dW H dW^T / 2 equals the returned error exactly (the
+        algebra of the Cholesky update: it caught a transposed factor); every value sits on its
+        group's 16-level grid; the output error on correlated inputs is below round-to-nearest's;
+        dead inputs give zero columns and act_order walks the columns by decreasing activity.
+        The reference runs these loops in fp32 on the GPU: its decisions near rounding ties
+        are not pinned bit for bit (GPU agreement is asserted for >= 97 % of the nibbles).
   awq_inference_engine.gemm_forward_cuda (third-party, huggingface/llm-awq @ bd1dc2d5,
   not in the reference tree): parity unpinned by any runnable reference test; covered
   through the in-tree equivalence fast_awq_to_gptq (awq/conversion_utils.py:83-97).
