@@ -385,9 +385,11 @@ def main():
         for Mb in (4, 16, 18, 32, 64):
             batch[f"gptq_m{Mb}"] = step_us(weights, Mb)
         # act_order: rows put into group order at load time (what the layers do by default),
-        # x read through the permutation; act_order_lookup: checkpoint order, g_idx in the kernel
-        for kind in ("awq", "act_order", "act_order_lookup"):
-            wl = [[make_weights_variant(pkg, torch, dev, K, N, 31 * c + i, "awq" if kind == "awq" else "act_order")
+        # x read through the permutation; act_order_lookup: checkpoint order, g_idx in the kernel;
+        # awq_native: the AWQ-layout kernels (the layers convert AWQ checkpoints to the GPTQ layout
+        # once and then run at the gptq_* figures)
+        for kind in ("awq_native", "act_order", "act_order_lookup"):
+            wl = [[make_weights_variant(pkg, torch, dev, K, N, 31 * c + i, "awq" if kind == "awq_native" else "act_order")
                    for i, (_, K, N) in enumerate(SHAPES)] for c in range(min(copies, 3))]
             if kind == "act_order":
                 wl = [[pkg.ops.make_sequential(w) for w in row] for row in wl]
