@@ -537,7 +537,14 @@ def moe_linear_gate_up(w: PackedMoeWeight, x: torch.Tensor, routing: MoeRouting,
     if x.dim() != 2 or tuple(x.shape) != (T, w.K):
         raise ValueError(f"x must be [{T}, {w.K}], got {tuple(x.shape)}")
     x = x.contiguous()
-    if T > 0 and w.perm is None:
+    x_rows = routing.sorted_tokens
+    if w.perm is not None and T > 0:
+        # experts in group order: sorted rows with their expert's column order, then as below
+        x = _moe_gather(w, x, routing, True)
+        x_rows = None
+        w = PackedMoeWeight(w.qweight, w.qzeros, w.scales, None, w.K, w.N, w.groupsize, w.num_groups,
+                            w.num_experts, w.layout)
+    if T > 0:
         lib = _lib.load()
         y = torch.empty((T * k, w.N // 2), dtype=x.dtype, device=x.device)
         with torch.cuda.device(x.device):
@@ -545,13 +552,14 @@ def moe_linear_gate_up(w: PackedMoeWeight, x: torch.Tensor, routing: MoeRouting,
             st = w.struct()
             ws = reserve_workspace(x.device, int(lib.q4_moe_workspace_bytes(ctypes.byref(st), T, k)), stream)
             rc = lib.q4_moe_linear_gate_up(
-                ctypes.byref(st), x.data_ptr(), routing.sorted_tokens.data_ptr(), routing.expert_offsets.data_ptr(),
+                ctypes.byref(st), x.data_ptr(), x_rows.data_ptr() if x_rows is not None else None,
+                routing.expert_offsets.data_ptr(),
                 y.data_ptr(), T, k, _DTYPES[x.dtype], _lib.ACTIVATIONS[act], ws.data_ptr(), ws.numel(), stream,
             )
         if rc != _lib.ERR_UNSUPPORTED:
             _lib.check(rc)
             return y
-    return act_mul(moe_linear(w, x, routing, gather=True), act)
+    return act_mul(moe_linear(w, x, routing, gather=x_rows is not None), act)
 
 
 def moe_combine(y_sorted: torch.Tensor, routing: MoeRouting) -> torch.Tensor:
