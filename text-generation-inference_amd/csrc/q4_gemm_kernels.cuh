@@ -453,8 +453,18 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restric
   for (long q = (long)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += (long)gridDim.x * blockDim.x) {
     const size_t e = (size_t)q * 4;
     const int n = (int)(e % (size_t)N);
+    // four splits' loads in flight at a time (the partial tiles come from other XCDs' write-backs:
+    // a load per loop iteration would pay one memory round trip per split); summed in split order
     float4_t sum = *(const float4_t*)(partials + e);
-    for (int sp = 1; sp < splits; ++sp) {
+    int sp = 1;
+    for (; sp + 4 <= splits; sp += 4) {
+      float4_t v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = *(const float4_t*)(partials + (size_t)(sp + u) * stride + e);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) { sum.x += v[u].x; sum.y += v[u].y; sum.z += v[u].z; sum.w += v[u].w; }
+    }
+    for (; sp < splits; ++sp) {
       const float4_t v = *(const float4_t*)(partials + (size_t)sp * stride + e);
       sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
     }
