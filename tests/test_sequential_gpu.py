@@ -186,3 +186,30 @@ def test_wqlinear_converts_to_the_gptq_layout_bit_exactly(pkg, oracle, gpu, M, m
     yn = native(x)
     assert not native.gptq_layout and native.packed().layout == 1
     assert max_rel_err(y.float().cpu().numpy(), yn.float().cpu().numpy()) <= TOL
+
+
+def test_out_of_range_permutation_entries_are_clamped(pkg, oracle, gpu):
+    """A permutation with entries outside 0..K-1 must not read outside x or qweight: such entries
+    are clamped to the nearest valid index in the repack kernel, the gather kernels and the
+    decode kernel's fused gather."""
+    K, N, gs = 1024, 256, 128
+    qw, qz, sc, _ = oracle.make_gptq(K, N, gs, seed=4, sym=False)
+    qd = to_dev(qw, gpu)
+    bad = torch.arange(K, dtype=torch.int32, device=gpu)
+    bad[3] = -7
+    bad[100] = K + 12345
+    bad[1023] = 2**31 - 1
+    clamped = bad.clamp(0, K - 1)
+    lib = pkg._lib.load()
+    out_bad, out_ok = torch.empty_like(qd), torch.empty_like(qd)
+    assert lib.q4_gptq_make_sequential(qd.data_ptr(), bad.data_ptr(), out_bad.data_ptr(), K, N, None) == 0
+    assert lib.q4_gptq_make_sequential(qd.data_ptr(), clamped.data_ptr(), out_ok.data_ptr(), K, N, None) == 0
+    assert torch.equal(out_bad, out_ok)
+    x = to_dev(oracle.make_x(2, K, seed=1), gpu)
+    assert torch.equal(pkg.ops.gather_columns(x, bad), x[:, clamped.long()])
+    plain = pkg.ops.make_packed(qd, to_dev(qz, gpu), to_dev(sc, gpu), None, gs, 0)
+    with_bad = pkg.ops.PackedWeight(plain.qweight, plain.qzeros, plain.scales, None, K, N, gs, K // gs, 0, bad)
+    with_ok = pkg.ops.PackedWeight(plain.qweight, plain.qzeros, plain.scales, None, K, N, gs, K // gs, 0, clamped)
+    for M in (1, 2, 5, 40):  # fused gather (1, 2 rows), workspace gather, prefill
+        xm = to_dev(oracle.make_x(M, K, seed=M), gpu)
+        assert torch.equal(pkg.ops.linear(with_bad, xm), pkg.ops.linear(with_ok, xm))

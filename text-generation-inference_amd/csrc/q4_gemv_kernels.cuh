@@ -188,12 +188,13 @@ struct SlabStager {
       const uint16_t* row = xs + (size_t)mr * gp.p.K;
       const uint4_t p0 = *(const uint4_t*)(cols + kb * 8);
       const uint4_t p1 = *(const uint4_t*)(cols + kb * 8 + 4);
-      const uint32_t last = (uint32_t)(gp.p.K - 1);
+      const int last = gp.p.K - 1;
+      auto at = [&](uint32_t i) { return (uint32_t)row[min(max((int)i, 0), last)]; };
       uint4_t o;
-      o.x = (uint32_t)row[min(p0.x, last)] | ((uint32_t)row[min(p0.y, last)] << 16);
-      o.y = (uint32_t)row[min(p0.z, last)] | ((uint32_t)row[min(p0.w, last)] << 16);
-      o.z = (uint32_t)row[min(p1.x, last)] | ((uint32_t)row[min(p1.y, last)] << 16);
-      o.w = (uint32_t)row[min(p1.z, last)] | ((uint32_t)row[min(p1.w, last)] << 16);
+      o.x = at(p0.x) | (at(p0.y) << 16);
+      o.y = at(p0.z) | (at(p0.w) << 16);
+      o.z = at(p1.x) | (at(p1.y) << 16);
+      o.w = at(p1.z) | (at(p1.w) << 16);
       return o;
     }
     return *(const uint4_t*)(xs + (size_t)mr * gp.p.K + kb * 8);

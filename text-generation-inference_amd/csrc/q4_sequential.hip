@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void gather_columns_kernel(const uint16_t* __r
     const uint32_t idx[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
     uint32_t h[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) h[i] = row[min(idx[i], (uint32_t)(K - 1))];
+    for (int i = 0; i < 8; ++i) h[i] = row[min(max((int)idx[i], 0), K - 1)];
     uint4_t o;
     o.x = h[0] | (h[1] << 16);
     o.y = h[2] | (h[3] << 16);
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void moe_gather_columns_kernel(const uint16_t*
     const uint32_t idx[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
     uint32_t h[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) h[i] = row[min(idx[i], (uint32_t)(K - 1))];
+    for (int i = 0; i < 8; ++i) h[i] = row[min(max((int)idx[i], 0), K - 1)];
     uint4_t o;
     o.x = h[0] | (h[1] << 16);
     o.y = h[2] | (h[3] << 16);
