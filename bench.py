@@ -427,6 +427,28 @@ def main():
             moe[f"tokens_{T}"] = {"us_avg": round(avg * 1e6, 1), "experts_active": active,
                                   "weight_GBps": round(wbytes / avg / 1e9, 1), "TFLOPs": round(fl / avg / 1e12, 1)}
         out["moe_block"] = {"experts": E, "topk": topk, "hidden": H, "intermediate": I, "per_tokens": moe}
+        # the same block with act-order experts (the reference's Mixtral test checkpoint is one):
+        # rows put into group order when the layer is built, activations gathered per sorted row
+        del gate_up, down
+        torch.cuda.empty_cache()
+
+        def act_order_experts(K, N):
+            w = experts(K, N)
+            g_idx = torch.stack([(torch.randperm(K, device=dev, generator=gen) // GROUPSIZE).to(torch.int32)
+                                 for _ in range(E)])
+            w = pkg.ops.make_packed_moe(w.qweight, w.qzeros, w.scales, GROUPSIZE, g_idx)
+            return pkg.ops.make_sequential_moe(w)
+
+        gate_up, down = act_order_experts(H, 2 * I), act_order_experts(I, H)
+        torch.cuda.empty_cache()
+        moe_act = {}
+        for T in (1, 16, 1024):
+            xm = torch.randn((T, H), device=dev, dtype=torch.float16)
+            logits = torch.randn((T, E), device=dev, dtype=torch.float32, generator=gen)
+            fn = lambda: pkg.ops.moe_forward(gate_up, down, xm, logits, topk, True, "silu")
+            avg, _ = time_kernel_launches(torch, [fn], 10)
+            moe_act[f"tokens_{T}"] = {"us_avg": round(avg * 1e6, 1)}
+        out["moe_block"]["act_order_experts"] = moe_act
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(M)
