@@ -116,6 +116,12 @@ def test_gather_columns_is_exact(pkg, gpu):
     assert torch.equal(pkg.ops.gather_columns(x, perm), x[:, perm.long()])
     xb = x.to(torch.bfloat16)
     assert torch.equal(pkg.ops.gather_columns(xb, perm), xb[:, perm.long()])
+    # many rows: the kernel that stages each row in LDS; K = 40000 does not fit and falls back
+    big = torch.randn((300, 1024), device=gpu, dtype=torch.float16, generator=g)
+    assert torch.equal(pkg.ops.gather_columns(big, perm), big[:, perm.long()])
+    wide = torch.randn((130, 40000), device=gpu, dtype=torch.float16, generator=g)
+    pw = torch.randperm(40000, device=gpu, generator=g).to(torch.int32)
+    assert torch.equal(pkg.ops.gather_columns(wide, pw), wide[:, pw.long()])
 
 
 def test_groups_of_unequal_size_are_left_alone(pkg, oracle, gpu):

@@ -86,9 +86,65 @@ __global__ __launch_bounds__(256) void moe_gather_columns_kernel(const uint16_t*
   }
 }
 
+// Many rows: a workgroup stages one row of x in LDS with 16-byte loads and gathers from there,
+// so that global memory sees only coalesced traffic (the direct kernels above read 2-byte
+// elements scattered over the row).  perms == one permutation when offsets is nullptr.
+__global__ __launch_bounds__(256) void gather_rows_lds_kernel(const uint16_t* __restrict__ x,
+                                                              const int32_t* __restrict__ x_rows,
+                                                              const int32_t* __restrict__ offsets,
+                                                              const int32_t* __restrict__ perms,
+                                                              uint16_t* __restrict__ out, int num_experts, int rows,
+                                                              int K) {
+  extern __shared__ __align__(16) uint16_t row_lds[];  // [K]
+  const int vec_per_row = K >> 3;
+  for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+    const int32_t* perm = perms;
+    if (offsets != nullptr) {
+      int lo = 0, hi = num_experts;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (offsets[mid] <= r) lo = mid; else hi = mid;
+      }
+      perm += (size_t)lo * K;
+    }
+    const uint16_t* src = x + (size_t)(x_rows != nullptr ? x_rows[r] : r) * K;
+    for (int v = threadIdx.x; v < vec_per_row; v += 256) ((uint4_t*)row_lds)[v] = ((const uint4_t*)src)[v];
+    __syncthreads();
+    for (int v = threadIdx.x; v < vec_per_row; v += 256) {
+      const uint4_t p0 = *(const uint4_t*)(perm + v * 8);
+      const uint4_t p1 = *(const uint4_t*)(perm + v * 8 + 4);
+      const uint32_t idx[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+      uint32_t h[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) h[i] = row_lds[min(max((int)idx[i], 0), K - 1)];
+      uint4_t o;
+      o.x = h[0] | (h[1] << 16);
+      o.y = h[2] | (h[3] << 16);
+      o.z = h[4] | (h[5] << 16);
+      o.w = h[6] | (h[7] << 16);
+      ((uint4_t*)(out + (size_t)r * K))[v] = o;
+    }
+    __syncthreads();
+  }
+}
+
 }  // namespace q4
 
 namespace q4host {
+
+// rows from which the LDS-staged kernel is used (fewer rows leave most CUs without a workgroup)
+static constexpr int kGatherLdsRows = 128;
+
+static bool launch_gather_lds(const void* x, const int32_t* x_rows, const int32_t* offsets, const int32_t* perms,
+                              void* out, int num_experts, int rows, int K, hipStream_t stream) {
+  const size_t smem = (size_t)K * 2;
+  if (rows < kGatherLdsRows || smem > 64 * 1024) return false;
+  const int blocks = rows < 2048 ? rows : 2048;
+  hipLaunchKernelGGL(q4::gather_rows_lds_kernel, dim3((unsigned)blocks), dim3(256), smem, stream, (const uint16_t*)x,
+                     x_rows, offsets, perms, (uint16_t*)out, num_experts, rows, K);
+  return true;
+}
+
 
 int launch_moe_gather_columns(const void* x, const int32_t* x_rows, const int32_t* offsets, const int32_t* perms,
                               void* out, int num_experts, int pairs, int K, hipStream_t stream) {
@@ -96,8 +152,10 @@ int launch_moe_gather_columns(const void* x, const int32_t* x_rows, const int32_
   long blocks = (total + 255) / 256;
   if (blocks > 8192) blocks = 8192;
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL(q4::moe_gather_columns_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t*)x,
-                     x_rows, offsets, perms, (uint16_t*)out, num_experts, pairs, K);
+  if (!launch_gather_lds(x, x_rows, offsets, perms, out, num_experts, pairs, K, stream)) {
+    hipLaunchKernelGGL(q4::moe_gather_columns_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                       (const uint16_t*)x, x_rows, offsets, perms, (uint16_t*)out, num_experts, pairs, K);
+  }
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {
     set_error("q4_moe_gather_columns: launch failed: %s", hipGetErrorString(err));
@@ -124,8 +182,10 @@ int launch_gather_columns(const void* x, const int32_t* perm, void* out, int M, 
   long blocks = (total + 255) / 256;
   if (blocks > 8192) blocks = 8192;
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL(q4::gather_columns_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t*)x, perm,
-                     (uint16_t*)out, M, K);
+  if (!launch_gather_lds(x, nullptr, nullptr, perm, out, 1, M, K, stream)) {
+    hipLaunchKernelGGL(q4::gather_columns_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t*)x,
+                       perm, (uint16_t*)out, M, K);
+  }
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {
     set_error("q4_gather_columns: launch failed: %s", hipGetErrorString(err));
