@@ -139,6 +139,10 @@ int q4_gather_columns(const void* x, const int32_t* perm, void* out, int M, int 
 int q4_linear_perm(const q4_weight* w, const int32_t* perm, const void* x, const void* bias, void* y, int M,
                    int dtype, void* workspace, size_t workspace_bytes, int path, void* stream);
 size_t q4_workspace_bytes_perm(int M, int K, int N);
+/* q4_linear_gate_up for a weight in group order, x in checkpoint order (see q4_linear_perm);
+ * Q4_ERR_UNSUPPORTED where the fused kernel does not apply: then q4_linear_perm + q4_act_mul. */
+int q4_linear_gate_up_perm(const q4_weight* w, const int32_t* perm, const void* x, const void* bias, void* y, int M,
+                           int dtype, int act, void* workspace, size_t workspace_bytes, void* stream);
 /*
  * One block of the GPTQ solver's column loop (GPTQ.fasterquant,
  * server/text_generation_server/layers/gptq/quantize.py:294-331; the quantizer's range rule,

@@ -219,3 +219,22 @@ def test_out_of_range_permutation_entries_are_clamped(pkg, oracle, gpu):
     for M in (1, 2, 5, 40):  # fused gather (1, 2 rows), workspace gather, prefill
         xm = to_dev(oracle.make_x(M, K, seed=M), gpu)
         assert torch.equal(pkg.ops.linear(with_bad, xm), pkg.ops.linear(with_ok, xm))
+
+
+@pytest.mark.parametrize("K,M", [(2048, 1), (2048, 2), (8192, 1), (2048, 5), (2048, 300)])
+def test_gated_mlp_first_half_on_rows_in_group_order(pkg, oracle, gpu, K, M):
+    """act(gate) * up with a [gate | up] weight in group order: the fused decode kernel gathers
+    while staging (K <= 4096) or after a gather pass (longer K); more rows take linear + act_mul.
+    All agree with the same computation on hand-gathered activations and with the oracle."""
+    N, gs = 512, 128
+    qw, qz, sc, gi, pk = build(pkg, oracle, gpu, K, N, gs, seed=K // 256 + M)
+    seq = pkg.ops.make_sequential(pk)
+    xh = oracle.make_x(M, K, seed=M + 11)
+    x = to_dev(xh, gpu)
+    got = pkg.ops.linear_gate_up(seq, x, "silu")
+    plain = pkg.ops.PackedWeight(seq.qweight, seq.qzeros, seq.scales, None, K, N, gs, K // gs, 0)
+    want = pkg.ops.linear_gate_up(plain, x[:, seq.perm.long()].contiguous(), "silu")
+    assert torch.equal(got, want)
+    w = oracle.dequant_gptq(qw, qz, sc, gi, gs, "f16")
+    _, ref = oracle.gate_up_forward(xh, w, "silu", None, "f16")
+    assert max_rel_err(got.float().cpu().numpy(), oracle.to_f32(ref, "f16")) <= TOL

@@ -91,6 +91,8 @@ SIGNATURES = {
     "q4_linear_perm": (c_int, [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                 c_size_t, c_int, c_void_p]),
     "q4_workspace_bytes_perm": (c_size_t, [c_int, c_int, c_int]),
+    "q4_linear_gate_up_perm": (c_int, [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                        c_void_p, c_size_t, c_void_p]),
     "q4_gptq_solve_block": (c_int, [c_void_p] * 7 + [c_int] * 7 + [c_void_p]),
     "q4_moe_gather_columns": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "q4_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),

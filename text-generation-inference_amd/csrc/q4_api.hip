@@ -285,6 +285,47 @@ int q4_linear_perm(const q4_weight* w, const int32_t* perm, const void* x, const
   return q4_linear_ex(w, x_seq, bias, y, M, dtype, workspace, offset, path, stream);
 }
 
+int q4_linear_gate_up_perm(const q4_weight* w, const int32_t* perm, const void* x, const void* bias, void* y, int M,
+                           int dtype, int act, void* workspace, size_t workspace_bytes, void* stream) {
+  if (perm == nullptr) return q4_linear_gate_up(w, x, bias, y, M, dtype, act, workspace, workspace_bytes, stream);
+  int rc = validate_weight(w, "q4_linear_gate_up_perm");
+  if (rc == Q4_OK) rc = validate_dtype(dtype, "q4_linear_gate_up_perm");
+  if (rc != Q4_OK) return rc;
+  if (act != Q4_ACT_SILU && act != Q4_ACT_GELU_TANH && act != Q4_ACT_GELU) {
+    set_error("q4_linear_gate_up_perm: unknown activation %d", act);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M < 0 || (w->N & 1) || w->layout != Q4_LAYOUT_GPTQ || w->g_idx != nullptr) {
+    set_error("q4_linear_gate_up_perm: bad M=%d, odd N=%d, or a weight that is not a GPTQ matrix in group order", M,
+              w->N);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M == 0 || w->N == 0) return Q4_OK;
+  if (y == nullptr || x == nullptr) {
+    set_error("q4_linear_gate_up_perm: null x or y");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (!(q4_select_path(w, M, dtype) == Q4_PATH_GEMV && gemv_gate_up_supported(w, M, dtype))) {
+    set_error("q4_linear_gate_up_perm: no fused kernel for this problem (M=%d K=%d N=%d groupsize=%d)", M, w->K, w->N,
+              w->groupsize);
+    return Q4_ERR_UNSUPPORTED;
+  }
+  // the fused kernel runs for one or two rows: with a short K it gathers while staging (see q4_linear_perm)
+  if (w->K <= 4096)
+    return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, nullptr, (hipStream_t)stream, act + 1, perm);
+  const size_t offset = perm_gather_offset(M, w->K, w->N);
+  const size_t need = offset + (size_t)M * w->K * 2;
+  if (workspace == nullptr || workspace_bytes < need || w->K % 8 != 0) {
+    set_error("q4_linear_gate_up_perm: workspace of %zu bytes needed (q4_workspace_bytes_perm), %zu given", need,
+              workspace_bytes);
+    return Q4_ERR_WORKSPACE;
+  }
+  void* x_seq = (char*)workspace + offset;
+  rc = launch_gather_columns(x, perm, x_seq, M, w->K, (hipStream_t)stream);
+  if (rc != Q4_OK) return rc;
+  return launch_gemv(w, x_seq, bias, y, M, dtype, workspace, offset, nullptr, (hipStream_t)stream, act + 1);
+}
+
 int q4_linear_gate_up(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                       int act, void* workspace, size_t workspace_bytes, void* stream) {
   int rc = validate_weight(w, "q4_linear_gate_up");

@@ -325,9 +325,6 @@ def linear_gate_up(
     if act not in _lib.ACTIVATIONS:
         raise ValueError(f"unknown activation {act!r}; known: {sorted(_lib.ACTIVATIONS)}")
     x = x.contiguous()
-    if w.perm is not None:
-        x = gather_columns(x, w.perm)
-        w = PackedWeight(w.qweight, w.qzeros, w.scales, None, w.K, w.N, w.groupsize, w.num_groups, w.layout)
     M, inter = x.shape[0], w.N // 2
     y = out if out is not None else torch.empty((M, inter), dtype=x.dtype, device=x.device)
     if tuple(y.shape) != (M, inter) or y.dtype != x.dtype or y.device != x.device or not y.is_contiguous():
@@ -339,10 +336,12 @@ def linear_gate_up(
         lib = _lib.load()
         with torch.cuda.device(x.device):
             stream = _stream_handle(x.device)
-            ws = reserve_workspace(x.device, workspace_bytes(M, w.K, w.N), stream)
+            need = workspace_bytes(M, w.K, w.N) if w.perm is None else int(lib.q4_workspace_bytes_perm(M, w.K, w.N))
+            ws = reserve_workspace(x.device, need, stream)
             st = w.struct()
-            rc = lib.q4_linear_gate_up(
-                ctypes.byref(st), x.data_ptr(), bias.contiguous().data_ptr() if bias is not None else None,
+            rc = lib.q4_linear_gate_up_perm(
+                ctypes.byref(st), w.perm.data_ptr() if w.perm is not None else None, x.data_ptr(),
+                bias.contiguous().data_ptr() if bias is not None else None,
                 y.data_ptr(), M, _DTYPES[x.dtype], _lib.ACTIVATIONS[act], ws.data_ptr(), ws.numel(), stream,
             )
         if rc != _lib.ERR_UNSUPPORTED or fused:
