@@ -5,13 +5,15 @@
 // Output rows are independent: one wave owns one row and keeps the block's 128 weights in
 // registers (two per lane), so the 128 dependent steps cost a broadcast, a handful of VALU
 // operations and one LDS row read each instead of several kernel launches.  The block of U
-// sits in LDS, shared by the waves of a workgroup.  The update of the columns behind the
+// sits in LDS, shared by the sixteen waves of a workgroup (the loop is a chain of dependent
+// operations: many resident waves per CU hide its latency).  The update of the columns behind the
 // block (W[:, i2:] -= Err @ U[i1:i2, i2:]) is a plain GEMM and stays with the caller.
 #include "q4_common.cuh"
 
 namespace q4 {
 
 constexpr int kSolveBlock = 128;  // columns per block (two per lane)
+constexpr int kSolveWaves = 16;   // rows (waves) per workgroup: they share the LDS copy of the block of U
 
 struct SolveParams {
   float* __restrict__ W;          // [rows, K] row-major, current weights; block columns are read
@@ -37,16 +39,16 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
-__global__ __launch_bounds__(256) void gptq_solve_block_kernel(SolveParams sp) {
+__global__ __launch_bounds__(64 * kSolveWaves) void gptq_solve_block_kernel(SolveParams sp) {
   extern __shared__ __align__(16) float u_lds[];  // [count][kSolveBlock]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int count = sp.count, K = sp.K;
-  for (int idx = tid; idx < count * kSolveBlock; idx += 256) {
+  for (int idx = tid; idx < count * kSolveBlock; idx += 64 * kSolveWaves) {
     const int r = idx / kSolveBlock, c = idx - r * kSolveBlock;
     u_lds[idx] = c < count ? sp.U[(size_t)(sp.i1 + r) * K + sp.i1 + c] : 0.f;
   }
   __syncthreads();
-  const int row = blockIdx.x * 4 + wave;
+  const int row = blockIdx.x * kSolveWaves + wave;
   if (row >= sp.rows) return;
   float* wrow = sp.W + (size_t)row * K;
   const int c0 = lane, c1 = lane + 64;
@@ -130,7 +132,8 @@ int launch_gptq_solve_block(float* W, const float* U, float* Q, float* Err, floa
   if (smem > 64 * 1024)
     (void)hipFuncSetAttribute((const void*)q4::gptq_solve_block_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)smem);
-  hipLaunchKernelGGL(q4::gptq_solve_block_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), smem, stream, sp);
+  hipLaunchKernelGGL(q4::gptq_solve_block_kernel, dim3((unsigned)((rows + q4::kSolveWaves - 1) / q4::kSolveWaves)),
+                     dim3(64 * q4::kSolveWaves), smem, stream, sp);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) {
     set_error("q4_gptq_solve_block: launch failed: %s", hipGetErrorString(err));
