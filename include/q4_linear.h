@@ -130,7 +130,7 @@ int q4_gptq_make_sequential(const uint32_t* qweight, const int32_t* perm, uint32
 int q4_gather_columns(const void* x, const int32_t* perm, void* out, int M, int K, void* stream);
 /*
  * q4_linear for a weight in group order, x in checkpoint order: y = x[:, perm] @ W (+ bias).
- * With one or two rows and K <= 4096 the decode kernel reads x through perm while it stages it
+ * With a few rows and K <= 4096 the decode kernel reads x through perm while it stages it
  * (no extra pass, as the reference's kernel does with b_q_perm); otherwise x is gathered once
  * into the tail of the workspace, which therefore must hold q4_workspace_bytes_perm(M, K, N)
  * bytes (its head is the zero-initialised area of q4_workspace_bytes).  `path` as for q4_linear_ex; perm NULL

@@ -260,12 +260,13 @@ int q4_linear_perm(const q4_weight* w, const int32_t* perm, const void* x, const
     return Q4_ERR_INVALID_ARGUMENT;
   }
   if (path == Q4_PATH_AUTO) path = q4_select_path(w, M, dtype);
-  // Decode of one or two rows with a short K: the kernel reads x through perm while it stages
-  // its activation slab.  Every workgroup gathers its own copy, so the saved launch (~2.5 us)
-  // is soon outweighed: measured against the separate pass at M = 1, 4096 x 4096 6.4 / 7.8 us,
-  // 4096 x 28672 15.8 / 17.3, but 14336 x 4096 13.4 / 12.3, 28672 x 8192 29.0 / 26.0, and at
-  // M = 16 4096 x 6144 18.1 / 14.3, 14336 x 4096 37.9 / 20.0.
-  if (path == Q4_PATH_GEMV && M <= 2 && w->K <= 4096)
+  // Decode of a few rows with a short K: the kernel reads x through perm while it stages its
+  // activation slab.  Every workgroup gathers its own copy, so the saved launch (~2.5 us) is
+  // soon outweighed: measured against the separate pass at M = 1, 4096 x 4096 6.4 / 7.8 us,
+  // 4096 x 28672 15.8 / 17.3, but 14336 x 4096 13.4 / 12.3, 28672 x 8192 29.0 / 26.0; at M = 4
+  // 4096 x 4096 9.1 / 10.6, 4096 x 6144 9.8 / 10.7, but 4096 x 28672 20.2 / 19.2; at M = 8
+  // 4096 x 6144 12.7 / 11.7; at M = 16 4096 x 6144 18.1 / 14.3, 14336 x 4096 37.9 / 20.0.
+  if (path == Q4_PATH_GEMV && w->K <= 4096 && (M <= 2 || (M <= 4 && w->N <= 8192)))
     return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, nullptr, (hipStream_t)stream, 0, perm);
   // otherwise one gather pass into the tail of the workspace, then the kernel of the plain call
   if (w->K % 8 != 0) {
