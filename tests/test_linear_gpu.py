@@ -528,3 +528,37 @@ def test_act_order_dispatch(pkg, oracle, gpu):
     assert pkg.ops.select_path(pk, 1024) == "gemm"
     assert pkg.ops.select_path(pk, 1024, torch.bfloat16) == "gemm"
     assert pkg.ops.select_path(pk, 4, torch.bfloat16) == "generic"  # the act-order decode kernel is fp16 only
+
+
+# --------------------------------------------------------------------------- full-size properties
+
+
+@pytest.mark.parametrize("K,N", [(4096, 6144), (4096, 4096), (4096, 28672), (14336, 4096)])
+def test_llama3_8b_shapes_size_independent_properties(pkg, oracle, gpu, K, N):
+    """At the benchmark's full sizes, properties that need no CPU matmul: one-hot activations read
+    single weight rows back bit for bit through every decode combine (cells for 1..3 rows, tickets,
+    two row blocks) and through the prefill GEMM; the decode and prefill kernels agree on random
+    activations; y is linear in x to rounding."""
+    g = torch.Generator(device=gpu).manual_seed(K + N)
+    qweight = torch.randint(-(2**31), 2**31 - 1, (K // 8, N), dtype=torch.int64, device=gpu, generator=g).to(torch.int32)
+    qzeros = torch.randint(-(2**31), 2**31 - 1, (K // 128, N // 8), dtype=torch.int64, device=gpu, generator=g).to(torch.int32)
+    scales = (torch.rand((K // 128, N), device=gpu, generator=g) * 0.019 + 0.001).half()
+    w = pkg.ops.make_packed(qweight, qzeros, scales, None, 128, 0)
+    dense = pkg.ops.dequantize(w)  # bit-exact against the oracle in the dequant tests
+    rows = torch.randint(0, K, (40,), device=gpu, generator=g)
+    for M in (1, 3, 8, 18, 40):
+        x = torch.zeros((M, K), dtype=torch.float16, device=gpu)
+        x[torch.arange(M, device=gpu), rows[:M]] = 1.0
+        y = pkg.ops.linear(w, x)
+        assert torch.equal(y, dense[rows[:M]]), f"one-hot rows, M={M}"
+    x = torch.zeros((40, K), dtype=torch.float16, device=gpu)
+    x[torch.arange(40, device=gpu), rows] = 1.0
+    assert torch.equal(pkg.ops.linear(w, x, path=2), dense[rows])
+    a = torch.randn((16, K), device=gpu, dtype=torch.float16, generator=g)
+    b = torch.randn((16, K), device=gpu, dtype=torch.float16, generator=g)
+    ya, yb = pkg.ops.linear(w, a, path=1).float(), pkg.ops.linear(w, b, path=1).float()
+    ga = pkg.ops.linear(w, a, path=2).float()
+    scale = float(ya.abs().max())
+    assert float((ya - ga).abs().max()) <= 2e-3 * scale          # decode against prefill kernel
+    yab = pkg.ops.linear(w, (a.float() * 0.5 + b.float() * 0.5).half(), path=1).float()
+    assert float((yab - 0.5 * (ya + yb)).abs().max()) <= 4e-3 * scale  # linearity to input/output rounding
