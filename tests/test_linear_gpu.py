@@ -342,6 +342,13 @@ def test_act_order_decode_llama70b(pkg, oracle, gpu, K, N, M):
     _run(pkg, oracle, gpu, K, N, 128, M, act=True, path=1, seed=K // 1024 + M)
 
 
+@pytest.mark.parametrize("K,N,M", [(4096, 14336, 1), (4096, 14336, 8), (4096, 28672, 16), (14336, 4096, 16)])
+def test_act_order_decode_picker_branches(pkg, oracle, gpu, K, N, M):
+    """The lookup kernels' picker: two column tiles per workgroup on wide layers, and the single
+    round of workgroups it takes with 12 rows or more when the slab leaves one workgroup per CU."""
+    _run(pkg, oracle, gpu, K, N, 128, M, act=True, sym=False, path=1, seed=N // 1024 + M)
+
+
 @pytest.mark.parametrize("M", [1, 5, 16, 33, 128])
 def test_act_order_small(pkg, oracle, gpu, M):
     _run(pkg, oracle, gpu, 1024, 256, 128, M, sym=False, act=True, bias=True, seed=M + 300)
