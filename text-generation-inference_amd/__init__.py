@@ -9,7 +9,7 @@ on sys.path.
 
 from . import _lib, ops  # noqa: F401
 from .layers.linear import get_linear  # noqa: F401
-from .layers.mlp import gate_up_act  # noqa: F401
+from .layers.mlp import fold_down_permutation, gate_up_act  # noqa: F401
 from .layers.gptq import (  # noqa: F401
     GPTQWeight,
     GPTQWeightsLoader,

@@ -145,6 +145,22 @@ def make_sequential(w: PackedWeight) -> Optional[PackedWeight]:
     return PackedWeight(out, w.qzeros, w.scales, None, K, w.N, w.groupsize, w.num_groups, w.layout, perm32)
 
 
+def permute_output_columns(w: PackedWeight, cols: torch.Tensor) -> PackedWeight:
+    """The same weight with its output columns reordered: column j of the result is column
+    cols[j] of w (GPTQ layout; load-time integer reshuffles, nothing is requantized)."""
+    from .layers.awq.conversion_utils import pack, unpack
+
+    if w.layout != LAYOUT_GPTQ:
+        raise ValueError("permute_output_columns handles the GPTQ layout")
+    cols = cols.to(torch.int64)
+    if cols.numel() != w.N:
+        raise ValueError(f"cols has {cols.numel()} entries, expected {w.N}")
+    qweight = w.qweight.index_select(1, cols).contiguous()
+    scales = w.scales.index_select(1, cols).contiguous()
+    qzeros = pack(unpack(w.qzeros, "column").index_select(1, cols), "column").contiguous()
+    return PackedWeight(qweight, qzeros, scales, w.g_idx, w.K, w.N, w.groupsize, w.num_groups, w.layout, w.perm)
+
+
 def gather_columns(x: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:
     """x[:, perm] for a contiguous fp16/bf16 [M, K] tensor, through the HIP gather kernel."""
     out = torch.empty_like(x)
