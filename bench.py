@@ -428,7 +428,8 @@ def main():
                                   "weight_GBps": round(wbytes / avg / 1e9, 1), "TFLOPs": round(fl / avg / 1e12, 1)}
         out["moe_block"] = {"experts": E, "topk": topk, "hidden": H, "intermediate": I, "per_tokens": moe}
         # the same block with act-order experts (the reference's Mixtral test checkpoint is one):
-        # rows put into group order when the layer is built, activations gathered per sorted row
+        # rows put into group order when the layer is built, activations gathered per sorted row for
+        # the first projection
         del gate_up, down
         torch.cuda.empty_cache()
 
@@ -440,6 +441,8 @@ def main():
             return pkg.ops.make_sequential_moe(w)
 
         gate_up, down = act_order_experts(H, 2 * I), act_order_experts(I, H)
+        # as the layer does: the down projections' input order goes into the gate_up columns
+        gate_up, down = pkg.ops.fold_moe_down_permutation(gate_up, down)
         torch.cuda.empty_cache()
         moe_act = {}
         for T in (1, 16, 1024):

@@ -413,7 +413,11 @@ def test_sparse_moe_layer_from_safetensors(pkg, oracle, gpu, tmp_path, desc_act)
         assert (layer._gate_up.g_idx is not None) == desc_act and layer._gate_up.perm is None
     else:  # act-order experts are put into group order once: no g_idx left, a permutation per expert
         assert layer._gate_up.g_idx is None and layer._down.g_idx is None
-        assert (layer._gate_up.perm is not None) == desc_act and (layer._down.perm is not None) == desc_act
+        assert (layer._gate_up.perm is not None) == desc_act
+    if desc_act and mode != "table":
+        # the down projections' input order went into the gate_up columns: no gather in between
+        assert layer._down.perm is None and layer._gate_up.perm is not None
+        assert layer.down_proj.rows_in_group_order and layer.down_proj.packed().g_idx is None
     rng = np.random.default_rng(5)
     x = oracle.make_x(6, H, seed=2)
     g = rng.standard_normal((6, E)).astype(np.float32)
@@ -421,6 +425,25 @@ def test_sparse_moe_layer_from_safetensors(pkg, oracle, gpu, tmp_path, desc_act)
     assert out.shape == (2, 3, H)
     ref32, _ = oracle.moe_forward(x, g, gu, dn, k, True, "silu", "f16")
     assert max_rel_err(to_f32(out).reshape(6, H), ref32) <= 2 * TOL
+
+
+@pytest.mark.parametrize("T", [1, 7, 90])
+def test_expert_down_permutations_folded_into_gate_up_columns(pkg, oracle, gpu, T):
+    """Folding every expert's down-projection permutation into its gate and up columns leaves the
+    block's output bit for bit as with the activation gather between the projections."""
+    E, k, H, I, gs = 4, 2, 1024, 512, 128
+    gu, _ = _packed_experts(pkg, oracle, gpu, "act", E, H, 2 * I, gs, "f16", seed=3)
+    dn, _ = _packed_experts(pkg, oracle, gpu, "act", E, I, H, gs, "f16", seed=9)
+    gu, dn = pkg.ops.make_sequential_moe(gu), pkg.ops.make_sequential_moe(dn)
+    fgu, fdn = pkg.ops.fold_moe_down_permutation(gu, dn)
+    assert fdn.perm is None and fgu.perm is not None
+    assert pkg.ops.fold_moe_down_permutation(fgu, fdn)[1] is fdn  # nothing left to fold
+    rng = np.random.default_rng(T)
+    g, _ = _gating(rng, T, E, "f32")
+    x = to_dev(oracle.make_x(T, H, seed=T), gpu)
+    want = pkg.ops.moe_forward(gu, dn, x, g.to(gpu), k, True, "silu")
+    got = pkg.ops.moe_forward(fgu, fdn, x, g.to(gpu), k, True, "silu")
+    assert torch.equal(got, want)
 
 
 def test_awq_layout_experts_are_converted_once(pkg, oracle, gpu):

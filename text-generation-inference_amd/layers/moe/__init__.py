@@ -40,6 +40,9 @@ class GPTQMoEWeight:
     use_awq_kernel: bool
 
     q_perm: Optional[torch.Tensor] = None  # set once the experts' rows are in group order
+    # rows in group order with the activations' order folded into the producer's columns:
+    # plain contiguous-group experts, g_idx no longer describes the stored rows
+    rows_in_group_order: bool = False
 
     def packed(self) -> ops.PackedMoeWeight:
         if self.use_awq_kernel and AWQ_MODE != "native" and self.qweight.is_cuda:
@@ -50,7 +53,7 @@ class GPTQMoEWeight:
             self.qzeros = torch.stack([c[1] for c in converted]).contiguous()
             self.use_awq_kernel = False
         g_idx = self.g_idx
-        if self.q_perm is not None or (
+        if self.rows_in_group_order or self.q_perm is not None or (
                 g_idx is not None and all(is_trivial_g_idx(g, self.groupsize) for g in g_idx)):
             g_idx = None  # sequential groups in every expert: the kernels index by k // groupsize
         pk = ops.make_packed_moe(self.qweight, self.qzeros, self.scales, self.groupsize, g_idx,
@@ -161,6 +164,15 @@ class GPTQSparseMoELayer(nn.Module):
         self.bits = 4
         self._gate_up = self.gate_up_proj.packed()
         self._down = self.down_proj.packed()
+        # act-order experts: the second projection's input order goes into the first one's
+        # output columns, expert by expert (no activation gather between the projections)
+        folded_gate_up, folded_down = ops.fold_moe_down_permutation(self._gate_up, self._down)
+        if folded_down is not self._down:
+            self.gate_up_proj.qweight, self.gate_up_proj.qzeros, self.gate_up_proj.scales = (
+                folded_gate_up.qweight, folded_gate_up.qzeros, folded_gate_up.scales)
+            self.down_proj.q_perm = None
+            self.down_proj.rows_in_group_order = True
+            self._gate_up, self._down = folded_gate_up, folded_down
 
     @torch.no_grad()
     def forward(self, x: torch.Tensor, *, gating_output: torch.Tensor) -> torch.Tensor:

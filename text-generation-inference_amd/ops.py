@@ -454,6 +454,30 @@ def make_sequential_moe(w: PackedMoeWeight) -> Optional[PackedMoeWeight]:
     return PackedMoeWeight(out, w.qzeros, w.scales, None, K, w.N, w.groupsize, w.num_groups, E, w.layout, perm32)
 
 
+def fold_moe_down_permutation(gate_up: PackedMoeWeight, down: PackedMoeWeight):
+    """Experts whose down projection is in group order: apply every expert's permutation to the
+    output columns of its gate and up halves instead (load time; see permute_output_columns), so
+    that the second projection needs no activation gather.  Returns (gate_up, down), unchanged
+    when there is nothing to fold."""
+    if down.perm is None or gate_up.layout != LAYOUT_GPTQ or gate_up.N != 2 * down.K \
+            or gate_up.num_experts != down.num_experts:
+        return gate_up, down
+    inter = down.K
+    parts = []
+    for e in range(gate_up.num_experts):
+        one = PackedWeight(gate_up.qweight[e], gate_up.qzeros[e], gate_up.scales[e], None, gate_up.K, gate_up.N,
+                           gate_up.groupsize, gate_up.num_groups, gate_up.layout)
+        perm = down.perm[e].to(torch.int64)
+        parts.append(permute_output_columns(one, torch.cat([perm, perm + inter])))
+    new_gate_up = PackedMoeWeight(
+        torch.stack([p.qweight for p in parts]), torch.stack([p.qzeros for p in parts]),
+        torch.stack([p.scales for p in parts]), gate_up.g_idx, gate_up.K, gate_up.N, gate_up.groupsize,
+        gate_up.num_groups, gate_up.num_experts, gate_up.layout, gate_up.perm)
+    new_down = PackedMoeWeight(down.qweight, down.qzeros, down.scales, None, down.K, down.N, down.groupsize,
+                               down.num_groups, down.num_experts, down.layout, None)
+    return new_gate_up, new_down
+
+
 def _moe_gather(w: PackedMoeWeight, x: torch.Tensor, routing: "MoeRouting", gather: bool) -> torch.Tensor:
     """Activations of every sorted row in its expert's row order: [tokens*k, K]."""
     T, k = routing.topk_ids.shape
