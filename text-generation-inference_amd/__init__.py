@@ -19,7 +19,7 @@ from .layers.gptq import (  # noqa: F401
     set_device,
 )
 from .layers.awq.quantize import WQLinear  # noqa: F401
-from .layers.gptq.solver import GPTQ  # noqa: F401
+from .layers.gptq.solver import GPTQ, quantize_linear  # noqa: F401
 from .layers.moe import GPTQSparseMoELayer, GPTQMoEWeight  # noqa: F401
 from .layers.awq import conversion_utils  # noqa: F401
 from .utils.weights import Weights, WeightsLoader, DefaultWeightsLoader, UnquantizedWeight  # noqa: F401

@@ -117,3 +117,23 @@ class GPTQ:
     def free(self):
         self.H = None
         torch.cuda.empty_cache()
+
+
+@torch.no_grad()
+def quantize_linear(layer: nn.Linear, calibration: torch.Tensor, groupsize: int = 128, act_order: bool = False,
+                    sym: bool = True, percdamp: float = 0.01):
+    """Calibrate, solve and pack one linear layer: the per-layer body of the reference's
+    `sequential` (layers/gptq/quantize.py:703-735: add_batch over the calibration inputs, fasterquant,
+    free) followed by `pack` (:780-791).  `calibration` is [..., in_features] on the layer's (GPU) device; returns
+    (QuantLinear on that device, error).  The layer's weight is left holding the quantized values."""
+    from .quant_linear import QuantLinear
+
+    solver = GPTQ(layer, sym=sym)
+    x = calibration.reshape(-1, calibration.shape[-1])
+    for chunk in x.split(4096):  # one "batch" per chunk keeps the Hessian update a bounded GEMM
+        solver.add_batch(chunk.unsqueeze(0))
+    scale, zero, g_idx, error = solver.fasterquant(percdamp=percdamp, groupsize=groupsize, act_order=act_order)
+    solver.free()
+    packed = QuantLinear.new(4, groupsize, layer.in_features, layer.out_features, layer.bias is not None)
+    packed.pack(layer, scale.cpu(), zero.cpu(), g_idx.cpu())
+    return packed.to(layer.weight.device), error
