@@ -174,12 +174,12 @@ def test_gpu_solver_rejects_cpu_layers_and_bad_blocks(pkg, gpu):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("act_order", [False, True])
-def test_quantize_linear_end_to_end(pkg, oracle, gpu, act_order):
+@pytest.mark.parametrize("act_order,gs,sym", [(False, 128, False), (True, 128, False), (False, -1, True), (True, 64, True)])
+def test_quantize_linear_end_to_end(pkg, oracle, gpu, act_order, gs, sym):
     """Calibrate -> solve -> pack -> run: the quantized layer tracks the dense one on held-out
     inputs of the calibration distribution better than round-to-nearest does."""
     rng = np.random.default_rng(4)
-    rows, K, gs = 192, 512, 128
+    rows, K = 192, 512
     X = calib(rng, K, 2048)
     W = rng.standard_normal((rows, K)) * 0.05
     lin = torch.nn.Linear(K, rows, bias=True)
@@ -187,10 +187,10 @@ def test_quantize_linear_end_to_end(pkg, oracle, gpu, act_order):
     b = lin.bias.data.clone()
     lin = lin.to(gpu)
     layer, err = pkg.quantize_linear(lin, torch.from_numpy(X[:1536].astype(np.float32)).to(gpu), groupsize=gs,
-                                     act_order=act_order, sym=False)
+                                     act_order=act_order, sym=sym)
     assert type(layer).__name__ == "QuantLinear" and err > 0
     held = X[1536:1600]
     y = layer(torch.from_numpy(held.astype(np.float16)).to(gpu)).float().cpu().numpy()
     want = held.astype(np.float16).astype(np.float64) @ W.T + b.numpy()
-    out_rtn = np.linalg.norm(held @ (W - rtn(oracle, W, gs, False)).T)
+    out_rtn = np.linalg.norm(held @ (W - rtn(oracle, W, gs, sym)).T)
     assert np.linalg.norm(y - want) < out_rtn
