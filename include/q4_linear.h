@@ -195,6 +195,19 @@ int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, 
 #define Q4_WORKSPACE_CELL_BYTES 1048576   /* 64-bit fixed-point accumulation cells (fp16 decode, few rows) */
 #define Q4_WORKSPACE_COUNTER_BYTES 1064960 /* = tickets + cells: the part that must start zero */
 size_t q4_workspace_bytes(int M, int K, int N);
+/*
+ * The same for one weight: exactly what q4_linear / q4_linear_gate_up need for `w` at M rows
+ * (either dtype).  q4_workspace_bytes is an upper bound over every weight of the shape.
+ */
+size_t q4_workspace_bytes_for(const q4_weight* w, int M);
+/*
+ * Everything a caller needs to know before q4_linear_ex(w, ..., M, dtype, ...) in one call:
+ * *path = q4_select_path(w, M, dtype), *workspace_bytes = q4_workspace_bytes_for(w, M).  Both are
+ * pure functions of (w's geometry, M, dtype): a caller may keep them per layer and batch size
+ * and pass `path` to q4_linear_ex.  Replaces the per-layer sizing the reference does once at
+ * Warmup (server/text_generation_server/layers/gptq/exllamav2.py:159-175, 233-240).
+ */
+int q4_linear_plan(const q4_weight* w, int M, int dtype, int* path, size_t* workspace_bytes);
 
 /*
  * ---- Mixture of experts: the same linear layer, grouped over experts -----------------

@@ -157,6 +157,44 @@ def test_workspace_sizing_covers_every_launch(pkg):
                     assert rc != L.ERR_WORKSPACE, ("moe fused", layout, g_idx, K, N, M, dt, lib.q4_last_error())
 
 
+def test_workspace_sizing_other_group_sizes_and_70b_shapes(pkg):
+    """Act-order weights with other group sizes than 128 pick other K splits (their parameter
+    table shares LDS with the slab): both the per-shape bound and the per-weight size must cover
+    what the launcher then asks for."""
+    lib = pkg._lib.load()
+    L = pkg._lib
+    for K, N in [(8192, 28672), (28672, 8192), (8192, 10240), (4096, 4096)]:
+        for gs in (32, 64, 128, 256):
+            for layout, g_idx in ((0, True), (0, False), (1, False)):
+                for M in (1, 2, 4, 8, 12, 16):
+                    for dt in (0, 1):
+                        w = _weight(pkg, K, N, gs, layout, g_idx)
+                        for ws in (lib.q4_workspace_bytes(M, K, N), lib.q4_workspace_bytes_for(ctypes.byref(w), M)):
+                            rc = lib.q4_linear(ctypes.byref(w), 0x10, None, 0x20, M, dt, 0x40, ws, None)
+                            assert rc != L.ERR_WORKSPACE, (layout, g_idx, K, N, gs, M, dt, lib.q4_last_error())
+                        if layout == 0 and not g_idx and N % 128 == 0:
+                            ws = lib.q4_workspace_bytes_for(ctypes.byref(w), M)
+                            rc = lib.q4_linear_gate_up(ctypes.byref(w), 0x10, None, 0x20, M, dt, 0, 0x40, ws, None)
+                            assert rc != L.ERR_WORKSPACE, ("gate_up", K, N, gs, M, dt, lib.q4_last_error())
+
+
+def test_linear_plan_matches_its_parts(pkg):
+    lib = pkg._lib.load()
+    L = pkg._lib
+    path, need = ctypes.c_int(0), ctypes.c_size_t(0)
+    for layout, g_idx in ((0, False), (0, True), (1, False)):
+        for M in (1, 16, 17, 64, 2048):
+            w = _weight(pkg, 4096, 6144, 128, layout, g_idx)
+            assert lib.q4_linear_plan(ctypes.byref(w), M, 0, ctypes.byref(path), ctypes.byref(need)) == 0
+            assert path.value == lib.q4_select_path(ctypes.byref(w), M, 0)
+            assert need.value == lib.q4_workspace_bytes_for(ctypes.byref(w), M)
+            assert L.WORKSPACE_COUNTER_BYTES <= need.value <= lib.q4_workspace_bytes(M, 4096, 6144)
+    w = _weight(pkg, 4096, 6144, 128)
+    assert lib.q4_linear_plan(ctypes.byref(w), 1, 0, None, ctypes.byref(need)) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_linear_plan(ctypes.byref(w), 1, 9, ctypes.byref(path), ctypes.byref(need)) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_linear_plan(None, 1, 0, ctypes.byref(path), ctypes.byref(need)) == L.ERR_INVALID_ARGUMENT
+
+
 def test_path_selection_and_workspace(pkg):
     lib = pkg._lib.load()
     L = pkg._lib

@@ -108,3 +108,35 @@ def test_moe_block_under_graph_replay(pkg, oracle, gpu):
 
     capture_and_check([call(c) for c in cases], gpu,
                       between=lambda: pkg.ops.moe_forward(*cases[0][:4], k, True, "silu"))
+
+
+@pytest.mark.parametrize("kind", ["act_order", "awq", "gptq"])
+@pytest.mark.parametrize("M", [1, 16])
+def test_first_forward_of_a_fresh_layer_is_capturable(pkg, oracle, gpu, kind, M):
+    """Everything that is not the matmul (act-order test on g_idx, validation, launch plan,
+    workspace) happens when the layer is built: its very first forward can be recorded into a
+    HIP graph, and every replay (with eager work and synchronizations in between) returns the
+    eager result bit for bit."""
+    K, N, gs = 2048, 1024, 128
+    if kind == "awq":
+        qw, qz, sc = oracle.make_awq(K, N, gs, seed=3)
+        build = lambda: pkg.WQLinear(4, gs, to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None)
+    else:
+        qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=4, sym=False, act_order=(kind == "act_order"))
+        g = to_dev(gi, gpu) if gi is not None else (torch.arange(K, device=gpu) // gs).to(torch.int32)
+        build = lambda: pkg.QuantLinear(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), g, None, 4, gs)
+    x = to_dev(oracle.make_x(M, K, seed=M), gpu)
+    want = build()(x).clone()  # eager result of an identical layer
+    layer = build()            # fresh: has never run
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = layer(x)
+    for i in range(3):
+        y.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), (kind, M, i)
+        _ = layer(x + 1.0)  # eager work between the replays
+        torch.cuda.synchronize()

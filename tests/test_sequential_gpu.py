@@ -146,35 +146,59 @@ def test_argument_validation(pkg, gpu):
     assert lib.q4_gather_columns(t.data_ptr(), t.data_ptr(), o.data_ptr(), 0, 12, None) == 0
 
 
-def test_quant_linear_repacks_once_and_keeps_memory_flat(pkg, oracle, gpu):
+def _act_order_mode(monkeypatch, mode):
+    import importlib
+    mod = importlib.import_module("text-generation-inference_amd.layers.gptq.quant_linear")
+    monkeypatch.setattr(mod, "ACT_ORDER_MODE", mode)
+
+
+@pytest.mark.parametrize("mode", ["table", "repack"])
+@pytest.mark.parametrize("cls", ["triton", "exllama"])
+def test_act_order_modules_leave_the_checkpoint_tensors_alone(pkg, oracle, gpu, monkeypatch, mode, cls):
+    """Both act-order routes of the modules: the default reads the checkpoint layout through
+    g_idx; Q4_ACT_ORDER=repack keeps a private copy with the rows in group order.  Either way
+    the tensors the loader handed in (and with them the state_dict) are never written."""
+    _act_order_mode(monkeypatch, mode)
     K, N, gs = 1024, 256, 128
     qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=5, sym=False, act_order=True)
-    import importlib
-    if importlib.import_module("text-generation-inference_amd.layers.gptq.quant_linear").ACT_ORDER_MODE == "table":
-        pytest.skip("Q4_ACT_ORDER=table keeps the checkpoint order")
-    layer = pkg.QuantLinear(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), None, 4, gs)
+    tq, tz, ts, tg = to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu)
+    if cls == "triton":
+        layer = pkg.QuantLinear(tq, tz, ts, tg, None, 4, gs)
+        pk = layer.packed()
+    else:
+        weight = pkg.GPTQWeight(qweight=tq, qzeros=tz, scales=ts, g_idx=tg, bits=4, groupsize=gs,
+                                use_awq_kernel=False, use_exllama=True)
+        layer = pkg.get_linear(weight, None)
+        pk = layer._packed
+    assert (pk.perm is not None) == (mode == "repack") and (pk.g_idx is not None) == (mode == "table")
     xh = oracle.make_x(4, K, seed=9)
     x = to_dev(xh, gpu)
     y1 = layer(x)
-    assert layer.q_perm is not None and layer.packed().g_idx is None
-    first = layer.qweight.data_ptr()
     y2 = layer(x)
-    assert layer.qweight.data_ptr() == first and torch.equal(y1, y2)
+    assert torch.equal(y1, y2)
     w = oracle.dequant_gptq(qw, qz, sc, gi, gs, "f16")
     y32, _ = oracle.linear_forward(xh, w, None, "f16")
     assert max_rel_err(y1.float().cpu().numpy(), y32) <= TOL
     assert np.array_equal(layer.dequantize().cpu().numpy().view(np.uint16), w.view(np.uint16))
-    # a copy of the module (new storage) keeps working: the permutation travels as a buffer
-    import copy
-    twin = copy.deepcopy(layer)
-    assert torch.equal(twin(x), y1)
+    # the loader's tensors are what they were
+    assert np.array_equal(tq.cpu().numpy().view(np.uint32), qw.view(np.uint32)) and np.array_equal(tg.cpu().numpy(), gi)
+    if cls == "triton":
+        assert layer.qweight.data_ptr() == tq.data_ptr() and layer.g_idx.data_ptr() == tg.data_ptr()
+        sd = layer.state_dict()
+        assert np.array_equal(sd["qweight"].cpu().numpy().view(np.uint32), qw.view(np.uint32)) and np.array_equal(sd["g_idx"].cpu().numpy(), gi)
+        # a copy of the module (new storage) rebuilds its kernel view and keeps working
+        import copy
+        twin = copy.deepcopy(layer)
+        assert torch.equal(twin(x), y1)
+    else:
+        assert layer.q_tensors.qweight.data_ptr() == tq.data_ptr()
 
 
 @pytest.mark.parametrize("M", [1, 16, 200])
-def test_wqlinear_converts_to_the_gptq_layout_bit_exactly(pkg, oracle, gpu, M, monkeypatch):
-    """The AWQ module serves its checkpoint through the GPTQ layout by default: same dense
-    matrix bit for bit (zero point 0 included: stored 15, read back as 0), same outputs as the
-    native AWQ kernels to rounding, AWQ-layout tensors dropped."""
+def test_wqlinear_both_routes_agree_and_keep_the_checkpoint_layout(pkg, oracle, gpu, M, monkeypatch):
+    """The AWQ module reads its checkpoint layout directly by default; Q4_AWQ=convert serves a
+    private GPTQ-layout copy: same dense matrix bit for bit (zero point 0 included: stored 15,
+    read back as 0), same outputs to rounding, and `qweight` keeps its [K, N/8] shape."""
     K, N, gs = 1024, 512, 128
     aq, az, sc = oracle.make_awq(K, N, gs, seed=M)
     az = az.copy()
@@ -187,14 +211,17 @@ def test_wqlinear_converts_to_the_gptq_layout_bit_exactly(pkg, oracle, gpu, M, m
     xh = oracle.make_x(M, K, seed=M + 2)
     x = to_dev(xh, gpu)
     y = conv(x)
-    assert conv.gptq_layout and tuple(conv.qweight.shape) == (K // 8, N) and conv.packed().layout == 0
+    assert tuple(conv.qweight.shape) == (K, N // 8) and conv.packed().layout == 0
+    assert np.array_equal(conv.qweight.cpu().numpy().view(np.uint32), aq.view(np.uint32))
     assert np.array_equal(conv.dequantize().cpu().numpy().view(np.uint16), want.view(np.uint16))
     y32, _ = oracle.linear_forward(xh, want, None, "f16")
     assert max_rel_err(y.float().cpu().numpy(), y32) <= TOL
     monkeypatch.setattr(mod, "AWQ_MODE", "native")
     native = pkg.WQLinear(4, gs, to_dev(aq, gpu), to_dev(az, gpu), to_dev(sc, gpu), None)
     yn = native(x)
-    assert not native.gptq_layout and native.packed().layout == 1
+    assert native.packed().layout == 1 and native.packed().qweight.data_ptr() == native.qweight.data_ptr()
+    assert np.array_equal(native.dequantize().cpu().numpy().view(np.uint16), want.view(np.uint16))
+    assert max_rel_err(yn.float().cpu().numpy(), y32) <= TOL
     assert max_rel_err(y.float().cpu().numpy(), yn.float().cpu().numpy()) <= TOL
 
 
@@ -245,13 +272,11 @@ def test_gated_mlp_first_half_on_rows_in_group_order(pkg, oracle, gpu, K, M):
 
 
 @pytest.mark.parametrize("gate_up_act_order", [False, True])
-def test_down_permutation_folded_into_gate_up_columns(pkg, oracle, gpu, gate_up_act_order):
+def test_down_permutation_folded_into_gate_up_columns(pkg, oracle, gpu, gate_up_act_order, monkeypatch):
     """The gated MLP of an act-order model: applying the down projection's permutation to the
     gate and up output columns at load time leaves every output bit for bit as it was with the
     run-time gather, and the down projection becomes a plain contiguous-group layer."""
-    import importlib
-    if importlib.import_module("text-generation-inference_amd.layers.gptq.quant_linear").ACT_ORDER_MODE == "table":
-        pytest.skip("Q4_ACT_ORDER=table keeps the checkpoint order")
+    _act_order_mode(monkeypatch, "repack")
     H, I, gs = 1024, 2048, 128
     gq = oracle.make_gptq(H, 2 * I, gs, seed=1, sym=False, act_order=gate_up_act_order)
     dq = oracle.make_gptq(I, H, gs, seed=2, sym=False, act_order=True)

@@ -130,34 +130,72 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   return Q4_PATH_GENERIC;
 }
 
+// Bytes of split-K partial sums the decode kernels would write for this weight at M rows:
+// the launcher's own decomposition, for the plain call and (where it exists) the gated-MLP one.
+static size_t decode_partial_bytes(const q4_weight* w, int M) {
+  if (!gemv_supported(w, M, Q4_DTYPE_F16) && !gemv_supported(w, M, Q4_DTYPE_BF16)) return 0;
+  int splits = gemv_pick_config(w, M).splits;
+  if (w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && w->N % 128 == 0) {
+    const int s = gemv_pick_config(w, M, true).splits;
+    if (s > splits) splits = s;
+  }
+  return splits > 1 ? (size_t)splits * M * w->N * sizeof(float) : 0;
+}
+
+size_t q4_workspace_bytes_for(const q4_weight* w, int M) {
+  if (validate_weight(w, "q4_workspace_bytes_for") != Q4_OK || M < 1 || w->K == 0 || w->N == 0)
+    return Q4_WORKSPACE_COUNTER_BYTES;
+  const size_t decode = decode_partial_bytes(w, M);
+  const size_t prefill = gemm_workspace_bytes(M, w->K, w->N);
+  return (size_t)Q4_WORKSPACE_COUNTER_BYTES + (decode > prefill ? decode : prefill);
+}
+
+int q4_linear_plan(const q4_weight* w, int M, int dtype, int* path, size_t* workspace_bytes) {
+  int rc = validate_weight(w, "q4_linear_plan");
+  if (rc == Q4_OK) rc = validate_dtype(dtype, "q4_linear_plan");
+  if (rc != Q4_OK) return rc;
+  if (M < 0 || path == nullptr || workspace_bytes == nullptr) {
+    set_error("q4_linear_plan: negative M=%d or null output pointer", M);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  *path = (M == 0 || w->K == 0 || w->N == 0) ? Q4_PATH_GENERIC : q4_select_path(w, M, dtype);
+  *workspace_bytes = q4_workspace_bytes_for(w, M);
+  return Q4_OK;
+}
+
 size_t q4_workspace_bytes(int M, int K, int N) {
   if (M < 1 || K < 1 || N < 1) return Q4_WORKSPACE_COUNTER_BYTES;
-  // Upper bound over the three decode kernels (their column tiles and split choices differ).
-  int splits = 1;
+  // Upper bound over the three decode kernels (their column tiles and split choices differ)
+  // for every weight of this shape: the act-order kernel's choice also depends on the number
+  // of groups (its parameter table shares LDS with the activation slab), so it is bounded over
+  // the group sizes 32 .. 1024 and "one group".
+  size_t decode = 0;
   if (K % 128 == 0 && N % 64 == 0) {
     static const int32_t fake_idx = 0;
     q4_weight w = {};
     w.K = K;
     w.N = N;
-    w.groupsize = 128;
-    w.num_groups = K / 128;
     const int m_lo = M <= 16 ? 1 : M, m_hi = M;
     for (int variant = 0; variant < 3; ++variant) {
       w.layout = variant == 1 ? Q4_LAYOUT_AWQ : Q4_LAYOUT_GPTQ;
       w.g_idx = variant == 2 ? &fake_idx : nullptr;  // only tested against NULL
       if (variant == 1 && N % 256 != 0) continue;
-      for (int m = m_lo; m <= m_hi; ++m) {
-        int s = gemv_pick_config(&w, m).splits;
-        if (s > splits) splits = s;
-        if (variant == 0 && N % 128 == 0) {  // the gated-MLP variant tiles N differently
-          s = gemv_pick_config(&w, m, true).splits;
-          if (s > splits) splits = s;
+      static const int kGroupSizes[] = {128, 32, 64, 256, 512, 1024, 1 << 30};
+      for (int gs : kGroupSizes) {
+        // the AWQ kernel does not look at the group count; contiguous GPTQ groups shorter than a
+        // chunk run on a different kernel, with its own decomposition
+        if (gs != 128 && (variant == 1 || (variant == 0 && gs != 32))) continue;
+        if (gs < K && K % gs != 0) continue;
+        w.groupsize = gs < K ? gs : K;
+        w.num_groups = K / w.groupsize;
+        for (int m = m_lo; m <= m_hi; ++m) {
+          const size_t b = decode_partial_bytes(&w, m) / m * M;
+          if (b > decode) decode = b;
         }
       }
     }
   }
   // decode: split-K partial sums; prefill: split-K partial tiles of under-filled GEMM grids
-  const size_t decode = (size_t)splits * M * N * sizeof(float);
   const size_t prefill = gemm_workspace_bytes(M, K, N);
   return (size_t)Q4_WORKSPACE_COUNTER_BYTES + (decode > prefill ? decode : prefill);
 }
@@ -426,7 +464,10 @@ int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, 
     return Q4_ERR_INVALID_ARGUMENT;
   }
   GemvConfig cfg{wcol, wk, splits, words};
-  if (words == 4 && gemv_rows32_kernel(w, M)) cfg.rows_per_block = 32;  // one workgroup for all rows
+  if (words == 0) {  // the lean contiguous-group kernel
+    cfg.words = 4;
+    cfg.lean = 1;
+  } else if (words == 4 && gemv_rows32_kernel(w, M)) cfg.rows_per_block = 32;  // one workgroup for all rows
   return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, &cfg, (hipStream_t)stream);
 }
 

@@ -191,7 +191,9 @@ struct GemvConfig {
   int splits;  // workgroups across K (cross-workgroup reduction through the workspace)
   int words;   // GPTQ contiguous-group kernel: packed words per lane (4, 2, 1 -> 64/32/16-column tiles)
   int rows_per_block = 16;  // 32: GPTQ contiguous-group kernel with two MFMA row blocks (17..32 rows)
+  int lean = 0;  // 1: the instruction-lean contiguous-group kernel (groups of whole 128-row chunks, up to 16 waves)
 };
+bool gemv_lean_supported(const q4_weight* w, int dtype);
 bool gemv_supported(const q4_weight* w, int M, int dtype);
 bool gemv_rows32_supported(const q4_weight* w, int M);
 bool gemv_rows32_kernel(const q4_weight* w, int M);

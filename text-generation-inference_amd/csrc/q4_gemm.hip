@@ -110,8 +110,10 @@ void launch_gemm_reduce(const float* partials, const void* bias, void* y, int M,
 // fp32 partial tiles of the split-K variants: splits x M x N floats (upper bound over the
 // GPTQ kernel and the AWQ / act-order kernel, whose tiles differ).
 size_t gemm_workspace_bytes(int M, int K, int N) {
-  if (M <= 16 || K % q4::kBK != 0 || N % 128 != 0) return 0;
-  int splits = gemm_plan(M, K, N).splits;
+  if (K % q4::kBK != 0 || N % 128 != 0) return 0;
+  // the GPTQ kernel runs from 17 rows on; the AWQ / act-order kernel may be forced at any M and
+  // is dispatched from 9 rows on for small AWQ layers
+  int splits = M > 16 ? gemm_plan(M, K, N).splits : 1;
   for (const bool one_per_cu : {false, true}) {
     const int other = gemm_awq_splits(M, K, N, one_per_cu);
     if (other > splits) splits = other;

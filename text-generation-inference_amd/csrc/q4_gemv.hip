@@ -10,6 +10,15 @@ using q4::Problem;
 // fused gated-MLP instantiations live in their own translation unit (q4_gemv_gate_up.hip)
 void launch_gemv_gate_up(const GemvParams& gp, int dtype, int rmax, bool static128, dim3 grid, dim3 block,
                          size_t smem, hipStream_t stream, bool grouped);
+// instruction-lean contiguous-group kernel (q4_gemv_lean.hip)
+void launch_gemv_lean(const GemvParams& gp, int dtype, int mp, dim3 grid, dim3 block, size_t smem, hipStream_t stream);
+
+// GPTQ layout, contiguous groups of whole 128-row chunks: what the lean kernel takes
+bool gemv_lean_supported(const q4_weight* w, int dtype) {
+  (void)dtype;
+  return w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && w->groupsize >= 128 && w->groupsize % 128 == 0 &&
+         w->K % 128 == 0 && w->N % 64 == 0;
+}
 
 static bool groupsize_ok_contiguous(int gs) {
   return gs == 32 || gs == 64 || (gs >= 128 && gs % 128 == 0);
@@ -69,9 +78,14 @@ bool gemv_rows32_supported(const q4_weight* w, int M) {
   return (long)M * (kr * 2 + 16) <= 150000;
 }
 
-GemvConfig gemv_pick_config(const q4_weight* w, int M) { return gemv_pick_config(w, M, false); }
+static GemvConfig pick_config(const q4_weight* w, int M, bool gate_up, bool allow_lean);
 
-GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
+// the plain call of q4_linear: any kernel of the family
+GemvConfig gemv_pick_config(const q4_weight* w, int M) { return pick_config(w, M, false, true); }
+// the kernels with the gated-MLP epilogue, two row blocks or an expert dimension (no lean variant)
+GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) { return pick_config(w, M, gate_up, false); }
+
+static GemvConfig pick_config(const q4_weight* w, int M, bool gate_up, bool allow_lean) {
   // Measured on MI355X (Llama-3-8B shapes, M=1): narrow column tiles with 4 waves along K
   // per workgroup and about two workgroups per CU (512 in flight) is the best point; wider
   // workgroups start too slowly and more splits lengthen the reduction tail.  The
@@ -79,13 +93,50 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) {
   GemvConfig c;
   c.words = 4;
   if (!gate_up && gemv_rows32_supported(w, M)) {
-    c = gemv_pick_config(w, 16, false);
+    c = pick_config(w, 16, false, false);
     c.rows_per_block = 32;
     return c;
   }
   const int rows = M < c.rows_per_block ? M : c.rows_per_block;
   const int mchunks = (M + c.rows_per_block - 1) / c.rows_per_block;
   const int chunks = w->K / 128;
+  // Large layers (from 32 M weights on), plain epilogue, up to 16 rows: the instruction-lean
+  // kernel.  Measured against the kernel below on MI355X (us, same box): 4096 x 28672 14.5 / 15.6
+  // at M = 1, 15.3 / 17.1 at M = 4, 18.2 / 20.1 at M = 16; 14336 x 4096 9.8 / 10.0, 12.9 / 13.5,
+  // 14.8 / 15.9.  On small layers (4096 x 4096, 4096 x 6144), which are bound by launch, first
+  // access and the split-K combine, it measured 0.5 us slower and is not taken.
+  if (allow_lean && !gate_up && M <= 16 && gemv_lean_supported(w, Q4_DTYPE_F16) && (long)w->K * w->N >= (1L << 25) && chunks >= 8) {
+    c.lean = 1;
+    const int n64 = w->N / 64;
+    if (n64 >= 384 && w->N % 128 == 0) {
+      // the column tiles alone fill the chip: two per workgroup, K whole
+      c.wcol = 2;
+      c.wk = (M >= 4 && chunks % 8 == 0) ? 8 : 4;
+      c.splits = 1;
+      // many rows: one slab per workgroup must fit LDS
+      while ((long)rows * ((long)w->K / c.splits * 2 + 16) > 150000 && c.splits * c.wk * 2 <= chunks) c.splits *= 2;
+      return c;
+    }
+    c.wcol = 1;
+    c.wk = 8;
+    // about one workgroup per CU; every wave keeps its own activations: rows x K / splits x 2 B in all
+    int best = 1;
+    double best_cost = -1.0;
+    for (int dv = 1; dv * c.wk <= chunks; ++dv) {
+      const long lds = (long)rows * c.wk * ((long)((chunks + dv * c.wk - 1) / (dv * c.wk)) * 256 + 16);
+      if (lds > 150000) continue;
+      const double wgs = (double)n64 * dv;
+      double cost = wgs > 256.0 ? wgs / 256.0 : 256.0 / wgs;
+      if (chunks % (dv * c.wk) != 0) cost *= 1.1;
+      if (best_cost < 0.0 || cost < best_cost) {
+        best_cost = cost;
+        best = dv;
+      }
+    }
+    c.splits = best;
+    if (best_cost >= 0.0) return c;
+    c.lean = 0;  // no split fits LDS: the kernel below, with its workgroup slab
+  }
   c.wcol = 1;
   c.wk = chunks >= 4 ? 4 : (chunks >= 2 ? 2 : 1);
   // wide layers with many rows: two column tiles per workgroup halve the slab staging
@@ -310,7 +361,7 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   }
   const bool awq = w->layout == Q4_LAYOUT_AWQ;
   const bool act = !awq && w->g_idx != nullptr;
-  GemvConfig cfg = cfg_in ? *cfg_in : gemv_pick_config(w, M, gate_up_act != 0);
+  GemvConfig cfg = cfg_in ? *cfg_in : (gate_up_act != 0 ? gemv_pick_config(w, M, true) : gemv_pick_config(w, M));
   const bool contiguous = !awq && !act;
   if (!contiguous || w->groupsize < 128) cfg.words = 4;  // only the contiguous-group kernel has narrow tiles
   if (gate_up_act != 0) cfg.words = 8;                    // four gate + four up words per lane
@@ -319,7 +370,12 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
     return Q4_ERR_INVALID_ARGUMENT;
   }
   const int wave_cols = awq ? 256 : 16 * cfg.words;
-  if (cfg.wcol < 1 || cfg.wk < 1 || cfg.splits < 1 || cfg.wcol * cfg.wk > 8 ||
+  const bool lean = cfg.lean != 0;
+  if (lean && !(gate_up_act == 0 && cfg.words == 4 && cfg.rows_per_block == 16 && gemv_lean_supported(w, dtype))) {
+    set_error("q4_linear(gemv): the lean kernel takes GPTQ weights with contiguous groups of a multiple of 128 rows");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (cfg.wcol < 1 || cfg.wk < 1 || cfg.splits < 1 || cfg.wcol * cfg.wk > (lean ? 16 : 8) ||
       w->N % (wave_cols * cfg.wcol) != 0 || w->K % 128 != 0 || (long)cfg.splits * cfg.wk > w->K / 128) {
     set_error("q4_linear(gemv): bad config wcol=%d wk=%d splits=%d for K=%d N=%d", cfg.wcol, cfg.wk,
               cfg.splits, w->K, w->N);
@@ -334,17 +390,15 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   const int rows = M < rpb ? M : rpb;
   const int mchunks = (M + rpb - 1) / rpb;
   // largest K range of a workgroup: K goes out in 128-row chunks over splits x wk wave slots
-  const long kchunks = w->K / 128, kslots = (long)cfg.splits * cfg.wk;
-  int KR = 0;
-  for (int sp = 0; sp < cfg.splits; ++sp) {
-    const int r = (int)(((long)(sp + 1) * cfg.wk * kchunks / kslots - (long)sp * cfg.wk * kchunks / kslots) * 128);
-    if (r > KR) KR = r;
-  }
-  const int slab_stride = KR * 2 + 16;
+  GemvParams gp;
+  const int KR = q4::set_k_deal(gp, w->K / 128, cfg.splits, cfg.wk);
+  // the lean kernel gives every wave its own piece of LDS for the K range it walks
+  const bool wave_slab = lean && (cfg.wcol == 1 || rows <= 2);
+  const int slab_stride = (wave_slab ? q4::max_wave_rows(gp) : KR) * 2 + 16;
   const int rmax = rpb == 32 ? 8 : (M <= 1 ? 1 : (M <= 2 ? 2 : 4));
   const int nt = awq ? 16 : cfg.words;
-  const size_t slab_bytes = ((size_t)rows * slab_stride + 15) & ~(size_t)15;
-  size_t smem = slab_bytes;
+  const size_t slab_bytes = ((size_t)rows * slab_stride * (wave_slab ? cfg.wcol * cfg.wk : 1) + 15) & ~(size_t)15;
+  size_t smem = slab_bytes + (lean ? 512 : 0);  // lean: a block of zeros behind the slab
   if (act) smem += (((size_t)KR * 2 + 15) & ~(size_t)15) + (size_t)w->num_groups * 64 * cfg.wcol * 4;
   const size_t red = (size_t)(cfg.wk - 1) * cfg.wcol * nt * rmax * 64 * sizeof(float);
   if (red > smem) smem = red;
@@ -364,7 +418,6 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
     tickets = (uint32_t*)workspace;
     partials = (float*)((char*)workspace + Q4_WORKSPACE_COUNTER_BYTES);
   }
-  GemvParams gp;
   gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, w->g_idx, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
   gp.p.gate_up_act = gate_up_act;
@@ -401,9 +454,15 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.partial_rows = M;
   gp.rows_per_block = rpb;
   gp.moe = q4::MoeView{};
+  gp.ntiles = ntiles;
+  gp.rows_per_block_alloc = rows;
+  gp.wave_slab = wave_slab ? 1 : 0;
   dim3 grid((unsigned)(ntiles * cfg.splits), (unsigned)mchunks);
   dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
-  if (gate_up_act != 0) {
+  if (lean) {
+    launch_gemv_lean(gp, dtype, rows <= 1 ? 1 : (rows <= 2 ? 2 : (rows <= 4 ? 4 : (rows <= 8 ? 8 : 16))), grid, block, smem,
+                     stream);
+  } else if (gate_up_act != 0) {
     launch_gemv_gate_up(gp, dtype, rmax, w->groupsize == 128, grid, block, smem, stream, false);
   } else if (rmax == 8) {
     if (dtype == Q4_DTYPE_F16) launch_rows32<Q4_DTYPE_F16>(w, gp, grid, block, smem, stream);

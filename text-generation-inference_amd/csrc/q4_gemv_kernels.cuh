@@ -56,7 +56,30 @@ struct GemvParams {
   int partial_rows;  // rows of one split's slice of `partials` (M; grouped launches: all pairs)
   int rows_per_block;  // activation rows per workgroup: 16, or 32 (two MFMA row blocks per unpacked word)
   MoeView moe;       // grouped launches only (MOE kernels): blockIdx.z is the expert
+  // How the K / 128 chunks are dealt out (set_k_deal): workgroup `split` takes kd_Q chunks, the
+  // first kd_R workgroups one more; inside a workgroup of kd_Q (+1) chunks wave wkk takes
+  // kd_q0 (kd_q1) chunks, the first kd_r0 (kd_r1) waves one more.  No division on the device.
+  int ntiles, kd_Q, kd_R, kd_q0, kd_r0, kd_q1, kd_r1;
+  int rows_per_block_alloc;  // lean kernel: activation rows every wave's piece of LDS has room for
+  int wave_slab;             // lean kernel: 1 = every wave stages its own K range, 0 = one slab per workgroup
 };
+
+// Fills the K partition of gp for `chunks` chunks over `splits` workgroups of `wk` waves
+// (splits * wk <= chunks) and returns the largest K range of a workgroup in rows.
+inline int set_k_deal(GemvParams& gp, int chunks, int splits, int wk) {
+  gp.kd_Q = chunks / splits;
+  gp.kd_R = chunks % splits;
+  gp.kd_q0 = gp.kd_Q / wk;
+  gp.kd_r0 = gp.kd_Q % wk;
+  gp.kd_q1 = (gp.kd_Q + 1) / wk;
+  gp.kd_r1 = (gp.kd_Q + 1) % wk;
+  return (gp.kd_Q + (gp.kd_R > 0 ? 1 : 0)) * 128;
+}
+// Largest K range of a wave under the same partition, in rows.
+inline int max_wave_rows(const GemvParams& gp) {
+  const int a = gp.kd_q0 + (gp.kd_r0 > 0 ? 1 : 0), b = gp.kd_R > 0 ? gp.kd_q1 + (gp.kd_r1 > 0 ? 1 : 0) : 0;
+  return (a > b ? a : b) * 128;
+}
 
 // Constants of the nibble splice, hidden from constant folding (empty asm, no instruction
 // is emitted): as literals the compiler must split (w & mask) | magic into v_and + v_or
@@ -133,20 +156,18 @@ __device__ __forceinline__ Decomp make_decomp(const GemvParams& gp, int wave_col
   d.kq = d.lane >> 4;
   d.nthreads = blockDim.x;
   d.tile_cols = wave_cols * gp.wcol;
-  d.ntiles = gp.p.N / d.tile_cols;
-  d.tile = blockIdx.x % d.ntiles;
-  d.split = blockIdx.x / d.ntiles;
-  // K is dealt out in chunks of 128 rows over splits x wk wave slots, as evenly as the chunk
-  // count allows (ranges differ by at most one chunk when it is not a multiple of the slots)
-  const long chunks = gp.p.K / kChunkRows;
-  const long slots = (long)gp.splits * gp.wk;
-  const long slot0 = (long)d.split * gp.wk;
-  const int g0 = (int)(slot0 * chunks / slots), g1 = (int)((slot0 + gp.wk) * chunks / slots);
-  const int c0 = (int)((slot0 + d.wkk) * chunks / slots), c1 = (int)((slot0 + d.wkk + 1) * chunks / slots);
+  d.ntiles = gp.ntiles;
+  d.tile = blockIdx.x % (unsigned)d.ntiles;
+  d.split = blockIdx.x / (unsigned)d.ntiles;
+  // K is dealt out in chunks of 128 rows, first over the `splits` workgroups, then over the wk
+  // waves of each, as evenly as the counts allow (ranges differ by at most one chunk)
+  const bool big = d.split < gp.kd_R;
+  const int g0 = d.split * gp.kd_Q + min(d.split, gp.kd_R);
+  const int wq = big ? gp.kd_q1 : gp.kd_q0, wr = big ? gp.kd_r1 : gp.kd_r0;
   d.kwg0 = g0 * kChunkRows;
-  d.KR = (g1 - g0) * kChunkRows;
-  d.kw0 = c0 * kChunkRows;
-  d.KW = (c1 - c0) * kChunkRows;
+  d.KR = (gp.kd_Q + (big ? 1 : 0)) * kChunkRows;
+  d.kw0 = (g0 + d.wkk * wq + min(d.wkk, wr)) * kChunkRows;
+  d.KW = (wq + (d.wkk < wr ? 1 : 0)) * kChunkRows;
   d.kwo = d.kw0 - d.kwg0;
   d.mb = blockIdx.y * gp.rows_per_block;
   d.mloc = min(gp.rows_per_block, gp.p.M - d.mb);

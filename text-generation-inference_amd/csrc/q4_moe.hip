@@ -444,6 +444,8 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
     gp.rows_per_block = kRowsPerBlock;
     gp.slab_stride = pl.kr_max * 2 + 16;
     gp.kr_max = pl.kr_max;
+    gp.ntiles = pl.ntiles;
+    (void)q4::set_k_deal(gp, e0->K / 128, cfg.splits, cfg.wk);
     gp.slab_bytes = (int)pl.slab_bytes;
     gp.partial_rows = pairs;
     gp.moe = mv;

@@ -2,13 +2,16 @@
 
 Mirrors server/text_generation_server/layers/awq/quantize/cuda.py:19-49.  The reference
 calls the third-party `awq_inference_engine.gemm_forward_cuda` and refuses to run on ROCm
-(gptq/__init__.py:39-43); here the HIP library reads the interleaved-nibble layout
-directly ("native"), or -- the default -- converts the tensors once to the GPTQ layout
-(fast_awq_to_gptq, the reference's own route for AWQ checkpoints on ROCm,
-gptq/__init__.py:186-204) and serves them with the GPTQ kernels, which are faster (decode
-step of the Llama-3-8B projections 36 against 51 us at one row, 57 against 105 us at 16;
-prefill 1.3x).  The two routes compute the same weights bit for bit: the GPTQ reader's +1
-undoes the -1 of the conversion for every zero point, 0 included (15 + 1 wraps to 0).
+(gptq/__init__.py:39-43); here the HIP kernels read the interleaved-nibble layout as it
+sits in the checkpoint: nothing is repacked and `qweight` / `qzeros` / `scales` stay the
+tensors the loader handed in.
+
+Q4_AWQ=convert opts into the reference's own route for AWQ checkpoints on ROCm
+(fast_awq_to_gptq, gptq/__init__.py:186-204): one conversion to the GPTQ layout at load time,
+kept in private tensors next to the checkpoint ones (twice the weight memory), served by the
+GPTQ kernels, which are faster at decode.  The two routes compute the same weights bit for
+bit: the GPTQ reader's +1 undoes the -1 of the conversion for every zero point, 0 included
+(15 + 1 wraps to 0).
 """
 
 from __future__ import annotations
@@ -23,8 +26,8 @@ from ... import ops
 from ..._lib import LAYOUT_AWQ, LAYOUT_GPTQ
 from .conversion_utils import fast_awq_to_gptq
 
-# "convert": GPTQ layout + GPTQ kernels (the AWQ-layout tensors are dropped); "native": AWQ kernels
-AWQ_MODE = os.environ.get("Q4_AWQ", "convert")
+# "native": the AWQ-layout kernels on the checkpoint tensors; "convert": GPTQ-layout copy + GPTQ kernels
+AWQ_MODE = os.environ.get("Q4_AWQ", "native")
 
 
 class WQLinear(nn.Module):
@@ -48,18 +51,29 @@ class WQLinear(nn.Module):
         self.scales = scales
         self.bias = bias
         self._packed: Optional[ops.PackedWeight] = None
-        self.gptq_layout = False  # set once qweight / qzeros have been converted
+        self._packed_of = None  # data pointer of the qweight the kernel view was built from
+        if qweight.is_cuda:
+            self.post_init()
+
+    def post_init(self) -> ops.PackedWeight:
+        """Everything that is not the matmul happens here, once, when the tensors are on the GPU:
+        validation, the optional layout conversion, the launch plans of the decode sizes and the
+        workspace.  The forward is then one library call."""
+        if AWQ_MODE == "convert" and self.qweight.is_cuda:
+            gq, gz = fast_awq_to_gptq(self.qweight, self.qzeros)
+            pk = ops.make_packed(gq.contiguous(), gz.contiguous(), self.scales, None, self.group_size, LAYOUT_GPTQ)
+        else:
+            pk = ops.make_packed(self.qweight, self.qzeros, self.scales, None, self.group_size, LAYOUT_AWQ)
+        pk.prepare()
+        self._packed = pk
+        self._packed_of = self.qweight.data_ptr()
+        return pk
 
     def packed(self) -> ops.PackedWeight:
+        """Kernel view of the tensors, rebuilt if they were replaced (e.g. moved to a device)."""
         pk = self._packed
-        if pk is None or pk.qweight.data_ptr() != self.qweight.data_ptr():
-            if not self.gptq_layout and AWQ_MODE != "native" and self.qweight.is_cuda:
-                gq, gz = fast_awq_to_gptq(self.qweight, self.qzeros)
-                self.qweight, self.qzeros = gq.contiguous(), gz.contiguous()
-                self.gptq_layout = True
-            layout = LAYOUT_GPTQ if self.gptq_layout else LAYOUT_AWQ
-            pk = ops.make_packed(self.qweight, self.qzeros, self.scales, None, self.group_size, layout)
-            self._packed = pk
+        if pk is None or self._packed_of != self.qweight.data_ptr():
+            pk = self.post_init()
         return pk
 
     @torch.no_grad()

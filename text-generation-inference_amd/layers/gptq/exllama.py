@@ -16,7 +16,8 @@ import torch.nn as nn
 
 from ... import ops
 from ..._lib import LAYOUT_GPTQ
-from .quant_linear import ACT_ORDER_MODE, is_trivial_g_idx
+from . import quant_linear
+from .quant_linear import is_trivial_g_idx
 
 DEVICE = None
 
@@ -54,32 +55,24 @@ class ExllamaQuantLinear(nn.Module):
         ):
             g_idx = None
         self.act_order = g_idx is not None
-        # a weight object that an earlier layer already put into group order carries its perm
-        q_perm = getattr(weight, "q_perm", None)
-        if q_perm is not None:
-            g_idx = None
         groupsize = weight.groupsize
         if g_idx is None and weight.scales.shape[0] == 1:
             groupsize = self.infeatures
-        self._packed = ops.make_packed(
-            weight.qweight, weight.qzeros, weight.scales, g_idx, groupsize, LAYOUT_GPTQ
-        )
-        self.q_perm = q_perm
-        if q_perm is not None:
-            self._packed.perm = q_perm
-        elif self.act_order and ACT_ORDER_MODE != "table" and weight.qweight.is_cuda:
-            # the reference shuffles q_weight in place when it builds its matrix
-            # (exllamav2.py:106-130 -> make_q_matrix -> QMatrix::make_sequential); here the
-            # reordered rows are a new tensor and the weight object is pointed at it
-            seq = ops.make_sequential(self._packed)
+        # The reference shuffles q_weight in place when it builds its matrix (exllamav2.py:106-130
+        # -> make_q_matrix -> QMatrix::make_sequential); here the checkpoint tensors are read as
+        # they are.  With Q4_ACT_ORDER=repack a second qweight with the rows in group order is
+        # kept privately and the weight object stays untouched.
+        pk = ops.make_packed(weight.qweight, weight.qzeros, weight.scales, g_idx, groupsize, LAYOUT_GPTQ)
+        if self.act_order and quant_linear.ACT_ORDER_MODE == "repack" and weight.qweight.is_cuda:
+            seq = ops.make_sequential(pk)
             if seq is not None:
-                weight.qweight = seq.qweight
-                weight.q_perm = seq.perm
-                self.q_perm = seq.perm
-                self._packed = seq
+                pk = seq
+        pk.prepare()
+        self._packed = pk
 
     def post_init(self, temp_dq=None):
-        """The reference builds its device matrix here (exllamav2.py:215-224); nothing to do."""
+        """The reference builds its device matrix here at Warmup (exllamav2.py:215-224); this
+        module has done its load-time work in the constructor."""
         return None
 
     @torch.no_grad()

@@ -21,10 +21,12 @@ from ... import ops
 from ..._lib import LAYOUT_GPTQ
 
 
-# Act-order layers: "repack" puts the rows of qweight into group order once (what the
-# reference's exllama matrices do) so that the contiguous-group kernels apply; "table" keeps
-# the checkpoint order and uses the kernels that look up every weight's group.
-ACT_ORDER_MODE = os.environ.get("Q4_ACT_ORDER", "repack")
+# Act-order layers: "table" (default) runs the kernels that read the checkpoint layout and look
+# every row's group up through g_idx; nothing is repacked.  "repack" opts into what the
+# reference's exllama matrices do at load time (QMatrix::make_sequential): a second qweight with
+# the rows in group order, kept privately next to the checkpoint tensor (twice the weight
+# memory), served by the contiguous-group kernels, which are faster at decode.
+ACT_ORDER_MODE = os.environ.get("Q4_ACT_ORDER", "table")
 
 
 def is_trivial_g_idx(g_idx: torch.Tensor, groupsize: int) -> bool:
@@ -61,10 +63,10 @@ class QuantLinear(nn.Module):
 
         self.outfeatures = qweight.shape[1]
         self.infeatures = qweight.shape[0] * 32 // self.bits
-        # set once the rows of qweight have been put into group order: row i is checkpoint row
-        # q_perm[i] and g_idx describes the stored (sequential) rows
-        self.register_buffer("q_perm", None)
         self._packed: Optional[ops.PackedWeight] = None
+        self._packed_of = None  # data pointer of the qweight the kernel view was built from
+        if qweight is not None and qweight.is_cuda:
+            self.post_init()
 
     @classmethod
     def new(cls, bits, groupsize, infeatures, outfeatures, bias):
@@ -94,7 +96,6 @@ class QuantLinear(nn.Module):
         """
         if g_idx is not None:
             self.g_idx = g_idx.clone()
-        self.q_perm = None  # the rows written below are in checkpoint order
         gi = self.g_idx.to(torch.int64).cpu()
         scales = scales.detach().cpu().t().contiguous()
         zeros = zeros.detach().cpu().t().contiguous()
@@ -117,27 +118,31 @@ class QuantLinear(nn.Module):
         self.qzeros = torch.from_numpy(qzeros.astype(np.int32))
         self._packed = None
 
+    def post_init(self) -> ops.PackedWeight:
+        """The load-time work of the layer (the reference's exllama modules do theirs in
+        post_init at Warmup, exllamav2.py:215-224): the act-order test on g_idx (one
+        device->host sync), validation, the optional row reorder, the launch plans of the
+        decode sizes and the workspace.  The registered buffers are never written: a
+        state_dict saved afterwards is still the checkpoint."""
+        g_idx = self.g_idx
+        if g_idx is not None and is_trivial_g_idx(g_idx, self.groupsize):
+            g_idx = None  # sequential groups: the kernels index by k // groupsize
+        pk = ops.make_packed(self.qweight, self.qzeros, self.scales, g_idx, self.groupsize, LAYOUT_GPTQ)
+        if pk.g_idx is not None and ACT_ORDER_MODE == "repack" and self.qweight.is_cuda:
+            seq = ops.make_sequential(pk)
+            if seq is not None:
+                pk = seq
+        pk.prepare()
+        self._packed = pk
+        self._packed_of = self.qweight.data_ptr()
+        return pk
+
     def packed(self) -> ops.PackedWeight:
-        """Validated kernel view of the buffers, rebuilt if they moved (e.g. `.to(device)`)."""
+        """Kernel view of the buffers, rebuilt if they moved (e.g. `.to(device)`) or were
+        rewritten (`pack`)."""
         pk = self._packed
-        if pk is None or pk.qweight.data_ptr() != self.qweight.data_ptr():
-            g_idx = self.g_idx
-            if g_idx is not None and is_trivial_g_idx(g_idx, self.groupsize):
-                g_idx = None  # sequential groups: the kernels index by k // groupsize
-            pk = ops.make_packed(self.qweight, self.qzeros, self.scales, g_idx, self.groupsize, LAYOUT_GPTQ)
-            if self.q_perm is not None:
-                pk.perm = self.q_perm.to(torch.int32).contiguous()
-            elif pk.g_idx is not None and ACT_ORDER_MODE != "table" and self.qweight.is_cuda:
-                seq = ops.make_sequential(pk)
-                if seq is not None:
-                    # like the reference's exllama matrix, the module now holds the reordered
-                    # rows (the checkpoint-order tensor is dropped: memory stays flat)
-                    K = self.infeatures
-                    self.qweight = seq.qweight
-                    self.g_idx = (torch.arange(K, device=seq.qweight.device, dtype=torch.int64) // pk.groupsize).to(torch.int32)
-                    self.q_perm = seq.perm
-                    pk = seq
-            self._packed = pk
+        if pk is None or self._packed_of != self.qweight.data_ptr():
+            pk = self.post_init()
         return pk
 
     @torch.no_grad()

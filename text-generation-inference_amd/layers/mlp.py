@@ -38,9 +38,11 @@ def fold_down_permutation(gate_up_layer, down_layer) -> bool:
     so the permutation can be applied once, at load time, to the output columns of the gate and
     the up half of the gate_up projection instead: the first half of the MLP then produces its
     result directly in the order the down projection's rows are in, and the down projection
-    becomes a plain contiguous-group layer.  Both layers must come from this package; returns
-    False (nothing changed) when the down projection has no permutation or the shapes do not
-    pair up.  Afterwards `down_layer.dequantize()` returns its matrix with the rows in group
+    becomes a plain contiguous-group layer.  Only the layers' private kernel views (and the
+    gate_up bias) change; the checkpoint tensors they were built from stay as they are.  Both
+    layers must come from this package; returns False (nothing changed) when the down projection
+    has no permutation (the default: rows stay in checkpoint order unless Q4_ACT_ORDER=repack) or
+    the shapes do not pair up.  Afterwards `down_layer.dequantize()` returns its matrix with the rows in group
     order, the one that multiplies the reordered activations."""
     gpk = gate_up_layer.packed() if callable(getattr(gate_up_layer, "packed", None)) else gate_up_layer._packed
     dpk = down_layer.packed() if callable(getattr(down_layer, "packed", None)) else down_layer._packed
@@ -53,18 +55,10 @@ def fold_down_permutation(gate_up_layer, down_layer) -> bool:
     bias = getattr(gate_up_layer, "bias", None)
     if bias is not None:
         gate_up_layer.bias = bias.index_select(0, cols.to(bias.device))
-    for name in ("qweight", "qzeros", "scales"):
-        if isinstance(getattr(gate_up_layer, name, None), torch.Tensor):
-            setattr(gate_up_layer, name, getattr(new, name))
-    tensors = getattr(gate_up_layer, "q_tensors", None)
-    if tensors is not None:
-        tensors.qweight, tensors.qzeros, tensors.scales = new.qweight, new.qzeros, new.scales
     gate_up_layer._packed = new
     plain = ops.PackedWeight(dpk.qweight, dpk.qzeros, dpk.scales, None, dpk.K, dpk.N, dpk.groupsize,
                              dpk.num_groups, dpk.layout)
-    if hasattr(down_layer, "q_perm"):
-        down_layer.q_perm = None
-    if getattr(down_layer, "q_tensors", None) is not None and hasattr(down_layer.q_tensors, "q_perm"):
-        down_layer.q_tensors.q_perm = None
+    new.prepare()
+    plain.prepare()
     down_layer._packed = plain
     return True

@@ -23,8 +23,16 @@ from ... import ops
 from ..._lib import LAYOUT_AWQ, LAYOUT_GPTQ
 from ..gptq import GPTQWeight
 from ..awq.conversion_utils import fast_awq_to_gptq
-from ..awq.quantize import AWQ_MODE
-from ..gptq.quant_linear import ACT_ORDER_MODE, is_trivial_g_idx
+import os
+
+from ..gptq.quant_linear import is_trivial_g_idx
+
+# The expert weights keep the load-time conversions as their default (the reference's MoE layer
+# repacks every expert into the Marlin layout when it is built, layers/moe/gptq_marlin.py:186-229):
+# AWQ-layout experts go to the GPTQ layout once, act-order experts get their rows put into
+# group order.  "native" / "table" keep the checkpoint layout and run the AWQ / lookup kernels.
+AWQ_MODE = os.environ.get("Q4_MOE_AWQ", "convert")
+ACT_ORDER_MODE = os.environ.get("Q4_MOE_ACT_ORDER", "repack")
 
 
 @dataclass

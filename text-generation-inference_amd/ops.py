@@ -7,7 +7,7 @@ kernels of libq4linear.so.  CPU tensors are rejected: there is no host fallback.
 from __future__ import annotations
 
 import ctypes
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Optional
 
 import torch
@@ -52,8 +52,55 @@ class PackedWeight:
     # Rows in group order (make_sequential): packed row i holds checkpoint row perm[i] and the
     # kernels take the activation columns in that order; None for checkpoint order.
     perm: Optional[torch.Tensor] = None
+    # (M, dtype code) -> (kernel path, workspace bytes): a pure function of the weight's geometry,
+    # asked of the library once and kept (one library call per forward afterwards)
+    _plans: dict = field(default_factory=dict, repr=False, compare=False)
+    _struct: Optional[Q4Weight] = field(default=None, repr=False, compare=False)
+
+    def __deepcopy__(self, memo):
+        import copy
+
+        # the cached ctypes struct holds device addresses: a copy gets its own, on first use
+        return PackedWeight(
+            copy.deepcopy(self.qweight, memo), copy.deepcopy(self.qzeros, memo), copy.deepcopy(self.scales, memo),
+            copy.deepcopy(self.g_idx, memo), self.K, self.N, self.groupsize, self.num_groups, self.layout,
+            copy.deepcopy(self.perm, memo), dict(self._plans), None)
 
     def struct(self) -> Q4Weight:
+        if self._struct is None:
+            self._struct = self._make_struct()
+        return self._struct
+
+    def plan(self, M: int, dtype_code: int) -> tuple:
+        """(Q4_PATH_* the library picks, workspace bytes the call needs) for M rows."""
+        key = (M, dtype_code)
+        got = self._plans.get(key)
+        if got is None:
+            lib = _lib.load()
+            path, need = ctypes.c_int(0), ctypes.c_size_t(0)
+            _lib.check(lib.q4_linear_plan(ctypes.byref(self.struct()), M, dtype_code, ctypes.byref(path), ctypes.byref(need)))
+            nbytes = int(need.value)
+            if self.perm is not None:
+                # weight in group order: x is gathered into the tail of the workspace (all but the
+                # shortest decode calls, which gather inside the kernel)
+                nbytes = max(nbytes, int(lib.q4_workspace_bytes_perm(M, self.K, self.N)))
+            got = (int(path.value), nbytes)
+            self._plans[key] = got
+        return got
+
+    def prepare(self, rows=tuple(range(1, 17)) + (32, 64)) -> None:
+        """Load-time step of a layer: fetch the launch plans of the decode row counts and
+        reserve the device's shared workspace for them, so that the first forward neither asks
+        the library for a plan nor allocates (it can be captured into a HIP graph)."""
+        if not self.qweight.is_cuda:
+            return
+        need = max(self.plan(M, DTYPE_F16)[1] for M in rows)
+        for M in rows:
+            self.plan(M, DTYPE_BF16)
+        with torch.cuda.device(self.qweight.device):
+            reserve_workspace(self.qweight.device, need, SHARED)
+
+    def _make_struct(self) -> Q4Weight:
         return Q4Weight(
             self.qweight.data_ptr(),
             self.qzeros.data_ptr(),
@@ -175,11 +222,18 @@ def _stream_handle(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+# stream key of a device's shared workspace (reserved at load time, used under graph capture)
+SHARED = -1
+
+
 def reserve_workspace(device: torch.device, nbytes: int, stream: Optional[int] = None) -> torch.Tensor:
     """Return this (device, stream)'s workspace, growing it to at least `nbytes`.
 
     The first bytes hold the split-K ticket counters: they must start at zero and the
     kernels leave them at zero, so a grown buffer is freshly zeroed and the old one dropped.
+    `stream=SHARED` names the device's shared workspace: the layers reserve it when they are
+    built, and calls made while a stream is capturing (where nothing may be allocated or
+    cleared) fall back to it.
     """
     if stream is None:
         stream = _stream_handle(device)
@@ -189,6 +243,27 @@ def reserve_workspace(device: torch.device, nbytes: int, stream: Optional[int] =
         ws = torch.zeros(int(nbytes), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+def _workspace_for_call(device: torch.device, need: int, stream: int) -> torch.Tensor:
+    """The workspace a kernel call on `stream` uses.  Outside graph capture: the stream's own,
+    grown on demand.  Under capture nothing is allocated: the stream's own if it is large
+    enough, else the device's shared workspace (calls that share it must be ordered, which the
+    nodes of one captured stream are)."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    ws = _workspaces.get(key)
+    if ws is not None and ws.numel() >= need:
+        return ws
+    if torch.cuda.is_current_stream_capturing():
+        shared = _workspaces.get((key[0], SHARED))
+        if shared is not None and (ws is None or shared.numel() > ws.numel()):
+            ws = shared
+        if ws is None:
+            raise RuntimeError(
+                "no workspace was reserved before the stream began capturing: build the layer on the GPU "
+                "(its post_init reserves one) or call ops.reserve_workspace(device, nbytes, ops.SHARED) first")
+        return ws  # a decode call that needs more reports it; a prefill call runs unsplit
+    return reserve_workspace(device, need, stream)
 
 
 def workspace_bytes(M: int, K: int, N: int) -> int:
@@ -252,20 +327,12 @@ def linear(
     lib = _lib.load()
     with torch.cuda.device(x.device):
         stream = _stream_handle(x.device)
-        st = w.struct()
         # decode: split-K partial sums, tickets, accumulation cells; prefill GEMM: split-K
         # partial tiles when the tile grid alone would leave CUs idle
-        chosen = path
-        if chosen == PATH_AUTO and gemv_config is None:
-            chosen = lib.q4_select_path(ctypes.byref(st), M, _DTYPES[x.dtype])
-        need = _lib.WORKSPACE_COUNTER_BYTES
-        if chosen in (_lib.PATH_GEMV, _lib.PATH_GEMM):
-            need = workspace_bytes(M, w.K, w.N)
-        if w.perm is not None:
-            # weight in group order: x is gathered into the tail of the workspace (all but the
-            # shortest decode calls, which gather inside the kernel)
-            need = int(lib.q4_workspace_bytes_perm(M, w.K, w.N))
-        ws = reserve_workspace(x.device, need, stream)
+        planned_path, need = w.plan(M, _DTYPES[x.dtype])
+        if path == PATH_AUTO and gemv_config is None:
+            path = planned_path
+        ws = _workspace_for_call(x.device, need, stream)
         st = w.struct()
         if gemv_config is not None:
             wcol, wk, splits = gemv_config[:3]
@@ -352,8 +419,7 @@ def linear_gate_up(
         lib = _lib.load()
         with torch.cuda.device(x.device):
             stream = _stream_handle(x.device)
-            need = workspace_bytes(M, w.K, w.N) if w.perm is None else int(lib.q4_workspace_bytes_perm(M, w.K, w.N))
-            ws = reserve_workspace(x.device, need, stream)
+            ws = _workspace_for_call(x.device, w.plan(M, _DTYPES[x.dtype])[1], stream)
             st = w.struct()
             rc = lib.q4_linear_gate_up_perm(
                 ctypes.byref(st), w.perm.data_ptr() if w.perm is not None else None, x.data_ptr(),
