@@ -210,6 +210,23 @@ size_t q4_workspace_bytes_for(const q4_weight* w, int M);
 int q4_linear_plan(const q4_weight* w, int M, int dtype, int* path, size_t* workspace_bytes);
 
 /*
+ * q4_linear for callers that cannot allocate device memory or hand over a workspace (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  The split-K scratch (tickets, accumulation cells, fp32
+ * partial sums) lives in a device array built into the library, Q4_NOALLOC_SCRATCH_BYTES per
+ * GPU, held until the process ends; the call allocates and frees nothing.  Decode problems
+ * whose partial sums do not fit return Q4_ERR_WORKSPACE (q4_linear_plan tells the size);
+ * prefill problems run unsplit where their partial tiles do not fit.  All calls on one GPU
+ * share the array: calls that overlap on one GPU (two streams) race; the kernels leave the
+ * counters at zero, so consecutive calls need no clearing.  q4_noalloc_init() looks the
+ * array's address up for the current device (the first q4_linear_noalloc on a device does
+ * it otherwise; call it before a stream capture begins).
+ */
+#define Q4_NOALLOC_SCRATCH_BYTES 16777216
+int q4_noalloc_init(void);
+int q4_linear_noalloc(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype, void* stream);
+
+/*
  * ---- Mixture of experts: the same linear layer, grouped over experts -----------------
  *
  * Replaces, for GPTQ and AWQ checkpoints, what the reference's sparse MoE layer

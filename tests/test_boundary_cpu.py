@@ -195,6 +195,16 @@ def test_linear_plan_matches_its_parts(pkg):
     assert lib.q4_linear_plan(None, 1, 0, ctypes.byref(path), ctypes.byref(need)) == L.ERR_INVALID_ARGUMENT
 
 
+def test_noalloc_entry_point_validation_without_gpu(pkg):
+    lib = pkg._lib.load()
+    L = pkg._lib
+    assert lib.q4_linear_noalloc(None, 0x10, None, 0x20, 1, 0, None) == L.ERR_INVALID_ARGUMENT
+    w = _weight(pkg, 4096, 4096, 128)
+    assert lib.q4_linear_noalloc(ctypes.byref(w), 0x10, None, 0x20, -1, 0, None) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_linear_noalloc(ctypes.byref(w), 0x10, None, 0x20, 1, 5, None) == L.ERR_INVALID_ARGUMENT
+    assert lib.q4_linear_noalloc(ctypes.byref(w), None, None, None, 0, 0, None) == 0  # no rows: nothing to do
+
+
 def test_path_selection_and_workspace(pkg):
     lib = pkg._lib.load()
     L = pkg._lib

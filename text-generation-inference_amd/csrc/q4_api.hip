@@ -4,6 +4,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "q4_common.cuh"
 
 namespace {
@@ -446,6 +448,69 @@ int q4_gather_columns(const void* x, const int32_t* perm, void* out, int M, int 
     return Q4_ERR_UNSUPPORTED;
   }
   return launch_gather_columns(x, perm, out, M, K, (hipStream_t)stream);
+}
+
+// ---- q4_linear without a caller-provided workspace -------------------------------------
+// The scratch memory of the split-K paths (tickets, accumulation cells, fp32 partial sums) lives
+// in a file-scope device array instead of a caller's buffer.  In host code the array's name
+// is only a stand-in for the symbol: its device address is looked up once per device.
+#define Q4_SCRATCH_BYTES Q4_NOALLOC_SCRATCH_BYTES
+static __device__ __align__(256) unsigned char scratch[Q4_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (looked up on first use), or nullptr with
+// the error set.
+void* scratch_of_current_device(const char* who) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("%s: cannot identify the current device (%s, device %d)", who,
+              err != hipSuccess ? hipGetErrorString(err) : "out of range", dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr) {
+      set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev, hipGetErrorString(err));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
+int q4_noalloc_init(void) { return scratch_of_current_device("q4_noalloc_init") != nullptr ? Q4_OK : Q4_ERR_LAUNCH; }
+
+int q4_linear_noalloc(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype, void* stream) {
+  int rc = validate_weight(w, "q4_linear_noalloc");
+  if (rc == Q4_OK) rc = validate_dtype(dtype, "q4_linear_noalloc");
+  if (rc != Q4_OK) return rc;
+  if (M < 0) {
+    set_error("q4_linear_noalloc: negative M=%d", M);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M == 0 || w->N == 0) return Q4_OK;
+  const int path = q4_select_path(w, M, dtype);
+  // the decode kernels need their whole workspace; the prefill kernels fall back to unsplit
+  // tiles when the partial tiles do not fit, so they run with whatever the array holds
+  const size_t need = path == Q4_PATH_GEMV ? (size_t)Q4_WORKSPACE_COUNTER_BYTES + decode_partial_bytes(w, M)
+                                           : (size_t)Q4_WORKSPACE_COUNTER_BYTES;
+  if (need > Q4_SCRATCH_BYTES) {
+    set_error("q4_linear_noalloc: M=%d K=%d N=%d needs %zu bytes of scratch, the built-in array holds %zu "
+              "(use q4_linear with a workspace of q4_workspace_bytes_for())", M, w->K, w->N, need,
+              (size_t)Q4_SCRATCH_BYTES);
+    return Q4_ERR_WORKSPACE;
+  }
+  void* ptr = scratch_of_current_device("q4_linear_noalloc");
+  if (ptr == nullptr) return Q4_ERR_LAUNCH;
+  return q4_linear_ex(w, x, bias, y, M, dtype, ptr, Q4_SCRATCH_BYTES, path, stream);
 }
 
 int q4_linear(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
