@@ -12,7 +12,10 @@ the 256 MB Infinity Cache.  Inputs are resident in HBM before the timed region.
 `roofline` = the decode kernel against the 8 TB/s HBM peak, from per-launch durations
 measured with HIP events on the launch stream inside this script.
 `gemm` (when the prefill kernel is built) = M=2048 TFLOP/s on the same shapes.
-`cpu_baseline` = the NumPy oracle (dequantize then fp32 matmul) on the host cores.
+`cfg4` / `cfg5` = the act-order (Llama-3-70B shapes) and AWQ (Mistral-7B shapes) configurations
+at their own sizes, checkpoint-layout kernels and the opt-in load-time conversions side by side.
+`cpu_baseline` = the PyTorch restatement of the reference's dequantize-then-matmul path on all
+host cores (torch thread pool), a bounded sample.
 
 Prints exactly one JSON line on stdout.
 """
@@ -33,8 +36,18 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E peak
 MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16/bf16 MFMA peak
 
-# FETCH_SIZE 14182.1 KiB x 2.000 (copy-kernel calibration) + WRITE_SIZE 321.0 KiB x 1.000
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 29373594
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE live next to the
+# profile summaries they come from (the file names the commit and the summary)
+TRAFFIC_FILE = ROOT / "profiles" / "hbm_traffic.json"
+
+
+def measured_traffic(key):
+    """Bytes per launch from the tracked counter summary, or None when there is none."""
+    try:
+        entry = json.loads(TRAFFIC_FILE.read_text())[key]
+        return int(entry["bytes_per_launch"])
+    except (OSError, KeyError, ValueError, TypeError):
+        return None
 
 SHAPES = [  # name, K, N
     ("qkv_proj", 4096, 6144),
@@ -135,48 +148,73 @@ def time_kernel_launches(torch, fn_list, reps):
     return tot / rounds, best
 
 
-def cpu_baseline(M):
-    """Oracle (dequantize -> fp32 matmul) on the host, one call per projection."""
-    import numpy as np
-    from oracle import q4_oracle as o
+def _blas_backend(torch):
+    """Name of the BLAS library torch's CPU matmul uses, from its build configuration."""
+    try:
+        for part in torch.__config__.show().replace("\n", ",").split(","):
+            part = part.strip()
+            if part.startswith("BLAS_INFO="):
+                return part.split("=", 1)[1]
+    except Exception:
+        pass
+    return "unknown"
 
-    total_bytes = 0
-    total_t = 0.0
-    detail = {}
-    reps = 8  # about 10 s of host work in total
-    for name, K, N in SHAPES:
+
+def cpu_baseline(M):
+    """The reference's dequantize-then-matmul path restated in PyTorch, on all host cores: the
+    decode step (four projections, M rows), plus cfg1 (K = N = 4096, M = 16) and one prefill shape
+    (o_proj at M = 2048) for context.  A bounded sample: a few repetitions each."""
+    import torch
+
+    from oracle import q4_oracle as o
+    from oracle import q4_oracle_torch as ot
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+
+    def tensors(K, N):
         qw, qz, sc, _ = o.make_gptq(K, N, GROUPSIZE, seed=1)
-        x = o.make_x(M, K, seed=1)
+        return (torch.from_numpy(qw.view("int32")), torch.from_numpy(qz.view("int32")), torch.from_numpy(sc))
+
+    def timed(K, N, rows, reps):
+        qw, qz, sc = tensors(K, N)
+        x = torch.from_numpy(o.make_x(rows, K, seed=1))
         td = tm = 0.0
         for _ in range(reps):
             t0 = time.perf_counter()
-            w = o.dequant_gptq(qw, qz, sc, None, GROUPSIZE, "f16")
+            w = ot.dequant_gptq(qw, qz, sc, None, GROUPSIZE)
             t1 = time.perf_counter()
-            o.linear_forward(x, w, None, "f16")
+            ot.linear_forward(x, w, None)
             t2 = time.perf_counter()
             td += t1 - t0
             tm += t2 - t1
             del w
-        detail[name] = {"dequant_ms": round(td / reps * 1e3, 1), "matmul_ms": round(tm / reps * 1e3, 1)}
-        total_bytes += gemv_bytes(M, K, N) * reps
-        total_t += td + tm
-    threads = os.cpu_count()
-    try:
-        from threadpoolctl import threadpool_info
-        pools = [p["num_threads"] for p in threadpool_info() if p.get("user_api") == "blas"]
-        if pools:
-            threads = max(pools)
-    except Exception:
-        pass
+        return td / reps, tm / reps
+
+    detail = {}
+    reps = 3
+    step_t = 0.0
+    step_bytes = 0
+    for name, K, N in SHAPES:
+        td, tm = timed(K, N, M, reps)
+        detail[name] = {"dequant_ms": round(td * 1e3, 1), "matmul_ms": round(tm * 1e3, 1)}
+        step_t += td + tm
+        step_bytes += gemv_bytes(M, K, N)
+    td, tm = timed(4096, 4096, 16, 2)
+    detail["cfg1_4096x4096_m16"] = {"dequant_ms": round(td * 1e3, 1), "matmul_ms": round(tm * 1e3, 1)}
+    td, tm = timed(4096, 4096, 2048, 2)
+    detail["o_proj_m2048"] = {"dequant_ms": round(td * 1e3, 1), "matmul_ms": round(tm * 1e3, 1),
+                              "TFLOPs": round(2.0 * 2048 * 4096 * 4096 / (td + tm) / 1e12, 3)}
     return {
-        "value": round(total_bytes / total_t / 1e9, 4),
+        "value": round(step_bytes / step_t / 1e9, 4),
         "unit": "GB/s",
-        "cores": threads,
+        "cores": cores,
         "kind": "port",
-        "sample": f"{reps} steps (4 Llama-3-8B projections each, M={M}) of the NumPy oracle: dequantize to fp16 "
-                  f"then fp32 matmul; {total_t:.1f} s of host time; unpacking is single-threaded NumPy, "
-                  f"the matmul uses the BLAS thread pool",
-        "ms_per_step": round(total_t / reps * 1e3, 1),
+        "sample": f"{reps} decode steps (4 Llama-3-8B projections each, M={M}) of the PyTorch restatement of the "
+                  f"reference path: unpack + dequantize to fp16, then x.float() @ W.float(); torch thread pool with "
+                  f"{cores} threads, BLAS backend {_blas_backend(torch)}; "
+                  f"plus cfg1 (M=16) and o_proj at M=2048, 2 repetitions each",
+        "ms_per_step": round(step_t * 1e3, 1),
         "detail": detail,
     }
 
@@ -281,10 +319,20 @@ def main():
         }
         all_durs.append(avg)
         all_bytes += b
+    # the same call outside a graph: Python + ctypes + launch per call (o_proj, M rows)
+    for _ in range(50):
+        pkg.ops.linear(weights[0][1], xs[1], None, out=ys[1])
+    torch.cuda.synchronize()
+    n_eager = 2000
+    t0 = time.perf_counter()
+    for c in range(n_eager):
+        pkg.ops.linear(weights[c % copies][1], xs[1], None, out=ys[1])
+    torch.cuda.synchronize()
+    per_shape["o_proj"]["eager_us_per_call"] = round((time.perf_counter() - t0) / n_eager * 1e6, 2)
     achieved = all_bytes / sum(all_durs) / 1e9
     roofline = {
         "bound": "hbm",
-        "kernel": "q4::gemv_gptq_kernel",
+        "kernel": "q4::gemv_gptq_kernel / q4::gemv_gptq_lean_kernel",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
@@ -292,7 +340,7 @@ def main():
         # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this
         # workload (mean over the four projections, calibrated with a 256 MiB copy kernel);
         # only valid for the default M=1 workload, null otherwise
-        "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if M == 1 else None,
+        "traffic": measured_traffic("decode_m1") if M == 1 else None,
         "bytes_per_launch": all_bytes // len(SHAPES),
         "us_per_launch": round(sum(all_durs) / len(SHAPES) * 1e6, 2),
     }
@@ -355,12 +403,33 @@ def main():
                 gm[name]["dense_fp16_matmul_TFLOPs"] = round(fl / davg / 1e12, 1)
                 del dense
             del xg, yg
+        power = None
+        if gm and not args.no_dense_ref:
+            # What bounds the GEMM: the same kernel (and the vendor library's dense GEMM) on all-zero
+            # operands, which toggle no data lines and draw far less power (gate_up, fp16)
+            name, K, N = SHAPES[2]
+            wz = [make_weights(pkg, torch, dev, K, N, seed=900 + c) for c in range(2)]
+            for w in wz:
+                w.qweight.zero_()
+            xz = torch.zeros((Mg, K), device=dev, dtype=torch.float16)
+            yz = torch.empty((Mg, N), device=dev, dtype=torch.float16)
+            zavg, _ = time_kernel_launches(torch, [(lambda c=c: pkg.ops.linear(wz[c], xz, None, out=yz)) for c in range(2)], 20)
+            dz = [torch.zeros((K, N), device=dev, dtype=torch.float16) for _ in range(2)]
+            dzavg, _ = time_kernel_launches(torch, [(lambda c=c: torch.matmul(xz, dz[c], out=yz)) for c in range(2)], 20)
+            fl = 2.0 * Mg * N * K
+            power = {"shape": name, "zero_operands_TFLOPs": round(fl / zavg / 1e12, 1),
+                     "random_operands_TFLOPs": gm[name]["TFLOPs"],
+                     "dense_fp16_matmul_zero_operands_TFLOPs": round(fl / dzavg / 1e12, 1),
+                     "dense_fp16_matmul_random_operands_TFLOPs": gm[name].get("dense_fp16_matmul_TFLOPs")}
+            del wz, xz, yz, dz
         if gm:
             out["gemm"] = {
                 "M": Mg, "per_shape": gm,
                 "roofline": {"bound": "mfma", "kernel": "q4::gemm_gptq_kernel", "achieved": round(tot_f / tot_t / 1e12, 1),
                              "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                             "frac": round(tot_f / tot_t / 1e12 / MFMA_PEAK_TFLOPS, 4), "traffic": None},
+                             "frac": round(tot_f / tot_t / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                             "traffic": measured_traffic(f"gemm_m{Mg}")},
+                "power_probe": power,
             }
 
     # ---- batched decode: the same four projections with more activation rows (the serving
@@ -384,14 +453,13 @@ def main():
 
         for Mb in (4, 16, 18, 32, 64):
             batch[f"gptq_m{Mb}"] = step_us(weights, Mb)
-        # act_order: rows put into group order at load time (what the layers do by default),
-        # x read through the permutation; act_order_lookup: checkpoint order, g_idx in the kernel;
-        # awq_native: the AWQ-layout kernels (the layers convert AWQ checkpoints to the GPTQ layout
-        # once and then run at the gptq_* figures)
-        for kind in ("awq_native", "act_order", "act_order_lookup"):
-            wl = [[make_weights_variant(pkg, torch, dev, K, N, 31 * c + i, "awq" if kind == "awq_native" else "act_order")
+        # awq / act_order: the kernels that read the checkpoint layout (what the layers run);
+        # *_converted / *_repacked: the opt-in load-time conversions (AWQ -> GPTQ layout, rows
+        # into group order with x read through the permutation)
+        for kind in ("awq", "act_order", "act_order_repacked"):
+            wl = [[make_weights_variant(pkg, torch, dev, K, N, 31 * c + i, "awq" if kind == "awq" else "act_order")
                    for i, (_, K, N) in enumerate(SHAPES)] for c in range(min(copies, 3))]
-            if kind == "act_order":
+            if kind == "act_order_repacked":
                 wl = [[pkg.ops.make_sequential(w) for w in row] for row in wl]
                 torch.cuda.empty_cache()
             for Mb in (1, 16):
@@ -399,6 +467,58 @@ def main():
             del wl
             torch.cuda.empty_cache()
         out["batched_decode"] = batch
+
+        # ---- BASELINE.json configs[3] and [4] at their own shapes
+        def shape_us(make, K, N, Mb, ncopies):
+            ws_ = [make(c) for c in range(ncopies)]
+            xb = torch.randn((Mb, K), device=dev, dtype=torch.float16)
+            yb = torch.empty((Mb, N), device=dev, dtype=torch.float16)
+            fns = [(lambda c=c: pkg.ops.linear(ws_[c], xb, None, out=yb)) for c in range(ncopies)]
+            avg, _ = time_kernel_launches(torch, fns, 48 if Mb <= 64 else 12)
+            path = pkg.ops.select_path(ws_[0], Mb)
+            del ws_, xb, yb
+            torch.cuda.empty_cache()
+            return avg, path
+
+        cfg4 = {}
+        for K, N in ((8192, 10240), (28672, 8192)):
+            nc = max(2, -(-600 * 1024 * 1024 // (K * N // 2)))
+            for Mb in (1, 16, 1024):
+                entry = {}
+                for label, seq in (("g_idx_kernels", False), ("rows_in_group_order", True)):
+                    def make(c, seq=seq):
+                        w = make_weights_variant(pkg, torch, dev, K, N, 71 * c + Mb, "act_order")
+                        return pkg.ops.make_sequential(w) if seq else w
+                    avg, path = shape_us(make, K, N, Mb, nc)
+                    entry[label] = {"us": round(avg * 1e6, 1), "path": path}
+                    if Mb <= 16:
+                        entry[label]["GBps"] = round(gemv_bytes(Mb, K, N, g_idx=True) / avg / 1e9, 1)
+                    else:
+                        entry[label]["TFLOPs"] = round(2.0 * Mb * N * K / avg / 1e12, 1)
+                cfg4[f"{K}x{N}_m{Mb}"] = entry
+        out["cfg4_act_order_llama70b"] = cfg4
+        cfg5 = {}
+        for K, N in ((4096, 14336), (14336, 4096)):
+            nc = max(2, -(-600 * 1024 * 1024 // (K * N // 2)))
+            conv = importlib.import_module(f"{pkg.__name__}.layers.awq.conversion_utils")
+            for Mb in (1, 16, 256):
+                entry = {}
+                for label, convert in (("awq_layout_kernels", False), ("converted_to_gptq_layout", True)):
+                    def make(c, convert=convert):
+                        w = make_weights_variant(pkg, torch, dev, K, N, 53 * c + Mb, "awq")
+                        if not convert:
+                            return w
+                        gq, gz = conv.fast_awq_to_gptq(w.qweight, w.qzeros)
+                        return pkg.ops.make_packed(gq.contiguous(), gz.contiguous(), w.scales, None, GROUPSIZE, 0)
+                    avg, path = shape_us(make, K, N, Mb, nc)
+                    e = {"us": round(avg * 1e6, 1), "path": path}
+                    if Mb <= 16:
+                        e["GBps"] = round(gemv_bytes(Mb, K, N) / avg / 1e9, 1)
+                    else:
+                        e["TFLOPs"] = round(2.0 * Mb * N * K / avg / 1e12, 1)
+                    entry[label] = e
+                cfg5[f"{K}x{N}_m{Mb}"] = entry
+        out["cfg5_awq_mistral7b"] = cfg5
 
     # ---- mixture-of-experts block (Mixtral-8x7B shapes: 8 experts, top-2, 4096 -> 2 x 14336 -> 4096):
     # routing, both grouped projections, activation and weighted sum, per block call

@@ -305,3 +305,33 @@ def test_gate_up_forward_roundings(oracle):
     assert out[0, 0] == np.float16(np.float32(s1) * np.float32(3.0))
     assert out[0, 1] == np.float16(np.float32(s2) * np.float32(-1.0))
     assert np.allclose(exact[0], [3.0 / (1.0 + np.exp(-1.0)), 2.0 / (1.0 + np.exp(2.0))], rtol=1e-6)
+
+
+def test_torch_restatement_matches_numpy_oracle():
+    """The PyTorch restatement used for the CPU baseline is the NumPy oracle in another idiom:
+    same dequantized bits, same fp32 products (GPTQ with and without g_idx, AWQ)."""
+    import torch
+
+    from oracle import q4_oracle as o
+    from oracle import q4_oracle_torch as ot
+
+    def t(a):
+        return torch.from_numpy(a.view(np.int32) if a.dtype == np.uint32 else a)
+
+    for act in (False, True):
+        qw, qz, sc, gi = o.make_gptq(512, 256, 128, seed=7, sym=False, act_order=act)
+        w = o.dequant_gptq(qw, qz, sc, gi, 128, "f16")
+        wt = ot.dequant_gptq(t(qw), t(qz), t(sc), t(gi) if gi is not None else None, 128)
+        assert np.array_equal(wt.numpy().view(np.uint16), w.view(np.uint16))
+    qw, qz, sc = o.make_awq(512, 256, 128, seed=8)
+    w = o.dequant_awq(qw, qz, sc, 128, "f16")
+    wt = ot.dequant_awq(t(qw), t(qz), t(sc), 128)
+    assert np.array_equal(wt.numpy().view(np.uint16), w.view(np.uint16))
+    x = o.make_x(5, 512, seed=3)
+    y32, y16 = o.linear_forward(x, w, None, "f16")
+    t32, t16 = ot.linear_forward(t(x), wt, None)
+    assert np.allclose(t32.numpy(), y32, rtol=1e-5, atol=1e-5)
+    assert np.array_equal(wt.numpy()[:1].view(np.uint16), w[:1].view(np.uint16))
+    # one-hot rows read the weights back exactly through the matmul
+    eye = torch.eye(512, dtype=torch.float16)[:7]
+    assert torch.equal(ot.linear_forward(eye, wt, None)[1], wt[:7])

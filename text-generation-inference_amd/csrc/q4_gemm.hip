@@ -18,6 +18,15 @@ bool gemm_supported(const q4_weight* w, int M, int dtype) {
   return true;
 }
 
+// two K groups per workgroup (eight waves), groups of at least 64 rows
+template <int DTYPE, int BM>
+static void launch_tile_kg2(const GemmParams& gp, dim3 grid, size_t smem, hipStream_t stream) {
+  auto k = q4::gemm_gptq_kernel<DTYPE, BM, 1, 2, false, 2>;
+  if (smem > 64 * 1024)
+    (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  hipLaunchKernelGGL(k, grid, dim3(512), smem, stream, gp);
+}
+
 template <int DTYPE, int BM, int NW>
 static void launch_tile(const GemmParams& gp, int gs, dim3 grid, size_t smem, hipStream_t stream) {
   using namespace q4;
@@ -37,14 +46,15 @@ static void launch_tile(const GemmParams& gp, int gs, dim3 grid, size_t smem, hi
 // Tile shape and split factor for a problem; shared by the launcher and the workspace sizing.
 struct GemmPlan {
   int bm, nw, splits;
+  int kg = 1;  // K groups per workgroup (2: eight waves, see gemm_gptq_kernel)
   long tiles;
 };
 
 static GemmPlan gemm_plan(int M, int K, int N) {
   // Tile choice (all with 4 waves side by side along N):
-  //   256 x 256  grids of at least two rounds over the 256 CUs: half the unpacking per flop,
-  //              one wave per SIMD, runs at a higher clock;
-  //   128 x 256  the default; two workgroups per CU once there are more than 256 of them;
+  //   128 x 256  the default; two workgroups per CU once there are more than 256 of them (a
+  //              256 x 256 tile with one wave per SIMD measured 0..12 % slower on every Llama-3-8B
+  //              projection at M = 512 .. 4096: 4096 x 28672 at M = 2048 501 against 446 us);
   //    64 x 256  up to 64 rows: half the accumulators, three workgroups per CU keep more weight
   //              loads in flight (4096 x 28672 at M = 32: 30.6 against 40.7 us; 8192 x 8192:
   //              23.4 against 28.5 us); a cost model of its own for the split factor measured
@@ -53,10 +63,8 @@ static GemmPlan gemm_plan(int M, int K, int N) {
   //              everywhere else: twice the activation-fragment reads per MFMA).
   GemmPlan g;
   const bool n256 = N % 256 == 0;
-  const long t256 = n256 ? (long)((M + 255) / 256) * (N / 256) : 0;
   g.bm = 128;
   g.nw = n256 ? 2 : 1;
-  if (t256 >= 512) g.bm = 256;
   if (M <= 64 && n256) g.bm = 64;
   const int bn = 128 * g.nw;
   g.tiles = (long)((M + g.bm - 1) / g.bm) * (N / bn);
@@ -70,6 +78,11 @@ static GemmPlan gemm_plan(int M, int K, int N) {
   // M = 512: 200 us unsplit, 78 us with eight.)
   g.splits = 1;
   if (g.bm <= 128 && g.tiles < 256) g.splits = gemm_pick_splits(g.tiles, K / q4::kBK, M, N, 0.9, 1.3);
+  // One workgroup per CU (the tiles, times the split factor, do not exceed the CU count): eight
+  // waves in two K groups put two waves on every SIMD.  Measured at M = 2048 on MI355X:
+  // 4096 x 4096 77.8 -> 70.2 us, 14336 x 4096 296 -> 246 us; with more workgroups than CUs the
+  // four-wave kernel, two to a CU, is the faster one (4096 x 6144: 115 against 127 us).
+  if (g.bm == 128 && g.nw == 2 && g.tiles * g.splits <= 256 && (K / q4::kBK) % (2 * g.splits) == 0) g.kg = 2;
   return g;
 }
 
@@ -148,17 +161,27 @@ int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, in
     set_error("q4_linear(gemm): grid too large");
     return Q4_ERR_UNSUPPORTED;
   }
-  const size_t smem = 2 * (size_t)bm * kAUnitsPerRow * 16;
+  size_t smem = 2 * (size_t)bm * kAUnitsPerRow * 16;
   dim3 grid((unsigned)total);
   const int gs = w->groupsize;
-  if (dtype == Q4_DTYPE_F16) {
+  const bool kg2 = g.kg == 2 && nw == 2 && bm <= 128 && gs >= 64 && (w->K / kBK) % (2 * g.splits) == 0;
+  if (kg2) {
+    smem *= 2;
+    const size_t xch = (size_t)(bm / 32) * 2 * 16 * 256 * sizeof(float);
+    if (xch > smem) smem = xch;
+    if (dtype == Q4_DTYPE_F16) {
+      if (bm == 64) launch_tile_kg2<Q4_DTYPE_F16, 64>(gp, grid, smem, stream);
+      else launch_tile_kg2<Q4_DTYPE_F16, 128>(gp, grid, smem, stream);
+    } else {
+      if (bm == 64) launch_tile_kg2<Q4_DTYPE_BF16, 64>(gp, grid, smem, stream);
+      else launch_tile_kg2<Q4_DTYPE_BF16, 128>(gp, grid, smem, stream);
+    }
+  } else if (dtype == Q4_DTYPE_F16) {
     if (bm == 64) launch_tile<Q4_DTYPE_F16, 64, 2>(gp, gs, grid, smem, stream);
-    else if (bm == 256) launch_tile<Q4_DTYPE_F16, 256, 2>(gp, gs, grid, smem, stream);
     else if (nw == 2) launch_tile<Q4_DTYPE_F16, 128, 2>(gp, gs, grid, smem, stream);
     else launch_tile<Q4_DTYPE_F16, 128, 1>(gp, gs, grid, smem, stream);
   } else {
     if (bm == 64) launch_tile<Q4_DTYPE_BF16, 64, 2>(gp, gs, grid, smem, stream);
-    else if (bm == 256) launch_tile<Q4_DTYPE_BF16, 256, 2>(gp, gs, grid, smem, stream);
     else if (nw == 2) launch_tile<Q4_DTYPE_BF16, 128, 2>(gp, gs, grid, smem, stream);
     else launch_tile<Q4_DTYPE_BF16, 128, 1>(gp, gs, grid, smem, stream);
   }

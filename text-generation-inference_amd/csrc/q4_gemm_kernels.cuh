@@ -121,8 +121,14 @@ __device__ __forceinline__ float16_t mfma32(const uint4_t a, const uint4_t b, fl
 // NW: packed words (columns) per lane and K step: 2 -> 256-column workgroup tile, 1 -> 128.
 // MOE: grouped launch, blockIdx.y is the expert; its row count is read from device memory, so
 // the grid covers the largest possible count and surplus workgroups leave at once.
-template <int DTYPE, int BM, int GPT, int NW, bool MOE = false>
-__global__ __launch_bounds__(256, (BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm_gptq_kernel(GemmParams gp) {
+// KG: K groups per workgroup (1 or 2).  With 2 the workgroup has eight waves: waves 0-3 take
+// the even K tiles of the workgroup's range, waves 4-7 the odd ones, each group with its own
+// activation buffers in LDS; the two accumulator sets meet through LDS at the end.  A grid of
+// one workgroup per CU then runs two waves per SIMD (one wave's fragment reads and unpacking
+// under the other's MFMAs) without any partial tile going through memory.
+template <int DTYPE, int BM, int GPT, int NW, bool MOE = false, int KG = 1>
+__global__ __launch_bounds__(256 * KG, (KG == 2 ? 1 : BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm_gptq_kernel(GemmParams gp) {
+  static_assert(KG == 1 || (KG == 2 && !MOE && BM <= 128), "two K groups: dense launches, at most 128 rows");
   int moe_row0 = 0;
   if constexpr (MOE) {
     moe_row0 = moe_enter(gp.p, gp.moe, blockIdx.y);
@@ -133,7 +139,8 @@ __global__ __launch_bounds__(256, (BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) 
   constexpr int A_TILE_BYTES = BM * kAUnitsPerRow * 16;
   extern __shared__ __align__(16) unsigned char smem[];  // two activation tiles
   const Problem& p = gp.p;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x & 255;  // thread of its K group
+  const int grp = KG == 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int j = lane & 31;
@@ -181,9 +188,14 @@ __global__ __launch_bounds__(256, (BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) 
 
   const SpliceK splice = gemm_splice_consts();
   const int KT_all = K / kBK;
-  // this workgroup's K tiles [kt_begin, KT)
-  const int kt_begin = (int)((long)split * KT_all / gp.splits);
-  const int KT = (int)((long)(split + 1) * KT_all / gp.splits);
+  // this workgroup's K tiles [kt_begin, kt_end); group grp walks kt_begin + grp, + KG, ...
+  // (KG == 2: the host makes the count even).  Below, tile indices are positions in the group's
+  // own sequence: tile i is K tile kt0 + i * KG.
+  const int kt0 = (int)((long)split * KT_all / gp.splits) + grp;
+  const int kt_end = (int)((long)(split + 1) * KT_all / gp.splits);
+  const int kt_begin = 0;
+  const int KT = (kt_end - kt0 + KG - 1) / KG;
+  auto ktile = [&](int i) { return kt0 + i * KG; };
 
   // ---- packed-weight stream: words [K/8 + kq][ncol, ncol+1], two K tiles ahead
   const char* wbase = (const char*)p.qweight;
@@ -195,7 +207,7 @@ __global__ __launch_bounds__(256, (BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) 
 #pragma unroll
     for (int s = 0; s < kKSteps; ++s)
     {
-      const char* addr = wbase + (size_t)(kt * kKSteps + s) * kstep_bytes + w_lane;
+      const char* addr = wbase + (size_t)(ktile(kt) * kKSteps + s) * kstep_bytes + w_lane;
       if constexpr (NW == 2) {
         const uint2_t t = *(const uint2_t*)addr;
         dst[s].v[0] = t.x; dst[s].v[1] = t.y;
@@ -213,7 +225,7 @@ __global__ __launch_bounds__(256, (BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) 
   auto load_group_raw = [&](int kt) {
 #pragma unroll
     for (int g = 0; g < GPT; ++g) {
-      int gi = (kt * kBK + g * (kBK / GPT)) / p.groupsize;
+      int gi = (ktile(kt) * kBK + g * (kBK / GPT)) / p.groupsize;
       gi = min(gi, p.num_groups - 1);
       if constexpr (NW == 2) sraw[g] = *(const uint32_t*)(p.scales + (size_t)gi * N + ncol);
       else sraw[g] = *(const uint16_t*)(p.scales + (size_t)gi * N + ncol);
@@ -252,12 +264,12 @@ __global__ __launch_bounds__(256, (BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) 
       const int m = u >> 3, kb = u & 7;
       // rows past M re-read the last row: their results are never stored
       const int row = MOE ? moe_xrow[i] : min(m0 + m, M - 1);
-      areg[set][i] = *(const uint4_t*)(xs + (size_t)row * K + kt * kBK + kb * 8);
+      areg[set][i] = *(const uint4_t*)(xs + (size_t)row * K + ktile(kt) * kBK + kb * 8);
     }
   };
   auto store_a = [&](int buf, auto set_c) {
     constexpr int set = decltype(set_c)::value % ASETS;
-    unsigned char* base = smem + buf * A_TILE_BYTES;
+    unsigned char* base = smem + (grp * 2 + buf) * A_TILE_BYTES;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
       const int u = tid + 256 * i;
@@ -284,7 +296,7 @@ __global__ __launch_bounds__(256, (BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) 
   uint4_t afrag[2][MT];  // A fragments of the current / next MFMA K step
   uint4_t bfrag[2][NW];  // unpacked B fragments of the current / next step
   auto read_a = [&](int buf, int s, uint4_t (&dst)[MT]) {
-    const unsigned char* abase = smem + buf * A_TILE_BYTES + a_lane_off;
+    const unsigned char* abase = smem + (grp * 2 + buf) * A_TILE_BYTES + a_lane_off;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
       dst[mt] = *(const uint4_t*)(abase + (mt * 32 * kAUnitsPerRow + 2 * s) * 16);
@@ -386,6 +398,29 @@ __global__ __launch_bounds__(256, (BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) 
       tile_step(kt + 1, std::integral_constant<int, 1>{});
     }
     if (kt < KT) tile_step(kt, std::integral_constant<int, 0>{});
+  }
+
+  if constexpr (KG == 2) {
+    // the odd-tile group hands its sums over through LDS (the activation buffers are dead):
+    // accumulator register by register, consecutive threads at consecutive addresses
+    __syncthreads();
+    float* xch = (float*)smem;
+    if (grp == 1) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int f = 0; f < NW; ++f)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) xch[((mt * NW + f) * 16 + r) * 256 + tid] = acc[mt][f][r];
+    }
+    __syncthreads();
+    if (grp == 1) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int f = 0; f < NW; ++f)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mt][f][r] += xch[((mt * NW + f) * 16 + r) * 256 + tid];
   }
 
   // ---- epilogue: C layout of the 32x32 MFMA: register r of lane (j, kq) is row
