@@ -151,10 +151,11 @@ def time_kernel_launches(torch, fn_list, reps):
 def _blas_backend(torch):
     """Name of the BLAS library torch's CPU matmul uses, from its build configuration."""
     try:
-        for part in torch.__config__.show().replace("\n", ",").split(","):
-            part = part.strip()
-            if part.startswith("BLAS_INFO="):
-                return part.split("=", 1)[1]
+        import re
+
+        m = re.search(r"BLAS_INFO=([A-Za-z0-9_]+)", torch.__config__.show())
+        if m:
+            return m.group(1)
     except Exception:
         pass
     return "unknown"
