@@ -79,6 +79,8 @@ def parse_args():
     ap.add_argument("--copies", type=int, default=0, help="weight copies to rotate over (0 = auto)")
     ap.add_argument("--no-dense-ref", action="store_true",
                     help="skip timing torch's dense fp16 matmul (hipBLASLt) on the GEMM shapes")
+    ap.add_argument("--floor-probe", action="store_true",
+                    help="time read-only kernels (q4_probe_read) on buffers of the projections' sizes and print a table")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="eager launches only (a 256 MiB copy kernel, then each decode shape and one GEMM), "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs; prints no JSON line")
@@ -220,6 +222,92 @@ def cpu_baseline(M):
     }
 
 
+def read_floor_configs(K, N):
+    """Grids of the read-only tile kernel for a [K/8, N] matrix of packed words: (workgroups,
+    threads, unroll) with the row steps dividing evenly, around the decode kernels' own grids."""
+    ntiles = N // 64
+    steps_total = K // 32  # four packed rows per wave load
+    out = []
+    for wk in (4, 8, 16):
+        for splits in (1, 2, 4, 7, 8, 14, 16):
+            slots = wk * splits
+            if steps_total % slots:
+                continue
+            per = steps_total // slots
+            wgs = ntiles * splits
+            if wgs < 192 or wgs > 4096:
+                continue
+            for unroll in (2, 4, 8):
+                if per % unroll == 0:
+                    out.append((wgs, 64 * wk, unroll))
+    return out
+
+
+def time_read_floor(pkg, torch, lib, dev, pool, sink, nbytes, pattern, n_words, wgs, threads, unroll, hot, reps=24):
+    """Average us of one read-only launch over `nbytes`; the launches of a graph walk through
+    `pool` (larger than the last-level cache) unless `hot`."""
+    pieces = max(1, pool.numel() // nbytes)
+    stream = torch.cuda.Stream()
+    fns = []
+    for r in range(1 if hot else min(pieces, reps)):
+        ptr = pool.data_ptr() + r * nbytes
+
+        def fn(ptr=ptr):
+            rc = lib.q4_probe_read(ptr, nbytes, pattern, n_words, wgs, threads, unroll, sink.data_ptr(),
+                                   torch.cuda.current_stream().cuda_stream)
+            pkg._lib.check(rc)
+        fns.append(fn)
+    avg, best = time_kernel_launches(torch, fns, reps)
+    return avg * 1e6, best * 1e6
+
+
+def floor_probe(pkg, torch, lib, dev):
+    """Table of read-only launches: empty grids, linear reads and the decode tile pattern at the
+    four projections' sizes, HBM-rotating (1 GiB pool) and cache-hot."""
+    pool = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+    sink = torch.zeros(4, dtype=torch.uint8, device=dev)
+    rows = []
+    for wgs in (256, 1024, 4096):
+        for threads in (256, 512):
+            us, _ = time_read_floor(pkg, torch, lib, dev, pool, sink, 4096, 2, 0, wgs, threads, 1, True)
+            rows.append({"what": "empty", "workgroups": wgs, "threads": threads, "us": round(us, 2)})
+            print(f"empty kernel           wgs {wgs:5d} x {threads:4d}                       {us:7.2f} us", flush=True)
+    summary = {}
+    for name, K, N in SHAPES:
+        nbytes = K * N // 2
+        best = {}
+        for wgs in (256, 512, 1024, 2048):
+            for threads in (256, 512):
+                for unroll in (2, 4, 8):
+                    # the linear kernel reads whole rounds of threads x unroll vectors per workgroup
+                    rnd = threads * unroll
+                    if (nbytes // 16 // wgs // rnd * rnd) * 16 * wgs != nbytes:
+                        continue
+                    for hot in (False, True):
+                        us, _ = time_read_floor(pkg, torch, lib, dev, pool, sink, nbytes, 0, 0, wgs, threads, unroll, hot)
+                        key = "linear_hot" if hot else "linear"
+                        if key not in best or us < best[key]["us"]:
+                            best[key] = {"workgroups": wgs, "threads": threads, "unroll": unroll, "us": round(us, 2)}
+                        rows.append({"what": key, "shape": name, "workgroups": wgs, "threads": threads, "unroll": unroll,
+                                     "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1)})
+        for wgs, threads, unroll in read_floor_configs(K, N):
+            for hot in (False, True):
+                us, _ = time_read_floor(pkg, torch, lib, dev, pool, sink, nbytes, 1, N, wgs, threads, unroll, hot)
+                key = "tile_hot" if hot else "tile"
+                if key not in best or us < best[key]["us"]:
+                    best[key] = {"workgroups": wgs, "threads": threads, "unroll": unroll, "us": round(us, 2)}
+                rows.append({"what": key, "shape": name, "workgroups": wgs, "threads": threads, "unroll": unroll,
+                             "bytes_in_flight_per_wave": unroll * 1024, "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1)})
+                print(f"{name:13s} {key:9s} wgs {wgs:5d} x {threads:4d} unroll {unroll}  {nbytes / 1e6:6.1f} MB  {us:7.2f} us  "
+                      f"{nbytes / us / 1e3:7.1f} GB/s", flush=True)
+        for key, b in best.items():
+            b["GBps"] = round(nbytes / b["us"] / 1e3, 1)
+        summary[name] = {"bytes": nbytes, **best}
+        print(f"== {name}: " + "  ".join(f"{k} {v['us']} us ({v['GBps']} GB/s, {v['workgroups']}x{v['threads']} u{v['unroll']})"
+                                          for k, v in best.items()), flush=True)
+    print(json.dumps({"read_floor": summary}))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -250,6 +338,10 @@ def main():
     def step(c):
         for i in range(len(SHAPES)):
             pkg.ops.linear(weights[c % copies][i], xs[i], None, out=ys[i])
+
+    if args.floor_probe:
+        floor_probe(pkg, torch, lib, dev)
+        return
 
     if args.traffic_probe:
         # calibration: a plain device-to-device copy of known size (reads and writes 256 MiB)
@@ -320,6 +412,16 @@ def main():
         }
         all_durs.append(avg)
         all_bytes += b
+    # read-only launches over the same weight bytes (decode tile pattern, rotating through
+    # HBM like the weights): the time such a launch takes when it computes nothing
+    if M == 1:
+        pool = torch.empty(1 << 29, dtype=torch.uint8, device=dev).random_(0, 255)
+        sink = torch.zeros(4, dtype=torch.uint8, device=dev)
+        for name, K, N in SHAPES:
+            floor = min(time_read_floor(pkg, torch, lib, dev, pool, sink, K * N // 2, 1, N, wgs, threads, unroll, False)[0]
+                        for wgs, threads, unroll in read_floor_configs(K, N) if unroll == 4)
+            per_shape[name]["read_only_floor_us"] = round(floor, 2)
+        del pool
     # the same call outside a graph: Python + ctypes + launch per call (o_proj, M rows)
     for _ in range(50):
         pkg.ops.linear(weights[0][1], xs[1], None, out=ys[1])

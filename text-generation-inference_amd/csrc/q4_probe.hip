@@ -1,0 +1,115 @@
+// Measurement aid: kernels that only read.  They give the time a launch of the decode
+// kernel's shape needs when it does nothing but pull its weight bytes out of HBM, which is
+// the floor the decode kernels are compared with.  Nothing in the product path calls them.
+#include <hip/hip_runtime.h>
+
+#include "q4_common.cuh"
+#include "q4_linear.h"
+
+namespace q4 {
+
+// One workgroup per contiguous range; every wave instruction reads 1 KB of consecutive bytes.
+template <int U>
+__global__ __launch_bounds__(1024) void probe_read_linear_kernel(const uint4_t* __restrict__ p, size_t vec_per_wg, uint32_t* sink) {
+  const uint4_t* base = p + (size_t)blockIdx.x * vec_per_wg;
+  uint4_t acc = {0u, 0u, 0u, 0u};
+  const size_t nt = blockDim.x;
+  for (size_t i = threadIdx.x; i < vec_per_wg; i += nt * U) {
+    uint4_t v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(base + i + (size_t)u * nt);
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u];
+  }
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) sink[0] = 1u;  // keeps the loads alive
+}
+
+// The decode kernels' pattern on a [rows, n_words] matrix of packed words: a wave load covers
+// four rows x 64 words (256 B per row); wave (tile, K slot) walks `steps` such loads down the
+// rows.  grid = ntiles * splits, block = 64 * wk.
+template <int U>
+__global__ __launch_bounds__(1024) void probe_read_tile_kernel(const uint32_t* __restrict__ p, int n_words, int wk, int steps,
+                                                               int ntiles, uint32_t* sink) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int tile = blockIdx.x % ntiles, split = blockIdx.x / ntiles;
+  const int col = tile * 64 + (lane & 15) * 4;
+  const size_t row0 = ((size_t)split * wk + wave) * steps * 4 + (lane >> 4);
+  const uint4_t* q = (const uint4_t*)(p + row0 * n_words + col);
+  const size_t stride = (size_t)n_words;  // uint4 units between loads: 4 rows * n_words / 4
+  uint4_t acc = {0u, 0u, 0u, 0u};
+  for (int s = 0; s < steps; s += U) {
+    uint4_t v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(q + (size_t)(s + u) * stride);
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u];
+  }
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) sink[0] = 1u;
+}
+
+__global__ void probe_empty_kernel(uint32_t* sink) {
+  if (sink == nullptr) sink[0] = 1u;
+}
+
+}  // namespace q4
+
+using namespace q4;
+using q4host::set_error;
+
+extern "C" int q4_probe_read(const void* buf, size_t bytes, int pattern, int n_words, int workgroups, int threads, int unroll,
+                             void* sink, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (sink == nullptr || workgroups <= 0 || threads <= 0 || threads > 1024 || threads % 64 != 0) {
+    set_error("q4_probe_read: needs a sink, a positive grid and a block of whole waves (<= 1024 threads)");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (pattern == 2) {
+    hipLaunchKernelGGL(probe_empty_kernel, dim3(workgroups), dim3(threads), 0, st, (uint32_t*)sink);
+    return hipGetLastError() == hipSuccess ? Q4_OK : Q4_ERR_LAUNCH;
+  }
+  if (buf == nullptr || (unroll != 1 && unroll != 2 && unroll != 4 && unroll != 8)) {
+    set_error("q4_probe_read: needs a buffer and an unroll of 1, 2, 4 or 8");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (pattern == 0) {
+    // every workgroup reads the same whole number of (threads x unroll) vector rounds
+    const size_t round = (size_t)threads * unroll;
+    const size_t vec_per_wg = bytes / 16 / workgroups / round * round;
+    if (vec_per_wg == 0) {
+      set_error("q4_probe_read: %zu bytes are less than one round of %d workgroups", bytes, workgroups);
+      return Q4_ERR_INVALID_ARGUMENT;
+    }
+    auto launch = [&](auto k) { hipLaunchKernelGGL(k, dim3(workgroups), dim3(threads), 0, st, (const uint4_t*)buf, vec_per_wg, (uint32_t*)sink); };
+    if (unroll == 1) launch(probe_read_linear_kernel<1>);
+    else if (unroll == 2) launch(probe_read_linear_kernel<2>);
+    else if (unroll == 4) launch(probe_read_linear_kernel<4>);
+    else launch(probe_read_linear_kernel<8>);
+  } else if (pattern == 1) {
+    const int wk = threads / 64;
+    if (n_words <= 0 || n_words % 64 != 0 || bytes % ((size_t)n_words * 16) != 0) {
+      set_error("q4_probe_read: tile pattern needs n_words %% 64 == 0 and a whole number of four-row steps");
+      return Q4_ERR_INVALID_ARGUMENT;
+    }
+    const int ntiles = n_words / 64;
+    const size_t steps_total = bytes / ((size_t)n_words * 16);
+    if (workgroups % ntiles != 0) {
+      set_error("q4_probe_read: %d workgroups are not a multiple of the %d column tiles", workgroups, ntiles);
+      return Q4_ERR_INVALID_ARGUMENT;
+    }
+    const size_t slots = (size_t)(workgroups / ntiles) * wk;
+    if (steps_total % slots != 0 || (steps_total / slots) % unroll != 0) {
+      set_error("q4_probe_read: %zu row steps do not divide over %zu wave slots x unroll %d", steps_total, slots, unroll);
+      return Q4_ERR_INVALID_ARGUMENT;
+    }
+    const int steps = (int)(steps_total / slots);
+    auto launch = [&](auto k) { hipLaunchKernelGGL(k, dim3(workgroups), dim3(threads), 0, st, (const uint32_t*)buf, n_words, wk, steps, ntiles, (uint32_t*)sink); };
+    if (unroll == 1) launch(probe_read_tile_kernel<1>);
+    else if (unroll == 2) launch(probe_read_tile_kernel<2>);
+    else if (unroll == 4) launch(probe_read_tile_kernel<4>);
+    else launch(probe_read_tile_kernel<8>);
+  } else {
+    set_error("q4_probe_read: unknown pattern %d", pattern);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  return hipGetLastError() == hipSuccess ? Q4_OK : Q4_ERR_LAUNCH;
+}
