@@ -529,7 +529,7 @@ int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, 
     return Q4_ERR_INVALID_ARGUMENT;
   }
   GemvConfig cfg{wcol, wk, splits, words};
-  if (words == 0) {  // the lean contiguous-group kernel
+  if (words == 0) {  // the lean contiguous-group kernel / the AWQ kernel that feeds the words as stored
     cfg.words = 4;
     cfg.lean = 1;
   } else if (words == 4 && gemv_rows32_kernel(w, M)) cfg.rows_per_block = 32;  // one workgroup for all rows

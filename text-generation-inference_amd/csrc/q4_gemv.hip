@@ -12,6 +12,7 @@ void launch_gemv_gate_up(const GemvParams& gp, int dtype, int rmax, bool static1
                          size_t smem, hipStream_t stream, bool grouped);
 // instruction-lean contiguous-group kernel (q4_gemv_lean.hip)
 void launch_gemv_lean(const GemvParams& gp, int dtype, int mp, dim3 grid, dim3 block, size_t smem, hipStream_t stream);
+void launch_gemv_awq_diag(const GemvParams& gp, int dtype, int row_groups, dim3 grid, dim3 block, size_t smem, hipStream_t stream);
 
 // GPTQ layout, contiguous groups of whole 128-row chunks: what the lean kernel takes
 bool gemv_lean_supported(const q4_weight* w, int dtype) {
@@ -81,7 +82,16 @@ bool gemv_rows32_supported(const q4_weight* w, int M) {
 static GemvConfig pick_config(const q4_weight* w, int M, bool gate_up, bool allow_lean);
 
 // the plain call of q4_linear: any kernel of the family
-GemvConfig gemv_pick_config(const q4_weight* w, int M) { return pick_config(w, M, false, true); }
+GemvConfig gemv_pick_config(const q4_weight* w, int M) {
+  GemvConfig c = pick_config(w, M, false, true);
+  // AWQ layout, plain call, up to 8 rows: the kernel that feeds the stored words to the matrix
+  // core (its MFMA count grows with the rows).  Same decomposition, us on MI355X, new / old:
+  // 4096 x 14336 12.0 / 13.3 at M = 1, 13.2 / 15.3 at M = 2, 15.0 / 18.4 at M = 4, 21.1 / 21.4 at
+  // M = 8, 35.6 / 27.6 at M = 16; 14336 x 4096 11.8 / 13.0, 13.1 / 15.3, 17.1 / 20.2, 22.8 / 23.0,
+  // 37.8 / 31.0; 4096 x 4096 8.5 / 9.0, 9.8 / 10.7, 11.6 / 13.5, 16.0 / 16.2, 21.3 / 27.3.
+  if (w->layout == Q4_LAYOUT_AWQ && c.rows_per_block == 16 && M <= 8) c.lean = 1;
+  return c;
+}
 // the kernels with the gated-MLP epilogue, two row blocks or an expert dimension (no lean variant)
 GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) { return pick_config(w, M, gate_up, false); }
 
@@ -370,7 +380,8 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
     return Q4_ERR_INVALID_ARGUMENT;
   }
   const int wave_cols = awq ? 256 : 16 * cfg.words;
-  const bool lean = cfg.lean != 0;
+  const bool diag = awq && cfg.lean != 0 && gate_up_act == 0 && M <= 8;  // AWQ: words straight into the MFMA
+  const bool lean = !awq && cfg.lean != 0;
   if (lean && !(gate_up_act == 0 && cfg.words == 4 && cfg.rows_per_block == 16 && gemv_lean_supported(w, dtype))) {
     set_error("q4_linear(gemv): the lean kernel takes GPTQ weights with contiguous groups of a multiple of 128 rows");
     return Q4_ERR_INVALID_ARGUMENT;
@@ -395,7 +406,9 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   // the lean kernel gives every wave its own piece of LDS for the K range it walks
   const bool wave_slab = lean && (cfg.wcol == 1 || rows <= 2);
   const int slab_stride = (wave_slab ? q4::max_wave_rows(gp) : KR) * 2 + 16;
-  const int rmax = rpb == 32 ? 8 : (M <= 1 ? 1 : (M <= 2 ? 2 : 4));
+  // accumulator rows per lane: rows 4 kq .. 4 kq + 3 of an MFMA block (AWQ words-as-stored
+  // kernel: rows kq, kq + 4, ..)
+  const int rmax = diag ? (rows <= 4 ? 1 : 2) : (rpb == 32 ? 8 : (M <= 1 ? 1 : (M <= 2 ? 2 : 4)));
   const int nt = awq ? 16 : cfg.words;
   const size_t slab_bytes = ((size_t)rows * slab_stride * (wave_slab ? cfg.wcol * cfg.wk : 1) + 15) & ~(size_t)15;
   size_t smem = slab_bytes + (lean ? 512 : 0);  // lean: a block of zeros behind the slab
@@ -439,7 +452,8 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.fixed_point_split = cfg.splits > 1 && cfg.splits <= 14 && dtype == Q4_DTYPE_F16 && gate_up_act == 0 &&
                          (nt >= 4 ? M <= kCellRowsMax : M == 1) && (size_t)M * w->N * 8 <= Q4_WORKSPACE_CELL_BYTES;
   if (gp.fixed_point_split && nt >= 4) {
-    const size_t tile = red + (size_t)cfg.wcol * (rmax < 4 ? rmax : kRowsPerBlock) * 16 * nt * sizeof(float);
+    const int tile_rows = diag ? (4 * rmax < kRowsPerBlock ? 4 * rmax : kRowsPerBlock) : (rmax < 4 ? rmax : kRowsPerBlock);
+    const size_t tile = red + (size_t)cfg.wcol * tile_rows * 16 * nt * sizeof(float);
     if (tile > smem) smem = tile;
   }
   const size_t smem_limit = 160 * 1024 - 1024;  // gfx950: 160 KB of LDS per workgroup
@@ -459,7 +473,9 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.wave_slab = wave_slab ? 1 : 0;
   dim3 grid((unsigned)(ntiles * cfg.splits), (unsigned)mchunks);
   dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
-  if (lean) {
+  if (diag) {
+    launch_gemv_awq_diag(gp, dtype, rmax, grid, block, smem, stream);
+  } else if (lean) {
     launch_gemv_lean(gp, dtype, rows <= 1 ? 1 : (rows <= 2 ? 2 : (rows <= 4 ? 4 : (rows <= 8 ? 8 : 16))), grid, block, smem,
                      stream);
   } else if (gate_up_act != 0) {

@@ -259,13 +259,19 @@ struct SlabStager {
 
 // Row (relative to the workgroup's first) of accumulator slot r of a lane: an MFMA row block
 // gives a lane rows 4*kq .. 4*kq + 3; slots 4..7 are the second block of 16 rows.
-__device__ __forceinline__ int out_row(const Decomp& d, int r) { return 4 * d.kq + (r & 3) + ((r >> 2) << 4); }
+// KQROWS (the AWQ kernel, whose MFMA rows are (activation row, column) pairs): lane block kq
+// holds rows kq, kq + 4, ..
+template <bool KQROWS = false>
+__device__ __forceinline__ int out_row(const Decomp& d, int r) {
+  if constexpr (KQROWS) return d.kq + 4 * r;
+  return 4 * d.kq + (r & 3) + ((r >> 2) << 4);
+}
 
 // Everything after the K loop.  out[t][r] is the fp32 sum of output row out_row(r) (relative
 // to the workgroup's first row) and column col0 + t: every lane owns NT adjacent columns.
 // FUSE (NT = 8): gated-MLP epilogue.  out[0..3] are four gate columns col0 .. col0 + 3 and
 // out[4..7] the matching up columns N/2 + col0 ..; the output is act(gate) * up, [M, N/2].
-template <int DTYPE, int NT, int RMAX, bool FUSE = false>
+template <int DTYPE, int NT, int RMAX, bool FUSE = false, bool KQROWS = false>
 __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& d,
                                             float (&out)[NT][RMAX], int col0,
                                             unsigned char* smem) {
@@ -301,7 +307,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
       if (d.wkk == 0) {
 #pragma unroll
         for (int r = 0; r < RMAX; ++r) {
-          const int m = out_row(d, r);
+          const int m = out_row<KQROWS>(d, r);
           if (m < d.mloc) {
             uint32_t o[NT / 2];
 #pragma unroll
@@ -324,7 +330,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
     if (d.wkk == 0) {
 #pragma unroll
       for (int r = 0; r < RMAX; ++r) {
-        const int m = out_row(d, r);
+        const int m = out_row<KQROWS>(d, r);
         if (m < d.mloc) {
           uint16_t* dst = y + (size_t)(d.mb + m) * N + col0;
           uint16_t o[NT];
@@ -371,13 +377,13 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
         // consecutive cells with all lanes active.  The tiles sit behind the K-wave partials.
         constexpr int PER_LANE = NT >= 4 ? NT / 4 : 1;  // 16 * NT columns over 64 lanes
         constexpr int TW = 16 * NT;
-        constexpr int TILE_ROWS = RMAX < 4 ? RMAX : kRowsPerBlock;
+        constexpr int TILE_ROWS = KQROWS ? (4 * RMAX < kRowsPerBlock ? 4 * RMAX : kRowsPerBlock) : (RMAX < 4 ? RMAX : kRowsPerBlock);
         if (gp.wk == 1 && gp.wcol > 1) __syncthreads();  // other column waves may still read the slab
         if (d.wkk == 0) {
           float* tile = (float*)smem + (size_t)(gp.wk - 1) * gp.wcol * NT * RMAX * 64 + (size_t)d.wc * TILE_ROWS * TW;
 #pragma unroll
           for (int r = 0; r < RMAX; ++r) {
-            const int m = out_row(d, r);
+            const int m = out_row<KQROWS>(d, r);
             if (m < d.mloc) {
 #pragma unroll
               for (int t = 0; t < NT; ++t) tile[m * TW + d.j * NT + t] = out[t][r];
@@ -415,7 +421,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
         unsigned long long* cells = gp.cells;
 #pragma unroll
         for (int r = 0; r < RMAX; ++r) {
-          const int m = out_row(d, r);
+          const int m = out_row<KQROWS>(d, r);
           if (m < d.mloc) {
             unsigned long long* cell = cells + (size_t)(d.mb + m) * N + col0;
             unsigned long long before[NT], inc[NT];
@@ -453,7 +459,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
   if (d.wkk == 0) {
 #pragma unroll
     for (int r = 0; r < RMAX; ++r) {
-      const int m = out_row(d, r);
+      const int m = out_row<KQROWS>(d, r);
       if (m < d.mloc) {
         float* dst = gp.partials + ((size_t)d.split * gp.partial_rows + d.mb + m) * N + col0;
 #pragma unroll
