@@ -403,6 +403,9 @@ def gptq_fasterquant(W, H, blocksize=128, percdamp=0.01, groupsize=-1, act_order
     W = np.array(W, dtype=np.float64)
     H = np.array(H, dtype=np.float64)
     rows, K = W.shape
+    # one group for all of K: the range comes from the weights as given, dead inputs included
+    # (quantizer.find_params(W) runs before the dead columns are cleared, quantize.py:257-264)
+    whole = gptq_find_params(W, sym) if groupsize == -1 else None
     dead = np.diag(H) == 0
     H[dead, dead] = 1.0
     W[:, dead] = 0.0
@@ -421,7 +424,7 @@ def gptq_fasterquant(W, H, blocksize=128, percdamp=0.01, groupsize=-1, act_order
     scale = np.zeros((rows, G))
     zero = np.zeros((rows, G))
     if groupsize == -1:
-        scale[:, 0], zero[:, 0] = gptq_find_params(W, sym)
+        scale[:, 0], zero[:, 0] = whole
     for i1 in range(0, K, blocksize):
         i2 = min(i1 + blocksize, K)
         Err = np.zeros((rows, i2 - i1))

@@ -569,3 +569,55 @@ def test_llama3_8b_shapes_size_independent_properties(pkg, oracle, gpu, K, N):
     assert float((ya - ga).abs().max()) <= 2e-3 * scale          # decode against prefill kernel
     yab = pkg.ops.linear(w, (a.float() * 0.5 + b.float() * 0.5).half(), path=1).float()
     assert float((yab - 0.5 * (ya + yb)).abs().max()) <= 4e-3 * scale  # linearity to input/output rounding
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
+@pytest.mark.parametrize("poison", ["+inf", "-inf", "nan", "+inf,-inf"])
+def test_decode_non_finite_activations_keep_their_class(pkg, oracle, gpu, M, poison):
+    """inf / NaN activations through split-K (accumulation cells up to 3 rows, tickets from 4):
+    every output is NaN, +inf or -inf exactly where fp32 arithmetic on the dequantized weights
+    gives that class, and the rows without poison stay finite and correct."""
+    K, N = 4096, 4096
+    qw, qz, sc, _ = oracle.make_gptq(K, N, 128, seed=77, sym=False)
+    w = oracle.dequant_gptq(qw, qz, sc, None, 128, "f16")
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
+    x = oracle.make_x(M, K, seed=M).copy()
+    vals = {"+inf": np.inf, "-inf": -np.inf, "nan": np.nan}
+    for i, name in enumerate(poison.split(",")):
+        x[M - 1, 100 + 1500 * i] = np.float16(vals[name])
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = x.astype(np.float32) @ w.astype(np.float32)
+    got = to_f32(pkg.ops.linear(pk, to_dev(x, gpu), None, path=1))
+    torch.cuda.synchronize()
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    assert np.array_equal(np.isposinf(got), np.isposinf(ref))
+    assert np.array_equal(np.isneginf(got), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    if fin.any():
+        assert np.abs(got[fin] - ref[fin]).max() <= TOL * np.abs(ref[fin]).max()
+    # a later clean call finds the cells and tickets as the kernels must leave them
+    xc = oracle.make_x(M, K, seed=M + 40)
+    clean = to_f32(pkg.ops.linear(pk, to_dev(xc, gpu), None, path=1))
+    assert np.isfinite(clean).all()
+    assert max_rel_err(clean, xc.astype(np.float32) @ w.astype(np.float32)) <= TOL
+
+
+@pytest.mark.parametrize("layout", ["gptq", "awq"])
+def test_decode_offset_kernels_stay_non_finite_on_poisoned_rows(pkg, oracle, gpu, layout):
+    """The kernels that keep the splice offsets in the sums (large GPTQ layers, AWQ up to 8 rows)
+    subtract inf from inf on a poisoned row: its outputs are non-finite (NaN where the reference
+    may say +-inf); other rows are untouched."""
+    K, N, M = 4096, 14336, 2
+    if layout == "gptq":
+        qw, qz, sc, _ = oracle.make_gptq(K, N, 128, seed=5)
+        w = oracle.dequant_gptq(qw, qz, sc, None, 128, "f16")
+    else:
+        qw, qz, sc = oracle.make_awq(K, N, 128, seed=5)
+        w = oracle.dequant_awq(qw, qz, sc, 128, "f16")
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0 if layout == "gptq" else 1)
+    x = oracle.make_x(M, K, seed=9).copy()
+    x[1, 333] = np.float16(np.inf)
+    got = to_f32(pkg.ops.linear(pk, to_dev(x, gpu), None, path=1))
+    assert not np.isfinite(got[1]).any()
+    assert np.isfinite(got[0]).all()
+    assert max_rel_err(got[0:1], x[0:1].astype(np.float32) @ w.astype(np.float32)) <= TOL

@@ -86,6 +86,23 @@ def test_oracle_dead_inputs_and_act_order_permutation(oracle):
     assert np.array_equal(g_idx[perm], np.arange(K) // 8)
 
 
+def test_oracle_whole_row_range_includes_dead_input_columns(oracle):
+    """groupsize -1: the row range is taken before dead columns are cleared (quantize.py:257-264),
+    so an extreme weight in a dead input column still sets the row's scale."""
+    rng = np.random.default_rng(4)
+    rows, K, n = 3, 16, 50
+    X = calib(rng, K, n)
+    X[:, 5] = 0.0
+    H = 2.0 / n * X.T @ X
+    W = rng.standard_normal((rows, K)) * 0.05
+    W[1, 5] = 3.0  # far outside the other weights of row 1
+    _, scale, zero, _, _, _, _ = oracle.gptq_fasterquant(W, H, blocksize=8, groupsize=-1, sym=False)
+    lo, hi = np.minimum(W.min(axis=1), 0), np.maximum(W.max(axis=1), 0)
+    assert np.allclose(scale[:, 0], (hi - lo) / 15)
+    assert scale[1, 0] > 0.19  # (3.0 - lo) / 15
+    assert np.array_equal(zero[:, 0], np.rint(-lo / scale[:, 0]))
+
+
 # --------------------------------------------------------------------------- GPU
 
 
@@ -133,6 +150,23 @@ def test_gpu_solver_identity_and_oracle_agreement(pkg, oracle, gpu, rows, K, gs,
     assert np.mean(lv == olv) >= 0.97
     assert abs(err - oerr) <= 2e-2 * oerr
     assert np.allclose(scale, oscale, rtol=2e-2, atol=1e-7) and np.mean(zero == ozero) >= 0.97
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sym", [True, False])
+def test_gpu_solver_whole_row_range_with_dead_input(pkg, oracle, gpu, sym):
+    """groupsize -1 with an all-zero calibration column that holds a row's extreme weight."""
+    rng = np.random.default_rng(12)
+    rows, K, n = 8, 128, 64
+    X = calib(rng, K, n)
+    X[:, 17] = 0.0
+    W = rng.standard_normal((rows, K)) * 0.05
+    W[2, 17] = 2.5
+    Q, scale, zero, _, _, H = _solve(pkg, gpu, W, X, -1, False, sym)
+    _, s_ref, z_ref, _, _, _, _ = oracle.gptq_fasterquant(W.astype(np.float32).astype(np.float64), H, groupsize=-1, sym=sym)
+    assert np.allclose(scale[:, 0], s_ref[:, 0], rtol=1e-6)
+    assert np.array_equal(zero[:, 0], z_ref[:, 0])
+    assert np.all(Q[:, 17] == 0.0)
 
 
 @pytest.mark.gpu

@@ -267,6 +267,33 @@ __device__ __forceinline__ int out_row(const Decomp& d, int r) {
   return 4 * d.kq + (r & 3) + ((r >> 2) << 4);
 }
 
+// 64-bit accumulation cell of the fixed-point split-K combine (up to 14 splits):
+//   bits 60..63  arrivals
+//   bits 55..58  arrivals whose partial sum was -inf or NaN
+//   bits 51..54  arrivals whose partial sum was +inf or NaN
+//   bits  0..50  sum of the finite partial sums, 28 fractional bits, two's complement running
+//                into the fields above (read back with a bias of 2^50)
+// A partial sum beyond +-2^17 (twice the largest fp16) counts as an infinity of its sign, so 14
+// finite ones stay below 2^49.  The combined value is NaN when both non-finite fields are set
+// (a NaN partial, or +inf meeting -inf), else +-inf when one is, else the fixed-point sum: what
+// fp32 addition of the partials gives in any order, as long as no partial leaves +-2^17 (one
+// that does makes the fp16 output infinite or, when such partials cancel, NaN).
+__device__ __forceinline__ unsigned long long cell_increment(float v) {
+  constexpr unsigned long long kArrival = 1ull << 60, kPos = 1ull << 51, kNeg = 1ull << 55;
+  if (fabsf(v) <= 131072.f) return kArrival + (unsigned long long)__float2ll_rn(v * 268435456.f);
+  return kArrival + (v < 0.f ? 0ull : kPos) + (v > 0.f ? 0ull : kNeg);  // NaN compares false both ways
+}
+__device__ __forceinline__ bool cell_complete(unsigned long long now, int splits) {
+  return (int)((now + (1ull << 50)) >> 60) == splits;
+}
+__device__ __forceinline__ float cell_value(unsigned long long now) {
+  const unsigned long long t = now + (1ull << 50);
+  const bool pos = ((t >> 51) & 15ull) != 0, neg = ((t >> 55) & 15ull) != 0;
+  const float f = (float)((long long)(t & ((1ull << 51) - 1)) - (1ll << 50)) * (1.0f / 268435456.f);
+  if (pos || neg) return pos && neg ? __builtin_nanf("") : (pos ? __builtin_inff() : -__builtin_inff());
+  return f;
+}
+
 // Everything after the K loop.  out[t][r] is the fp32 sum of output row out_row(r) (relative
 // to the workgroup's first row) and column col0 + t: every lane owns NT adjacent columns.
 // FUSE (NT = 8): gated-MLP epilogue.  out[0..3] are four gate columns col0 .. col0 + 3 and
@@ -356,19 +383,14 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
   }
 
   // ---- cross-workgroup split-K, fp16: one 64-bit atomic per output element and workgroup.
-  // The cell of an element accumulates the partial sums in fixed point (28 fractional bits,
-  // integer addition: the total does not depend on the arrival order) and, in its top byte,
-  // the number of arrivals.  The add returns the previous contents, so the workgroup that
-  // brings the count to `splits` holds the complete sum, writes the output and clears the
-  // cell: one memory round trip where partial store -> ticket -> re-read takes three.
-  // Finite partials are clamped to +-2^17 (twice the largest fp16) and a non-finite partial
-  // (inf or NaN activations) counts as +2^23, more than all finite partials of up to 14
-  // splits can cancel: the output is then +inf where the reference's would be inf or NaN.
-  // |sum| stays below 2^55 fixed-point units, clear of the count.  The cells must be zero
-  // before the first call; they are left zero.
+  // The cell of an element accumulates the partial sums in fixed point (integer addition: the
+  // total does not depend on the arrival order) next to the number of arrivals (cell_increment
+  // above).  The add returns the previous contents, so the workgroup that brings the count to
+  // `splits` holds the complete sum, writes the output and clears the cell: one memory round
+  // trip where partial store -> ticket -> re-read takes three.  The cells must be zero before
+  // the first call; they are left zero.
   if constexpr (DTYPE == Q4_DTYPE_F16 && !FUSE) {
     if (gp.fixed_point_split) {
-      constexpr unsigned long long kOne = 1ull << 56, kHalf = 1ull << 55;
       if constexpr (NT >= 4) {
         // A row's sums sit in the 16 lanes of one K block, NT adjacent columns each: issued
         // from there, an atomic instruction touches 16 separate groups of cells (with the AWQ
@@ -397,19 +419,15 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
             unsigned long long before[PER_LANE], inc[PER_LANE];
 #pragma unroll
             for (int u = 0; u < PER_LANE; ++u) {
-              const float v = tile[m * TW + d.lane + 64 * u];
-              long long q = 1ll << 51;  // non-finite
-              if (fabsf(v) <= 3.0e38f) q = __float2ll_rn(fminf(fmaxf(v, -131072.f), 131072.f) * 268435456.f);
-              inc[u] = kOne + (unsigned long long)q;
+              inc[u] = cell_increment(tile[m * TW + d.lane + 64 * u]);
               before[u] = __hip_atomic_fetch_add(cell + 64 * u, inc[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
 #pragma unroll
             for (int u = 0; u < PER_LANE; ++u) {
               const unsigned long long now = before[u] + inc[u];
-              if ((long long)(now + kHalf) >> 56 == (long long)gp.splits) {
-                const long long sum = (long long)(now - ((unsigned long long)gp.splits << 56));
+              if (cell_complete(now, gp.splits)) {
                 const int n = nbase + d.lane + 64 * u;
-                y[(size_t)(d.mb + m) * N + n] = finish_output<DTYPE>((float)sum * (1.0f / 268435456.f), p.bias, n);
+                y[(size_t)(d.mb + m) * N + n] = finish_output<DTYPE>(cell_value(now), p.bias, n);
                 __hip_atomic_store(cell + 64 * u, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
               }
             }
@@ -427,19 +445,14 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
             unsigned long long before[NT], inc[NT];
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-              const float v = out[t][r];
-              long long q = 1ll << 51;  // non-finite
-              if (fabsf(v) <= 3.0e38f) q = __float2ll_rn(fminf(fmaxf(v, -131072.f), 131072.f) * 268435456.f);
-              inc[t] = kOne + (unsigned long long)q;
+              inc[t] = cell_increment(out[t][r]);
               before[t] = __hip_atomic_fetch_add(cell + t, inc[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
               const unsigned long long now = before[t] + inc[t];
-              if ((long long)(now + kHalf) >> 56 == (long long)gp.splits) {
-                const long long sum = (long long)(now - ((unsigned long long)gp.splits << 56));
-                y[(size_t)(d.mb + m) * N + col0 + t] =
-                    finish_output<DTYPE>((float)sum * (1.0f / 268435456.f), p.bias, col0 + t);
+              if (cell_complete(now, gp.splits)) {
+                y[(size_t)(d.mb + m) * N + col0 + t] = finish_output<DTYPE>(cell_value(now), p.bias, col0 + t);
                 __hip_atomic_store(cell + t, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
               }
             }

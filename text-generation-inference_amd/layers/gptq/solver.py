@@ -55,6 +55,10 @@ class GPTQ:
             raise ValueError(f"blocksize must be 1..{BLOCK}, got {blocksize}")
         K, rows = self.columns, self.rows
         W = self.layer.weight.data.clone().float().contiguous()
+        # one group for all of K: the row ranges come from the weights as given, before the
+        # columns of dead inputs are cleared (quantize.py:257-264)
+        row_lo = W.min(dim=1).values if groupsize == -1 else None
+        row_hi = W.max(dim=1).values if groupsize == -1 else None
         H = self.H.clone()
         dead = torch.diag(H) == 0
         H[dead, dead] = 1
@@ -84,8 +88,8 @@ class GPTQ:
         err = torch.zeros((rows, BLOCK), device=self.dev, dtype=torch.float32)
         if groupsize == -1:
             # one range per row, from the weights as they are before any column is quantized
-            lo = torch.clamp(W.min(dim=1).values, max=0)
-            hi = torch.clamp(W.max(dim=1).values, min=0)
+            lo = torch.clamp(row_lo, max=0)
+            hi = torch.clamp(row_hi, min=0)
             if self.sym:
                 hi = torch.maximum(lo.abs(), hi)
                 lo = torch.where(lo < 0, -hi, lo)
