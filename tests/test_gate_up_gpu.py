@@ -86,7 +86,8 @@ def test_activations_decode_and_prefill(pkg, oracle, gpu, act, dtype):
         x = oracle.make_x(M, K, seed=9, dtype=dtype)
         _, want = oracle.gate_up_forward(x, w, oracle_act, None, dtype)
         pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, gs, 0)
-        # decode sizes run the fused kernel, prefill sizes the GEMM + elementwise kernel
+        # decode sizes run the fused decode kernel; this prefill size splits K (few tiles) and
+        # takes the GEMM + elementwise kernel
         got = to_f32(pkg.ops.linear_gate_up(pk, to_dev(x, gpu, bf16=bf), act, fused=True if M == 2 else None))
         assert max_rel_err(got, oracle.to_f32(want, dtype)) <= (TOL_BF16 if bf else TOL)
 
@@ -103,9 +104,41 @@ def test_prefill_bf16_groupsize_64(pkg, oracle, gpu):
     _case(pkg, oracle, gpu, 2048, 1024, 64, 640, dtype="bf16", seed=4)
 
 
-def test_prefill_sizes_have_no_fused_kernel(pkg, oracle, gpu):
+def test_prefill_fused_kernel_where_k_is_not_split(pkg, oracle, gpu):
+    """Enough tiles to run unsplit: the MFMA kernel with the gated epilogue; a small grid that
+    splits K keeps the two-kernel route and refuses `fused=True`."""
+    _case(pkg, oracle, gpu, 1024, 4096, 128, 2048, fused=True, seed=1)
+    _case(pkg, oracle, gpu, 1024, 4096, 128, 2048, fused=True, bias=True, act="gelu", seed=2)
+    _case(pkg, oracle, gpu, 1024, 4096, 128, 512, fused=True, dtype="bf16", seed=3)
     with pytest.raises(pkg._lib.Q4Error):
-        _case(pkg, oracle, gpu, 1024, 4096, 128, 2048, fused=True, seed=1)
+        _case(pkg, oracle, gpu, 4096, 512, 128, 128, fused=True, seed=1)
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu_tanh", "gelu"])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("K,N,gs,M,bitwise", [(4096, 28672, 128, 2048, True), (4096, 28672, 128, 777, True),
+                                              (2048, 8192, 64, 1024, False), (512, 65536, 256, 64, True),
+                                              (512, 65536, 128, 33, True)])
+def test_prefill_fused_equals_two_kernels_bitwise(pkg, oracle, gpu, act, dtype, K, N, gs, M, bitwise):
+    """Same MFMA sequence per column, same roundings, same activation routine: the fused
+    epilogue and GEMM + act_mul agree bit for bit (ragged last row tile included).  Where the
+    plain GEMM of the two-kernel route runs with two K groups per workgroup (a grid of one
+    workgroup per CU) its summation order differs: compared to the parity bar there."""
+    bf = dtype == "bf16"
+    qw, qz, sc, _ = oracle.make_gptq(K, N, gs, seed=M, sym=False)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, gs, 0)
+    x = to_dev(oracle.make_x(M, K, seed=M + 1, dtype=dtype), gpu, bf16=bf)
+    rng = np.random.default_rng(M)
+    b32 = rng.standard_normal(N).astype(np.float32)
+    b = to_dev(b32.astype(np.float16) if not bf else oracle.f32_to_bf16_bits(b32), gpu, bf16=bf)
+    for bias in (None, b):
+        one = pkg.ops.linear_gate_up(pk, x, act, bias, fused=True)
+        two = pkg.ops.linear_gate_up(pk, x, act, bias, fused=False)
+        torch.cuda.synchronize()
+        if bitwise:
+            assert torch.equal(one.view(torch.int16), two.view(torch.int16))
+        else:
+            assert max_rel_err(to_f32(one), to_f32(two)) <= (TOL_BF16 if bf else TOL)
 
 
 @pytest.mark.parametrize("layout,act_order", [("awq", False), ("gptq", True)])

@@ -534,7 +534,14 @@ def test_act_order_dispatch(pkg, oracle, gpu):
     assert pkg.ops.select_path(pk, 16) == "gemv"
     assert pkg.ops.select_path(pk, 1024) == "gemm"
     assert pkg.ops.select_path(pk, 1024, torch.bfloat16) == "gemm"
-    assert pkg.ops.select_path(pk, 4, torch.bfloat16) == "generic"  # the act-order decode kernel is fp16 only
+    assert pkg.ops.select_path(pk, 4, torch.bfloat16) == "gemm"  # the act-order decode kernel is fp16 only
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("K,N", [(1024, 1024), (8192, 10240)])
+def test_act_order_bf16_small_m(pkg, oracle, gpu, K, N, M):
+    """g_idx with bf16 activations at decode sizes: the MFMA kernel that reads through g_idx."""
+    _run(pkg, oracle, gpu, K, N, 128, M, dtype="bf16", act=True, seed=M + 2)
 
 
 # --------------------------------------------------------------------------- full-size properties

@@ -128,7 +128,8 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   }
   if (!small && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
   if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
-  if (M > 16 && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
+  // (act-order with bf16 activations has no decode kernel: the MFMA kernel takes any M)
+  if (gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
   return Q4_PATH_GENERIC;
 }
 
@@ -346,6 +347,20 @@ int q4_linear_gate_up_perm(const q4_weight* w, const int32_t* perm, const void* 
     set_error("q4_linear_gate_up_perm: null x or y");
     return Q4_ERR_INVALID_ARGUMENT;
   }
+  if (q4_select_path(w, M, dtype) == Q4_PATH_GEMM && gemm_gate_up_supported(w, M, dtype)) {
+    // prefill: gather the activation columns into the workspace tail, then the fused MFMA kernel
+    const size_t offset = perm_gather_offset(M, w->K, w->N);
+    const size_t need = offset + (size_t)M * w->K * 2;
+    if (workspace == nullptr || workspace_bytes < need || w->K % 8 != 0) {
+      set_error("q4_linear_gate_up_perm: workspace of %zu bytes needed (q4_workspace_bytes_perm), %zu given", need,
+                workspace_bytes);
+      return Q4_ERR_WORKSPACE;
+    }
+    void* x_seq = (char*)workspace + offset;
+    rc = launch_gather_columns(x, perm, x_seq, M, w->K, (hipStream_t)stream);
+    if (rc != Q4_OK) return rc;
+    return launch_gemm_gate_up(w, x_seq, bias, y, M, dtype, act, (hipStream_t)stream);
+  }
   if (!(q4_select_path(w, M, dtype) == Q4_PATH_GEMV && gemv_gate_up_supported(w, M, dtype))) {
     set_error("q4_linear_gate_up_perm: no fused kernel for this problem (M=%d K=%d N=%d groupsize=%d)", M, w->K, w->N,
               w->groupsize);
@@ -385,13 +400,13 @@ int q4_linear_gate_up(const q4_weight* w, const void* x, const void* bias, void*
     set_error("q4_linear_gate_up: null x or y");
     return Q4_ERR_INVALID_ARGUMENT;
   }
-  // Fused on the decode path only.  In the prefill GEMM the exp / tanh of a 256 x 256 tile
-  // would run with the matrix cores idle and the lane's gate and up columns are no longer
-  // neighbours in memory; measured slower (571 us against 476 + 36 us for the Llama-3-8B
-  // gate_up projection at M = 2048) than the GEMM followed by q4_act_mul, so the caller gets
-  // Q4_ERR_UNSUPPORTED there and runs the two kernels.
-  if (q4_select_path(w, M, dtype) == Q4_PATH_GEMV && gemv_gate_up_supported(w, M, dtype))
+  // Decode: the kernels with eight words per lane.  Prefill: the MFMA kernel with a lane's two
+  // columns set to (gate c, up c), where it runs unsplit.
+  const int path = q4_select_path(w, M, dtype);
+  if (path == Q4_PATH_GEMV && gemv_gate_up_supported(w, M, dtype))
     return launch_gemv(w, x, bias, y, M, dtype, workspace, workspace_bytes, nullptr, (hipStream_t)stream, act + 1);
+  if (path == Q4_PATH_GEMM && gemm_gate_up_supported(w, M, dtype))
+    return launch_gemm_gate_up(w, x, bias, y, M, dtype, act, (hipStream_t)stream);
   set_error("q4_linear_gate_up: no fused kernel for this problem (layout=%d g_idx=%p M=%d K=%d N=%d groupsize=%d)",
             w->layout, (const void*)w->g_idx, M, w->K, w->N, w->groupsize);
   return Q4_ERR_UNSUPPORTED;

@@ -107,8 +107,25 @@ __device__ __forceinline__ uint16_t finish_output(float acc, const void* bias, i
 // evaluated in fp32 and rounded, then the product is rounded):
 // server/text_generation_server/models/custom_modeling/flash_llama_modeling.py:400-404.
 // `act` is a Q4_ACT_* value.
-template <int DTYPE>
-__device__ __forceinline__ uint16_t act_mul(uint16_t g_bits, uint16_t u_bits, int act) {
+// ACT is a Q4_ACT_* value.  silu and the tanh form of gelu are both g * sigmoid(t) (t = g, or
+// t = 2 * sqrt(2/pi) * (g + 0.044715 g^3): 0.5 * (1 + tanh(t/2)) is sigmoid(t), without the
+// cancellation of 1 + tanh for negative inputs); the exponential and the reciprocal are the
+// hardware ones (about 1 ulp each in fp32, far inside the half rounding that follows).
+template <int ACT>
+__device__ __forceinline__ float act_value(float g) {
+  if constexpr (ACT == Q4_ACT_GELU) {
+    return 0.5f * g * (1.0f + erff(g * 0.7071067811865476f));
+  } else {
+    // (written so that no multiply-add pair is left to the compiler's choice of contraction:
+    // every kernel that inlines this rounds alike)
+    float t = g;
+    if constexpr (ACT == Q4_ACT_GELU_TANH) t = (1.5957691216057308f * g) * __builtin_fmaf(0.044715f, g * g, 1.0f);
+    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * t));
+  }
+}
+
+template <int DTYPE, int ACT>
+__device__ __forceinline__ uint16_t act_mul_as(uint16_t g_bits, uint16_t u_bits) {
   float g, u;
   if constexpr (DTYPE == Q4_DTYPE_F16) {
     g = (float)__builtin_bit_cast(half_t, g_bits);
@@ -117,20 +134,24 @@ __device__ __forceinline__ uint16_t act_mul(uint16_t g_bits, uint16_t u_bits, in
     g = bf16_bits_to_f32(g_bits);
     u = bf16_bits_to_f32(u_bits);
   }
-  float a;
-  if (act == Q4_ACT_SILU) {
-    a = g / (1.0f + expf(-g));
-  } else if (act == Q4_ACT_GELU_TANH) {
-    const float inner = 0.7978845608028654f * (g + 0.044715f * g * g * g);
-    a = 0.5f * g * (1.0f + tanhf(inner));
-  } else {
-    a = 0.5f * g * (1.0f + erff(g * 0.7071067811865476f));
-  }
+  // The activation is rounded to fp32 and then to the half type, as an fp32 routine followed
+  // by a cast does.  The empty asm keeps the compiler from folding the last multiply and the
+  // cast into one mixed-precision multiply-add, which rounds once (and loses the sign of a
+  // zero): every kernel that inlines this then gives the same bits.
+  float a = act_value<ACT>(g);
+  asm("" : "+v"(a));
   const uint16_t a_bits = store_act<DTYPE>(a);
   float ar;
   if constexpr (DTYPE == Q4_DTYPE_F16) ar = (float)__builtin_bit_cast(half_t, a_bits);
   else ar = bf16_bits_to_f32(a_bits);
   return store_act<DTYPE>(ar * u);
+}
+
+template <int DTYPE>
+__device__ __forceinline__ uint16_t act_mul(uint16_t g_bits, uint16_t u_bits, int act) {
+  if (act == Q4_ACT_SILU) return act_mul_as<DTYPE, Q4_ACT_SILU>(g_bits, u_bits);
+  if (act == Q4_ACT_GELU_TANH) return act_mul_as<DTYPE, Q4_ACT_GELU_TANH>(g_bits, u_bits);
+  return act_mul_as<DTYPE, Q4_ACT_GELU>(g_bits, u_bits);
 }
 
 // Kernel-side view of q4_weight plus the activation-side pointers.
@@ -204,6 +225,9 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
                 int gate_up_act = 0, const int32_t* x_perm = nullptr);
 bool gemv_gate_up_supported(const q4_weight* w, int M, int dtype);
 int launch_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, hipStream_t stream);
+bool gemm_gate_up_supported(const q4_weight* w, int M, int dtype);
+int launch_gemm_gate_up(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype, int act,
+                        hipStream_t stream);
 int launch_make_sequential(const uint32_t* qweight, const int32_t* perm, uint32_t* out, int K, int N, hipStream_t stream);
 int launch_gather_columns(const void* x, const int32_t* perm, void* out, int M, int K, hipStream_t stream);
 int launch_gptq_solve_block(float* W, const float* U, float* Q, float* Err, float* loss, float* scale, float* zero,

@@ -43,6 +43,15 @@ static void launch_tile(const GemmParams& gp, int gs, dim3 grid, size_t smem, hi
   }
 }
 
+// gated-MLP epilogue: 128 gate + 128 up columns per workgroup, groups of at least 64 rows
+template <int DTYPE, int BM>
+static void launch_tile_fused(const GemmParams& gp, dim3 grid, size_t smem, hipStream_t stream) {
+  auto k = q4::gemm_gptq_kernel<DTYPE, BM, 1, 2, false, 1, true>;
+  if (smem > 64 * 1024)
+    (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  hipLaunchKernelGGL(k, grid, dim3(256), smem, stream, gp);
+}
+
 // Tile shape and split factor for a problem; shared by the launcher and the workspace sizing.
 struct GemmPlan {
   int bm, nw, splits;
@@ -132,6 +141,50 @@ size_t gemm_workspace_bytes(int M, int K, int N) {
     if (other > splits) splits = other;
   }
   return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+}
+
+// The prefill kernel with the gated-MLP epilogue: one launch where the plain kernel would run
+// unsplit (the fused tile cannot leave partial sums), groups of at least 64 rows.
+bool gemm_gate_up_supported(const q4_weight* w, int M, int dtype) {
+  if (!gemm_supported(w, M, dtype) || w->N % 512 != 0 || w->groupsize < 64) return false;
+  const GemmPlan g = gemm_plan(M, w->K, w->N);
+  return g.splits == 1 && g.nw == 2 && g.bm <= 128;
+}
+
+int launch_gemm_gate_up(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype, int act,
+                        hipStream_t stream) {
+  using namespace q4;
+  if (!gemm_gate_up_supported(w, M, dtype)) {
+    set_error("q4_linear_gate_up(gemm): no fused prefill kernel for this problem (M=%d K=%d N=%d groupsize=%d)", M, w->K,
+              w->N, w->groupsize);
+    return Q4_ERR_UNSUPPORTED;
+  }
+  GemmParams gp;
+  gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, nullptr, x, bias, y,
+                 M,          w->K,      w->N,                     w->groupsize, w->num_groups};
+  gp.p.gate_up_act = act + 1;
+  gp.moe = q4::MoeView{};
+  gp.partial_rows = M;
+  gp.splits = 1;
+  gp.partials = nullptr;
+  const GemmPlan g = gemm_plan(M, w->K, w->N);
+  size_t smem = 2 * (size_t)g.bm * kAUnitsPerRow * 16;
+  const size_t exchange = (size_t)4 * (g.bm / 32) * 16 * 64 * 4;  // every wave's rounded tile
+  if (exchange > smem) smem = exchange;
+  dim3 grid((unsigned)g.tiles);
+  if (dtype == Q4_DTYPE_F16) {
+    if (g.bm == 64) launch_tile_fused<Q4_DTYPE_F16, 64>(gp, grid, smem, stream);
+    else launch_tile_fused<Q4_DTYPE_F16, 128>(gp, grid, smem, stream);
+  } else {
+    if (g.bm == 64) launch_tile_fused<Q4_DTYPE_BF16, 64>(gp, grid, smem, stream);
+    else launch_tile_fused<Q4_DTYPE_BF16, 128>(gp, grid, smem, stream);
+  }
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    set_error("q4_linear_gate_up(gemm): launch failed: %s", hipGetErrorString(err));
+    return Q4_ERR_LAUNCH;
+  }
+  return Q4_OK;
 }
 
 int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,

@@ -126,9 +126,14 @@ __device__ __forceinline__ float16_t mfma32(const uint4_t a, const uint4_t b, fl
 // activation buffers in LDS; the two accumulator sets meet through LDS at the end.  A grid of
 // one workgroup per CU then runs two waves per SIMD (one wave's fragment reads and unpacking
 // under the other's MFMAs) without any partial tile going through memory.
-template <int DTYPE, int BM, int GPT, int NW, bool MOE = false, int KG = 1>
+// FUSE: the weight packs [gate | up] and the output is act(gate) * up, [M, N/2].  A workgroup
+// covers 128 gate columns (waves 0, 1) and the 128 up columns that go with them (waves 2, 3):
+// the K loop is the plain one, at the end the up waves hand their rounded tile to the gate
+// waves through LDS (the activation tiles are dead by then).
+template <int DTYPE, int BM, int GPT, int NW, bool MOE = false, int KG = 1, bool FUSE = false>
 __global__ __launch_bounds__(256 * KG, (KG == 2 ? 1 : BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm_gptq_kernel(GemmParams gp) {
   static_assert(KG == 1 || (KG == 2 && !MOE && BM <= 128), "two K groups: dense launches, at most 128 rows");
+  static_assert(!FUSE || (NW == 2 && KG == 1 && !MOE), "gated epilogue: two columns per lane, dense launches, one K group");
   int moe_row0 = 0;
   if constexpr (MOE) {
     moe_row0 = moe_enter(gp.p, gp.moe, blockIdx.y);
@@ -183,8 +188,10 @@ __global__ __launch_bounds__(256 * KG, (KG == 2 ? 1 : BM == 64 ? 3 : BM == 128 ?
   }
   const int m0 = tm * BM;
   const int n0 = tn * BN;
-  const int nw = n0 + wave * 32 * NW;  // first column of this wave
-  const int ncol = nw + NW * j;        // first of this lane's NW columns
+  const int up_off = N >> 1;  // FUSE: first up column
+  // first column of this wave
+  const int nw = FUSE ? (n0 >> 1) + (wave & 1) * 32 * NW + (wave >> 1) * up_off : n0 + wave * 32 * NW;
+  const int ncol = nw + NW * j;  // first of this lane's NW columns
 
   const SpliceK splice = gemm_splice_consts();
   const int KT_all = K / kBK;
@@ -460,6 +467,37 @@ __global__ __launch_bounds__(256 * KG, (KG == 2 ? 1 : BM == 64 ? 3 : BM == 128 ?
     }
     return o;
   };
+  if constexpr (FUSE) {
+    // act(gate) * up on the rounded halves (what the two-kernel route computes).  Every wave
+    // leaves its tile in LDS, two halves per word, under (wave, row tile, register, lane); then
+    // all threads walk the gate words, each with the up word 2 waves further on.
+    constexpr int WORDS = 2 * MT * 16 * 64;  // gate words of the workgroup (as many up words)
+    uint32_t* xch = (uint32_t*)smem;
+    __syncthreads();  // every wave is done with the activation tiles
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        xch[((wave * MT + mt) * 16 + r) * 64 + lane] = finish(acc[mt][0][r], bias_f[0]) | (finish(acc[mt][1][r], bias_f[1]) << 16);
+    __syncthreads();
+    auto product = [&](auto act_c) {
+      constexpr int ACT = decltype(act_c)::value;
+#pragma unroll 4
+      for (int idx = tid; idx < WORDS; idx += 256) {
+        const uint32_t g = xch[idx], u = xch[idx + WORDS];
+        const int ln = idx & 63, rr = (idx >> 6) & 15, mtt = (idx >> 10) % MT, wv = idx / (1024 * MT);
+        const int m = m0 + mtt * 32 + 8 * (rr >> 2) + 4 * (ln >> 5) + (rr & 3);
+        const uint32_t lo = act_mul_as<DTYPE, ACT>((uint16_t)(g & 0xFFFFu), (uint16_t)(u & 0xFFFFu));
+        const uint32_t hi = act_mul_as<DTYPE, ACT>((uint16_t)(g >> 16), (uint16_t)(u >> 16));
+        if (m < M) *(uint32_t*)(y + (size_t)m * up_off + (n0 >> 1) + wv * 64 + 2 * (ln & 31)) = lo | (hi << 16);
+      }
+    };
+    const int act = p.gate_up_act - 1;
+    if (act == Q4_ACT_SILU) product(std::integral_constant<int, Q4_ACT_SILU>{});
+    else if (act == Q4_ACT_GELU_TANH) product(std::integral_constant<int, Q4_ACT_GELU_TANH>{});
+    else product(std::integral_constant<int, Q4_ACT_GELU>{});
+    return;
+  }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
