@@ -506,6 +506,23 @@ def main():
                 gm[name]["dense_fp16_matmul_TFLOPs"] = round(fl / davg / 1e12, 1)
                 del dense
             del xg, yg
+        # gated MLP first half (gate_up projection + act(gate) * up): one fused launch against
+        # the GEMM followed by the elementwise kernel, fp16
+        gated = None
+        if "gate_up_proj" in gm:
+            name, K, N = SHAPES[2]
+            xg = torch.randn((Mg, K), device=dev, dtype=torch.float16)
+            yh = torch.empty((Mg, N // 2), device=dev, dtype=torch.float16)
+            gated = {"shape": f"{K}x{N}", "M": Mg}
+            for key, fused in (("fused_us", True), ("gemm_plus_act_mul_us", False)):
+                try:
+                    fns = [(lambda c=c: pkg.ops.linear_gate_up(weights[c][2], xg, "silu", None, out=yh, fused=fused))
+                           for c in range(copies)]
+                    avg, _ = time_kernel_launches(torch, fns, 20)
+                    gated[key] = round(avg * 1e6, 1)
+                except pkg._lib.Q4Error:
+                    gated[key] = None
+            del xg, yh
         power = None
         if gm and not args.no_dense_ref:
             # What bounds the GEMM: the same kernel (and the vendor library's dense GEMM) on all-zero
@@ -533,6 +550,7 @@ def main():
                              "frac": round(tot_f / tot_t / 1e12 / MFMA_PEAK_TFLOPS, 4),
                              "traffic": measured_traffic(f"gemm_m{Mg}")},
                 "power_probe": power,
+                "gated_mlp": gated,
             }
 
     # ---- batched decode: the same four projections with more activation rows (the serving
