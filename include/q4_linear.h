@@ -155,6 +155,9 @@ int q4_linear_gate_up_perm(const q4_weight* w, const int32_t* perm, const void* 
  * of the block.  W itself is not written; the caller follows with
  * W[:, i1+count:] -= err @ U[i1:i1+count, i1+count:].  groupsize <= 0: scale / zero [rows]
  * are given; else they are [rows, num_groups] and the groups starting in the block are written.
+ * sym: bit 0 = symmetric range; bit 1 = the parameters of the groups that start in the block
+ * are given too (the caller found them, e.g. with the quantizer's mse search, :101-123, from
+ * W as it is when the block starts) and the kernel only reads them.
  */
 int q4_gptq_solve_block(float* W, const float* U, float* Q, float* err, float* loss, float* scale, float* zero,
                         int rows, int K, int i1, int count, int groupsize, int num_groups, int sym, void* stream);

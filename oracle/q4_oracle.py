@@ -370,9 +370,16 @@ def moe_forward(x, gating, gate_up_w, down_w, topk, renormalize=True, act="silu"
 # --------------------------------------------------------------------------- synthetic inputs
 
 
-def gptq_find_params(x, sym):
-    """Range rule of the reference's quantizer with mse off (quantize.py:60-101): per row of x
-    (float64), the range always contains 0; sym mirrors it; an all-zero row gets [-1, 1].
+def _gptq_round(x, scale, zero):
+    """Quantizer._quantize (quantize.py:54-58): scale * (clamp(round(x / scale) + zero, 0, 15) - zero)."""
+    return scale * (np.clip(np.rint(x / scale) + zero, 0, 15) - zero)
+
+
+def gptq_find_params(x, sym, mse=False, norm=2.4, grid=100, maxshrink=0.8):
+    """Range rule of the reference's quantizer (quantize.py:60-130): per row of x (float64), the
+    range always contains 0; sym mirrors it; an all-zero row gets [-1, 1].  With mse the range
+    is shrunk by p = 1 - i / grid for i = 0 .. maxshrink * grid - 1 and a row keeps the first
+    candidate with the smallest sum of |quantized - x| ** norm (:101-123; sym keeps zero = 8).
     Returns (scale, zero) per row, 4 bits."""
     x = np.asarray(x, dtype=np.float64)
     lo = np.minimum(x.min(axis=1), 0.0)
@@ -385,10 +392,22 @@ def gptq_find_params(x, sym):
     hi = np.where(dead, 1.0, hi)
     scale = (hi - lo) / 15.0
     zero = np.full_like(scale, 8.0) if sym else np.rint(-lo / scale)
+    if mse:
+        best = np.full(x.shape[0], np.inf)
+        zero0 = zero.copy()
+        for i in range(int(maxshrink * grid)):
+            p = 1 - i / grid
+            scale1 = (p * hi - p * lo) / 15.0
+            zero1 = zero0 if sym else np.rint(-(p * lo) / scale1)
+            err = np.sum(np.abs(_gptq_round(x, scale1[:, None], zero1[:, None]) - x) ** norm, axis=1)
+            better = err < best
+            best = np.where(better, err, best)
+            scale = np.where(better, scale1, scale)
+            zero = np.where(better, zero1, zero)
     return scale, zero
 
 
-def gptq_fasterquant(W, H, blocksize=128, percdamp=0.01, groupsize=-1, act_order=False, sym=True):
+def gptq_fasterquant(W, H, blocksize=128, percdamp=0.01, groupsize=-1, act_order=False, sym=True, mse=False):
     """The GPTQ solver in float64, column by column (quantize.py:243-351).
 
     W [rows, K] (one row per output feature), H [K, K] the accumulated Hessian 2/n X X^T.
@@ -405,7 +424,7 @@ def gptq_fasterquant(W, H, blocksize=128, percdamp=0.01, groupsize=-1, act_order
     rows, K = W.shape
     # one group for all of K: the range comes from the weights as given, dead inputs included
     # (quantizer.find_params(W) runs before the dead columns are cleared, quantize.py:257-264)
-    whole = gptq_find_params(W, sym) if groupsize == -1 else None
+    whole = gptq_find_params(W, sym, mse) if groupsize == -1 else None
     dead = np.diag(H) == 0
     H[dead, dead] = 1.0
     W[:, dead] = 0.0
@@ -433,7 +452,7 @@ def gptq_fasterquant(W, H, blocksize=128, percdamp=0.01, groupsize=-1, act_order
             g = i // gs
             if groupsize != -1 and i % gs == 0:
                 # from W, which has the updates of finished blocks only (quantize.py:308-312)
-                scale[:, g], zero[:, g] = gptq_find_params(W[:, i:i + gs], sym)
+                scale[:, g], zero[:, g] = gptq_find_params(W[:, i:i + gs], sym, mse)
             w = W1[:, i - i1]
             d = U[i, i]
             q = scale[:, g] * (np.clip(np.rint(w / scale[:, g]) + zero[:, g], 0, 15) - zero[:, g])

@@ -26,6 +26,7 @@ struct SolveParams {
   int rows, K, i1, count;
   int groupsize;                  // <= 0: one set of parameters per row, already in scale / zero
   int G, sym;
+  int given;                      // groups starting in the block: parameters already in scale / zero
 };
 
 __device__ __forceinline__ float wave_min(float v) {
@@ -72,7 +73,10 @@ __global__ __launch_bounds__(64 * kSolveWaves) void gptq_solve_block_kernel(Solv
   }
   for (int i = 0; i < count; ++i) {
     const int col = sp.i1 + i;
-    if (gs > 0 && col % gs == 0) {
+    if (gs > 0 && col % gs == 0 && sp.given) {
+      scale = sp.scale[(size_t)row * sp.G + col / gs];
+      zero = sp.zero[(size_t)row * sp.G + col / gs];
+    } else if (gs > 0 && col % gs == 0) {
       // range of the group's values: the block's part as it was at block entry, the rest from W
       const int end = min(col + gs, K);       // one past the group's last column
       const int in_block = min(end - sp.i1, count);
@@ -127,7 +131,7 @@ namespace q4host {
 
 int launch_gptq_solve_block(float* W, const float* U, float* Q, float* Err, float* loss, float* scale, float* zero,
                             int rows, int K, int i1, int count, int groupsize, int G, int sym, hipStream_t stream) {
-  q4::SolveParams sp{W, U, Q, Err, loss, scale, zero, rows, K, i1, count, groupsize, G, sym};
+  q4::SolveParams sp{W, U, Q, Err, loss, scale, zero, rows, K, i1, count, groupsize, G, sym & 1, (sym >> 1) & 1};
   const size_t smem = (size_t)count * q4::kSolveBlock * sizeof(float);
   if (smem > 64 * 1024)
     (void)hipFuncSetAttribute((const void*)q4::gptq_solve_block_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
