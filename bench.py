@@ -536,8 +536,17 @@ def main():
             zavg, _ = time_kernel_launches(torch, [(lambda c=c: pkg.ops.linear(wz[c], xz, None, out=yz)) for c in range(2)], 20)
             dz = [torch.zeros((K, N), device=dev, dtype=torch.float16) for _ in range(2)]
             dzavg, _ = time_kernel_launches(torch, [(lambda c=c: torch.matmul(xz, dz[c], out=yz)) for c in range(2)], 20)
+            # in between: real activations, weights whose dequantized values are small integers
+            # (all scales 1.0: few mantissa bits switch in the B operand)
+            wi = [make_weights(pkg, torch, dev, K, N, seed=950 + c) for c in range(2)]
+            for w in wi:
+                w.scales.fill_(1.0)
+            xr = torch.randn((Mg, K), device=dev, dtype=torch.float16)
+            iavg, _ = time_kernel_launches(torch, [(lambda c=c: pkg.ops.linear(wi[c], xr, None, out=yz)) for c in range(2)], 20)
+            del wi, xr
             fl = 2.0 * Mg * N * K
             power = {"shape": name, "zero_operands_TFLOPs": round(fl / zavg / 1e12, 1),
+                     "unit_scale_weights_random_activations_TFLOPs": round(fl / iavg / 1e12, 1),
                      "random_operands_TFLOPs": gm[name]["TFLOPs"],
                      "dense_fp16_matmul_zero_operands_TFLOPs": round(fl / dzavg / 1e12, 1),
                      "dense_fp16_matmul_random_operands_TFLOPs": gm[name].get("dense_fp16_matmul_TFLOPs")}
