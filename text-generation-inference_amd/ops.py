@@ -218,8 +218,35 @@ def gather_columns(x: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:
     return out
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_handle(device: torch.device) -> int:
+    """The current HIP stream of `device` as an integer handle."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)  # one C call; Stream objects cost about 1 us more
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _NoSwitch:
+    """Stand-in for torch.cuda.device(...) when the device is already current."""
+
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(device: torch.device):
+    """Context that makes `device` current for the launches inside it; entering and leaving
+    torch.cuda.device costs about 2 us per call, so nothing is switched when it already is."""
+    if device.index is None or torch.cuda.current_device() == device.index:
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 # stream key of a device's shared workspace (reserved at load time, used under graph capture)
@@ -325,7 +352,7 @@ def linear(
     fused_bias = bias is not None and bias.dtype == x.dtype and bias.is_cuda and bias.numel() == w.N
     bias_ptr = bias.contiguous().data_ptr() if fused_bias else None
     lib = _lib.load()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         stream = _stream_handle(x.device)
         # decode: split-K partial sums, tickets, accumulation cells; prefill GEMM: split-K
         # partial tiles when the tile grid alone would leave CUs idle
@@ -417,7 +444,7 @@ def linear_gate_up(
     fusable_bias = bias is None or (bias.dtype == x.dtype and bias.is_cuda and bias.numel() == w.N)
     if fused is not False and fusable_bias:
         lib = _lib.load()
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             stream = _stream_handle(x.device)
             ws = _workspace_for_call(x.device, w.plan(M, _DTYPES[x.dtype])[1], stream)
             st = w.struct()
