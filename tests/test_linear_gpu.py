@@ -534,14 +534,34 @@ def test_act_order_dispatch(pkg, oracle, gpu):
     assert pkg.ops.select_path(pk, 16) == "gemv"
     assert pkg.ops.select_path(pk, 1024) == "gemm"
     assert pkg.ops.select_path(pk, 1024, torch.bfloat16) == "gemm"
-    assert pkg.ops.select_path(pk, 4, torch.bfloat16) == "gemm"  # the act-order decode kernel is fp16 only
+    assert pkg.ops.select_path(pk, 4, torch.bfloat16) == "gemv"
 
 
 @pytest.mark.parametrize("M", [1, 4, 16])
 @pytest.mark.parametrize("K,N", [(1024, 1024), (8192, 10240)])
 def test_act_order_bf16_small_m(pkg, oracle, gpu, K, N, M):
-    """g_idx with bf16 activations at decode sizes: the MFMA kernel that reads through g_idx."""
+    """g_idx with bf16 activations at decode sizes: the lookup decode kernel with bf16 weights
+    rounded once from the fp32 product, and the MFMA kernel forced on the same problem."""
     _run(pkg, oracle, gpu, K, N, 128, M, dtype="bf16", act=True, seed=M + 2)
+    _run(pkg, oracle, gpu, K, N, 128, M, dtype="bf16", act=True, seed=M + 2, path=2)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_act_order_decode_one_hot_reads_weights_back(pkg, oracle, gpu, dtype):
+    """x = rows of the identity through the lookup decode kernel: the dequantized rows, bit for bit."""
+    K, N, gs = 1024, 512, 128
+    bf = dtype == "bf16"
+    qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=11, sym=False, act_order=True)
+    w = oracle.dequant_gptq(qw, qz, sc, gi, gs, dtype)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), gs, 0)
+    ks = np.random.default_rng(2).choice(K, size=8, replace=False)
+    x = torch.zeros((8, K), dtype=torch.bfloat16 if bf else torch.float16, device=gpu)
+    for i, k in enumerate(ks):
+        x[i, k] = 1.0
+    y = pkg.ops.linear(pk, x, None, path=1)
+    torch.cuda.synchronize()
+    got = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, w[ks].view(np.uint16))
 
 
 # --------------------------------------------------------------------------- full-size properties

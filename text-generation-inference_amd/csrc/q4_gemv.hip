@@ -41,7 +41,6 @@ bool gemv_supported(const q4_weight* w, int M, int dtype) {
   if (chunks * (w->N / tile) > Q4_WORKSPACE_TICKET_BYTES / 4 && M > 16) return false;
   if (w->g_idx != nullptr) {
     // act-order: the table of all groups for 64 columns must fit LDS next to the slab
-    if (dtype != Q4_DTYPE_F16) return false;
     return w->num_groups <= 65535 && (long)w->num_groups * 64 * 4 <= 96 * 1024;
   }
   if (!groupsize_ok_contiguous(w->groupsize)) return false;
@@ -327,7 +326,7 @@ static void launch_rmax(const q4_weight* w, const GemvParams& gp, int words, dim
   if (w->layout == Q4_LAYOUT_AWQ) {
     launch_kernel(gemv_awq_kernel<DTYPE, RMAX>, gp, grid, block, smem, stream);
   } else if (w->g_idx != nullptr) {
-    launch_kernel(gemv_gptq_act_kernel<RMAX>, gp, grid, block, smem, stream);
+    launch_kernel(gemv_gptq_act_kernel<DTYPE, RMAX>, gp, grid, block, smem, stream);
   } else if (gs == 128) {
     if (words == 4) launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, true, 4>, gp, grid, block, smem, stream);
     else if (words == 2) launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, true, 2>, gp, grid, block, smem, stream);

@@ -790,7 +790,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
 // ---------------------------------------------------------------------------------------
 // GPTQ with g_idx (act-order), fp16.  LDS: [slab][g_idx slice as uint16][table G x tile_cols].
 // Table entry (g, column) = fp16 scale | fp16 -(1024 + zero) << 16.
-template <int RMAX, bool MOE = false>
+template <int DTYPE, int RMAX, bool MOE = false>
 __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int32_t* moe_rows = nullptr;
@@ -879,7 +879,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
     const uint32_t words[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      half2_t b[4];
+      uint32_t b[4];
 #pragma unroll
       for (int pr = 0; pr < 4; ++pr) {
         // rows pr and pr + 4 of the K block share one splice (nibbles 16 bits apart)
@@ -889,10 +889,20 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
         const uint32_t c2 = __builtin_amdgcn_perm(eb, ea, 0x07060302u);
         const uint32_t q2 = ((words[t] >> (4 * pr)) & splice.mask_lo) | splice.magic;
         const half2_t dq = as_half2(q2) + as_half2(c2);  // exact q - z
-        b[pr] = dq * as_half2(s2);                       // one fp16 rounding, as the reference
+        if constexpr (DTYPE == Q4_DTYPE_F16) {
+          b[pr] = as_u32(dq * as_half2(s2));  // one fp16 rounding, as the reference
+        } else {
+          // bf16: the exact fp32 product, rounded once
+          const half2_t sc = as_half2(s2);
+          b[pr] = (uint32_t)f32_to_bf16_rne((float)dq.x * (float)sc.x) | ((uint32_t)f32_to_bf16_rne((float)dq.y * (float)sc.y) << 16);
+        }
       }
       // b is in K order [0,4,1,5,2,6,3,7], the order of the staged activations
-      acc[t] = mfma16<Q4_DTYPE_F16>(a, b, acc[t]);
+      const uint4_t bu = {b[0], b[1], b[2], b[3]};
+      if constexpr (DTYPE == Q4_DTYPE_F16)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, bu), acc[t], 0, 0, 0);
+      else
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, bu), acc[t], 0, 0, 0);
     }
   };
 
@@ -912,7 +922,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
   for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int r = 0; r < RMAX; ++r) out[t][r] = acc[t][r];
-  gemv_finish<Q4_DTYPE_F16, 4, RMAX>(gp, d, out, nl, smem);
+  gemv_finish<DTYPE, 4, RMAX>(gp, d, out, nl, smem);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -324,8 +324,7 @@ void launch_moe_gemv_dtype(const q4_weight* e0, dim3 grid, dim3 block, size_t sm
     return;
   }
   if (e0->g_idx != nullptr) {
-    // fp16 only (checked by the plan through gemv_supported)
-    launch_with_smem(gemv_gptq_act_kernel<4, true>, grid, block, smem, stream, gp);
+    launch_with_smem(gemv_gptq_act_kernel<DTYPE, 4, true>, grid, block, smem, stream, gp);
     return;
   }
   if (gs == 128) launch_with_smem(gemv_gptq_kernel<DTYPE, 4, 4, true, 4, false, true>, grid, block, smem, stream, gp);
