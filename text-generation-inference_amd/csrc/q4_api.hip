@@ -128,7 +128,7 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   }
   if (!small && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
   if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
-  // (act-order with bf16 activations has no decode kernel: the MFMA kernel takes any M)
+  // (what the decode kernels do not take, e.g. an act-order table too large for LDS: the MFMA kernel takes any M)
   if (gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
   return Q4_PATH_GENERIC;
 }
