@@ -64,7 +64,8 @@ __device__ __forceinline__ SpliceK gemm_splice_consts() {
 struct ColConsts {
   half2_t czlo, czhi;  // -(1024 + z), -(64 + z), both halves equal
   half2_t s2;          // (s, s)
-  float sf;            // float(s), bf16 path
+  // bf16 path: float(s), float(s) / 16, -(1024 + z) * float(s), -(64 + z) * float(s) (all exact)
+  float sf, sf16, clo, chi;
 };
 
 __device__ __forceinline__ ColConsts make_col_consts(uint32_t z, half_t s) {
@@ -73,32 +74,44 @@ __device__ __forceinline__ ColConsts make_col_consts(uint32_t z, half_t s) {
   c.czhi = as_half2(0xD400D400u | (z << 4) | (z << 20));
   c.s2 = half2_t{s, s};
   c.sf = (float)s;
+  c.sf16 = c.sf * 0.0625f;
+  c.clo = -(1024.f + (float)z) * c.sf;
+  c.chi = -(64.f + (float)z) * c.sf;
   return c;
 }
 
 // One packed word -> MFMA B fragment (8 weights of one column, K order 0,4,1,5,2,6,3,7).
 template <int DTYPE>
 __device__ __forceinline__ uint4_t dequant_word(uint32_t w, const ColConsts& c, const SpliceK& k) {
-  const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
   const uint32_t w8 = w >> 8;
-  half2_t d[4];  // exact (q - z)
-  d[0] = as_half2((w & k.mask_lo) | k.magic) + c.czlo;
-  d[1] = as_half2((w & k.mask_hi) | k.magic) * sixteenth + c.czhi;
-  d[2] = as_half2((w8 & k.mask_lo) | k.magic) + c.czlo;
-  d[3] = as_half2((w8 & k.mask_hi) | k.magic) * sixteenth + c.czhi;
   uint4_t out;
   if constexpr (DTYPE == Q4_DTYPE_F16) {
+    const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+    half2_t d[4];  // exact (q - z)
+    d[0] = as_half2((w & k.mask_lo) | k.magic) + c.czlo;
+    d[1] = as_half2((w & k.mask_hi) | k.magic) * sixteenth + c.czhi;
+    d[2] = as_half2((w8 & k.mask_lo) | k.magic) + c.czlo;
+    d[3] = as_half2((w8 & k.mask_hi) | k.magic) * sixteenth + c.czhi;
     // one fp16 multiply per weight: the reference's rounding
     out.x = as_u32(d[0] * c.s2);
     out.y = as_u32(d[1] * c.s2);
     out.z = as_u32(d[2] * c.s2);
     out.w = as_u32(d[3] * c.s2);
   } else {
-    // bf16: exact fp32 product, rounded once to nearest even by the packed convert
+    // bf16: the exact fp32 value float(s) * (q - z), rounded once to nearest even by the packed
+    // convert.  One mixed-precision multiply-add per weight gives it straight from the spliced
+    // half: (1024 + q) * s - (1024 + z) * s, or (1024 + 16 q) * s / 16 - (64 + z) * s; both
+    // products and both addends are exact in fp32 (the compiler would emit a convert, a
+    // subtraction and a multiply instead).
+    const uint32_t v[4] = {(w & k.mask_lo) | k.magic, (w & k.mask_hi) | k.magic, (w8 & k.mask_lo) | k.magic,
+                           (w8 & k.mask_hi) | k.magic};
     uint32_t o[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const gemm_float2_t f = {(float)d[i].x * c.sf, (float)d[i].y * c.sf};
+      const float sc = (i & 1) ? c.sf16 : c.sf, add = (i & 1) ? c.chi : c.clo;
+      gemm_float2_t f;
+      asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(f.x) : "v"(v[i]), "v"(sc), "v"(add));
+      asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(f.y) : "v"(v[i]), "v"(sc), "v"(add));
       o[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, gemm_bf16x2_t));
     }
     out.x = o[0]; out.y = o[1]; out.z = o[2]; out.w = o[3];
