@@ -419,10 +419,17 @@ def test_awq_dispatch_large_m(pkg, oracle, gpu):
     assert pkg.ops.select_path(pk, 8) == "gemv"
     assert pkg.ops.select_path(pk, 9) == "gemm"
     assert pkg.ops.select_path(pk, 64) == "gemm"
-    # the first row count that goes to the GEMM moves with the shape (measured crossovers)
+    # the kernel that unpacks the words in registers (groups of 64 rows or more, N a multiple of
+    # 256) takes over from 9 rows on whatever the shape
+    for K, N in [(4096, 4096), (4096, 6144), (14336, 4096), (4096, 14336), (8192, 28672), (28672, 8192)]:
+        w = pkg.ops.PackedWeight(pk.qweight, pk.qzeros, pk.scales, None, K, N, 128, K // 128, 1)  # geometry only
+        assert pkg.ops.select_path(w, 8) == "gemv", (K, N)
+        assert pkg.ops.select_path(w, 9) == "gemm", (K, N)
+    # groups of 32 rows go through the kernel that unpacks through LDS: the first row count that
+    # goes to it moves with the shape (measured crossovers)
     for K, N, first in [(4096, 4096, 9), (4096, 6144, 14), (11008, 4096, 10), (14336, 4096, 17), (4096, 14336, 17),
                         (8192, 10240, 17), (8192, 28672, 33), (28672, 8192, 33)]:
-        w = pkg.ops.PackedWeight(pk.qweight, pk.qzeros, pk.scales, None, K, N, 128, K // 128, 1)  # geometry only
+        w = pkg.ops.PackedWeight(pk.qweight, pk.qzeros, pk.scales, None, K, N, 32, K // 32, 1)  # geometry only
         assert pkg.ops.select_path(w, first - 1) == "gemv", (K, N)
         assert pkg.ops.select_path(w, first) == "gemm", (K, N)
 

@@ -109,14 +109,14 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   // 67 us at M = 24, 52 against 140 us at M = 64; the kernel's time is flat in M up to 128
   // rows), from about M = 48 on when it has to gather scales and zero points from global
   // memory (~2x slower per tile).
-  // AWQ: the decode kernel's time grows with every row (16 accumulator sets, ~250 VGPRs)
-  // while the split-K GEMM is flat in M (17.2 us for 4096 x 4096, 20.4 us for 4096 x 6144,
-  // 27 us for 11008 x 4096, 30 us for 4096 x 14336, 40 us for 8192 x 10240, 92 / 108 us for
-  // 28672 x 8192 / 8192 x 28672: it unpacks every weight through LDS once per 128 rows).
-  // First M at which the GEMM was faster: 4096 x 4096 9, 4096 x 6144 14, 5120 x 5120 16,
-  // 11008 x 4096 10; above 16 for 4096 x 11008, 4096 x 14336, 14336 x 4096, 8192 x 8192,
-  // 8192 x 10240, 5120 x 13824, 13824 x 5120; 28672 x 8192 and 8192 x 28672 in two row
-  // chunks up to 32 rows (96 against 95 / 131 us at M = 32).
+  // AWQ: up to 8 rows the decode kernel that feeds the words to the MFMA as stored; from 9 rows on
+  // the MFMA kernel that unpacks them in registers wherever it applies (split-K on small tile
+  // grids, flat in M up to 32 rows: 17.4 against 28.3 us for 4096 x 14336 at M = 16, 17.9 against
+  // 31.4 us for 14336 x 4096, 12.5 against 12.7 us for 4096 x 4096).  Other AWQ weights (N not a
+  // multiple of 256, groups shorter than 64 rows): the general decode kernel, whose time grows
+  // with every row, up to the M at which the kernel that unpacks through LDS measured faster:
+  // 4096 x 4096 9, 4096 x 6144 14, 5120 x 5120 16, 11008 x 4096 10; above 16 for the larger
+  // layers; 28672 x 8192 and 8192 x 28672 up to 32 rows.
   bool small = M <= 16 || (w->layout == Q4_LAYOUT_GPTQ && M <= 48 && !gemm_act_order_table(w));
   if (w->layout == Q4_LAYOUT_AWQ) {
     int first_gemm_m = 17;
@@ -124,6 +124,7 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
     else if (weights <= (1L << 24)) first_gemm_m = 9;
     else if (weights <= (1L << 25)) first_gemm_m = 14;
     else if ((w->K / 128) % 8 != 0 && weights <= (1L << 26)) first_gemm_m = 10;
+    if (gemm_awq_direct_supported(w, M, dtype)) first_gemm_m = 9;
     small = M < first_gemm_m;
   }
   if (!small && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;

@@ -246,6 +246,11 @@ struct MoeLaunch {
 int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                     void* workspace, size_t workspace_bytes, hipStream_t stream, const MoeLaunch* moe = nullptr);
 size_t gemm_awq_moe_workspace_bytes(const q4_weight* w, const MoeLaunch* moe);
+// AWQ layout, dense launches: the kernel that unpacks the checkpoint words in registers
+bool gemm_awq_direct_supported(const q4_weight* w, int M, int dtype);
+int launch_gemm_awq_direct(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
+                           void* workspace, size_t workspace_bytes, hipStream_t stream);
+size_t gemm_awq_direct_workspace_bytes(int M, int K, int N);
 bool gemm_supported(const q4_weight* w, int M, int dtype);
 int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                 void* workspace, size_t workspace_bytes, hipStream_t stream);

@@ -140,7 +140,9 @@ size_t gemm_workspace_bytes(int M, int K, int N) {
     const int other = gemm_awq_splits(M, K, N, one_per_cu);
     if (other > splits) splits = other;
   }
-  return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+  const size_t bytes = splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+  const size_t direct = gemm_awq_direct_workspace_bytes(M, K, N);
+  return direct > bytes ? direct : bytes;
 }
 
 // The prefill kernel with the gated-MLP epilogue: one launch where the plain kernel would run

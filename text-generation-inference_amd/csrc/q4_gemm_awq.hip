@@ -520,6 +520,9 @@ size_t gemm_awq_moe_workspace_bytes(const q4_weight* w, const MoeLaunch* moe) {
 int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                     void* workspace, size_t workspace_bytes, hipStream_t stream, const MoeLaunch* moe) {
   using namespace q4;
+  // dense AWQ launches go to the kernel that unpacks the words in registers where it applies
+  if (moe == nullptr && gemm_awq_direct_supported(w, M, dtype))
+    return launch_gemm_awq_direct(w, x, bias, y, M, dtype, workspace, workspace_bytes, stream);
   // grouped launch: M is the largest row count an expert can have (the number of tokens)
   if (!gemm_awq_supported(w, M, dtype)) {
     set_error("q4_linear(gemm/awq): unsupported problem (M=%d K=%d N=%d groupsize=%d)", M, w->K, w->N,
