@@ -81,6 +81,11 @@ def parse_args():
                     help="skip timing torch's dense fp16 matmul (hipBLASLt) on the GEMM shapes")
     ap.add_argument("--floor-probe", action="store_true",
                     help="time read-only kernels (q4_probe_read) on buffers of the projections' sizes and print a table")
+    ap.add_argument("--lds-probe", action="store_true",
+                    help="time 128-bit LDS reads (q4_probe_lds) under several lane-to-address maps and print a table")
+    ap.add_argument("--awq-probe", action="store_true",
+                    help="a few prefill launches (M = --gemm-m) of the AWQ-layout kernel and of the GPTQ-layout kernel on "
+                         "4096 x 14336, for counter runs under rocprofv3")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="eager launches only (a 256 MiB copy kernel, then each decode shape and one GEMM), "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs; prints no JSON line")
@@ -261,6 +266,44 @@ def time_read_floor(pkg, torch, lib, dev, pool, sink, nbytes, pattern, n_words, 
     return avg * 1e6, best * 1e6
 
 
+def lds_probe(pkg, torch, lib, dev):
+    """ns per wave-level ds_read_b128 (16 waves per CU, all CUs) for lane -> 16-byte-unit maps.
+    256 B per clock would be ~2.1 ns at the clock these launches run at."""
+    sink = torch.zeros(4, dtype=torch.uint8, device=dev)
+    blocks = lambda order: [u for b in order for u in range(8 * b, 8 * b + 8)]  # residues per 8-lane block
+    maps = [
+        ("linear: lane l at unit l", [l for l in range(64)]),
+        ("8-lane blocks at residues 0-7, 0-7, 8-15, 8-15 (free if lanes 0-7 pass with 24-31, 8-15 with 16-23)",
+         [(l & 7) + 8 * ((l >> 4) & 1) + 16 * (l >> 3) for l in range(64)]),
+        ("8-lane blocks at residues 0-7, 8-15, 8-15, 0-7 (free if lanes 0-15 pass together)",
+         [(l & 7) + 8 * (((l >> 3) & 1) ^ ((l >> 4) & 1)) + 16 * (l >> 3) for l in range(64)]),
+        ("32 rows x 2 units, rows of 9 units (prefill kernel of the GPTQ layout)", [(l & 31) * 9 + (l >> 5) for l in range(64)]),
+        ("16 rows x 4 units, rows of 9 units", [(l & 15) * 9 + (l >> 4) for l in range(64)]),
+        ("16 rows x 4 units, rows of 8 units, unit ^ (row >> 1) (prefill kernel of the AWQ layout)",
+         [(l & 15) * 8 + ((l >> 4) ^ ((l & 15) >> 1)) for l in range(64)]),
+        ("16 rows x 4 units, rows of 8 units, no swizzle", [(l & 15) * 8 + (l >> 4) for l in range(64)]),
+        ("all lanes on the same four banks", [l * 16 for l in range(64)]),
+    ]
+    iters = 2000
+    rows = []
+    for name, m in maps:
+        dm = torch.tensor(m, dtype=torch.int32, device=dev)
+        stream = torch.cuda.current_stream().cuda_stream
+        best = None
+        for rep in range(4):
+            pkg._lib.check(lib.q4_probe_lds(dm.data_ptr(), 10, 256, sink.data_ptr(), stream))
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            pkg._lib.check(lib.q4_probe_lds(dm.data_ptr(), iters, 256, sink.data_ptr(), stream))
+            e1.record()
+            e1.synchronize()
+            ns = e0.elapsed_time(e1) * 1e6 / (16.0 * iters * 8)
+            best = ns if best is None or ns < best else best
+        rows.append({"map": name, "ns_per_wave_read": round(best, 2)})
+        print(f"{best:6.2f} ns per wave read   {name}", flush=True)
+    return rows
+
+
 def floor_probe(pkg, torch, lib, dev):
     """Table of read-only launches: empty grids, linear reads and the decode tile pattern at the
     four projections' sizes, HBM-rotating (1 GiB pool) and cache-hot."""
@@ -339,6 +382,22 @@ def main():
         for i in range(len(SHAPES)):
             pkg.ops.linear(weights[c % copies][i], xs[i], None, out=ys[i])
 
+    if args.lds_probe:
+        print(json.dumps({"lds_probe": lds_probe(pkg, torch, lib, dev)}))
+        return
+    if args.awq_probe:
+        K, N, Mg = 4096, 14336, args.gemm_m
+        wa = make_weights_variant(pkg, torch, dev, K, N, 5, "awq")
+        wg = make_weights(pkg, torch, dev, K, N, 6)
+        xg = torch.randn((Mg, K), device=dev, dtype=torch.float16)
+        yg = torch.empty((Mg, N), device=dev, dtype=torch.float16)
+        for _ in range(6):
+            pkg.ops.linear(wa, xg, None, out=yg)
+            pkg.ops.linear(wg, xg, None, out=yg)
+        torch.cuda.synchronize()
+        print("awq probe done: 6 launches each of the AWQ-layout and the GPTQ-layout prefill kernel, %d x %d, M=%d"
+              % (K, N, Mg), file=sys.stderr)
+        return
     if args.floor_probe:
         floor_probe(pkg, torch, lib, dev)
         return
@@ -631,7 +690,7 @@ def main():
         for K, N in ((4096, 14336), (14336, 4096)):
             nc = max(2, -(-600 * 1024 * 1024 // (K * N // 2)))
             conv = importlib.import_module(f"{pkg.__name__}.layers.awq.conversion_utils")
-            for Mb in (1, 16, 256):
+            for Mb in (1, 16, 256, 2048):
                 entry = {}
                 for label, convert in (("awq_layout_kernels", False), ("converted_to_gptq_layout", True)):
                     def make(c, convert=convert):

@@ -245,6 +245,15 @@ int q4_probe_read(const void* buf, size_t bytes, int pattern, int n_words, int w
                   void* sink, void* stream);
 
 /*
+ * Measurement aid, no counterpart in the reference: every wave of `workgroups` workgroups of
+ * 1024 threads issues `iters` rounds of eight 128-bit LDS reads, lane l at the 16-byte unit
+ * lane_unit[l] (64 device ints, each 0..2887).  Timed with different maps it shows which
+ * lanes the LDS serves in the same pass, which is what the activation tiles' layouts of the
+ * prefill kernels are built on.  Synchronizes the stream once to validate the map.
+ */
+int q4_probe_lds(const int32_t* lane_unit, int iters, int workgroups, void* sink, void* stream);
+
+/*
  * ---- Mixture of experts: the same linear layer, grouped over experts -----------------
  *
  * Replaces, for GPTQ and AWQ checkpoints, what the reference's sparse MoE layer

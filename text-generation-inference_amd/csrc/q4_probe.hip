@@ -51,6 +51,27 @@ __global__ void probe_empty_kernel(uint32_t* sink) {
   if (sink == nullptr) sink[0] = 1u;
 }
 
+// 128-bit LDS reads with a caller-chosen lane -> 16-byte unit map: every wave of a 1024-thread
+// workgroup issues `iters` rounds of eight ds_read_b128 (one wait per round), lane l at unit
+// map[l] (+ 144 units per read of the round).  Timed, it tells which lane-to-address patterns
+// the LDS serves at full rate, i.e. which lanes share a pass.
+__global__ __launch_bounds__(1024) void probe_lds_read_kernel(const int* __restrict__ map, int iters, uint32_t* sink) {
+  extern __shared__ __align__(16) unsigned char probe_smem[];
+  for (int i = threadIdx.x; i < 16384; i += 1024) ((uint32_t*)probe_smem)[i] = (uint32_t)i;
+  __syncthreads();
+  const uint32_t addr = (uint32_t)map[threadIdx.x & 63] * 16u;
+  uint4_t acc = {0u, 0u, 0u, 0u};
+  for (int it = 0; it < iters; ++it) {
+    uint4_t v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v[u]) : "v"(addr), "n"(u * 2304));
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u];
+  }
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) sink[0] = 1u;  // keeps the reads alive
+}
+
 }  // namespace q4
 
 using namespace q4;
@@ -111,5 +132,28 @@ extern "C" int q4_probe_read(const void* buf, size_t bytes, int pattern, int n_w
     set_error("q4_probe_read: unknown pattern %d", pattern);
     return Q4_ERR_INVALID_ARGUMENT;
   }
+  return hipGetLastError() == hipSuccess ? Q4_OK : Q4_ERR_LAUNCH;
+}
+
+extern "C" int q4_probe_lds(const int32_t* lane_unit, int iters, int workgroups, void* sink, void* stream) {
+  if (lane_unit == nullptr || sink == nullptr || iters <= 0 || workgroups <= 0) {
+    set_error("q4_probe_lds: needs a 64-entry device map, a sink, positive iterations and workgroups");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  // the caller keeps every unit below (65536 - 7 * 2304) / 16 - 1 = 2887: checked on a host copy
+  int32_t host_map[64];
+  if (hipMemcpyAsync(host_map, lane_unit, sizeof(host_map), hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess ||
+      hipStreamSynchronize((hipStream_t)stream) != hipSuccess) {
+    set_error("q4_probe_lds: cannot read the lane map");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  for (int l = 0; l < 64; ++l) {
+    if (host_map[l] < 0 || host_map[l] > 2887) {
+      set_error("q4_probe_lds: lane %d maps to unit %d, outside 0..2887", l, host_map[l]);
+      return Q4_ERR_INVALID_ARGUMENT;
+    }
+  }
+  hipLaunchKernelGGL(q4::probe_lds_read_kernel, dim3(workgroups), dim3(1024), 65536, (hipStream_t)stream, lane_unit, iters,
+                     (uint32_t*)sink);
   return hipGetLastError() == hipSuccess ? Q4_OK : Q4_ERR_LAUNCH;
 }
