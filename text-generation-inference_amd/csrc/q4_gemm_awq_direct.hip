@@ -30,6 +30,15 @@ static DirectPlan direct_plan(int M, int K, int N) {
   // on 4096 x 14336; from M = 256 on the larger tile wins or ties); 64 and 32 rows below that.
   g.bm = M <= 32 ? 32 : (M <= 64 ? 64 : 96);
   if (g.bm == 96 && (long)((M + 95) / 96) * 96 * 5 > (long)((M + 63) / 64) * 64 * 6) g.bm = 64;
+  // Several rounds of the chip: a CU works through ceil(tiles / 256) tiles whatever their height
+  // (two 96-row or three 64-row workgroups per CU take the same time per row), so the smaller
+  // tile wins where it leaves clearly fewer rows to the busiest CU (14336 x 4096 or 4096 x 4096
+  // at M = 2048: 352 tiles of 96 rows against 512 of 64; 310 -> 274 us and 89 -> 83 us).
+  if (g.bm == 96) {
+    const long cols = N / 256;
+    const long t96 = (long)((M + 95) / 96) * cols, t64 = (long)((M + 63) / 64) * cols;
+    if (t96 > 256 && ((t64 + 255) / 256) * 64 * 4 <= ((t96 + 255) / 256) * 96 * 3) g.bm = 64;
+  }
   g.tiles = (long)((M + g.bm - 1) / g.bm) * (N / 256);
   g.splits = 1;
   g.kg = 1;
