@@ -15,7 +15,16 @@ bool gemm_supported(const q4_weight* w, int M, int dtype) {
   const int gs = w->groupsize;
   if (!(gs == 32 || (gs >= 64 && gs % 64 == 0))) return false;
   if ((long)w->num_groups * gs < w->K) return false;
+  // the kernel addresses weights, scales and activations through 32-bit byte offsets (launch_gemm
+  // feeds longer activation matrices in row blocks)
+  if ((long)w->K * w->N >= (1L << 33) || (long)w->num_groups * w->N >= (1L << 31)) return false;
   return true;
+}
+
+// rows of x a single launch may address: M * K * 2 bytes below 4 GB
+static int gemm_max_rows(int K) {
+  const long rows = ((1L << 31) - 1) / (K > 0 ? K : 1);
+  return (int)(rows > (1L << 30) ? (1L << 30) : rows);
 }
 
 // two K groups per workgroup (eight waves), groups of at least 64 rows
@@ -148,7 +157,7 @@ size_t gemm_workspace_bytes(int M, int K, int N) {
 // The prefill kernel with the gated-MLP epilogue: one launch where the plain kernel would run
 // unsplit (the fused tile cannot leave partial sums), groups of at least 64 rows.
 bool gemm_gate_up_supported(const q4_weight* w, int M, int dtype) {
-  if (!gemm_supported(w, M, dtype) || w->N % 512 != 0 || w->groupsize < 64) return false;
+  if (!gemm_supported(w, M, dtype) || w->N % 512 != 0 || w->groupsize < 64 || M > gemm_max_rows(w->K)) return false;
   const GemmPlan g = gemm_plan(M, w->K, w->N);
   return g.splits == 1 && g.nw == 2 && g.bm <= 128;
 }
@@ -196,6 +205,17 @@ int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, in
     set_error("q4_linear(gemm): unsupported problem (layout=%d g_idx=%p M=%d K=%d N=%d groupsize=%d)",
               w->layout, (const void*)w->g_idx, M, w->K, w->N, w->groupsize);
     return Q4_ERR_UNSUPPORTED;
+  }
+  if (M > gemm_max_rows(w->K)) {
+    // beyond the 32-bit activation offsets of one launch: row blocks (a multiple of the tile height)
+    const int block = gemm_max_rows(w->K) / 256 * 256;
+    for (int m0 = 0; m0 < M; m0 += block) {
+      const int rows = M - m0 < block ? M - m0 : block;
+      const int rc = launch_gemm(w, (const uint16_t*)x + (size_t)m0 * w->K, bias, (uint16_t*)y + (size_t)m0 * w->N, rows, dtype,
+                                 workspace, workspace_bytes, stream);
+      if (rc != Q4_OK) return rc;
+    }
+    return Q4_OK;
   }
   GemmParams gp;
   gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, nullptr, x, bias, y,

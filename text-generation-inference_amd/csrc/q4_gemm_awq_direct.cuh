@@ -107,15 +107,6 @@ __device__ __forceinline__ float4_t mfma16(const uint4_t a, const uint4_t b, flo
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
-// Buffer loads: the base sits in a scalar resource descriptor, the lane's part of the address is
-// a 32-bit byte offset in one vector register that never changes, and what moves from load to
-// load is a scalar offset: no 64-bit vector address arithmetic and no address registers.
-typedef __amdgpu_buffer_rsrc_t buffer_rsrc_t;
-__device__ __forceinline__ buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
-__device__ __forceinline__ uint32_t uniform_u32(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
-
 // value of the neighbouring lane (lanes 2t and 2t + 1 swap)
 __device__ __forceinline__ float swap_neighbour(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));

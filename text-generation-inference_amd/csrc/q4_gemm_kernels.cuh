@@ -49,6 +49,15 @@ typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef float gemm_float2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 gemm_bf16x2_t __attribute__((ext_vector_type(2)));
 
+// Buffer loads: the base sits in a scalar resource descriptor, the lane's part of the address is
+// a 32-bit byte offset in one vector register that never changes, and what moves from load to
+// load is a scalar offset: no 64-bit vector address arithmetic and no address registers.
+typedef __amdgpu_buffer_rsrc_t buffer_rsrc_t;
+__device__ __forceinline__ buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint32_t uniform_u32(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+
 struct SpliceK {
   uint32_t mask_lo, mask_hi, magic;
 };
@@ -218,21 +227,23 @@ __global__ __launch_bounds__(256 * KG, (KG == 2 ? 1 : BM == 64 ? 3 : BM == 128 ?
   auto ktile = [&](int i) { return kt0 + i * KG; };
 
   // ---- packed-weight stream: words [K/8 + kq][ncol, ncol+1], two K tiles ahead
-  const char* wbase = (const char*)p.qweight;
+  // (buffer loads: scalar descriptor, constant lane offset, scalar step offset; the host keeps
+  // the weight and activation byte counts below 4 GB)
+  const buffer_rsrc_t wrsrc = make_rsrc(p.qweight, (uint32_t)(K >> 3) * (uint32_t)N * 4u);
   const uint32_t w_lane = ((uint32_t)kq * (uint32_t)N + (uint32_t)ncol) * 4u;
-  const size_t kstep_bytes = (size_t)N * 8;  // two packed rows per MFMA K step
+  const uint32_t kstep_bytes = (uint32_t)N * 8u;  // two packed rows per MFMA K step
   struct BWords { uint32_t v[NW]; };
   BWords bq[2][kKSteps];
   auto load_b = [&](int kt, BWords (&dst)[kKSteps]) {
 #pragma unroll
     for (int s = 0; s < kKSteps; ++s)
     {
-      const char* addr = wbase + (size_t)(ktile(kt) * kKSteps + s) * kstep_bytes + w_lane;
+      const uint32_t soff = uniform_u32((uint32_t)(ktile(kt) * kKSteps + s) * kstep_bytes);
       if constexpr (NW == 2) {
-        const uint2_t t = *(const uint2_t*)addr;
+        const uint2_t t = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(wrsrc, w_lane, soff, 0));
         dst[s].v[0] = t.x; dst[s].v[1] = t.y;
       } else {
-        dst[s].v[0] = *(const uint32_t*)addr;
+        dst[s].v[0] = __builtin_amdgcn_raw_buffer_load_b32(wrsrc, w_lane, soff, 0);
       }
     }
   };
@@ -241,15 +252,17 @@ __global__ __launch_bounds__(256 * KG, (KG == 2 ? 1 : BM == 64 ? 3 : BM == 128 ?
   // from two tiny (cached) loads, which keeps the steady-state loop free of branches.
   ColConsts cc[GPT][NW], cc_next[GPT][NW];
   uint32_t sraw[GPT], zraw[GPT];
+  const buffer_rsrc_t srsrc = make_rsrc(p.scales, (uint32_t)p.num_groups * (uint32_t)N * 2u);
+  const buffer_rsrc_t zrsrc = make_rsrc(p.qzeros, (uint32_t)p.num_groups * (uint32_t)(N >> 3) * 4u);
   const int zshift = (ncol & 7) * 4;
   auto load_group_raw = [&](int kt) {
 #pragma unroll
     for (int g = 0; g < GPT; ++g) {
       int gi = (ktile(kt) * kBK + g * (kBK / GPT)) / p.groupsize;
       gi = min(gi, p.num_groups - 1);
-      if constexpr (NW == 2) sraw[g] = *(const uint32_t*)(p.scales + (size_t)gi * N + ncol);
-      else sraw[g] = *(const uint16_t*)(p.scales + (size_t)gi * N + ncol);
-      zraw[g] = p.qzeros[(size_t)gi * (N >> 3) + (ncol >> 3)];
+      if constexpr (NW == 2) sraw[g] = __builtin_amdgcn_raw_buffer_load_b32(srsrc, (uint32_t)ncol * 2u, uniform_u32((uint32_t)gi * (uint32_t)N * 2u), 0);
+      else sraw[g] = __builtin_amdgcn_raw_buffer_load_b16(srsrc, (uint32_t)ncol * 2u, uniform_u32((uint32_t)gi * (uint32_t)N * 2u), 0);
+      zraw[g] = __builtin_amdgcn_raw_buffer_load_b32(zrsrc, (uint32_t)(ncol >> 3) * 4u, uniform_u32((uint32_t)gi * (uint32_t)(N >> 3) * 4u), 0);
     }
   };
   auto make_group = [&](ColConsts (&dst)[GPT][NW]) {
@@ -263,29 +276,31 @@ __global__ __launch_bounds__(256 * KG, (KG == 2 ? 1 : BM == 64 ? 3 : BM == 128 ?
   };
 
   // ---- activation tile: global -> registers -> (permuted) LDS
-  const uint16_t* xs = (const uint16_t*)p.x;
+  // rows of x behind p.x: M, or every token of a grouped launch (its row map points anywhere)
+  const buffer_rsrc_t xrsrc = make_rsrc(p.x, 0xFFFFFFFFu);
   // Register staging sets: with two sets (128-row tiles) a tile's loads are issued two
   // tiles before they are written to LDS; the 256-row tile has registers for one set only.
   constexpr int ASETS = BM <= 128 ? 2 : 1;
   uint4_t areg[ASETS][A_LOADS];
-  int moe_xrow[MOE ? A_LOADS : 1];  // grouped launch with a row map: x row of each staged row
-  if constexpr (MOE) {
+  uint32_t a_off[A_LOADS];  // byte offset of the thread's 16-byte units within x (below 4 GB: host)
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      const int row = min(m0 + ((tid + 256 * i) >> 3), M - 1);
-      moe_xrow[i] = gp.moe.x_rows != nullptr ? gp.moe.x_rows[moe_row0 + row] : row;
+  for (int i = 0; i < A_LOADS; ++i) {
+    const int u = tid + 256 * i;
+    const int m = u >> 3, kb = u & 7;
+    // rows past M re-read the last row: their results are never stored
+    int row = min(m0 + m, M - 1);
+    if constexpr (MOE) {
+      // grouped launch with a row map: x row of each staged row
+      if (gp.moe.x_rows != nullptr) row = gp.moe.x_rows[moe_row0 + row];
     }
+    a_off[i] = ((uint32_t)row * (uint32_t)K + (uint32_t)kb * 8u) * 2u;
   }
   auto load_a = [&](int kt, auto set_c) {
     constexpr int set = decltype(set_c)::value % ASETS;
+    const uint32_t tile_off = uniform_u32((uint32_t)ktile(kt) * (kBK * 2));
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      const int u = tid + 256 * i;
-      const int m = u >> 3, kb = u & 7;
-      // rows past M re-read the last row: their results are never stored
-      const int row = MOE ? moe_xrow[i] : min(m0 + m, M - 1);
-      areg[set][i] = *(const uint4_t*)(xs + (size_t)row * K + ktile(kt) * kBK + kb * 8);
-    }
+    for (int i = 0; i < A_LOADS; ++i)
+      areg[set][i] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, a_off[i], tile_off, 0));
   };
   auto store_a = [&](int buf, auto set_c) {
     constexpr int set = decltype(set_c)::value % ASETS;
@@ -295,11 +310,12 @@ __global__ __launch_bounds__(256 * KG, (KG == 2 ? 1 : BM == 64 ? 3 : BM == 128 ?
       const int u = tid + 256 * i;
       const int m = u >> 3, kb = u & 7;
       const uint4_t v = areg[set][i];
+      // K order [0,4,1,5,2,6,3,7] of the splice: one byte permute per register
       uint4_t o;
-      o.x = (v.x & 0xFFFFu) | (v.z << 16);
-      o.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
-      o.z = (v.y & 0xFFFFu) | (v.w << 16);
-      o.w = (v.y >> 16) | (v.w & 0xFFFF0000u);
+      o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+      o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+      o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+      o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
       *(uint4_t*)(base + (m * kAUnitsPerRow + kb) * 16) = o;
     }
   };

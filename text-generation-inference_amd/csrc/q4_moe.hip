@@ -351,6 +351,12 @@ int moe_gemm_bm(const q4_moe_weight* w, int tokens, int topk) {
 // it plans for an even spread (tokens * topk / experts rows each) and splits K when those
 // tiles alone would leave CUs idle (Mixtral down projection at 64 tokens: 8 experts x 16
 // column tiles, 224 K tiles each).
+// the grouped GPTQ prefill kernel addresses the activation rows (tokens, or token-expert pairs)
+// through 32-bit byte offsets
+static bool moe_gemm_ok(const q4_weight* e0, int tokens, int topk, int dtype) {
+  return gemm_supported(e0, tokens, dtype) && (long)tokens * topk * e0->K < (1L << 31);
+}
+
 int moe_gemm_splits(const q4_moe_weight* w, int tokens, int topk) {
   const q4_weight* e0 = &w->expert0;
   const long pairs = (long)tokens * topk;
@@ -390,7 +396,7 @@ size_t moe_workspace_bytes(const q4_moe_weight* w, int tokens, int topk) {
     if (plain.ok) take(plain.cfg.splits);
     if (fused.ok) take(fused.cfg.splits);
     if (!plain.ok) {
-      if (gemm_supported(e0, tokens, dtype)) {
+      if (moe_gemm_ok(e0, tokens, topk, dtype)) {
         take(moe_gemm_splits(w, tokens, topk));
       } else if (gemm_awq_supported(e0, tokens, dtype)) {
         const MoeLaunch ml{MoeView{}, w->num_experts, tokens, tokens * topk};
@@ -454,7 +460,7 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
       launch_gemv_gate_up(gp, dtype, tokens <= 1 ? 1 : 2, e0->groupsize == 128, grid, block, pl.smem, stream, true);
     else if (dtype == Q4_DTYPE_F16) launch_moe_gemv_dtype<Q4_DTYPE_F16>(e0, grid, block, pl.smem, stream, gp);
     else launch_moe_gemv_dtype<Q4_DTYPE_BF16>(e0, grid, block, pl.smem, stream, gp);
-  } else if (gemm_supported(e0, tokens, dtype)) {
+  } else if (moe_gemm_ok(e0, tokens, topk, dtype)) {
     GemmParams gp;
     gp.p = Problem{e0->qweight, e0->qzeros, (const half_t*)e0->scales, nullptr, x, nullptr, y,
                    0,           e0->K,      e0->N,                     e0->groupsize, e0->num_groups};
