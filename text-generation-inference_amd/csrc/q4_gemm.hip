@@ -17,7 +17,7 @@ bool gemm_supported(const q4_weight* w, int M, int dtype) {
   if ((long)w->num_groups * gs < w->K) return false;
   // the kernel addresses weights, scales and activations through 32-bit byte offsets (launch_gemm
   // feeds longer activation matrices in row blocks)
-  if ((long)w->K * w->N >= (1L << 33) || (long)w->num_groups * w->N >= (1L << 31)) return false;
+  if ((long)w->K * w->N >= (1L << 33) || (long)w->num_groups * w->N >= (1L << 31) || w->K > (1 << 22)) return false;
   return true;
 }
 
