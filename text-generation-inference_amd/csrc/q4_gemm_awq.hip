@@ -207,11 +207,11 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   // Phase 3: o holds rows (0,4),(1,5),(2,6),(3,7): back to natural K order, one 16-byte unit.
   auto word_store = [&](int buf, int i, const uint32_t (&o)[4]) {
     unsigned char* base = smem + 2 * A_TILE + buf * B_TILE;
-    uint4_t unit;
-    unit.x = (o[0] & 0xFFFFu) | (o[1] << 16);
-    unit.y = (o[2] & 0xFFFFu) | (o[3] << 16);
-    unit.z = (o[0] >> 16) | (o[1] & 0xFFFF0000u);
-    unit.w = (o[2] >> 16) | (o[3] & 0xFFFF0000u);
+    uint4_t unit;  // one byte permute per register
+    unit.x = __builtin_amdgcn_perm(o[1], o[0], 0x05040100u);
+    unit.y = __builtin_amdgcn_perm(o[3], o[2], 0x05040100u);
+    unit.z = __builtin_amdgcn_perm(o[1], o[0], 0x07060302u);
+    unit.w = __builtin_amdgcn_perm(o[3], o[2], 0x07060302u);
     *(uint4_t*)(base + ((size_t)(pkb0 + 2 * i) * kABN + b_slot(pn)) * 16) = unit;
   };
   auto store_b_act_word = [&](int buf, int kt, int i) {
