@@ -142,9 +142,50 @@ static GemvConfig pick_config(const q4_weight* w, int M, bool gate_up, bool allo
         best = dv;
       }
     }
+    // 160 column tiles or more over a short K (up to 4096 rows), four rows or more: every split
+    // costs more in partial sums than the idle CUs do (4096 x 11008, 172 tiles: 10.2 / 10.7 / 11.9 us
+    // unsplit at M = 4 / 8 / 16 against 13.5 / 14.2 / 16.4 us with two splits)
+    if (M >= 4 && n64 >= 160 && chunks <= 32 && (long)rows * c.wk * ((long)((chunks + c.wk - 1) / c.wk) * 256 + 16) <= 150000)
+      best = 1;
     c.splits = best;
     if (best_cost >= 0.0) return c;
     c.lean = 0;  // no split fits LDS: the kernel below, with its workgroup slab
+  }
+  // Small layers, 4 to 16 rows, K a multiple of 1024 from 2048 on: 32-column wave tiles (two words per lane)
+  // in eight-wave workgroups, about one workgroup per CU (two up to 8 rows); tiles that fill
+  // the chip on their own are not split.  Swept on MI355X against the rule below (us, new /
+  // old): 4096 x 4096 8.1 / 8.5 at M = 4, 8.3 / 9.2 at M = 8, 8.4 / 9.9 at M = 9, 8.9 / 9.5 at
+  // M = 16; 4096 x 6144 9.8 / 10.7 at M = 9, 10.5 / 11.9 at M = 16; 8192 x 1024 7.5 / 9.1,
+  // 7.8 / 10.1, 8.3 / 9.5 at M = 4, 8, 16; 2048 x 8192 6.4 / 8.2, 7.1 / 8.2, 7.9 / 9.7.
+  if (allow_lean && !gate_up && w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && w->groupsize >= 128 &&
+      w->groupsize % 128 == 0 && M >= 4 && M <= 16 && chunks % 8 == 0 && chunks >= 16 && w->N % 64 == 0 &&
+      // (4096 x 6144 up to 8 rows: no better than the rule below)
+      (M >= 9 || w->N <= 4096 || w->N / 32 >= 256)) {
+    const bool narrow = w->N / 32 >= 256 || w->N <= 2048;  // one 32-column tile per workgroup, eight waves along K
+    GemvConfig t = c;
+    t.words = 2;
+    t.wcol = narrow ? 1 : 2;
+    t.wk = narrow ? 8 : 4;
+    const long tiles = w->N / (32 * t.wcol);
+    const int per = chunks / t.wk;
+    const double target = (M <= 8 && !narrow) ? 512.0 : 256.0;
+    int pick = -1;
+    double pick_cost = -1.0;
+    for (int dv = 1; dv <= per; ++dv) {
+      if (per % dv != 0) continue;
+      if ((long)rows * ((long)w->K / dv * 2 + 16) > 150000) continue;  // the workgroup's slab
+      const double wgs = (double)tiles * dv;
+      if (tiles >= 256 && dv > 1) break;
+      const double cost = wgs >= target ? wgs / target : 1.5 * target / wgs;
+      if (pick_cost < 0.0 || cost < pick_cost) {
+        pick_cost = cost;
+        pick = dv;
+      }
+    }
+    if (pick > 0) {
+      t.splits = pick;
+      return t;
+    }
   }
   c.wcol = 1;
   c.wk = chunks >= 4 ? 4 : (chunks >= 2 ? 2 : 1);
