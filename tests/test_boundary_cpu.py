@@ -222,6 +222,17 @@ def test_probe_read_rejects_shapes_that_do_not_divide(pkg):
     assert b"q4_probe_read" in lib.q4_last_error()
 
 
+def test_probe_lds_rejects_missing_arguments(pkg):
+    """The LDS probe validates its arguments before it touches the device."""
+    lib = pkg._lib.load()
+    L = pkg._lib
+    assert lib.q4_probe_lds(None, 10, 256, 0x2000, None) == L.ERR_INVALID_ARGUMENT    # no lane map
+    assert lib.q4_probe_lds(0x1000, 10, 256, None, None) == L.ERR_INVALID_ARGUMENT    # no sink
+    assert lib.q4_probe_lds(0x1000, 0, 256, 0x2000, None) == L.ERR_INVALID_ARGUMENT   # no iterations
+    assert lib.q4_probe_lds(0x1000, 10, 0, 0x2000, None) == L.ERR_INVALID_ARGUMENT    # no workgroups
+    assert b"q4_probe_lds" in lib.q4_last_error()
+
+
 def test_path_selection_and_workspace(pkg):
     lib = pkg._lib.load()
     L = pkg._lib
