@@ -153,3 +153,27 @@ def test_cfg5_wqlinear_module_mistral(pkg, oracle, gpu, K, N):
         torch.cuda.synchronize()
         _rows_check(oracle, x, w, got, "f16", np.arange(min(M, 24)))
     assert tuple(layer.qweight.shape) == (K, N // 8)
+
+
+def test_prefill_activation_matrix_beyond_4gb_runs_in_row_blocks(pkg, gpu):
+    """The prefill kernel addresses activations through 32-bit byte offsets; a matrix of more than
+    4 GB goes through the launcher's row blocks.  Rows on both sides of the block boundary and at
+    both ends must agree with what the same rows give on their own (a split-K launch there: same
+    fp16 weights, another fp32 summation order)."""
+    K, N = 4096, 128
+    M = 524032 + 100  # the first block is 524032 rows at K = 4096
+    g = torch.Generator(device=gpu).manual_seed(11)
+    qweight = torch.randint(-(2**31), 2**31 - 1, (K // 8, N), dtype=torch.int64, device=gpu, generator=g).to(torch.int32)
+    qzeros = torch.randint(-(2**31), 2**31 - 1, (K // 128, N // 8), dtype=torch.int64, device=gpu, generator=g).to(torch.int32)
+    scales = (torch.rand((K // 128, N), device=gpu, generator=g) * 0.019 + 0.001).half()
+    w = pkg.ops.make_packed(qweight, qzeros, scales, None, 128, 0)
+    x = torch.empty((M, K), dtype=torch.float16, device=gpu)
+    x.normal_(generator=g)
+    y = pkg.ops.linear(w, x)
+    torch.cuda.synchronize()
+    for lo, hi in [(0, 200), (524032 - 150, 524032 + 100), (M - 100, M)]:
+        ref = pkg.ops.linear(w, x[lo:hi].contiguous(), path=2).float()
+        err = float((y[lo:hi].float() - ref).abs().max() / ref.abs().max())
+        assert err <= TOL, (lo, hi, err)
+    del x, y
+    torch.cuda.empty_cache()
