@@ -200,46 +200,34 @@ static GemvConfig pick_config(const q4_weight* w, int M, bool gate_up, bool allo
     c.wcol = 2;
   const bool act = w->layout == Q4_LAYOUT_GPTQ && w->g_idx != nullptr;
   if (act) {
-    // Act-order: the kernel is bound by its per-weight table lookups (VALU + LDS), wants two
-    // 512-thread workgroups per CU and builds the table of all groups once per workgroup.
-    // Eight waves along K share table and slab; from 192 column tiles on (128 from 12 rows on)
-    // two column tiles of four waves do.  The split count aims at 448 workgroups within the
-    // LDS budget; with 12 rows or more, when the slab leaves room for one workgroup per CU
-    // only, a single round of at most 256 is taken instead if K splits that way.  Fitted on a
-    // sweep of 14 layer shapes x M = 1..16 on MI355X: 3.4 % above the best measured
-    // configuration on average (the rule before: 10 %; 11008 x 4096 at M = 4: 24.0 -> 19.2 us,
-    // 8192 x 28672 at M = 4: 64.7 -> 47.7 us, 4096 x 28672 at M = 8: 37.8 -> 28.7 us).
-    const int n64 = w->N / 64;
+    // Act-order: the kernel is bound by its per-weight table lookups (VALU + LDS), not by
+    // memory, and keeps no activation slab (its lanes fetch their activations themselves), so
+    // its LDS use - the table of all groups for 64 columns and the g_idx slice - is the same
+    // for every M.  Eight waves along K share the table; the split count aims at two workgroups
+    // per CU (512; 256 when the table leaves room for one) and is charged the imbalance of
+    // its K deal.  Against a sweep of 7 layer shapes x M = 1, 4, 16 x every (column waves,
+    // K waves, splits) on MI355X this rule is 4 % above the best measured configuration on
+    // average (worst: 8192 x 10240 and 4096 x 11008 at M = 1, 11-12 %, where four-wave
+    // workgroups in more splits win).
+    c.wcol = 1;
+    c.wk = chunks >= 8 ? 8 : c.wk;
     const long table1 = (long)w->num_groups * 64 * 4;
-    c.wcol = (w->N % 128 == 0 && (n64 >= 192 || (M >= 12 && n64 >= 128)) && 2 * table1 <= 64 * 1024) ? 2 : 1;
-    c.wk = c.wcol == 2 ? 4 : (chunks >= 8 ? 8 : c.wk);
-    const int tiles = (w->N / (64 * c.wcol)) * mchunks;
+    const int tiles = (w->N / 64) * mchunks;
     const int max_dv = chunks / c.wk;
-    auto lds_bytes = [&](int dv) {
-      const long kr = (long)((chunks + dv - 1) / dv) * 128;
-      return (long)rows * (kr * 2 + 16) + kr * 2 + table1 * c.wcol + 32;
-    };
-    const long lds_limit = 160 * 1024 - 1024;
+    auto lds_bytes = [&](int dv) { return (long)((chunks + dv - 1) / dv) * 256 + table1 + 32; };
     int best_dv = max_dv;
     double best = -1.0;
     for (int dv = 1; dv <= max_dv; ++dv) {
       if (lds_bytes(dv) > 150000) continue;
+      const double slots = lds_bytes(dv) > 80 * 1024 ? 256.0 : 512.0;
       const double wgs = (double)tiles * dv;
-      double cost = wgs >= 448.0 ? wgs / 448.0 : 448.0 / wgs;
-      if (chunks % (dv * c.wk) != 0) cost *= 1.15;
-      if (lds_bytes(dv) > 80 * 1024) cost *= 1.5;  // one workgroup per CU: half the waves to hide the lookups
-      if (best < 0.0 || cost < best) {
+      double cost = wgs >= slots ? wgs / slots : slots / wgs;
+      const int per_wave = (chunks + dv * c.wk - 1) / (dv * c.wk);  // chunks of the busiest wave
+      cost *= (double)per_wave * dv * c.wk / chunks;
+      if (slots < 512.0) cost *= 1.5;  // one workgroup per CU: half the waves to hide the lookups
+      if (best < 0.0 || cost <= best) {
         best = cost;
         best_dv = dv;
-      }
-    }
-    if (M >= 12 && lds_bytes(best_dv) > 80 * 1024) {
-      for (int dv = best_dv - 1; dv >= 1; --dv) {
-        const long wgs = (long)tiles * dv;
-        if (wgs > 256) continue;
-        if (wgs < 224 || lds_bytes(dv) > lds_limit) break;
-        best_dv = dv;
-        break;
       }
     }
     c.splits = best_dv;
@@ -367,7 +355,7 @@ static void launch_rmax(const q4_weight* w, const GemvParams& gp, int words, dim
   if (w->layout == Q4_LAYOUT_AWQ) {
     launch_kernel(gemv_awq_kernel<DTYPE, RMAX>, gp, grid, block, smem, stream);
   } else if (w->g_idx != nullptr) {
-    launch_kernel(gemv_gptq_act_kernel<DTYPE, RMAX>, gp, grid, block, smem, stream);
+    launch_kernel(gemv_gptq_act_kernel<DTYPE, RMAX, false, true>, gp, grid, block, smem, stream);
   } else if (gs == 128) {
     if (words == 4) launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, true, 4>, gp, grid, block, smem, stream);
     else if (words == 2) launch_kernel(gemv_gptq_kernel<DTYPE, RMAX, 4, true, 2>, gp, grid, block, smem, stream);
@@ -432,6 +420,10 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
               cfg.splits, w->K, w->N);
     return Q4_ERR_INVALID_ARGUMENT;
   }
+  if (w->g_idx != nullptr && (cfg.wcol & (cfg.wcol - 1)) != 0) {
+    set_error("q4_linear(gemv): the act-order kernel takes 1, 2 or 4 column waves (wcol=%d)", cfg.wcol);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
   if (cfg.rows_per_block != 16 && !(cfg.rows_per_block == 32 && contiguous && gate_up_act == 0 && cfg.words == 4)) {
     set_error("q4_linear(gemv): %d rows per workgroup need the contiguous-group kernel with 64-column waves",
               cfg.rows_per_block);
@@ -450,7 +442,9 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   // kernel: rows kq, kq + 4, ..)
   const int rmax = diag ? (rows <= 4 ? 1 : 2) : (rpb == 32 ? 8 : (M <= 1 ? 1 : (M <= 2 ? 2 : 4)));
   const int nt = awq ? 16 : cfg.words;
-  const size_t slab_bytes = ((size_t)rows * slab_stride * (wave_slab ? cfg.wcol * cfg.wk : 1) + 15) & ~(size_t)15;
+  // act-order: no slab, the lanes fetch their activations themselves
+  const bool x_direct = act;
+  const size_t slab_bytes = x_direct ? 0 : ((size_t)rows * slab_stride * (wave_slab ? cfg.wcol * cfg.wk : 1) + 15) & ~(size_t)15;
   size_t smem = slab_bytes + (lean ? 512 : 0);  // lean: a block of zeros behind the slab
   if (act) smem += (((size_t)KR * 2 + 15) & ~(size_t)15) + (size_t)w->num_groups * 64 * cfg.wcol * 4;
   const size_t red = (size_t)(cfg.wk - 1) * cfg.wcol * nt * rmax * 64 * sizeof(float);

@@ -790,8 +790,13 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
 // ---------------------------------------------------------------------------------------
 // GPTQ with g_idx (act-order), fp16.  LDS: [slab][g_idx slice as uint16][table G x tile_cols].
 // Table entry (g, column) = fp16 scale | fp16 -(1024 + zero) << 16.
-template <int DTYPE, int RMAX, bool MOE = false>
-__global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
+// XDIRECT: no activation slab.  A lane fetches the 16 bytes of its (row, K block) per 32-row step
+// from global memory (the activations stay in L2) beside its weight words, so the LDS a
+// workgroup needs does not grow with the rows: this kernel is bound by the per-weight work,
+// not by memory, and what it wants is resident waves.
+template <int DTYPE, int RMAX, bool MOE = false, bool XDIRECT = false>
+__global__ __launch_bounds__(512, 4) void gemv_gptq_act_kernel(GemvParams gp) {
+  static_assert(!(MOE && XDIRECT), "grouped launches stage their (mapped) rows in LDS");
   extern __shared__ __align__(16) unsigned char smem[];
   const int32_t* moe_rows = nullptr;
   if constexpr (MOE) {
@@ -804,8 +809,18 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
   const int nsteps = d.KW / 32;
   constexpr int PF = 2;  // 32-row steps of weight loads in flight per wave
 
+  const bool row_live = d.j < d.mloc;
   SlabStager<true> slab;
-  slab.issue(gp, d, moe_rows);
+  if constexpr (!XDIRECT) slab.issue(gp, d, moe_rows);
+  // XDIRECT: the lane's activations of a step, issued ahead of the weight words they meet
+  // (memory returns in issue order: an L2 hit must not queue behind the weight stream)
+  const uint16_t* x_lane = (const uint16_t*)p.x + (size_t)(d.mb + (row_live ? d.j : 0)) * p.K + d.kw0 + d.kq * 8;
+  uint4_t aq[PF] = {};
+  auto load_x = [&](int st) {
+    uint4_t v = {0u, 0u, 0u, 0u};
+    if (row_live) v = *(const uint4_t*)(x_lane + st * 32);
+    return v;
+  };
 
   const char* wbase = (const char*)(p.qweight + (size_t)(d.kw0 / 8) * N);
   const uint32_t w_lane = ((uint32_t)d.kq * (uint32_t)N + (uint32_t)nl) * 4u;
@@ -816,16 +831,39 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
   };
 #pragma unroll
   for (int b = 0; b < PF; ++b)
-    if (b < nsteps) wq[b] = load_step(b);
+    if (b < nsteps) {
+      if constexpr (XDIRECT) aq[b] = load_x(b);
+      wq[b] = load_step(b);
+    }
 
-  slab.store(gp, d, smem);
+  if constexpr (!XDIRECT) slab.store(gp, d, smem);
 
-  // ---- g_idx slice of this workgroup, clamped to the table, as uint16
+  // ---- g_idx slice of this workgroup, clamped to the table, as uint16; four entries per
+  // thread and load, up to four loads in flight (a loop of dependent single loads costs one
+  // memory round trip per iteration: 14 of them for a 7168-row range)
   uint16_t* gidx_s = (uint16_t*)(smem + gp.slab_bytes);
-  for (int i = d.tid; i < d.KR; i += d.nthreads) {
-    int g = p.g_idx[d.kwg0 + i];
-    g = min(max(g, 0), p.num_groups - 1);
-    gidx_s[i] = (uint16_t)g;
+  constexpr int PU = 4;
+  {
+    const int32_t* gsrc = p.g_idx + d.kwg0;
+    const int quads = d.KR >> 2;
+    const int gmax = p.num_groups - 1;
+    for (int i0 = d.tid; i0 < quads; i0 += PU * d.nthreads) {
+      uint4_t v[PU];
+#pragma unroll
+      for (int u = 0; u < PU; ++u) {
+        const int i = i0 + u * d.nthreads;
+        if (i < quads) v[u] = *(const uint4_t*)(gsrc + 4 * i);
+      }
+#pragma unroll
+      for (int u = 0; u < PU; ++u) {
+        const int i = i0 + u * d.nthreads;
+        if (i < quads) {
+          const uint32_t g0 = (uint32_t)min(max((int)v[u].x, 0), gmax), g1 = (uint32_t)min(max((int)v[u].y, 0), gmax);
+          const uint32_t g2 = (uint32_t)min(max((int)v[u].z, 0), gmax), g3 = (uint32_t)min(max((int)v[u].w, 0), gmax);
+          *(uint2_t*)(gidx_s + 4 * i) = uint2_t{g0 | (g1 << 16), g2 | (g3 << 16)};
+        }
+      }
+    }
   }
   // ---- scale / zero table of the workgroup's columns, all groups
   uint32_t* table = (uint32_t*)(smem + gp.slab_bytes + ((gp.kr_max * 2 + 15) & ~15));
@@ -833,39 +871,67 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
   {
     const int nbase = d.tile * tc;
     const int words_per_row = tc >> 3;  // one qzeros word covers 8 columns
-    for (int i = d.tid; i < p.num_groups * words_per_row; i += d.nthreads) {
-      const int g = i / words_per_row;
-      const int c8 = i - g * words_per_row;
-      const uint32_t z8 = gptq_zero_plus_one(p.qzeros[(size_t)g * (N >> 3) + (nbase >> 3) + c8]);
-      const uint4_t s8 = *(const uint4_t*)(p.scales + (size_t)g * N + nbase + c8 * 8);
-      const uint32_t su[4] = {s8.x, s8.y, s8.z, s8.w};
-      uint32_t e[8];
+    const int items = p.num_groups * words_per_row;
+    for (int i0 = d.tid; i0 < items; i0 += PU * d.nthreads) {
+      uint32_t zr[PU];
+      uint4_t sr[PU];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const uint32_t s16 = (u & 1) ? (su[u >> 1] >> 16) : (su[u >> 1] & 0xFFFFu);
-        const uint32_t z = (z8 >> (4 * u)) & 0xFu;
-        e[u] = s16 | ((0xE400u | z) << 16);
+      for (int u = 0; u < PU; ++u) {
+        const int i = i0 + u * d.nthreads;
+        if (i < items) {
+          const int g = i / words_per_row;
+          const int c8 = i - g * words_per_row;
+          zr[u] = p.qzeros[(size_t)g * (N >> 3) + (nbase >> 3) + c8];
+          sr[u] = *(const uint4_t*)(p.scales + (size_t)g * N + nbase + c8 * 8);
+        }
       }
-      uint4_t* dst = (uint4_t*)(table + (size_t)g * tc + c8 * 8);
-      dst[0] = uint4_t{e[0], e[1], e[2], e[3]};
-      dst[1] = uint4_t{e[4], e[5], e[6], e[7]};
+#pragma unroll
+      for (int u = 0; u < PU; ++u) {
+        const int i = i0 + u * d.nthreads;
+        if (i < items) {
+          const int g = i / words_per_row;
+          const int c8 = i - g * words_per_row;
+          const uint32_t z8 = gptq_zero_plus_one(zr[u]);
+          const uint32_t su[4] = {sr[u].x, sr[u].y, sr[u].z, sr[u].w};
+          uint32_t e[8];
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            const uint32_t s16 = (q & 1) ? (su[q >> 1] >> 16) : (su[q >> 1] & 0xFFFFu);
+            const uint32_t z = (z8 >> (4 * q)) & 0xFu;
+            e[q] = s16 | ((0xE400u | z) << 16);
+          }
+          uint4_t* dst = (uint4_t*)(table + (size_t)g * tc + c8 * 8);
+          dst[0] = uint4_t{e[0], e[1], e[2], e[3]};
+          dst[1] = uint4_t{e[4], e[5], e[6], e[7]};
+        }
+      }
     }
   }
   __syncthreads();
 
-  const bool row_live = d.j < d.mloc;
   const unsigned char* a_base =
       smem + (size_t)d.j * gp.slab_stride + (size_t)(d.kwo + d.kq * 8) * 2;
   const uint16_t* g_base = gidx_s + d.kwo + d.kq * 8;
-  const uint32_t* t_lane = table + d.wc * 64 + 4 * d.j;
+  const unsigned char* t_lane = (const unsigned char*)(table + d.wc * 64 + 4 * d.j);
+  // a table row is 64 or 128 columns of 4 bytes: group -> byte offset is a shift (a 32-bit
+  // integer multiply issues at a quarter of the rate)
+  const int row_shift = __builtin_ctz((unsigned)tc) + 2;
 
   const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   float4_t acc[4] = {zero4, zero4, zero4, zero4};
   const SpliceConsts splice = splice_consts();
 
-  auto process_step = [&](int st, const uint4_t w) {
+  auto process_step = [&](int st, const uint4_t w, const uint4_t xa) {
     uint4_t a = {0u, 0u, 0u, 0u};
-    if (row_live) a = *(const uint4_t*)(a_base + (size_t)st * 64);
+    if constexpr (XDIRECT) {
+      // K order [0,4,1,5,2,6,3,7] of the splice
+      a.x = __builtin_amdgcn_perm(xa.z, xa.x, 0x05040100u);
+      a.y = __builtin_amdgcn_perm(xa.z, xa.x, 0x07060302u);
+      a.z = __builtin_amdgcn_perm(xa.w, xa.y, 0x05040100u);
+      a.w = __builtin_amdgcn_perm(xa.w, xa.y, 0x07060302u);
+    } else {
+      if (row_live) a = *(const uint4_t*)(a_base + (size_t)st * 64);
+    }
     // groups of the 8 rows of this lane's K block, then their table rows (4 columns each)
     const uint4_t g8 = *(const uint4_t*)(g_base + st * 32);
     const uint32_t gw[4] = {g8.x, g8.y, g8.z, g8.w};
@@ -873,7 +939,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       const uint32_t g = (r & 1) ? (gw[r >> 1] >> 16) : (gw[r >> 1] & 0xFFFFu);
-      const uint4_t row = *(const uint4_t*)(t_lane + (size_t)g * tc);
+      const uint4_t row = *(const uint4_t*)(t_lane + (g << row_shift));
       e[r][0] = row.x; e[r][1] = row.y; e[r][2] = row.z; e[r][3] = row.w;
     }
     const uint32_t words[4] = {w.x, w.y, w.z, w.w};
@@ -892,9 +958,14 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
         if constexpr (DTYPE == Q4_DTYPE_F16) {
           b[pr] = as_u32(dq * as_half2(s2));  // one fp16 rounding, as the reference
         } else {
-          // bf16: the exact fp32 product, rounded once
-          const half2_t sc = as_half2(s2);
-          b[pr] = (uint32_t)f32_to_bf16_rne((float)dq.x * (float)sc.x) | ((uint32_t)f32_to_bf16_rne((float)dq.y * (float)sc.y) << 16);
+          // bf16: the exact fp32 products (mixed-precision multiplies that read the fp16 halves
+          // where they lie: no scale pair needed), rounded once by the packed convert
+          // (the compiler would emit two converts and a multiply per weight instead)
+          const uint32_t dqu = as_u32(dq);
+          float2_t f;
+          asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[0,0,0] op_sel_hi:[1,1,0]" : "=v"(f.x) : "v"(dqu), "v"(ea));
+          asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,1,0]" : "=v"(f.y) : "v"(dqu), "v"(eb));
+          b[pr] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
         }
       }
       // b is in K order [0,4,1,5,2,6,3,7], the order of the staged activations
@@ -911,8 +982,11 @@ __global__ __launch_bounds__(512) void gemv_gptq_act_kernel(GemvParams gp) {
     for (int b = 0; b < PF; ++b) {
       const int st = s0 + b;
       if (st < nsteps) {
-        process_step(st, wq[b]);
-        if (st + PF < nsteps) wq[b] = load_step(st + PF);
+        process_step(st, wq[b], aq[b]);
+        if (st + PF < nsteps) {
+          if constexpr (XDIRECT) aq[b] = load_x(st + PF);
+          wq[b] = load_step(st + PF);
+        }
       }
     }
   }
