@@ -105,10 +105,12 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   // AWQ and act-order: the decode kernels take any M in row chunks of 16; the MFMA kernel
   // that unpacks the weights into LDS (split-K when its tile grid is small) takes over where
   // it measured faster on MI355X.
-  // Act-order: from M = 17 on when its parameter table fits in LDS (8192 x 10240: 57 against
-  // 67 us at M = 24, 52 against 140 us at M = 64; the kernel's time is flat in M up to 128
-  // rows), from about M = 48 on when it has to gather scales and zero points from global
-  // memory (~2x slower per tile).
+  // Act-order: from M = 33 on when its parameter table fits in LDS (two 16-row blocks of the
+  // decode kernel, which is flat in M within a block, against the MFMA kernel, flat in M up to
+  // 128 rows, us at M = 32: 4096 x 4096 14.2 / 20.3, 14336 x 4096 27.0 / 43.4, 8192 x 10240
+  // 41.6 / 56.4, 28672 x 8192 92.7 / 153; at M = 48 the three blocks win on some shapes, 18.5 /
+  // 21.3 and 45.8 / 55.5, and lose on others, 46.6 / 42.7 and 182 / 155), from about M = 48 on
+  // when it has to gather scales and zero points from global memory (~2x slower per tile).
   // AWQ: up to 8 rows the decode kernel that feeds the words to the MFMA as stored; from 9 rows on
   // the MFMA kernel that unpacks them in registers wherever it applies (split-K on small tile
   // grids, flat in M up to 32 rows: 17.4 against 28.3 us for 4096 x 14336 at M = 16, 17.9 against
@@ -117,7 +119,7 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   // with every row, up to the M at which the kernel that unpacks through LDS measured faster:
   // 4096 x 4096 9, 4096 x 6144 14, 5120 x 5120 16, 11008 x 4096 10; above 16 for the larger
   // layers; 28672 x 8192 and 8192 x 28672 up to 32 rows.
-  bool small = M <= 16 || (w->layout == Q4_LAYOUT_GPTQ && M <= 48 && !gemm_act_order_table(w));
+  bool small = M <= 16 || (w->layout == Q4_LAYOUT_GPTQ && (M <= 32 || (M <= 48 && !gemm_act_order_table(w))));
   if (w->layout == Q4_LAYOUT_AWQ) {
     int first_gemm_m = 17;
     if (weights >= (1L << 27)) first_gemm_m = 33;

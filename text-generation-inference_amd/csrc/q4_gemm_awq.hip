@@ -76,8 +76,14 @@ constexpr int kActNarrowGroupBytes = kABN * 3;  // 128 fp16 scales, then 128 zer
 // MOE: grouped launch, blockIdx.y is the expert; its row count is read from device memory, so
 // the grid covers the largest possible count and surplus workgroups leave at once.
 template <int DTYPE, int MODE, bool MOE = false>
-__global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
+__global__ __launch_bounds__(MODE == kModeAwq ? 256 : 512, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   constexpr bool ACT = MODE != kModeAwq;
+  // AWQ: 4 waves, 2 x 2, a 64 x 64 block each.  Act-order: 8 waves, 4 x 2, a 32 x 64 block each: the
+  // parameter table leaves room for one workgroup per CU, and a single wave per SIMD cannot hide
+  // its own LDS and unpack latencies behind its MFMAs; two can hide each other's.
+  constexpr int WAVES = ACT ? 8 : 4;
+  constexpr int NTH = 64 * WAVES;
+  constexpr int MT = ACT ? 1 : 2;  // MFMA row tiles per wave
   int moe_row0 = 0;
   if constexpr (MOE) {
     moe_row0 = moe_enter(gp.p, gp.moe, blockIdx.y);
@@ -87,7 +93,7 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   constexpr int GROUP_BYTES = MODE == kModeActWide ? kActWideGroupBytes : kActNarrowGroupBytes;
   constexpr int A_TILE = kABM * kAUnits * 16;   // bytes
   constexpr int B_TILE = (kABK / 8) * kABN * 16;
-  constexpr int A_LOADS = kABM * (kABK / 8) / 256;  // 16-byte activation loads per thread
+  constexpr int A_LOADS = kABM * (kABK / 8) / NTH;  // 16-byte activation loads per thread
   extern __shared__ __align__(16) unsigned char smem[];  // [A0][A1][B0][B1]
   const Problem& p = gp.p;
   const int tid = threadIdx.x;
@@ -117,37 +123,33 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
 
   // ---- producer state
   // AWQ: threads 0..127 own K block pb (8 rows) x word pc (8 columns).
-  // act-order: every thread owns column pn and K blocks pkb0, pkb0 + 2, pkb0 + 4, pkb0 + 6.
+  // act-order: wave w owns K block w (8 rows), its lane pq the two adjacent columns 2 pq, 2 pq + 1:
+  // one 8-byte load fetches the two packed words and one LDS read per row the parameters of both
+  // columns; the rows' groups are the same for the whole wave.
   const bool producer = ACT || tid < 128;
   const int pb = (tid >> 4) & 7;
   const int pc = tid & 15;
-  const int pn = tid & 127;
-  const int pkb0 = __builtin_amdgcn_readfirstlane(tid >> 7);  // wave-uniform
-  const uint32_t* wsrc = ACT ? p.qweight + (size_t)pkb0 * N + n0 + pn
+  const int pq = lane;
+  const int pkb = wave;
+  const uint32_t* wsrc = ACT ? p.qweight + (size_t)pkb * N + n0 + 2 * pq
                              : p.qweight + (size_t)(pb * 8) * NC + (n0 >> 3) + pc;
-  uint32_t braw[8];  // AWQ: 8 rows of one word column; act-order: 4 words (K blocks)
+  uint32_t braw[8];  // AWQ: 8 rows of one word column
   uint4_t sraw;      // AWQ: 8 fp16 scales of the word's columns
   uint32_t zraw;     // AWQ: 8 zero-point nibbles
-  int graw[4][8];    // act-order table modes: groups of the thread's 32 rows
-  // The groups are the same in every lane, but they are wanted in vector registers (LDS
-  // addresses are per lane): an offset the compiler cannot see through keeps the loads
-  // and the address arithmetic on the vector unit instead of a detour through scalars.
-  int lane_zero = 0;
-  asm volatile("" : "+v"(lane_zero));
-  // act-order: word i of the thread (K block pkb0 + 2 i) and, in table modes, its rows' groups
-  auto load_b_word = [&](int kt, int i) {
-    braw[i] = wsrc[(size_t)(kt * (kABK / 8) + 2 * i) * N];
+  // act-order: two register sets, the tile being unpacked and the one requested behind it
+  uint2_t bw[2];     // packed words of the thread's two columns
+  int gr[2][8];      // table modes: groups of the block's 8 rows
+  auto load_b_act = [&](int kt, auto st_c) {
+    constexpr int ST = decltype(st_c)::value;
+    bw[ST] = *(const uint2_t*)(wsrc + (size_t)(kt * (kABK / 8)) * N);
     if constexpr (TABLE) {
-      const int* gsrc = p.g_idx + kt * kABK + (pkb0 + 2 * i) * 8 + lane_zero;
+      const int* gsrc = p.g_idx + kt * kABK + pkb * 8;
 #pragma unroll
-      for (int r = 0; r < 8; ++r) graw[i][r] = gsrc[r];
+      for (int r = 0; r < 8; ++r) gr[ST][r] = gsrc[r];
     }
   };
   auto load_b = [&](int kt) {
-    if constexpr (ACT) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) load_b_word(kt, i);
-    } else if (producer) {
+    if (producer) {
 #pragma unroll
       for (int r = 0; r < 8; ++r) braw[r] = wsrc[(size_t)(kt * kABK + r) * NC];
       const int g = min((kt * kABK + pb * 8) / p.groupsize, p.num_groups - 1);
@@ -157,69 +159,90 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   };
   const unsigned char* table = smem + 2 * A_TILE + 2 * B_TILE;  // act-order table modes only
   const int last_group = p.num_groups - 1;
-  // The act-order producer works on one word (8 K rows of the thread's column) in three
-  // phases, so that the main loop can place MFMAs between them.
-  // Phase 1: the parameters of the word's 8 rows.  Wide table: ra = scale | -(1024 + zero) << 16.
-  // Otherwise ra = scale bits, rb = zero point.
-  auto word_params = [&](int kt, int i, uint32_t (&ra)[8], uint32_t (&rb)[8]) {
-    const int n = n0 + pn;
-    const int zshift = (n & 7) * 4;
-    const int k0 = kt * kABK + (pkb0 + 2 * i) * 8;
+  // The act-order producer works in three phases, so that the main loop can place MFMAs
+  // between them.
+  // Phase 1, once per tile: the parameters of the block's 8 rows for the two columns.  Wide
+  // table: a[r][t] = scale | -(1024 + zero) << 16 of column t.  Otherwise a[r][0] = the two
+  // fp16 scales, z[r] = the two zero points, one byte each.
+  struct ActRows {
+    uint32_t a[8][2];
+    uint32_t z[8];
+  };
+  auto tile_params = [&](int kt, auto st_c, ActRows& ar) {
+    constexpr int ST = decltype(st_c)::value;
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       if constexpr (TABLE) {
-        // a corrupt index stays inside the table: clamp to [0, groups - 1] in one instruction
-        int g;
-        asm("v_med3_i32 %0, %1, 0, %2" : "=v"(g) : "v"(graw[i][r]), "s"(last_group));
+        // a corrupt index stays inside the table
+        const int g = min(max(gr[ST][r], 0), last_group);
         if constexpr (MODE == kModeActWide) {
-          ra[r] = *(const uint32_t*)(table + g * GROUP_BYTES + 4 * pn);
+          const uint2_t e = *(const uint2_t*)(table + g * GROUP_BYTES + 8 * pq);
+          ar.a[r][0] = e.x; ar.a[r][1] = e.y;
         } else {
-          ra[r] = *(const uint16_t*)(table + g * GROUP_BYTES + 2 * pn);
-          rb[r] = table[g * GROUP_BYTES + 2 * kABN + pn];
+          ar.a[r][0] = *(const uint32_t*)(table + g * GROUP_BYTES + 4 * pq);
+          ar.z[r] = *(const uint16_t*)(table + g * GROUP_BYTES + 2 * kABN + 2 * pq);
         }
       } else {
-        int g = p.g_idx[k0 + r];
-        g = min(max(g, 0), p.num_groups - 1);
-        ra[r] = *(const uint16_t*)(p.scales + (size_t)g * N + n);
-        rb[r] = (gptq_zero_plus_one(p.qzeros[(size_t)g * NC + (n >> 3)]) >> zshift) & 0xFu;
+        int g = p.g_idx[kt * kABK + pkb * 8 + r];
+        g = min(max(g, 0), last_group);
+        ar.a[r][0] = *(const uint32_t*)(p.scales + (size_t)g * N + n0 + 2 * pq);
+        // the word holds 8 columns: this thread's two are one byte of it
+        const uint32_t zw = (gptq_zero_plus_one(p.qzeros[(size_t)g * NC + ((n0 + 2 * pq) >> 3)]) >> ((pq & 3) * 8)) & 0xFFu;
+        ar.z[r] = (zw & 0xFu) | ((zw & 0xF0u) << 4);
       }
     }
   };
-  // Phase 2: rows pr and pr + 4 share one splice (their nibbles sit 16 bits apart).
-  auto word_pair = [&](uint32_t w, int pr, const uint32_t (&ra)[8], const uint32_t (&rb)[8]) -> uint32_t {
+  // Phase 2: rows pr and pr + 4 of column t share one splice (their nibbles sit 16 bits apart).
+  auto word_pair = [&](uint32_t w, auto t_c, int pr, const ActRows& ar) -> uint32_t {
+    constexpr int T = decltype(t_c)::value;
     const uint32_t q2 = ((w >> (4 * pr)) & splice.mask_lo) | splice.magic;
-    half2_t s2, cz2;
+    uint32_t s2, cz2;
     if constexpr (MODE == kModeActWide) {
-      s2 = as_half2(__builtin_amdgcn_perm(ra[pr + 4], ra[pr], 0x05040100u));
-      cz2 = as_half2(__builtin_amdgcn_perm(ra[pr + 4], ra[pr], 0x07060302u));
+      s2 = __builtin_amdgcn_perm(ar.a[pr + 4][T], ar.a[pr][T], 0x05040100u);
+      cz2 = __builtin_amdgcn_perm(ar.a[pr + 4][T], ar.a[pr][T], 0x07060302u);
     } else {
-      s2 = as_half2(ra[pr] | (ra[pr + 4] << 16));
-      cz2 = as_half2(0xE400E400u | rb[pr] | (rb[pr + 4] << 16));
+      s2 = __builtin_amdgcn_perm(ar.a[pr + 4][0], ar.a[pr][0], (T & 1) ? 0x07060302u : 0x05040100u);
+      cz2 = 0xE400E400u | __builtin_amdgcn_perm(ar.z[pr + 4], ar.z[pr], 0x0C000C00u | (uint32_t)T | ((uint32_t)(4 + T) << 16));
     }
-    const half2_t dq = as_half2(q2) + cz2;  // exact q - z
+    const half2_t dq = as_half2(q2) + as_half2(cz2);  // exact q - z
     if constexpr (DTYPE == Q4_DTYPE_F16) {
-      return as_u32(dq * s2);  // one fp16 rounding
+      return as_u32(dq * as_half2(s2));  // one fp16 rounding
     } else {
-      const awq_float2_t f = {(float)dq.x * (float)s2.x, (float)dq.y * (float)s2.y};
+      // bf16: the exact fp32 product, one mixed-precision multiply per weight straight from the
+      // fp16 halves (the compiler would emit two converts and a multiply), rounded once
+      const uint32_t dqu = as_u32(dq);
+      awq_float2_t f;
+      asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[0,0,0] op_sel_hi:[1,1,0]" : "=v"(f.x) : "v"(dqu), "v"(s2));
+      asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,1,0] op_sel_hi:[1,1,0]" : "=v"(f.y) : "v"(dqu), "v"(s2));
       return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, awq_bf16x2_t));
     }
   };
-  // Phase 3: o holds rows (0,4),(1,5),(2,6),(3,7): back to natural K order, one 16-byte unit.
-  auto word_store = [&](int buf, int i, const uint32_t (&o)[4]) {
+  // Phase 3: o holds rows (0,4),(1,5),(2,6),(3,7) of column t: back to natural K order, one
+  // 16-byte unit.
+  auto word_store = [&](int buf, int t, const uint32_t (&o)[4]) {
     unsigned char* base = smem + 2 * A_TILE + buf * B_TILE;
     uint4_t unit;  // one byte permute per register
     unit.x = __builtin_amdgcn_perm(o[1], o[0], 0x05040100u);
     unit.y = __builtin_amdgcn_perm(o[3], o[2], 0x05040100u);
     unit.z = __builtin_amdgcn_perm(o[1], o[0], 0x07060302u);
     unit.w = __builtin_amdgcn_perm(o[3], o[2], 0x07060302u);
-    *(uint4_t*)(base + ((size_t)(pkb0 + 2 * i) * kABN + b_slot(pn)) * 16) = unit;
+    *(uint4_t*)(base + ((size_t)pkb * kABN + b_slot(2 * pq + t)) * 16) = unit;
   };
-  auto store_b_act_word = [&](int buf, int kt, int i) {
-    uint32_t ra[8], rb[8], o[4];
-    word_params(kt, i, ra, rb);
+  auto word_of = [&](const uint2_t& w, int t) { return t == 0 ? w.x : w.y; };
+  // whole tile at once (prologue only)
+  auto store_b_act = [&](int buf, int kt, auto st_c) {
+    constexpr int ST = decltype(st_c)::value;
+    ActRows ar;
+    tile_params(kt, st_c, ar);
+    auto one = [&](auto t_c) {
+      constexpr int T = decltype(t_c)::value;
+      uint32_t o[4];
 #pragma unroll
-    for (int pr = 0; pr < 4; ++pr) o[pr] = word_pair(braw[i], pr, ra, rb);
-    word_store(buf, i, o);
+      for (int pr = 0; pr < 4; ++pr) o[pr] = word_pair(word_of(bw[ST], T), t_c, pr, ar);
+      word_store(buf, T, o);
+    };
+    one(std::integral_constant<int, 0>{});
+    one(std::integral_constant<int, 1>{});
   };
   auto store_b_awq = [&](int buf) {
     if (!producer) return;
@@ -262,14 +285,6 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
     }
   };
 
-  auto store_b = [&](int buf, int kt) {
-    if constexpr (ACT) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) store_b_act_word(buf, kt, i);
-    } else {
-      store_b_awq(buf);
-    }
-  };
 
   // ---- activation tile: global -> registers -> LDS (natural K order)
   const uint16_t* xs = (const uint16_t*)p.x;
@@ -278,14 +293,14 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   if constexpr (MOE) {
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
-      const int row = min(m0 + ((tid + 256 * i) >> 3), M - 1);
+      const int row = min(m0 + ((tid + NTH * i) >> 3), M - 1);
       moe_xrow[i] = gp.moe.x_rows != nullptr ? gp.moe.x_rows[moe_row0 + row] : row;
     }
   }
   auto load_a = [&](int kt) {
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
-      const int u = tid + 256 * i;
+      const int u = tid + NTH * i;
       const int m = u >> 3, kb = u & 7;
       // rows past M re-read the last row, never stored
       const int row = MOE ? moe_xrow[i] : min(m0 + m, M - 1);
@@ -296,15 +311,15 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
     unsigned char* base = smem + buf * A_TILE;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
-      const int u = tid + 256 * i;
+      const int u = tid + NTH * i;
       const int m = u >> 3, kb = u & 7;
       *(uint4_t*)(base + (m * kAUnits + kb) * 16) = areg[i];
     }
   };
 
-  float16_t acc[2][2];
+  float16_t acc[MT][2];
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < MT; ++a)
 #pragma unroll
     for (int b = 0; b < 2; ++b)
 #pragma unroll
@@ -313,7 +328,7 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   if constexpr (TABLE) {
     // every group's parameters for this tile's 128 columns: 16 scale units + 16 zero words each
     unsigned char* tab = smem + 2 * A_TILE + 2 * B_TILE;
-    for (int u = tid; u < p.num_groups * 16; u += 256) {
+    for (int u = tid; u < p.num_groups * 16; u += NTH) {
       const int g = u >> 4, c = u & 15;
       const uint4_t s8 = *(const uint4_t*)(p.scales + (size_t)g * N + n0 + c * 8);
       const uint32_t zw = gptq_zero_plus_one(p.qzeros[(size_t)g * NC + (n0 >> 3) + c]);
@@ -338,20 +353,30 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
     }
     __syncthreads();
   }
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
   load_a(kt_begin);
-  load_b(kt_begin);
-  store_a(0);
-  store_b(0, kt_begin);
+  if constexpr (ACT) {
+    // set 1 takes the first tile, set 0 the second: iteration i of the loop unpacks set i & 1
+    load_b_act(kt_begin, I1{});
+    load_b_act(min(kt_begin + 1, last_tile), I0{});
+    store_a(0);
+    store_b_act(0, kt_begin, I1{});
+  } else {
+    load_b(kt_begin);
+    store_a(0);
+    store_b_awq(0);
+    load_b(min(kt_begin + 1, last_tile));
+  }
   load_a(min(kt_begin + 1, last_tile));
-  load_b(min(kt_begin + 1, last_tile));
   __syncthreads();
 
-  const int a_off = ((wm * 64 + j) * kAUnits + kq) * 16;
+  const int a_off = ((wm * 32 * MT + j) * kAUnits + kq) * 16;
   const int b_off[2] = {(kq * kABN + b_slot(wn * 64 + j)) * 16, (kq * kABN + b_slot(wn * 64 + 32 + j)) * 16};
 
-  auto read_frags = [&](const unsigned char* ab, const unsigned char* bb, int s, uint4_t (&af)[2], uint4_t (&bf)[2]) {
+  auto read_frags = [&](const unsigned char* ab, const unsigned char* bb, int s, uint4_t (&af)[MT], uint4_t (&bf)[2]) {
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) af[mt] = *(const uint4_t*)(ab + (mt * 32 * kAUnits + 2 * s) * 16);
+    for (int mt = 0; mt < MT; ++mt) af[mt] = *(const uint4_t*)(ab + (mt * 32 * kAUnits + 2 * s) * 16);
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) bf[nt] = *(const uint4_t*)(bb + b_off[nt] + (2 * s) * kABN * 16);
   };
@@ -362,19 +387,22 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
       c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
     }
   };
-  auto mfma_frags = [&](const uint4_t (&af)[2], const uint4_t (&bf)[2]) {
+  auto mfma_frags = [&](const uint4_t (&af)[MT], const uint4_t (&bf)[2]) {
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) mfma_one(af[mt], bf[nt], acc[mt][nt]);
   };
   auto mfma_step = [&](const unsigned char* ab, const unsigned char* bb, int s) {
-    uint4_t af[2], bf[2];
+    uint4_t af[MT], bf[2];
     read_frags(ab, bb, s, af, bf);
     mfma_frags(af, bf);
   };
 
-  for (int kt = kt_begin; kt < KT; ++kt) {
+  // One K tile.  ST: the act-order register set that holds the next tile's packed words (also
+  // the parity of the LDS buffer being multiplied).
+  auto tile_step = [&](int kt, auto st_c) {
+    constexpr int ST = decltype(st_c)::value;
     const int cur = (kt - kt_begin) & 1;
     const int kt1 = min(kt + 1, last_tile);
     const int kt2 = min(kt + 2, last_tile);
@@ -384,43 +412,49 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
     store_a(cur ^ 1);
     load_a(kt2);
     if constexpr (ACT) {
-      // one word of the next tile is unpacked in phases with one MFMA of this tile's K step
-      // between them (the order is pinned: the matrix pipe runs under the unpack even when
-      // the LDS table leaves room for a single workgroup per CU), then the word two tiles
-      // ahead is requested
-      static_assert(kABK / 16 == 4, "one producer word per MFMA K step");
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        uint4_t af[2], bf[2];
-        uint32_t ra[8], rb[8], o[4];
-        read_frags(ab, bb, s, af, bf);
-        word_params(kt1, s, ra, rb);
+      // the set unpacked in the previous tile is free: request the tile after the next
+      load_b_act(kt2, std::integral_constant<int, ST ^ 1>{});
+      // the next tile's parameters first, then half a column (two row pairs) per MFMA K step,
+      // unpacked in phases with this tile's MFMAs between them (the order is pinned)
+      static_assert(kABK / 16 == 4 && MT == 1, "half a producer column per MFMA K step");
+      ActRows ar;
+      // fragments one K step ahead
+      uint4_t af[2][MT], bf[2][2];
+      uint32_t o[4];
+      tile_params(kt1, st_c, ar);
+      read_frags(ab, bb, 0, af[0], bf[0]);
+      auto step = [&](auto s_c) {
+        constexpr int S = decltype(s_c)::value;
+        constexpr int P = S & 1;
+        constexpr int H = S & 1;  // which two row pairs of the column
+        using T = std::integral_constant<int, (S >> 1)>;
+        if constexpr (S < 3) read_frags(ab, bb, S + 1, af[P ^ 1], bf[P ^ 1]);
+        const uint32_t w = word_of(bw[ST], S >> 1);
         __builtin_amdgcn_sched_barrier(0);
-        mfma_one(af[0], bf[0], acc[0][0]);
+        mfma_one(af[P][0], bf[P][0], acc[0][0]);
         __builtin_amdgcn_sched_barrier(0);
-        o[0] = word_pair(braw[s], 0, ra, rb);
-        o[1] = word_pair(braw[s], 1, ra, rb);
+        o[2 * H] = word_pair(w, T{}, 2 * H, ar);
+        o[2 * H + 1] = word_pair(w, T{}, 2 * H + 1, ar);
         __builtin_amdgcn_sched_barrier(0);
-        mfma_one(af[0], bf[1], acc[0][1]);
+        mfma_one(af[P][0], bf[P][1], acc[0][1]);
         __builtin_amdgcn_sched_barrier(0);
-        o[2] = word_pair(braw[s], 2, ra, rb);
-        o[3] = word_pair(braw[s], 3, ra, rb);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_one(af[1], bf[0], acc[1][0]);
-        __builtin_amdgcn_sched_barrier(0);
-        word_store(cur ^ 1, s, o);
-        load_b_word(kt2, s);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_one(af[1], bf[1], acc[1][1]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+        if constexpr (H == 1) word_store(cur ^ 1, S >> 1, o);
+      };
+      step(std::integral_constant<int, 0>{});
+      step(std::integral_constant<int, 1>{});
+      step(std::integral_constant<int, 2>{});
+      step(std::integral_constant<int, 3>{});
     } else {
-      store_b(cur ^ 1, kt1);
+      store_b_awq(cur ^ 1);
       load_b(kt2);
 #pragma unroll
       for (int s = 0; s < kABK / 16; ++s) mfma_step(ab, bb, s);
     }
     __syncthreads();
+  };
+  for (int kt = kt_begin; kt < KT; kt += 2) {
+    tile_step(kt, I0{});
+    if (kt + 1 < KT) tile_step(kt + 1, I1{});
   }
 
   // ---- epilogue: register r of lane (j, kq) is row 8*(r/4) + 4*kq + r%4, column j
@@ -430,10 +464,10 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
     for (int nt = 0; nt < 2; ++nt) {
       const int n = n0 + wn * 64 + nt * 32 + j;
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
+      for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * 64 + mt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
+          const int m = m0 + wm * 32 * MT + mt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
           if (m < M) part[(size_t)m * N + n] = acc[mt][nt][r];
         }
       }
@@ -445,10 +479,10 @@ __global__ __launch_bounds__(256, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   for (int nt = 0; nt < 2; ++nt) {
     const int n = n0 + wn * 64 + nt * 32 + j;
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 64 + mt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
+        const int m = m0 + wm * 32 * MT + mt * 32 + 8 * (r >> 2) + 4 * kq + (r & 3);
         if (m < M) y[(size_t)m * N + n] = finish_output<DTYPE>(acc[mt][nt][r], p.bias, n);
       }
     }
@@ -555,7 +589,7 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
   const dim3 grid((unsigned)total, (unsigned)experts);
   auto launch = [&](auto k) {
     (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipLaunchKernelGGL(k, grid, dim3(256), smem, stream, gp);
+    hipLaunchKernelGGL(k, grid, dim3(mode == kModeAwq ? 256 : 512), smem, stream, gp);
   };
   auto launch_mode = [&](auto dt, auto grouped) {
     constexpr int DT = decltype(dt)::value;
