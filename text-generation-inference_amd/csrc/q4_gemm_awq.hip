@@ -5,23 +5,25 @@
 // rows that each belong to a different group.  In both cases the weight tile is unpacked
 // cooperatively into LDS (the classic dequantize-to-LDS stage) and both MFMA operands are
 // read from there:
-//   * workgroup = 4 waves in a 2 x 2 arrangement, tile 128 x 128, K tile 64; each wave owns
+//   * AWQ workgroup = 4 waves in a 2 x 2 arrangement, tile 128 x 128, K tile 64; each wave owns
 //     a 64 x 64 block = 2 x 2 MFMA tiles of v_mfma_f32_32x32x16 (64 accumulator VGPRs),
-//     so two or three workgroups share a CU and cover each other's barriers;
-//   * producer: thread t < 128 owns an 8-row x 1-word patch (8 rows of one K block, 8
+//     so two workgroups share a CU and cover each other's barriers;
+//   * AWQ producer: thread t < 128 owns an 8-row x 1-word patch (8 rows of one K block, 8
 //     columns).  One byte permute per row pair and byte puts the same nibble positions of
 //     two rows side by side, the mantissa splice turns them into halves, zero points are
 //     subtracted exactly and each weight is multiplied once by its fp16 scale (the
 //     reference's rounding).  The patch becomes eight 16-byte units (one per column,
 //     8 consecutive K values each) written to LDS at [K block][column];
-//   * act-order producer: every thread owns 4 packed words (8 K rows x 1 column each).  The
-//     groups of the 8 rows (g_idx[k], the same for every lane, requested one tile ahead)
-//     index a per-workgroup LDS table of all groups x the tile's 128 columns, filled once
-//     in the prologue, and scale and zero point are applied per weight -- no row of
-//     qweight is ever moved.  The table holds one 32-bit entry per group and column
-//     (fp16 scale | fp16 -(1024 + zero), one LDS read per row) for up to 184 groups, or
-//     an fp16 scale and a zero-point byte (two reads per row) for up to 245 groups;
-//     layers with more groups gather the two values per row from the checkpoint tensors;
+//   * act-order workgroup = 8 waves, 4 x 2, a 32 x 64 block each, same tile.  Producer: wave w
+//     owns K block w of the tile, its lanes two adjacent columns each (one 8-byte load for the
+//     two packed words).  The groups of the 8 rows (g_idx[k], the same for the whole wave,
+//     requested two tiles ahead) index a per-workgroup LDS table of all groups x the tile's
+//     128 columns, filled once in the prologue: one LDS read per row fetches the parameters of
+//     both columns, and scale and zero point are applied per weight -- no row of qweight is
+//     ever moved.  The table holds one 32-bit entry per group and column (fp16 scale | fp16
+//     -(1024 + zero)) for up to 184 groups, or an fp16 scale and a zero-point byte for up to
+//     245 groups; layers with more groups gather the two values per row from the checkpoint
+//     tensors;
 //   * LDS layouts: activations [row][K block] with the row stride padded to 9 units,
 //     weights [K block][column] with the low column bits XORed with the word index; both
 //     give conflict-free 128-bit fragment reads, and the swizzle spreads the AWQ
