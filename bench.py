@@ -86,6 +86,10 @@ def parse_args():
     ap.add_argument("--awq-probe", action="store_true",
                     help="a few prefill launches (M = --gemm-m) of the AWQ-layout kernel and of the GPTQ-layout kernel on "
                          "4096 x 14336, for counter runs under rocprofv3")
+    ap.add_argument("--act-probe", action="store_true",
+                    help="a few launches of the act-order kernels that read the checkpoint through g_idx: decode at "
+                         "M = 1 and 16 on 28672 x 8192, prefill (M = --gemm-m) on 8192 x 10240, for counter runs "
+                         "under rocprofv3")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="eager launches only (a 256 MiB copy kernel, then each decode shape and one GEMM), "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs; prints no JSON line")
@@ -397,6 +401,28 @@ def main():
         torch.cuda.synchronize()
         print("awq probe done: 6 launches each of the AWQ-layout and the GPTQ-layout prefill kernel, %d x %d, M=%d"
               % (K, N, Mg), file=sys.stderr)
+        return
+    if args.act_probe:
+        Kd, Nd = 28672, 8192
+        wd = [make_weights_variant(pkg, torch, dev, Kd, Nd, 5 + c, "act_order") for c in range(3)]
+        for Md in (1, 16):
+            xd = torch.randn((Md, Kd), device=dev, dtype=torch.float16)
+            yd = torch.empty((Md, Nd), device=dev, dtype=torch.float16)
+            for _ in range(4):
+                for w in wd:
+                    pkg.ops.linear(w, xd, None, out=yd)
+        torch.cuda.synchronize()
+        del wd
+        Kp, Np, Mg = 8192, 10240, args.gemm_m
+        wp = [make_weights_variant(pkg, torch, dev, Kp, Np, 9 + c, "act_order") for c in range(2)]
+        xg = torch.randn((Mg, Kp), device=dev, dtype=torch.float16)
+        yg = torch.empty((Mg, Np), device=dev, dtype=torch.float16)
+        for _ in range(3):
+            for w in wp:
+                pkg.ops.linear(w, xg, None, out=yg)
+        torch.cuda.synchronize()
+        print("act probe done: 12 decode launches each at M=1 and M=16 on %d x %d, 6 prefill launches at M=%d on %d x %d"
+              % (Kd, Nd, Mg, Kp, Np), file=sys.stderr)
         return
     if args.floor_probe:
         floor_probe(pkg, torch, lib, dev)
