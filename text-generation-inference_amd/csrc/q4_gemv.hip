@@ -122,7 +122,13 @@ static GemvConfig pick_config(const q4_weight* w, int M, bool gate_up, bool allo
       c.wcol = 2;
       c.wk = (M >= 4 && chunks % 8 == 0) ? 8 : 4;
       c.splits = 1;
-      // many rows: one slab per workgroup must fit LDS
+      // many rows: one slab per workgroup must fit LDS.  When K has to be split for that, four
+      // column tiles of four waves share each slab (8192 x 28672: 38.7 / 37.6 -> 30.2 / 31.3 us at
+      // M = 12 / 16, 5120 x 27648 at M = 16: 29.9 -> 23.0 us against two tiles of eight waves).
+      if ((long)rows * ((long)w->K * 2 + 16) > 150000 && w->N % 256 == 0 && chunks >= 8) {
+        c.wcol = 4;
+        c.wk = 4;
+      }
       while ((long)rows * ((long)w->K / c.splits * 2 + 16) > 150000 && c.splits * c.wk * 2 <= chunks) c.splits *= 2;
       return c;
     }
@@ -148,6 +154,57 @@ static GemvConfig pick_config(const q4_weight* w, int M, bool gate_up, bool allo
     if (M >= 4 && n64 >= 160 && chunks <= 32 && (long)rows * c.wk * ((long)((chunks + c.wk - 1) / c.wk) * 256 + 16) <= 150000)
       best = 1;
     c.splits = best;
+    if (M >= 4) {
+      // Four rows and more: the activation staging (per wave with one column wave, one slab per
+      // workgroup with several) decides how many workgroups a CU holds, and the rule above knows
+      // neither that nor rounds.  A small cost model fitted to sweeps on MI355X (us) searches every
+      // (column waves, K waves, splits): a launch floor, the 128-row x 64-column chunk-tiles the
+      // busiest CU walks (0.19 us each, up to 15 % more when fewer than 16 waves are resident
+      // there), 2.5 us per further round when its workgroups do not fit together, the staged
+      // activation bytes, the barrier of a shared slab, the slow start of 1024-thread workgroups
+      // and the split-K combine.  Its pick replaces the rule's only where it predicts 12 % or
+      // more: below that its error decides (measured on 11 layer shapes x M = 4..16: every pick
+      // with a smaller predicted gain was 10-23 % slower than the rule's; the ones taken are
+      // 8192 x 10240 17.5 / 18.7 / 24.5 -> 15.2 / 17.2 / 20.6 us at M = 4 / 8 / 16 and
+      // 28672 x 8192 38.8 / 34.2 / 47.6 -> 27.3 / 28.6 / 34.1 us at M = 6 / 8 / 16).
+      auto model_us = [&](int wcol, int wk, int dv) -> double {
+        if (n64 % wcol != 0 || wcol * wk > 16 || dv * wk > chunks) return -1.0;
+        const bool wave_slab = wcol == 1 || rows <= 2;
+        const int per_wave = (chunks + dv * wk - 1) / (dv * wk);
+        const int per_wg = (chunks + dv - 1) / dv;
+        const long lds = (wave_slab ? (long)rows * wcol * wk * (per_wave * 256 + 16) : (long)rows * (per_wg * 256 + 16)) + 512;
+        if (lds > 150000) return -1.0;
+        long res = (160 * 1024) / (lds + 1024);
+        if (res > 16 / (wcol * wk)) res = 16 / (wcol * wk);
+        if (res < 1) res = 1;
+        const long wgs = (long)(n64 / wcol) * dv;
+        const long per_cu = (wgs + 255) / 256;
+        const long waves = (per_cu < res ? per_cu : res) * wcol * wk;
+        const double occ = 1.0 + 0.3 * (waves < 16 ? 16 - waves : 0) / 16.0;
+        const long rounds = (per_cu + res - 1) / res;
+        double t = 3.5 + 0.19 * (double)per_cu * per_wave * wk * wcol * occ + 2.5 * (rounds - 1);
+        t += 0.015 * (double)per_cu * rows * per_wg * 256 / 1024.0;
+        if (!wave_slab) t += 1.5;
+        if (wcol * wk > 8) t += 1.2;
+        if (dv > 1) t += 2.0 + 0.3 * dv * (M / 16.0);
+        return t;
+      };
+      const double t_rule = best_cost >= 0.0 ? model_us(c.wcol, c.wk, c.splits) : -1.0;
+      double best_t = -1.0;
+      GemvConfig pick = c;
+      for (int wcol = 1; wcol <= 4; wcol *= 2)
+        for (int wk = 2; wk <= 16; wk *= 2)
+          for (int dv = 1; dv <= 32; ++dv) {
+            const double t = model_us(wcol, wk, dv);
+            if (t >= 0.0 && (best_t < 0.0 || t < best_t)) {
+              best_t = t;
+              pick.wcol = wcol;
+              pick.wk = wk;
+              pick.splits = dv;
+            }
+          }
+      if (best_t >= 0.0 && (t_rule < 0.0 || best_t < 0.88 * t_rule)) return pick;
+    }
     if (best_cost >= 0.0) return c;
     c.lean = 0;  // no split fits LDS: the kernel below, with its workgroup slab
   }
