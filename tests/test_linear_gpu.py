@@ -554,12 +554,20 @@ def test_act_order_bf16_small_m(pkg, oracle, gpu, K, N, M):
     _run(pkg, oracle, gpu, K, N, 128, M, dtype="bf16", act=True, seed=M + 2, path=2)
 
 
+@pytest.mark.parametrize("zeros", ["random", "one", "one_but_a_column"])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-def test_act_order_decode_one_hot_reads_weights_back(pkg, oracle, gpu, dtype):
-    """x = rows of the identity through the lookup decode kernel: the dequantized rows, bit for bit."""
+def test_act_order_decode_one_hot_reads_weights_back(pkg, oracle, gpu, dtype, zeros):
+    """x = rows of the identity through the lookup decode kernel: the dequantized rows, bit for bit.
+    The kernel takes a shorter loop when every zero point of a workgroup's 64 columns is the same
+    (symmetric quantization): random zero points, one zero point everywhere, and one zero point
+    except in a single (group, column) - whose column tile must take the general loop while its
+    neighbours take the short one."""
     K, N, gs = 1024, 512, 128
     bf = dtype == "bf16"
-    qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=11, sym=False, act_order=True)
+    qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=11, sym=(zeros != "random"), act_order=True)
+    if zeros == "one_but_a_column":
+        qz = qz.copy()
+        qz[5, 200 // 8] ^= np.int32(0x3 << (4 * (200 % 8)))  # group 5, column 200: stored zero 7 -> 4
     w = oracle.dequant_gptq(qw, qz, sc, gi, gs, dtype)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), gs, 0)
     ks = np.random.default_rng(2).choice(K, size=8, replace=False)

@@ -868,10 +868,13 @@ __global__ __launch_bounds__(512, 4) void gemv_gptq_act_kernel(GemvParams gp) {
   // ---- scale / zero table of the workgroup's columns, all groups
   uint32_t* table = (uint32_t*)(smem + gp.slab_bytes + ((gp.kr_max * 2 + 15) & ~15));
   const int tc = d.tile_cols;
+  uint32_t zref, zdiff;
   {
     const int nbase = d.tile * tc;
     const int words_per_row = tc >> 3;  // one qzeros word covers 8 columns
     const int items = p.num_groups * words_per_row;
+    zref = gptq_zero_plus_one(p.qzeros[nbase >> 3]);
+    zdiff = zref ^ ((zref & 0xFu) * 0x11111111u);
     for (int i0 = d.tid; i0 < items; i0 += PU * d.nthreads) {
       uint32_t zr[PU];
       uint4_t sr[PU];
@@ -892,6 +895,7 @@ __global__ __launch_bounds__(512, 4) void gemv_gptq_act_kernel(GemvParams gp) {
           const int g = i / words_per_row;
           const int c8 = i - g * words_per_row;
           const uint32_t z8 = gptq_zero_plus_one(zr[u]);
+          zdiff |= z8 ^ zref;
           const uint32_t su[4] = {sr[u].x, sr[u].y, sr[u].z, sr[u].w};
           uint32_t e[8];
 #pragma unroll
@@ -907,7 +911,11 @@ __global__ __launch_bounds__(512, 4) void gemv_gptq_act_kernel(GemvParams gp) {
       }
     }
   }
-  __syncthreads();
+  // One zero point for every group and column of the tile (symmetric quantization, the usual
+  // companion of act-order): the zero pair of a weight pair is then a constant and its byte
+  // permute drops out of the loop below (16 of ~137 vector instructions per 32-row step).
+  const bool one_zero = __syncthreads_or((int)(zdiff != 0u)) == 0;
+  const uint32_t c_const = 0xE400E400u | (zref & 0xFu) | ((zref & 0xFu) << 16);
 
   const unsigned char* a_base =
       smem + (size_t)d.j * gp.slab_stride + (size_t)(d.kwo + d.kq * 8) * 2;
@@ -921,7 +929,8 @@ __global__ __launch_bounds__(512, 4) void gemv_gptq_act_kernel(GemvParams gp) {
   float4_t acc[4] = {zero4, zero4, zero4, zero4};
   const SpliceConsts splice = splice_consts();
 
-  auto process_step = [&](int st, const uint4_t w, const uint4_t xa) {
+  auto process_step = [&](int st, const uint4_t w, const uint4_t xa, auto one_zero_c) {
+    constexpr bool ONE_ZERO = decltype(one_zero_c)::value;
     uint4_t a = {0u, 0u, 0u, 0u};
     if constexpr (XDIRECT) {
       // K order [0,4,1,5,2,6,3,7] of the splice
@@ -951,11 +960,11 @@ __global__ __launch_bounds__(512, 4) void gemv_gptq_act_kernel(GemvParams gp) {
         // rows pr and pr + 4 of the K block share one splice (nibbles 16 bits apart)
         // one byte permute each: the low halves (scales) and the high halves (-(1024 + z))
         const uint32_t ea = e[pr][t], eb = e[pr + 4][t];
-        const uint32_t s2 = __builtin_amdgcn_perm(eb, ea, 0x05040100u);
-        const uint32_t c2 = __builtin_amdgcn_perm(eb, ea, 0x07060302u);
+        const uint32_t c2 = ONE_ZERO ? c_const : __builtin_amdgcn_perm(eb, ea, 0x07060302u);
         const uint32_t q2 = ((words[t] >> (4 * pr)) & splice.mask_lo) | splice.magic;
         const half2_t dq = as_half2(q2) + as_half2(c2);  // exact q - z
         if constexpr (DTYPE == Q4_DTYPE_F16) {
+          const uint32_t s2 = __builtin_amdgcn_perm(eb, ea, 0x05040100u);
           b[pr] = as_u32(dq * as_half2(s2));  // one fp16 rounding, as the reference
         } else {
           // bf16: the exact fp32 products (mixed-precision multiplies that read the fp16 halves
@@ -977,19 +986,23 @@ __global__ __launch_bounds__(512, 4) void gemv_gptq_act_kernel(GemvParams gp) {
     }
   };
 
-  for (int s0 = 0; s0 < nsteps; s0 += PF) {
+  auto walk = [&](auto one_zero_c) {
+    for (int s0 = 0; s0 < nsteps; s0 += PF) {
 #pragma unroll
-    for (int b = 0; b < PF; ++b) {
-      const int st = s0 + b;
-      if (st < nsteps) {
-        process_step(st, wq[b], aq[b]);
-        if (st + PF < nsteps) {
-          if constexpr (XDIRECT) aq[b] = load_x(st + PF);
-          wq[b] = load_step(st + PF);
+      for (int b = 0; b < PF; ++b) {
+        const int st = s0 + b;
+        if (st < nsteps) {
+          process_step(st, wq[b], aq[b], one_zero_c);
+          if (st + PF < nsteps) {
+            if constexpr (XDIRECT) aq[b] = load_x(st + PF);
+            wq[b] = load_step(st + PF);
+          }
         }
       }
     }
-  }
+  };
+  if (one_zero) walk(std::true_type{});
+  else walk(std::false_type{});
 
   float out[4][RMAX];
 #pragma unroll
