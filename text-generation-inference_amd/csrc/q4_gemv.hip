@@ -189,6 +189,38 @@ static GemvConfig pick_config(const q4_weight* w, int M, bool gate_up, bool allo
         if (dv > 1) t += 2.0 + 0.3 * dv * (M / 16.0);
         return t;
       };
+      // Nine rows and more, and no single round of one-column-wave workgroups whose per-wave
+      // activations fit LDS: one round of 1024-thread workgroups, two column tiles x eight K
+      // waves (four x four next) around one shared slab.  Swept at M = 16 (us, this / the rule's
+      // choice): 13824 x 5120 16.9 / 21.3, 5120 x 13824 16.5 / 22.1, 8192 x 10240 19.5 / 24.6.
+      if (rows >= 9) {
+        bool one_round = false;
+        for (int dv = 1; dv * 8 <= chunks && (long)n64 * dv <= 256; ++dv)
+          if ((long)rows * 8 * (((chunks + dv * 8 - 1) / (dv * 8)) * 256 + 16) + 512 <= 150000) one_round = true;
+        if (!one_round) {
+          for (int wcol = 2; wcol <= 4; wcol *= 2) {
+            const int wk = 16 / wcol;
+            if (n64 % wcol != 0 || wk > chunks) continue;
+            int pick_dv = 0;
+            double pick_cost = -1.0;
+            for (int dv = 1; dv * wk <= chunks && (long)(n64 / wcol) * dv <= 256; ++dv) {
+              if ((long)rows * (((chunks + dv - 1) / dv) * 256 + 16) + 512 > 150000) continue;
+              const int per_wave = (chunks + dv * wk - 1) / (dv * wk);
+              const double cost = 256.0 / ((double)(n64 / wcol) * dv) * ((double)per_wave * dv * wk / chunks);
+              if (pick_cost < 0.0 || cost < pick_cost) {
+                pick_cost = cost;
+                pick_dv = dv;
+              }
+            }
+            if (pick_dv > 0) {
+              c.wcol = wcol;
+              c.wk = wk;
+              c.splits = pick_dv;
+              return c;
+            }
+          }
+        }
+      }
       const double t_rule = best_cost >= 0.0 ? model_us(c.wcol, c.wk, c.splits) : -1.0;
       double best_t = -1.0;
       GemvConfig pick = c;
