@@ -66,3 +66,26 @@ def test_lean_period_boundaries(pkg, oracle, gpu, chunks, M):
     _run(pkg, oracle, gpu, chunks * 128, 128, 128, M, sym=False, cfg=(1, 1, 1, 0), seed=chunks + M)
     if chunks >= 4:
         _run(pkg, oracle, gpu, chunks * 128, 128, 128, M, sym=False, cfg=(1, 2, 2, 0), seed=chunks + M + 1)
+
+
+@pytest.mark.parametrize("K,N", [(8192, 10240), (5120, 13824), (13824, 5120), (28672, 8192), (8192, 28672), (6656, 17920)])
+def test_large_layer_decode_decompositions_picked(pkg, gpu, K, N):
+    """The decompositions the picker takes for 4..16 rows on large layers (several column tiles
+    around one slab, 1024-thread workgroups, splits of an uneven K deal): one-hot rows read the
+    dequantized weights back bit for bit, and random activations agree with the prefill kernel."""
+    g = torch.Generator(device=gpu).manual_seed(K + N)
+    qweight = torch.randint(-(2**31), 2**31 - 1, (K // 8, N), dtype=torch.int64, device=gpu, generator=g).to(torch.int32)
+    qzeros = torch.randint(-(2**31), 2**31 - 1, (K // 128, N // 8), dtype=torch.int64, device=gpu, generator=g).to(torch.int32)
+    scales = (torch.rand((K // 128, N), device=gpu, generator=g) * 0.019 + 0.001).half()
+    w = pkg.ops.make_packed(qweight, qzeros, scales, None, 128, 0)
+    dense = pkg.ops.dequantize(w)
+    rows = torch.randint(0, K, (16,), device=gpu, generator=g)
+    for M in (4, 6, 9, 12, 16):
+        assert pkg.ops.select_path(w, M) == "gemv"
+        x = torch.zeros((M, K), dtype=torch.float16, device=gpu)
+        x[torch.arange(M, device=gpu), rows[:M]] = 1.0
+        assert torch.equal(pkg.ops.linear(w, x), dense[rows[:M]]), f"one-hot rows, M={M}"
+        x = torch.randn((M, K), dtype=torch.float16, device=gpu, generator=g)
+        y, ref = pkg.ops.linear(w, x).float(), pkg.ops.linear(w, x, path=2).float()
+        err = float((y - ref).abs().max() / ref.abs().max())
+        assert err <= 2e-3, f"M={M}: {err:.2e}"
