@@ -49,7 +49,10 @@ extern "C" {
 #define Q4_PATH_GEMM 2    /* dequant-to-LDS + MFMA GEMM, prefill (large M) */
 #define Q4_PATH_GENERIC 3 /* shape-agnostic kernel for unaligned K / N */
 
-/* Problem description shared by every entry point. */
+/* Problem description shared by every entry point.  All device pointers handed to this library
+ * (the four tensors below, activations, outputs, workspaces) must be 16-byte aligned, a bias
+ * 2-byte aligned: the kernels fetch with 16-byte loads, and the entry points refuse anything
+ * else with Q4_ERR_INVALID_ARGUMENT. */
 typedef struct q4_weight {
   const uint32_t* qweight; /* packed nibbles, see layout above */
   const uint32_t* qzeros;  /* packed zero points [G, N/8] */

@@ -370,3 +370,23 @@ def test_conversion_utils_match_oracle(pkg, oracle):
 def test_exllama_hooks_are_noops(pkg):
     pkg.set_device(torch.device("cpu"))
     assert pkg.create_exllama_buffers(4096) is None
+
+
+def test_misaligned_pointers_are_refused(pkg):
+    """The kernels fetch with 16-byte loads: tensors, activations, outputs and workspaces off a
+    16-byte boundary are turned away before anything is launched (fake pointers, never read)."""
+    L = pkg._lib
+    lib = L.load()
+    good = _weight(pkg, 4096, 4096, 128)
+    for field in ("qweight", "qzeros", "scales"):
+        w = _weight(pkg, 4096, 4096, 128)
+        setattr(w, field, getattr(w, field) + 4)
+        assert lib.q4_linear(ctypes.byref(w), 0x100, None, 0x200, 1, 0, 0x400, 1 << 20, None) == L.ERR_INVALID_ARGUMENT
+        assert b"aligned" in lib.q4_last_error()
+    w = _weight(pkg, 4096, 4096, 128, g_idx=True)
+    w.g_idx = w.g_idx + 8
+    assert lib.q4_linear(ctypes.byref(w), 0x100, None, 0x200, 1, 0, 0x400, 1 << 20, None) == L.ERR_INVALID_ARGUMENT
+    for x, bias, y, ws in [(0x102, None, 0x200, 0x400), (0x100, None, 0x208, 0x400), (0x100, 0x301, 0x200, 0x400),
+                           (0x100, None, 0x200, 0x404)]:
+        assert lib.q4_linear(ctypes.byref(good), x, bias, y, 1, 0, ws, 1 << 20, None) == L.ERR_INVALID_ARGUMENT
+        assert b"aligned" in lib.q4_last_error()

@@ -664,3 +664,22 @@ def test_decode_offset_kernels_stay_non_finite_on_poisoned_rows(pkg, oracle, gpu
     assert not np.isfinite(got[1]).any()
     assert np.isfinite(got[0]).all()
     assert max_rel_err(got[0:1], x[0:1].astype(np.float32) @ w.astype(np.float32)) <= TOL
+
+
+def test_activation_view_off_a_16_byte_boundary_is_copied(pkg, oracle, gpu):
+    """x that starts 2 bytes into its storage (a contiguous view): the host side hands the kernels
+    an aligned copy, the result is that of the aligned tensor bit for bit; the C entry point
+    itself refuses such a pointer."""
+    import ctypes
+    K, N, M = 1024, 512, 3
+    qw, qz, sc, _ = oracle.make_gptq(K, N, 128, seed=4, sym=False)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
+    flat = torch.randn(M * K + 1, dtype=torch.float16, device=gpu)
+    x_off = flat[1:].view(M, K)
+    assert x_off.is_contiguous() and x_off.data_ptr() % 16 != 0
+    assert torch.equal(pkg.ops.linear(pk, x_off), pkg.ops.linear(pk, x_off.clone()))
+    L = pkg._lib
+    y = torch.empty((M, N), dtype=torch.float16, device=gpu)
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=gpu)
+    rc = L.load().q4_linear(ctypes.byref(pk.struct()), x_off.data_ptr(), None, y.data_ptr(), M, 0, ws.data_ptr(), ws.numel(), None)
+    assert rc == L.ERR_INVALID_ARGUMENT

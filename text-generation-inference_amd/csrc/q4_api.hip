@@ -41,6 +41,11 @@ static int validate_weight(const q4_weight* w, const char* who) {
     set_error("%s: null qweight/qzeros/scales", who);
     return Q4_ERR_INVALID_ARGUMENT;
   }
+  // the kernels fetch all tensors with 16-byte loads
+  if ((((uintptr_t)w->qweight | (uintptr_t)w->qzeros | (uintptr_t)w->scales | (uintptr_t)w->g_idx) & 15u) != 0) {
+    set_error("%s: qweight, qzeros, scales and g_idx must be 16-byte aligned", who);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
   if (w->groupsize < 1 || w->num_groups < 1) {
     set_error("%s: groupsize=%d num_groups=%d must be positive", who, w->groupsize, w->num_groups);
     return Q4_ERR_INVALID_ARGUMENT;
@@ -220,6 +225,10 @@ int q4_linear_ex(const q4_weight* w, const void* x, const void* bias, void* y, i
     set_error("q4_linear: null x or y");
     return Q4_ERR_INVALID_ARGUMENT;
   }
+  if ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)workspace) & 15u) != 0 || ((uintptr_t)bias & 1u) != 0) {
+    set_error("q4_linear: x, y and the workspace must be 16-byte aligned (bias: 2-byte)");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
   if (path == Q4_PATH_AUTO) path = q4_select_path(w, M, dtype);
   switch (path) {
     case Q4_PATH_GEMV:
@@ -303,6 +312,10 @@ int q4_linear_perm(const q4_weight* w, const int32_t* perm, const void* x, const
     set_error("q4_linear_perm: null x or y");
     return Q4_ERR_INVALID_ARGUMENT;
   }
+  if ((((uintptr_t)x | (uintptr_t)y) & 15u) != 0 || ((uintptr_t)bias & 1u) != 0) {
+    set_error("q4_linear_perm: x and y must be 16-byte aligned (bias: 2-byte)");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
   if (path == Q4_PATH_AUTO) path = q4_select_path(w, M, dtype);
   // Decode of a few rows with a short K: the kernel reads x through perm while it stages its
   // activation slab.  Every workgroup gathers its own copy, so the saved launch (~2.5 us) is
@@ -348,6 +361,10 @@ int q4_linear_gate_up_perm(const q4_weight* w, const int32_t* perm, const void* 
   if (M == 0 || w->N == 0) return Q4_OK;
   if (y == nullptr || x == nullptr) {
     set_error("q4_linear_gate_up_perm: null x or y");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if ((((uintptr_t)x | (uintptr_t)y) & 15u) != 0 || ((uintptr_t)bias & 1u) != 0) {
+    set_error("q4_linear_gate_up_perm: x and y must be 16-byte aligned (bias: 2-byte)");
     return Q4_ERR_INVALID_ARGUMENT;
   }
   if (q4_select_path(w, M, dtype) == Q4_PATH_GEMM && gemm_gate_up_supported(w, M, dtype)) {
@@ -401,6 +418,10 @@ int q4_linear_gate_up(const q4_weight* w, const void* x, const void* bias, void*
   if (M == 0 || w->N == 0) return Q4_OK;
   if (y == nullptr || (x == nullptr && w->K > 0)) {
     set_error("q4_linear_gate_up: null x or y");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if ((((uintptr_t)x | (uintptr_t)y) & 15u) != 0 || ((uintptr_t)bias & 1u) != 0) {
+    set_error("q4_linear_gate_up: x and y must be 16-byte aligned (bias: 2-byte)");
     return Q4_ERR_INVALID_ARGUMENT;
   }
   // Decode: the kernels with eight words per lane.  Prefill: the MFMA kernel with a lane's two

@@ -36,6 +36,13 @@ def _require_cuda(t: torch.Tensor, name: str) -> None:
         )
 
 
+def _dense16(t: torch.Tensor) -> torch.Tensor:
+    """Contiguous and on a 16-byte boundary (the kernels fetch with 16-byte loads): a view that
+    starts elsewhere in its storage is copied."""
+    t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 @dataclass
 class PackedWeight:
     """Validated view of one quantized weight, ready to be passed through the C ABI."""
@@ -149,7 +156,7 @@ def make_packed(qweight, qzeros, scales, g_idx, groupsize: int, layout: int) -> 
             g_idx = g_idx.to(torch.int32)
         if g_idx.numel() != K:
             raise ValueError(f"g_idx has {g_idx.numel()} entries, expected {K}")
-        g_idx = g_idx.contiguous()
+        g_idx = _dense16(g_idx)
     elif G * groupsize < K:
         raise ValueError(f"{G} groups of {groupsize} rows do not cover K={K}")
     dev = qweight.device
@@ -157,7 +164,7 @@ def make_packed(qweight, qzeros, scales, g_idx, groupsize: int, layout: int) -> 
         if t is not None and t.device != dev:
             raise ValueError(f"{name} is on {t.device}, qweight on {dev}")
     return PackedWeight(
-        qweight.contiguous(), qzeros.contiguous(), scales.contiguous(), g_idx, K, N, groupsize, G, layout
+        _dense16(qweight), _dense16(qzeros), _dense16(scales), g_idx, K, N, groupsize, G, layout
     )
 
 
@@ -337,7 +344,7 @@ def linear(
         raise TypeError(f"x must be float16 or bfloat16, got {x.dtype}")
     if x.dim() != 2 or x.shape[1] != w.K:
         raise ValueError(f"x must be [M, {w.K}], got {tuple(x.shape)}")
-    x = x.contiguous()
+    x = _dense16(x)
     if w.perm is not None and gemv_config is not None:
         x = gather_columns(x, w.perm)  # explicit decode configurations take x in row order
     M = x.shape[0]
@@ -399,7 +406,7 @@ def act_mul(gate_up: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor
         raise ValueError(f"gate_up must be [M, 2I], got {tuple(gate_up.shape)}")
     if act not in _lib.ACTIVATIONS:
         raise ValueError(f"unknown activation {act!r}; known: {sorted(_lib.ACTIVATIONS)}")
-    gate_up = gate_up.contiguous()
+    gate_up = _dense16(gate_up)
     M, inter = gate_up.shape[0], gate_up.shape[1] // 2
     y = out if out is not None else torch.empty((M, inter), dtype=gate_up.dtype, device=gate_up.device)
     if tuple(y.shape) != (M, inter) or y.dtype != gate_up.dtype or not y.is_contiguous():
@@ -434,7 +441,7 @@ def linear_gate_up(
         raise ValueError(f"N={w.N} cannot hold a gate and an up half")
     if act not in _lib.ACTIVATIONS:
         raise ValueError(f"unknown activation {act!r}; known: {sorted(_lib.ACTIVATIONS)}")
-    x = x.contiguous()
+    x = _dense16(x)
     M, inter = x.shape[0], w.N // 2
     y = out if out is not None else torch.empty((M, inter), dtype=x.dtype, device=x.device)
     if tuple(y.shape) != (M, inter) or y.dtype != x.dtype or y.device != x.device or not y.is_contiguous():
@@ -637,7 +644,7 @@ def moe_linear(w: PackedMoeWeight, x: torch.Tensor, routing: MoeRouting, gather:
     rows = T if gather else T * k
     if x.dim() != 2 or tuple(x.shape) != (rows, w.K):
         raise ValueError(f"x must be [{rows}, {w.K}], got {tuple(x.shape)}")
-    x = x.contiguous()
+    x = _dense16(x)
     if w.perm is not None and T > 0:
         x = _moe_gather(w, x, routing, gather)  # sorted rows, columns in each expert's row order
         gather = False
@@ -668,7 +675,7 @@ def moe_linear_gate_up(w: PackedMoeWeight, x: torch.Tensor, routing: MoeRouting,
     T, k = routing.topk_ids.shape
     if x.dim() != 2 or tuple(x.shape) != (T, w.K):
         raise ValueError(f"x must be [{T}, {w.K}], got {tuple(x.shape)}")
-    x = x.contiguous()
+    x = _dense16(x)
     x_rows = routing.sorted_tokens
     if w.perm is not None and T > 0:
         # experts in group order: sorted rows with their expert's column order, then as below
