@@ -84,6 +84,10 @@ int q4_dequant(const q4_weight* w, void* w_out, int dtype, void* stream) {
     set_error("q4_dequant: null output");
     return Q4_ERR_INVALID_ARGUMENT;
   }
+  if (((uintptr_t)w_out & 15u) != 0) {
+    set_error("q4_dequant: the output must be 16-byte aligned");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
   return launch_dequant(w, w_out, dtype, (hipStream_t)stream);
 }
 

@@ -590,6 +590,10 @@ int q4_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_rows, 
     set_error("q4_moe_linear: null x / y / expert_offsets");
     return Q4_ERR_INVALID_ARGUMENT;
   }
+  if ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)workspace) & 15u) != 0) {
+    set_error("q4_moe_linear: x, y and the workspace must be 16-byte aligned");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
   return launch_moe_linear(w, x, x_rows, expert_offsets, y, tokens, topk, dtype, workspace, workspace_bytes,
                            (hipStream_t)stream);
 }
@@ -610,6 +614,10 @@ int q4_moe_linear_gate_up(const q4_moe_weight* w, const void* x, const int32_t* 
   if (tokens == 0) return Q4_OK;
   if (x == nullptr || y == nullptr || expert_offsets == nullptr) {
     set_error("q4_moe_linear_gate_up: null x / y / expert_offsets");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)workspace) & 15u) != 0) {
+    set_error("q4_moe_linear_gate_up: x, y and the workspace must be 16-byte aligned");
     return Q4_ERR_INVALID_ARGUMENT;
   }
   return launch_moe_linear(w, x, x_rows, expert_offsets, y, tokens, topk, dtype, workspace, workspace_bytes,
