@@ -1,5 +1,8 @@
 // Decode path, host side: kernel choice, work decomposition and launch.  The kernels are in
 // q4_gemv_kernels.cuh.
+#include <cstring>
+#include <initializer_list>
+
 #include "q4_gemv_kernels.cuh"
 
 namespace q4host {
@@ -94,7 +97,35 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M) {
 // the kernels with the gated-MLP epilogue, two row blocks or an expert dimension (no lean variant)
 GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up) { return pick_config(w, M, gate_up, false); }
 
+static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bool allow_lean);
+
+// The choice depends on the weight's shape fields and M only, and the search behind it costs
+// several microseconds on large layers - as much as a decode kernel runs: a small per-thread,
+// direct-mapped memo keeps it out of the eager launch path.
 static GemvConfig pick_config(const q4_weight* w, int M, bool gate_up, bool allow_lean) {
+  struct Key {
+    int32_t K, N, groupsize, num_groups, layout, act, M, flags;
+  };
+  struct Entry {
+    Key key;
+    GemvConfig cfg;
+    bool valid;
+  };
+  static thread_local Entry memo[128];
+  const Key key{w->K, w->N, w->groupsize, w->num_groups, w->layout, w->g_idx != nullptr ? 1 : 0, M,
+                (gate_up ? 1 : 0) | (allow_lean ? 2 : 0)};
+  uint32_t h = 2166136261u;
+  for (const int32_t v : {key.K, key.N, key.groupsize, key.num_groups, key.layout, key.act, key.M, key.flags}) h = (h ^ (uint32_t)v) * 16777619u;
+  Entry& e = memo[(h ^ (h >> 15)) & 127u];
+  if (e.valid && memcmp(&e.key, &key, sizeof(Key)) == 0) return e.cfg;
+  const GemvConfig cfg = pick_config_search(w, M, gate_up, allow_lean);
+  e.key = key;
+  e.cfg = cfg;
+  e.valid = true;
+  return cfg;
+}
+
+static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bool allow_lean) {
   // Measured on MI355X (Llama-3-8B shapes, M=1): narrow column tiles with 4 waves along K
   // per workgroup and about two workgroups per CU (512 in flight) is the best point; wider
   // workgroups start too slowly and more splits lengthen the reduction tail.  The
