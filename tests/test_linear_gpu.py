@@ -683,3 +683,25 @@ def test_activation_view_off_a_16_byte_boundary_is_copied(pkg, oracle, gpu):
     ws = torch.empty(1 << 20, dtype=torch.uint8, device=gpu)
     rc = L.load().q4_linear(ctypes.byref(pk.struct()), x_off.data_ptr(), None, y.data_ptr(), M, 0, ws.data_ptr(), ws.numel(), None)
     assert rc == L.ERR_INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("zeros_sym", [True, False])
+def test_act_order_prefill_tall_tiles(pkg, oracle, gpu, dtype, zeros_sym):
+    """288 tiles of 128 x 128 would be two rounds of the chip, 160 tiles of 256 x 128 are one: the act-order
+    prefill kernel takes the 256-row tiles (last row tile ragged).  One-hot rows read the dequantized
+    weights back bit for bit, random activations match the oracle."""
+    K, N, M, gs = 512, 4096, 1100, 128
+    bf = dtype == "bf16"
+    qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=21, sym=zeros_sym, act_order=True)
+    w = oracle.dequant_gptq(qw, qz, sc, gi, gs, dtype)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), gs, 0)
+    assert pkg.ops.select_path(pk, M, torch.bfloat16 if bf else torch.float16) == "gemm"
+    ks = np.random.default_rng(5).integers(0, K, size=M)
+    x = torch.zeros((M, K), dtype=torch.bfloat16 if bf else torch.float16, device=gpu)
+    x[torch.arange(M, device=gpu), torch.as_tensor(ks, device=gpu)] = 1.0
+    y = pkg.ops.linear(pk, x)
+    torch.cuda.synchronize()
+    got = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, w[ks].view(np.uint16))
+    _run(pkg, oracle, gpu, K, N, gs, M, dtype=dtype, sym=zeros_sym, act=True, bias=True, seed=33)

@@ -259,7 +259,7 @@ size_t gemm_workspace_bytes(int M, int K, int N);
 // workgroup alone on its CU / sharing it).
 int gemm_pick_splits(long tiles, int KT, int M, int N, double us_alone, double us_shared, int per_cu = 2);
 bool gemm_act_order_table(const q4_weight* w);  // act-order GEMM reads its parameters from LDS
-int gemm_awq_splits(int M, int K, int N, bool one_per_cu);
+int gemm_awq_splits(int M, int K, int N, bool one_per_cu, bool tall = false);
 void launch_gemm_reduce(const float* partials, const void* bias, void* y, int M, int N, int splits, int dtype,
                         hipStream_t stream);
 }  // namespace q4host

@@ -149,6 +149,10 @@ size_t gemm_workspace_bytes(int M, int K, int N) {
     const int other = gemm_awq_splits(M, K, N, one_per_cu);
     if (other > splits) splits = other;
   }
+  {
+    const int other = gemm_awq_splits(M, K, N, true, true);  // act-order, 256-row tiles
+    if (other > splits) splits = other;
+  }
   const size_t bytes = splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
   const size_t direct = gemm_awq_direct_workspace_bytes(M, K, N);
   return direct > bytes ? direct : bytes;

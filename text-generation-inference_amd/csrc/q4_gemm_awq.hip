@@ -77,15 +77,16 @@ constexpr int kActNarrowGroupBytes = kABN * 3;  // 128 fp16 scales, then 128 zer
 
 // MOE: grouped launch, blockIdx.y is the expert; its row count is read from device memory, so
 // the grid covers the largest possible count and surplus workgroups leave at once.
-template <int DTYPE, int MODE, bool MOE = false>
+template <int DTYPE, int MODE, bool MOE = false, int BM = kABM>
 __global__ __launch_bounds__(MODE == kModeAwq ? 256 : 512, 2) void gemm_awq_kernel(AwqGemmParams gp) {
   constexpr bool ACT = MODE != kModeAwq;
+  static_assert(BM == kABM || (BM == 2 * kABM && ACT), "256-row tiles: act-order only");
   // AWQ: 4 waves, 2 x 2, a 64 x 64 block each.  Act-order: 8 waves, 4 x 2, a 32 x 64 block each: the
   // parameter table leaves room for one workgroup per CU, and a single wave per SIMD cannot hide
   // its own LDS and unpack latencies behind its MFMAs; two can hide each other's.
   constexpr int WAVES = ACT ? 8 : 4;
   constexpr int NTH = 64 * WAVES;
-  constexpr int MT = ACT ? 1 : 2;  // MFMA row tiles per wave
+  constexpr int MT = ACT ? BM / 128 : 2;  // MFMA row tiles per wave
   int moe_row0 = 0;
   if constexpr (MOE) {
     moe_row0 = moe_enter(gp.p, gp.moe, blockIdx.y);
@@ -93,9 +94,9 @@ __global__ __launch_bounds__(MODE == kModeAwq ? 256 : 512, 2) void gemm_awq_kern
   }
   constexpr bool TABLE = MODE == kModeActWide || MODE == kModeActNarrow;
   constexpr int GROUP_BYTES = MODE == kModeActWide ? kActWideGroupBytes : kActNarrowGroupBytes;
-  constexpr int A_TILE = kABM * kAUnits * 16;   // bytes
+  constexpr int A_TILE = BM * kAUnits * 16;   // bytes
   constexpr int B_TILE = (kABK / 8) * kABN * 16;
-  constexpr int A_LOADS = kABM * (kABK / 8) / NTH;  // 16-byte activation loads per thread
+  constexpr int A_LOADS = BM * (kABK / 8) / NTH;  // 16-byte activation loads per thread
   extern __shared__ __align__(16) unsigned char smem[];  // [A0][A1][B0][B1]
   const Problem& p = gp.p;
   const int tid = threadIdx.x;
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(MODE == kModeAwq ? 256 : 512, 2) void gemm_awq_kern
   const int kq = lane >> 5;
   const int N = p.N, K = p.K, M = p.M;
   const int NC = N >> 3;
-  const int tiles_m = (M + kABM - 1) / kABM;
+  const int tiles_m = (M + BM - 1) / BM;
   const int tiles_all = tiles_m * (N / kABN);
   if constexpr (MOE) {
     if ((int)blockIdx.x >= tiles_all * gp.splits) return;
@@ -115,7 +116,7 @@ __global__ __launch_bounds__(MODE == kModeAwq ? 256 : 512, 2) void gemm_awq_kern
   const int tile_id = blockIdx.x - split * tiles_all;
   const int tm = tile_id % tiles_m;
   const int tn = tile_id / tiles_m;
-  const int m0 = tm * kABM;
+  const int m0 = tm * BM;
   const int n0 = tn * kABN;
   const int KT_all = K / kABK;
   const int kt_begin = (int)((long)split * KT_all / gp.splits);  // this workgroup's K tiles
@@ -418,7 +419,7 @@ __global__ __launch_bounds__(MODE == kModeAwq ? 256 : 512, 2) void gemm_awq_kern
       load_b_act(kt2, std::integral_constant<int, ST ^ 1>{});
       // the next tile's parameters first, then half a column (two row pairs) per MFMA K step,
       // unpacked in phases with this tile's MFMAs between them (the order is pinned)
-      static_assert(kABK / 16 == 4 && MT == 1, "half a producer column per MFMA K step");
+      static_assert(kABK / 16 == 4, "half a producer column per MFMA K step");
       ActRows ar;
       // fragments one K step ahead
       uint4_t af[2][MT], bf[2][2];
@@ -441,6 +442,12 @@ __global__ __launch_bounds__(MODE == kModeAwq ? 256 : 512, 2) void gemm_awq_kern
         mfma_one(af[P][0], bf[P][1], acc[0][1]);
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (H == 1) word_store(cur ^ 1, S >> 1, o);
+        if constexpr (MT == 2) {
+          __builtin_amdgcn_sched_barrier(0);
+          mfma_one(af[P][1], bf[P][0], acc[1][0]);
+          mfma_one(af[P][1], bf[P][1], acc[1][1]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       };
       step(std::integral_constant<int, 0>{});
       step(std::integral_constant<int, 1>{});
@@ -506,16 +513,18 @@ bool gemm_awq_supported(const q4_weight* w, int M, int dtype) {
 }
 
 constexpr size_t kAwqTilesLdsBytes = 2 * (size_t)q4::kABM * q4::kAUnits * 16 + 2 * (size_t)(q4::kABK / 8) * q4::kABN * 16;
+// with 256-row tiles (act-order, table modes)
+constexpr size_t kActTallTilesLdsBytes = 4 * (size_t)q4::kABM * q4::kAUnits * 16 + 2 * (size_t)(q4::kABK / 8) * q4::kABN * 16;
 
 // Kernel variant for a weight: act-order takes the 32-bit parameter table where it fits
 // beside the tiles, except that the smaller table is taken when only it leaves room for two
 // workgroups per CU and the grid has more than one workgroup per CU to offer; layers with
 // too many groups for either table gather from global memory.
-static int gemm_awq_mode(const q4_weight* w, long workgroups) {
+static int gemm_awq_mode(const q4_weight* w, long workgroups, size_t tiles_bytes = kAwqTilesLdsBytes) {
   using namespace q4;
   if (w->layout != Q4_LAYOUT_GPTQ) return kModeAwq;
-  const size_t wide = kAwqTilesLdsBytes + (size_t)w->num_groups * kActWideGroupBytes;
-  const size_t narrow = kAwqTilesLdsBytes + (size_t)w->num_groups * kActNarrowGroupBytes;
+  const size_t wide = tiles_bytes + (size_t)w->num_groups * kActWideGroupBytes;
+  const size_t narrow = tiles_bytes + (size_t)w->num_groups * kActNarrowGroupBytes;
   const bool narrow_doubles =
       workgroups > 256 && wide > kLdsBytesPerWorkgroup / 2 && narrow <= kLdsBytesPerWorkgroup / 2;
   if (wide <= kLdsBytesPerWorkgroup && !narrow_doubles) return kModeActWide;
@@ -532,9 +541,24 @@ bool gemm_act_order_table(const q4_weight* w) {
 // workgroup per CU (~1.0 us per K tile).  There a grid of a few hundred tiles runs in
 // rounds of 256 and a last, mostly empty round costs as much as a full one, so split-K is
 // also weighed above 256 tiles (8192 x 10240 at M = 512: 320 tiles, 2 rounds).
-int gemm_awq_splits(int M, int K, int N, bool one_per_cu) {
+// Act-order with its table in LDS, dense launches: 256-row tiles (the unpacked weight tile serves
+// twice the rows; a K tile takes about 1.5x as long) where they fit beside the table and save
+// rounds of 256 workgroups.  Measured on MI355X, 256- against 128-row tiles (us): 8192 x 10240
+// 158 / 201 at M = 512, 302 / 345 at M = 1024, 493 / 558 at M = 2048, 846 / 1067 at M = 4096, but
+// 162 / 137 at M = 384; 4096 x 14336 88 / 101 at M = 512, 177 / 201 at M = 1024, but 169 / 152 at M = 768.
+bool gemm_act_order_tall(const q4_weight* w, int M) {
+  if (w->layout != Q4_LAYOUT_GPTQ || w->g_idx == nullptr || M <= q4::kABM) return false;
+  if (kActTallTilesLdsBytes + (size_t)w->num_groups * q4::kActNarrowGroupBytes > q4::kLdsBytesPerWorkgroup) return false;
+  const long cols = w->N / q4::kABN;
+  const long rounds_short = (((M + q4::kABM - 1) / q4::kABM) * cols + 255) / 256;
+  const long rounds_tall = (((M + 2 * q4::kABM - 1) / (2 * q4::kABM)) * cols + 255) / 256;
+  return 3 * rounds_tall < 2 * rounds_short;
+}
+
+int gemm_awq_splits(int M, int K, int N, bool one_per_cu, bool tall) {
   if (K % q4::kABK != 0 || N % q4::kABN != 0) return 1;
-  const long tiles = (long)((M + q4::kABM - 1) / q4::kABM) * (N / q4::kABN);
+  const int bm = tall ? 2 * q4::kABM : q4::kABM;
+  const long tiles = (long)((M + bm - 1) / bm) * (N / q4::kABN);
   if (one_per_cu) return tiles < 1024 ? gemm_pick_splits(tiles, K / q4::kABK, M, N, 1.0, 1.0, 1) : 1;
   return tiles < 256 ? gemm_pick_splits(tiles, K / q4::kABK, M, N, 1.0, 1.9) : 1;
 }
@@ -569,7 +593,9 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
   gp.p = Problem{w->qweight, w->qzeros, (const half_t*)w->scales, w->g_idx, x, bias, y,
                  M,          w->K,      w->N,                     w->groupsize, w->num_groups};
   const int out_rows = moe != nullptr ? moe->pairs : M;  // rows of y (and of one split's partials)
-  int splits = moe != nullptr ? moe_awq_splits(w, moe) : gemm_awq_splits(M, w->K, w->N, gemm_act_order_table(w));
+  const bool tall = moe == nullptr && gemm_act_order_tall(w, M);
+  const int bm = tall ? 2 * kABM : kABM;
+  int splits = moe != nullptr ? moe_awq_splits(w, moe) : gemm_awq_splits(M, w->K, w->N, gemm_act_order_table(w), tall);
   if (splits > 1 && (workspace == nullptr ||
                      workspace_bytes < Q4_WORKSPACE_COUNTER_BYTES + (size_t)splits * out_rows * w->N * sizeof(float)))
     splits = 1;  // no room for partial tiles: one workgroup per whole tile
@@ -577,14 +603,14 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
   gp.partial_rows = out_rows;
   gp.partials = splits > 1 ? (float*)((char*)workspace + Q4_WORKSPACE_COUNTER_BYTES) : nullptr;
   gp.moe = moe != nullptr ? moe->view : MoeView{};
-  const long total = (long)((M + kABM - 1) / kABM) * (w->N / kABN) * splits;
+  const long total = (long)((M + bm - 1) / bm) * (w->N / kABN) * splits;
   const long experts = moe != nullptr ? moe->num_experts : 1;
   if (total > 0x7fffffffL || experts > 65535) {
     set_error("q4_linear(gemm/awq): grid too large");
     return Q4_ERR_UNSUPPORTED;
   }
-  const size_t tiles_smem = kAwqTilesLdsBytes;
-  const int mode = gemm_awq_mode(w, total * experts);
+  const size_t tiles_smem = tall ? kActTallTilesLdsBytes : kAwqTilesLdsBytes;
+  const int mode = gemm_awq_mode(w, total * experts, tiles_smem);
   const size_t smem = tiles_smem + (mode == kModeActWide     ? (size_t)w->num_groups * kActWideGroupBytes
                                     : mode == kModeActNarrow ? (size_t)w->num_groups * kActNarrowGroupBytes
                                                              : 0);
@@ -596,6 +622,13 @@ int launch_gemm_awq(const q4_weight* w, const void* x, const void* bias, void* y
   auto launch_mode = [&](auto dt, auto grouped) {
     constexpr int DT = decltype(dt)::value;
     constexpr bool G = decltype(grouped)::value;
+    if constexpr (!G) {
+      if (tall) {
+        if (mode == kModeActWide) launch(gemm_awq_kernel<DT, kModeActWide, false, 2 * kABM>);
+        else launch(gemm_awq_kernel<DT, kModeActNarrow, false, 2 * kABM>);
+        return;
+      }
+    }
     switch (mode) {
       case kModeAwq: launch(gemm_awq_kernel<DT, kModeAwq, G>); break;
       case kModeActWide: launch(gemm_awq_kernel<DT, kModeActWide, G>); break;
