@@ -542,17 +542,31 @@ bool gemm_act_order_table(const q4_weight* w) {
 // rounds of 256 and a last, mostly empty round costs as much as a full one, so split-K is
 // also weighed above 256 tiles (8192 x 10240 at M = 512: 320 tiles, 2 rounds).
 // Act-order with its table in LDS, dense launches: 256-row tiles (the unpacked weight tile serves
-// twice the rows; a K tile takes about 1.5x as long) where they fit beside the table and save
-// rounds of 256 workgroups.  Measured on MI355X, 256- against 128-row tiles (us): 8192 x 10240
-// 158 / 201 at M = 512, 302 / 345 at M = 1024, 493 / 558 at M = 2048, 846 / 1067 at M = 4096, but
-// 162 / 137 at M = 384; 4096 x 14336 88 / 101 at M = 512, 177 / 201 at M = 1024, but 169 / 152 at M = 768.
+// twice the rows; a K tile takes about 1.5x as long) where they fit beside the table and the
+// estimate below, rounds of 256 workgroups and split-K included, is the shorter one.  Measured on
+// MI355X, 256- against 128-row tiles (us): 8192 x 10240 158 / 201 at M = 512, 302 / 345 at M = 1024,
+// 493 / 558 at M = 2048, 846 / 1067 at M = 4096, but 162 / 137 at M = 384; 4096 x 14336 88 / 101 at
+// M = 512, 177 / 201 at M = 1024, but 169 / 152 at M = 768.
+// estimated time (us) of a dense act-order launch with one workgroup per CU: the split-K cost
+// model of gemm_pick_splits with the measured time of a K tile (0.85 us at 128 rows, 1.28 us at 256)
+static double act_estimate_us(int M, int K, int N, int bm, double us_tile) {
+  static const int kCandidates[] = {1, 2, 3, 4, 6, 8, 12, 16};
+  const long tiles = (long)((M + bm - 1) / bm) * (N / q4::kABN);
+  const int KT = K / q4::kABK;
+  double best = -1.0;
+  for (int sp : kCandidates) {
+    if (sp > 1 && (KT / sp < 8 || tiles >= 1024)) break;
+    double t = (double)((tiles * sp + 255) / 256) * ((KT + sp - 1) / sp) * us_tile;
+    if (sp > 1) t += 5.0 + (double)sp * M * N * 8.0 / 5.0e6;
+    if (best < 0.0 || t < best) best = t;
+  }
+  return best;
+}
 bool gemm_act_order_tall(const q4_weight* w, int M) {
-  if (w->layout != Q4_LAYOUT_GPTQ || w->g_idx == nullptr || M <= q4::kABM) return false;
+  // (below 512 rows the launches are split-K heavy and the estimate is not good enough to choose)
+  if (w->layout != Q4_LAYOUT_GPTQ || w->g_idx == nullptr || M < 4 * q4::kABM) return false;
   if (kActTallTilesLdsBytes + (size_t)w->num_groups * q4::kActNarrowGroupBytes > q4::kLdsBytesPerWorkgroup) return false;
-  const long cols = w->N / q4::kABN;
-  const long rounds_short = (((M + q4::kABM - 1) / q4::kABM) * cols + 255) / 256;
-  const long rounds_tall = (((M + 2 * q4::kABM - 1) / (2 * q4::kABM)) * cols + 255) / 256;
-  return 3 * rounds_tall < 2 * rounds_short;
+  return act_estimate_us(M, w->K, w->N, 2 * q4::kABM, 1.28) < 0.95 * act_estimate_us(M, w->K, w->N, q4::kABM, 0.85);
 }
 
 int gemm_awq_splits(int M, int K, int N, bool one_per_cu, bool tall) {
