@@ -351,6 +351,32 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
       }
     }
     c.splits = best_dv;
+    // One 1024-thread workgroup per CU - two column tiles x eight K waves around one table of 128
+    // columns - where 200 to 256 such workgroups make one round and their decomposition costs no more:
+    // half the table builds and half the splits of two 512-thread workgroups per CU (us at M = 1 /
+    // 16: 14336 x 4096 14.5 / 18.3 against 16.2 / 20.3, 8192 x 10240 18.0 / 21.4 against 19.6 / 24.2,
+    // level on 28672 x 8192 and 4096 x 28672).
+    if (w->N % 128 == 0 && chunks >= 8) {
+      const int tiles2 = (w->N / 128) * mchunks;
+      int pick = 0;
+      double pick_cost = -1.0;
+      for (int dv = 1; dv * 8 <= chunks; ++dv) {
+        if ((long)((chunks + dv - 1) / dv) * 256 + 2 * table1 + 32 > 150000) continue;
+        const double wgs = (double)tiles2 * dv;
+        if (wgs < 200.0 || wgs > 256.0) continue;  // a single round (4096 x 11008 in 344: 17.9 against 15.0 us)
+        const int per_wave = (chunks + dv * 8 - 1) / (dv * 8);
+        const double cost = (wgs >= 256.0 ? wgs / 256.0 : 256.0 / wgs) * ((double)per_wave * dv * 8 / chunks);
+        if (pick_cost < 0.0 || cost <= pick_cost) {
+          pick_cost = cost;
+          pick = dv;
+        }
+      }
+      if (pick > 0 && best >= 0.0 && pick_cost <= 1.02 * best) {
+        c.wcol = 2;
+        c.wk = 8;
+        c.splits = pick;
+      }
+    }
     return c;
   }
   // many rows, one column tile per workgroup: eight waves along K share one activation slab
@@ -534,7 +560,7 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
     set_error("q4_linear(gemv): the lean kernel takes GPTQ weights with contiguous groups of a multiple of 128 rows");
     return Q4_ERR_INVALID_ARGUMENT;
   }
-  if (cfg.wcol < 1 || cfg.wk < 1 || cfg.splits < 1 || cfg.wcol * cfg.wk > (lean ? 16 : 8) ||
+  if (cfg.wcol < 1 || cfg.wk < 1 || cfg.splits < 1 || cfg.wcol * cfg.wk > ((lean || act) ? 16 : 8) ||
       w->N % (wave_cols * cfg.wcol) != 0 || w->K % 128 != 0 || (long)cfg.splits * cfg.wk > w->K / 128) {
     set_error("q4_linear(gemv): bad config wcol=%d wk=%d splits=%d for K=%d N=%d", cfg.wcol, cfg.wk,
               cfg.splits, w->K, w->N);

@@ -795,7 +795,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
 // workgroup needs does not grow with the rows: this kernel is bound by the per-weight work,
 // not by memory, and what it wants is resident waves.
 template <int DTYPE, int RMAX, bool MOE = false, bool XDIRECT = false>
-__global__ __launch_bounds__(512, 4) void gemv_gptq_act_kernel(GemvParams gp) {
+__global__ __launch_bounds__(MOE ? 512 : 1024, 4) void gemv_gptq_act_kernel(GemvParams gp) {
   static_assert(!(MOE && XDIRECT), "grouped launches stage their (mapped) rows in LDS");
   extern __shared__ __align__(16) unsigned char smem[];
   const int32_t* moe_rows = nullptr;
