@@ -683,6 +683,26 @@ def main():
             torch.cuda.empty_cache()
         out["batched_decode"] = batch
 
+        # ---- BASELINE.json configs[2]: bf16 prefill away from the headline M
+        cfg3 = {}
+        for Mb in (512, 4096):
+            tot_f = 0.0
+            tot_t = 0.0
+            entry = {}
+            for i, (name, K, N) in enumerate(SHAPES):
+                xb = torch.randn((Mb, K), device=dev, dtype=torch.bfloat16)
+                yb = torch.empty((Mb, N), device=dev, dtype=torch.bfloat16)
+                fns = [(lambda c=c, i=i: pkg.ops.linear(weights[c][i], xb, None, out=yb)) for c in range(copies)]
+                avg, _ = time_kernel_launches(torch, fns, 12)
+                fl = 2.0 * Mb * N * K
+                entry[name] = {"us": round(avg * 1e6, 1), "TFLOPs": round(fl / avg / 1e12, 1)}
+                tot_f += fl
+                tot_t += avg
+                del xb, yb
+            entry["TFLOPs_aggregate"] = round(tot_f / tot_t / 1e12, 1)
+            cfg3[f"m{Mb}"] = entry
+        out["cfg3_bf16_prefill"] = cfg3
+
         # ---- BASELINE.json configs[3] and [4] at their own shapes
         def shape_us(make, K, N, Mb, ncopies):
             ws_ = [make(c) for c in range(ncopies)]
