@@ -226,6 +226,14 @@ def test_gemm_groupsizes(pkg, oracle, gpu, gs, dtype):
     _run(pkg, oracle, gpu, 1024, 256, gs, 96, dtype=dtype, sym=False, path=2, seed=gs + 200)
 
 
+@pytest.mark.parametrize("gs", [32, 64])
+@pytest.mark.parametrize("dtype,M", [("f16", 2048), ("bf16", 1000), ("f16", 300)])
+def test_gemm_two_k_groups_small_groupsizes(pkg, oracle, gpu, gs, dtype, M):
+    """A grid of at most 256 tiles of 128 x 256: two K groups of four waves per workgroup (128 rows
+    of K per round), with two and four quantisation groups to a round; M = 300 adds split-K."""
+    _run(pkg, oracle, gpu, 512, 4096, gs, M, dtype=dtype, sym=False, bias=True, path=2, seed=gs + M)
+
+
 def test_gemm_bit_exact_weights_through_identity(pkg, oracle, gpu):
     """x = identity rows: y[m, :] must be W[m, :] exactly (fp16 W is what the MFMA sees, and
     a one-hot fp32 accumulation adds nothing), so the in-register unpack of the GEMM kernel is
@@ -348,6 +356,18 @@ def test_act_order_decode_picker_branches(pkg, oracle, gpu, K, N, M):
     """The lookup kernels' picker: two column tiles per workgroup on wide layers, and the single
     round of workgroups it takes with 12 rows or more when the slab leaves one workgroup per CU."""
     _run(pkg, oracle, gpu, K, N, 128, M, act=True, sym=False, path=1, seed=N // 1024 + M)
+
+
+@pytest.mark.parametrize("K,gs", [(14336, 32), (17920, 32), (28672, 64)])
+@pytest.mark.parametrize("M,dtype", [(1, "f16"), (16, "f16"), (3, "bf16")])
+def test_act_order_decode_many_groups(pkg, oracle, gpu, K, gs, M, dtype):
+    """448 and 560 groups: the parameter table of a 64-column tile takes 112 / 140 KB of LDS and
+    the decode kernel still runs, beside a g_idx slice of a K range split far enough."""
+    N = 512
+    qw, qz, sc, gi = oracle.make_gptq(K, N, gs, seed=3, act_order=True)
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), gs, 0)
+    assert pkg.ops.select_path(pk, M) == "gemv"
+    _run(pkg, oracle, gpu, K, N, gs, M, dtype=dtype, act=True, sym=False, path=1, seed=K // 512 + M)
 
 
 @pytest.mark.parametrize("M", [1, 5, 16, 33, 128])

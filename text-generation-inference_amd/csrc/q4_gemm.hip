@@ -27,10 +27,10 @@ static int gemm_max_rows(int K) {
   return (int)(rows > (1L << 30) ? (1L << 30) : rows);
 }
 
-// two K groups per workgroup (eight waves), groups of at least 64 rows
+// two K groups per workgroup (eight waves)
 template <int DTYPE, int BM>
-static void launch_tile_kg2(const GemmParams& gp, dim3 grid, size_t smem, hipStream_t stream) {
-  auto k = q4::gemm_gptq_kernel<DTYPE, BM, 1, 2, false, 2>;
+static void launch_tile_kg2(const GemmParams& gp, int gs, dim3 grid, size_t smem, hipStream_t stream) {
+  auto k = gs == 32 ? q4::gemm_gptq_kernel<DTYPE, BM, 2, 2, false, 2> : q4::gemm_gptq_kernel<DTYPE, BM, 1, 2, false, 2>;
   if (smem > 64 * 1024)
     (void)hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   hipLaunchKernelGGL(k, grid, dim3(512), smem, stream, gp);
@@ -243,17 +243,17 @@ int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, in
   size_t smem = 2 * (size_t)bm * kAUnitsPerRow * 16;
   dim3 grid((unsigned)total);
   const int gs = w->groupsize;
-  const bool kg2 = g.kg == 2 && nw == 2 && bm <= 128 && gs >= 64 && (w->K / kBK) % (2 * g.splits) == 0;
+  const bool kg2 = g.kg == 2 && nw == 2 && bm <= 128 && (w->K / kBK) % (2 * g.splits) == 0;
   if (kg2) {
     smem *= 2;
     const size_t xch = (size_t)(bm / 32) * 2 * 16 * 256 * sizeof(float);
     if (xch > smem) smem = xch;
     if (dtype == Q4_DTYPE_F16) {
-      if (bm == 64) launch_tile_kg2<Q4_DTYPE_F16, 64>(gp, grid, smem, stream);
-      else launch_tile_kg2<Q4_DTYPE_F16, 128>(gp, grid, smem, stream);
+      if (bm == 64) launch_tile_kg2<Q4_DTYPE_F16, 64>(gp, gs, grid, smem, stream);
+      else launch_tile_kg2<Q4_DTYPE_F16, 128>(gp, gs, grid, smem, stream);
     } else {
-      if (bm == 64) launch_tile_kg2<Q4_DTYPE_BF16, 64>(gp, grid, smem, stream);
-      else launch_tile_kg2<Q4_DTYPE_BF16, 128>(gp, grid, smem, stream);
+      if (bm == 64) launch_tile_kg2<Q4_DTYPE_BF16, 64>(gp, gs, grid, smem, stream);
+      else launch_tile_kg2<Q4_DTYPE_BF16, 128>(gp, gs, grid, smem, stream);
     }
   } else if (dtype == Q4_DTYPE_F16) {
     if (bm == 64) launch_tile<Q4_DTYPE_F16, 64, 2>(gp, gs, grid, smem, stream);

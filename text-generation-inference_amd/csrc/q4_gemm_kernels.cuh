@@ -153,7 +153,7 @@ __device__ __forceinline__ float16_t mfma32(const uint4_t a, const uint4_t b, fl
 // the K loop is the plain one, at the end the up waves hand their rounded tile to the gate
 // waves through LDS (the activation tiles are dead by then).
 template <int DTYPE, int BM, int GPT, int NW, bool MOE = false, int KG = 1, bool FUSE = false>
-__global__ __launch_bounds__(256 * KG, (KG == 2 ? 1 : BM == 64 ? 3 : BM == 128 ? (NW == 1 ? 3 : 2) : 1)) void gemm_gptq_kernel(GemmParams gp) {
+__global__ __launch_bounds__(256 * KG, (KG == 2 ? 1 : BM == 64 ? 3 : BM == 128 ? (NW == 1 ? (GPT == 1 ? 3 : 1) : 2) : 1)) void gemm_gptq_kernel(GemmParams gp) {
   static_assert(KG == 1 || (KG == 2 && !MOE && BM <= 128), "two K groups: dense launches, at most 128 rows");
   static_assert(!FUSE || (NW == 2 && KG == 1 && !MOE), "gated epilogue: two columns per lane, dense launches, one K group");
   int moe_row0 = 0;

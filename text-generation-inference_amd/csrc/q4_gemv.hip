@@ -43,8 +43,9 @@ bool gemv_supported(const q4_weight* w, int M, int dtype) {
   const long tile = w->g_idx != nullptr ? 64 : 16;
   if (chunks * (w->N / tile) > Q4_WORKSPACE_TICKET_BYTES / 4 && M > 16) return false;
   if (w->g_idx != nullptr) {
-    // act-order: the table of all groups for 64 columns must fit LDS next to the slab
-    return w->num_groups <= 65535 && (long)w->num_groups * 64 * 4 <= 96 * 1024;
+    // act-order: the table of all groups for 64 columns must fit LDS next to the g_idx slice of
+    // a workgroup's K range (at most 16 chunks of 128 rows once K is split as far as it goes)
+    return w->num_groups <= 65535 && (long)w->num_groups * 64 * 4 + 16 * 256 + 32 <= 150000;
   }
   if (!groupsize_ok_contiguous(w->groupsize)) return false;
   return (long)w->num_groups * w->groupsize >= w->K;
