@@ -68,7 +68,8 @@ def test_lean_period_boundaries(pkg, oracle, gpu, chunks, M):
         _run(pkg, oracle, gpu, chunks * 128, 128, 128, M, sym=False, cfg=(1, 2, 2, 0), seed=chunks + M + 1)
 
 
-@pytest.mark.parametrize("K,N", [(8192, 10240), (5120, 13824), (13824, 5120), (28672, 8192), (8192, 28672), (6656, 17920)])
+@pytest.mark.parametrize("K,N", [(8192, 10240), (5120, 13824), (13824, 5120), (28672, 8192), (8192, 28672), (6656, 17920),
+                                 (3584, 37888), (3072, 9216), (2048, 9216), (8192, 1280)])
 def test_large_layer_decode_decompositions_picked(pkg, gpu, K, N):
     """The decompositions the picker takes for 4..16 rows on large layers (several column tiles
     around one slab, 1024-thread workgroups, splits of an uneven K deal): one-hot rows read the
@@ -80,7 +81,7 @@ def test_large_layer_decode_decompositions_picked(pkg, gpu, K, N):
     w = pkg.ops.make_packed(qweight, qzeros, scales, None, 128, 0)
     dense = pkg.ops.dequantize(w)
     rows = torch.randint(0, K, (16,), device=gpu, generator=g)
-    for M in (4, 6, 9, 12, 16):
+    for M in (1, 3, 4, 6, 9, 12, 16):
         assert pkg.ops.select_path(w, M) == "gemv"
         x = torch.zeros((M, K), dtype=torch.float16, device=gpu)
         x[torch.arange(M, device=gpu), rows[:M]] = 1.0

@@ -162,14 +162,29 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
         c.wk = 4;
       }
       while ((long)rows * ((long)w->K / c.splits * 2 + 16) > 150000 && c.splits * c.wk * 2 <= chunks) c.splits *= 2;
-      return c;
+      // From four rows on, a grid that spills into a second round it leaves mostly empty is handed
+      // to the cost model below: 296 such workgroups of 3584 x 37888 hold a 115 KB slab each at
+      // M = 16, one per CU (30.7 us; 25.9 us in 148 workgroups of four column tiles).  Elsewhere the
+      // model's picks for these layers measured no better than the rule's (6144 x 24576 at M = 16:
+      // 15 % slower).
+      if (M < 4) return c;
+      const long lds = (long)rows * ((long)((chunks + c.splits - 1) / c.splits) * 256 + 16) + 512;
+      long res = (160 * 1024) / (lds + 1024);
+      if (res > 16 / (c.wcol * c.wk)) res = 16 / (c.wcol * c.wk);
+      if (res < 1) res = 1;
+      const long wgs = (long)(n64 / c.wcol) * c.splits;
+      const long rounds = ((wgs + 255) / 256 + res - 1) / res;
+      if (rounds < 2 || wgs * 4 >= rounds * res * 256 * 3) return c;
     }
-    c.wcol = 1;
-    c.wk = 8;
-    // about one workgroup per CU; every wave keeps its own activations: rows x K / splits x 2 B in all
+    const bool wide = n64 >= 384 && w->N % 128 == 0;
     int best = 1;
     double best_cost = -1.0;
-    for (int dv = 1; dv * c.wk <= chunks; ++dv) {
+    if (!wide) {
+      c.wcol = 1;
+      c.wk = 8;
+    }
+    // about one workgroup per CU; every wave keeps its own activations: rows x K / splits x 2 B in all
+    for (int dv = 1; !wide && dv * c.wk <= chunks; ++dv) {
       const long lds = (long)rows * c.wk * ((long)((chunks + dv * c.wk - 1) / (dv * c.wk)) * 256 + 16);
       if (lds > 150000) continue;
       const double wgs = (double)n64 * dv;
@@ -183,9 +198,9 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
     // 160 column tiles or more over a short K (up to 4096 rows), four rows or more: every split
     // costs more in partial sums than the idle CUs do (4096 x 11008, 172 tiles: 10.2 / 10.7 / 11.9 us
     // unsplit at M = 4 / 8 / 16 against 13.5 / 14.2 / 16.4 us with two splits)
-    if (M >= 4 && n64 >= 160 && chunks <= 32 && (long)rows * c.wk * ((long)((chunks + c.wk - 1) / c.wk) * 256 + 16) <= 150000)
+    if (!wide && M >= 4 && n64 >= 160 && chunks <= 32 && (long)rows * c.wk * ((long)((chunks + c.wk - 1) / c.wk) * 256 + 16) <= 150000)
       best = 1;
-    c.splits = best;
+    if (!wide) c.splits = best;
     if (M >= 4) {
       // Four rows and more: the activation staging (per wave with one column wave, one slab per
       // workgroup with several) decides how many workgroups a CU holds, and the rule above knows
@@ -225,7 +240,7 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
       // activations fit LDS: one round of 1024-thread workgroups, two column tiles x eight K
       // waves (four x four next) around one shared slab.  Swept at M = 16 (us, this / the rule's
       // choice): 13824 x 5120 16.9 / 21.3, 5120 x 13824 16.5 / 22.1, 8192 x 10240 19.5 / 24.6.
-      if (rows >= 9) {
+      if (rows >= 9 && !wide) {
         bool one_round = false;
         for (int dv = 1; dv * 8 <= chunks && (long)n64 * dv <= 256; ++dv)
           if ((long)rows * 8 * (((chunks + dv * 8 - 1) / (dv * 8)) * 256 + 16) + 512 <= 150000) one_round = true;
@@ -253,7 +268,7 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
           }
         }
       }
-      const double t_rule = best_cost >= 0.0 ? model_us(c.wcol, c.wk, c.splits) : -1.0;
+      const double t_rule = (wide || best_cost >= 0.0) ? model_us(c.wcol, c.wk, c.splits) : -1.0;
       double best_t = -1.0;
       GemvConfig pick = c;
       for (int wcol = 1; wcol <= 4; wcol *= 2)
@@ -269,7 +284,7 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
           }
       if (best_t >= 0.0 && (t_rule < 0.0 || best_t < 0.88 * t_rule)) return pick;
     }
-    if (best_cost >= 0.0) return c;
+    if (wide || best_cost >= 0.0) return c;
     c.lean = 0;  // no split fits LDS: the kernel below, with its workgroup slab
   }
   // Small layers, 4 to 16 rows, K a multiple of 1024 from 2048 on: 32-column wave tiles (two words per lane)
@@ -305,6 +320,21 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
     }
     if (pick > 0) {
       t.splits = pick;
+      // A few workgroups more than CUs: the CUs that take two decide, and when the slab leaves
+      // room for one per CU they form a second, nearly empty round (3072 x 9216, 288 workgroups:
+      // 10.8 / 11.9 / 17.9 us at M = 4 / 8 / 16).  One round of the lean kernel's 64-column tiles,
+      // eight waves over the whole K with their own activations, takes 9.0 / 9.6 / 10.7 us.
+      const long wgs = tiles * pick;
+      const int per_wave = (chunks + 7) / 8;
+      if ((wgs + 255) / 256 * 256 * 2 > wgs * 3 && w->N / 64 <= 256 &&
+          (long)rows * 8 * (per_wave * 256 + 16) + 512 <= 150000) {
+        GemvConfig l = c;
+        l.lean = 1;
+        l.wcol = 1;
+        l.wk = 8;
+        l.splits = 1;
+        return l;
+      }
       return t;
     }
   }
