@@ -104,8 +104,20 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
     // 14336 x 4096 30.5 / 23.5 (at M = 17: 25.7 / 22.9).  From the third block on (M = 48) the
     // GEMM wins except on the smallest matrices (4096 x 4096: 12.6 / 17.9 at M = 64, 24.4 / 20.8
     // at M = 96; 2048 x 8192: 10.8 / 15.2 at M = 64).
-    const bool small = M <= 16 || gemv_rows32_supported(w, M) || (M <= 32 && w->K <= 8192 && weights <= (1L << 26)) ||
-                       (M <= 64 && weights <= (1L << 24));
+    // Three and four blocks on the smallest matrices only while the decode launch stays one round
+    // of workgroups (a slab that leaves room for one per CU and more workgroups than CUs: 5120 x 3072
+    // at M = 48 20.4 / 14.7), four blocks only up to K = 4096 (M = 64: 5120 x 2560 21.2 / 15.1,
+    // 8960 x 1536 22.6 / 15.4, 6912 x 2304 24.3 / 15.5, but 3072 x 5120 14.5 / 15.0, 2560 x 6144 12.8 / 15.2).
+    bool blocks34 = M > 32 && M <= 64 && weights <= (1L << 24) && (M <= 48 || w->K <= 4096) && gemv_supported(w, M, dtype);
+    if (blocks34) {
+      const GemvConfig c = gemv_pick_config(w, M);
+      const long mchunks = (M + c.rows_per_block - 1) / c.rows_per_block;
+      const long wgs = (long)(w->N / (16 * c.words * c.wcol)) * mchunks * c.splits;
+      const long chunks = w->K / 128;
+      const long slab = (long)c.rows_per_block * ((chunks + c.splits - 1) / c.splits * 256 + 16);
+      if (slab > 75 * 1024 && wgs > 256) blocks34 = false;
+    }
+    const bool small = M <= 16 || gemv_rows32_supported(w, M) || (M <= 32 && w->K <= 8192 && weights <= (1L << 26)) || blocks34;
     if (small && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
     if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;
     if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;

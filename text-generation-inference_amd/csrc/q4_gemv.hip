@@ -414,6 +414,14 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
   // (M = 16: 4096 x 6144 12.1 against 14.9 us, 14336 x 4096 18.8 against 22.4 us)
   const bool contiguous = w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr;
   if (contiguous && !gate_up && M >= 12 && c.wcol == 1 && (chunks % 8 == 0 || chunks >= 32)) c.wk = 8;
+  // Several 16-row blocks whose tiles outnumber the CUs while the unsplit slab leaves room for one
+  // workgroup per CU: two column tiles share each slab, one round instead of two (M = 64:
+  // 3072 x 5120 20.2 -> 15.5 us, 3584 x 4608 29.8 -> 16.7 us; M = 48: 2560 x 6144 23.2 us before)
+  if (contiguous && !gate_up && mchunks > 1 && c.wcol == 1 && w->N % 128 == 0 &&
+      (long)rows * ((long)w->K * 2 + 16) > 75 * 1024 && (long)(w->N / 64) * mchunks > 256) {
+    c.wcol = 2;
+    c.wk = 4;
+  }
   // 192..256 column tiles, 2..11 rows: one round of eight-wave workgroups over the whole K,
   // nothing to combine (4096 x 14336: 10.9 against 11.1 us at M = 2, 12.7 against 14.1 us at
   // M = 8; 5120 x 13824: 11.9 / 12.6 and 14.2 / 15.4 us; with 172 tiles it does not pay)
