@@ -351,10 +351,13 @@ def test_act_order_decode_llama70b(pkg, oracle, gpu, K, N, M):
     _run(pkg, oracle, gpu, K, N, 128, M, act=True, path=1, seed=K // 1024 + M)
 
 
-@pytest.mark.parametrize("K,N,M", [(4096, 14336, 1), (4096, 14336, 8), (4096, 28672, 16), (14336, 4096, 16)])
+@pytest.mark.parametrize("K,N,M", [(4096, 14336, 1), (4096, 14336, 8), (4096, 28672, 16), (14336, 4096, 16),
+                                   (18944, 3584, 1), (3584, 4608, 1), (3584, 4608, 16), (4096, 22016, 2)])
 def test_act_order_decode_picker_branches(pkg, oracle, gpu, K, N, M):
-    """The lookup kernels' picker: two column tiles per workgroup on wide layers, and the single
-    round of workgroups it takes with 12 rows or more when the slab leaves one workgroup per CU."""
+    """The lookup kernels' picker: two column tiles per workgroup on wide layers, the single
+    round of workgroups it takes with 12 rows or more when the slab leaves one workgroup per CU,
+    a split count held to one round of workgroups (18944 rows), four K waves on a short K that
+    does not deal out over eight (3584 rows), and a second round taken lightly at one or two rows."""
     _run(pkg, oracle, gpu, K, N, 128, M, act=True, sym=False, path=1, seed=N // 1024 + M)
 
 

@@ -1,5 +1,6 @@
 // Decode path, host side: kernel choice, work decomposition and launch.  The kernels are in
 // q4_gemv_kernels.cuh.
+#include <cmath>
 #include <cstring>
 #include <initializer_list>
 
@@ -364,23 +365,42 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
     c.wk = chunks >= 8 ? 8 : c.wk;
     const long table1 = (long)w->num_groups * 64 * 4;
     const int tiles = (w->N / 64) * mchunks;
-    const int max_dv = chunks / c.wk;
     auto lds_bytes = [&](int dv) { return (long)((chunks + dv - 1) / dv) * 256 + table1 + 32; };
-    int best_dv = max_dv;
+    // Workgroups beyond what the chip holds at once wait for a second round, which costs a
+    // third of a full one even when nearly empty (18944 x 3584 at M = 1, 56 column tiles: 16.5 us
+    // in 9 splits, 504 workgroups, against 21.7 us in 10).
+    // (One or two rows over a small table - short workgroups, next to no partial sums - take the
+    // extra round lightly: 4096 x 22016 at M = 1 21.1 us in two splits, 688 workgroups, against 22.9 us
+    // unsplit; at M = 16 27.1 against 24.3 us.)
+    const double late = (M <= 2 && table1 <= 16 * 1024) ? 0.1 : 0.35;
+    auto grid_cost = [late](double wgs, double slots) {
+      if (wgs <= slots) return slots / wgs;
+      const double full = floor(wgs / slots), rem = wgs - full * slots;
+      return full + (rem > 0.0 ? late + (1.0 - late) * rem / slots : 0.0);
+    };
+    int best_dv = chunks / c.wk;
+    int best_wk = c.wk;
     double best = -1.0;
-    for (int dv = 1; dv <= max_dv; ++dv) {
-      if (lds_bytes(dv) > 150000) continue;
-      const double slots = lds_bytes(dv) > 80 * 1024 ? 256.0 : 512.0;
-      const double wgs = (double)tiles * dv;
-      double cost = wgs >= slots ? wgs / slots : slots / wgs;
-      const int per_wave = (chunks + dv * c.wk - 1) / (dv * c.wk);  // chunks of the busiest wave
-      cost *= (double)per_wave * dv * c.wk / chunks;
-      if (slots < 512.0) cost *= 1.5;  // one workgroup per CU: half the waves to hide the lookups
-      if (best < 0.0 || cost <= best) {
-        best = cost;
-        best_dv = dv;
+    // a short K that deals out evenly over four waves but not over eight is also tried with four
+    // (3584 x 4608 at M = 1: 8.4 us as 4 x 7 against 10.2 us as 8 x 3, ragged)
+    const bool try4 = c.wk == 8 && chunks % 8 != 0 && chunks % 4 == 0 && chunks <= 32;
+    for (int wk = c.wk; wk >= (try4 ? 4 : c.wk); wk -= 4) {
+      for (int dv = 1; dv <= chunks / wk; ++dv) {
+        if (lds_bytes(dv) > 150000) continue;
+        const double slots = (lds_bytes(dv) > 80 * 1024 ? 256.0 : 512.0) * (wk == 4 ? 2.0 : 1.0);
+        double cost = grid_cost((double)tiles * dv, slots);
+        const int per_wave = (chunks + dv * wk - 1) / (dv * wk);  // chunks of the busiest wave
+        cost *= (double)per_wave * dv * wk / chunks;
+        if (lds_bytes(dv) > 80 * 1024) cost *= 1.5;  // one workgroup per CU: half the waves to hide the lookups
+        if (wk == 4) cost *= 1.1;             // twice the table builds
+        if (best < 0.0 || cost <= best) {
+          best = cost;
+          best_dv = dv;
+          best_wk = wk;
+        }
       }
     }
+    c.wk = best_wk;
     c.splits = best_dv;
     // One 1024-thread workgroup per CU - two column tiles x eight K waves around one table of 128
     // columns - where 200 to 256 such workgroups make one round and their decomposition costs no more:
