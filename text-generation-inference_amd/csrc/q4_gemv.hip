@@ -194,11 +194,12 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
       if (lds > 150000) continue;
       const double wgs = (double)n64 * dv;
       // Where some split count fills three quarters of the CUs or more in one round, going beyond
-      // one workgroup per CU lets the CUs that take one more decide (18944 x 3584 at M = 1: 11.6 us
-      // in 224 workgroups, 13.3 us in 280, 11.7 us in 504; 6144 x 6144: 8.6 us in 192, 10.1 us in
-      // 288).  Where none does, a round and a quarter beats a round that leaves a third of the chip
-      // idle (8192 x 10240: 15.1 us in 320 workgroups, 16.5 us in 160).
-      double cost = wgs > 256.0 ? (full_round ? 1.12 * ceil(wgs / 256.0) * 256.0 / wgs : wgs / 256.0) : 256.0 / wgs;
+      // one workgroup per CU lets the CUs that take one more decide and is charged as whole rounds
+      // (18944 x 3584 at M = 1: 11.6 us in 224 workgroups, 13.3 us in 280, 11.7 us in 504;
+      // 6144 x 6144: 8.6 us in 192, 10.1 us in 288).  Where none does, a round and a quarter beats
+      // a round that leaves a third of the chip idle (8192 x 10240: 15.1 us in 320 workgroups,
+      // 16.5 us in 160).
+      double cost = wgs > 256.0 ? (full_round ? ceil(wgs / 256.0) : wgs / 256.0) : 256.0 / wgs;
       if (chunks % (dv * c.wk) != 0) cost *= 1.1;
       if (best_cost < 0.0 || cost < best_cost) {
         best_cost = cost;
