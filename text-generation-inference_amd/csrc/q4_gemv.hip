@@ -334,10 +334,11 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
       // A few workgroups more than CUs: the CUs that take two decide, and when the slab leaves
       // room for one per CU they form a second, nearly empty round (3072 x 9216, 288 workgroups:
       // 10.8 / 11.9 / 17.9 us at M = 4 / 8 / 16).  One round of the lean kernel's 64-column tiles,
-      // eight waves over the whole K with their own activations, takes 9.0 / 9.6 / 10.7 us.
+      // eight waves over the whole K with their own activations, takes 9.0 / 9.6 / 10.7 us - where
+      // those tiles are half the CUs or more (8192 x 1280 has 20: 14 us against 7.9 us).
       const long wgs = tiles * pick;
       const int per_wave = (chunks + 7) / 8;
-      if ((wgs + 255) / 256 * 256 * 2 > wgs * 3 && w->N / 64 <= 256 &&
+      if (wgs > 256 && (wgs + 255) / 256 * 256 * 2 > wgs * 3 && w->N / 64 >= 128 && w->N / 64 <= 256 &&
           (long)rows * 8 * (per_wave * 256 + 16) + 512 <= 150000) {
         GemvConfig l = c;
         l.lean = 1;
@@ -393,7 +394,7 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
     double best = -1.0;
     // a short K that deals out evenly over four waves but not over eight is also tried with four
     // (3584 x 4608 at M = 1: 8.4 us as 4 x 7 against 10.2 us as 8 x 3, ragged)
-    const bool try4 = c.wk == 8 && chunks % 8 != 0 && chunks % 4 == 0 && chunks <= 32;
+    const bool try4 = c.wk == 8 && chunks % 8 != 0 && chunks % 4 == 0 && chunks <= 32 && mchunks == 1;
     for (int wk = c.wk; wk >= (try4 ? 4 : c.wk); wk -= 4) {
       for (int dv = 1; dv <= chunks / wk; ++dv) {
         if (lds_bytes(dv) > 150000) continue;
