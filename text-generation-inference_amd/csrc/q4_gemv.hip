@@ -189,6 +189,7 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
     for (int dv = 1; !wide && dv * c.wk <= chunks && (long)n64 * dv <= 256; ++dv)
       if ((long)n64 * dv >= 192 && (long)rows * c.wk * ((long)((chunks + dv * c.wk - 1) / (dv * c.wk)) * 256 + 16) <= 150000)
         full_round = true;
+    if (n64 >= 128 && chunks >= 64 && M <= 3) full_round = true;
     for (int dv = 1; !wide && dv * c.wk <= chunks; ++dv) {
       const long lds = (long)rows * c.wk * ((long)((chunks + dv * c.wk - 1) / (dv * c.wk)) * 256 + 16);
       if (lds > 150000) continue;
@@ -196,9 +197,10 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
       // Where some split count fills three quarters of the CUs or more in one round, going beyond
       // one workgroup per CU lets the CUs that take one more decide and is charged as whole rounds
       // (18944 x 3584 at M = 1: 11.6 us in 224 workgroups, 13.3 us in 280, 11.7 us in 504;
-      // 6144 x 6144: 8.6 us in 192, 10.1 us in 288).  Where none does, a round and a quarter beats
-      // a round that leaves a third of the chip idle (8192 x 10240: 15.1 us in 320 workgroups,
-      // 16.5 us in 160).
+      // 6144 x 6144: 8.6 us in 192, 10.1 us in 288), and so it is over a long K whose tiles cover
+      // half the CUs (8192 x 10240 at M = 1: 12.8 us in 160 workgroups, 14.7 us in 320, 16.5 us in
+      // 480).  A short K with fewer tiles than that keeps its round and a third (4096 x 11008 at
+      // M = 3: 12.9 us in 344 workgroups, 14.3 us in 172).
       double cost = wgs > 256.0 ? (full_round ? ceil(wgs / 256.0) : wgs / 256.0) : 256.0 / wgs;
       if (chunks % (dv * c.wk) != 0) cost *= 1.1;
       if (best_cost < 0.0 || cost < best_cost) {
