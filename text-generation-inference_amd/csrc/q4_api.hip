@@ -117,7 +117,11 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
       const long slab = (long)c.rows_per_block * ((chunks + c.splits - 1) / c.splits * 256 + 16);
       if (slab > 75 * 1024 && wgs > 256) blocks34 = false;
     }
-    const bool small = M <= 16 || gemv_rows32_supported(w, M) || (M <= 32 && w->K <= 8192 && weights <= (1L << 26)) || blocks34;
+    // Two blocks: up to K = 4096 (us at M = 32, decode / prefill: 4096 x 14336 18.7 / 19.3, 3072 x 16384
+    // 15.1 / 17.2, but 6144 x 6144 23.5 / 17.0, 8192 x 7168 31.0 / 19.5, 8192 x 8192 22.5 / 20.3, 5120 x 5120
+    // 21.3 / 15.2), beyond that on the smallest matrices only (5120 x 3072 12.1 / 13.6).
+    const bool blocks2 = M <= 32 && weights <= (w->K <= 4096 ? (1L << 26) : (1L << 24));
+    const bool small = M <= 16 || gemv_rows32_supported(w, M) || blocks2 || blocks34;
     if (small && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
     if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;
     if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;

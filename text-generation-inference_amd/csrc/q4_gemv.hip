@@ -80,7 +80,12 @@ bool gemv_rows32_supported(const q4_weight* w, int M) {
   const GemvConfig c = gemv_pick_config(w, 16, false);
   const long chunks = w->K / 128;
   const long kr = (chunks + c.splits - 1) / c.splits * 128;
-  return (long)M * (kr * 2 + 16) <= 150000;
+  const long slab = (long)M * (kr * 2 + 16);
+  if (slab > 150000) return false;
+  // a slab that leaves room for one workgroup per CU, and more workgroups than CUs: two rounds
+  // (8192 x 7168: 19.4 us at M = 17, 27.9 us at M = 20 against 18.4 us for the prefill kernel)
+  const long wgs = (long)(w->N / (16 * c.words * c.wcol)) * c.splits;
+  return !(slab > 75 * 1024 && wgs > 256);
 }
 
 static GemvConfig pick_config(const q4_weight* w, int M, bool gate_up, bool allow_lean);
