@@ -241,7 +241,7 @@ def test_path_selection_and_workspace(pkg):
         assert lib.q4_select_path(ctypes.byref(w), M, 0) == want
     # the decode kernel's reach depends on the shape (measured crossovers); 17..20 rows stay on it
     # while the activation slab of the 16-row configuration still fits LDS
-    for K, N, last_gemv in [(4096, 6144, 32), (4096, 14336, 32), (4096, 28672, 18), (8192, 8192, 32), (8192, 10240, 18), (14336, 4096, 20)]:
+    for K, N, last_gemv in [(4096, 6144, 32), (4096, 14336, 32), (4096, 28672, 18), (8192, 8192, 20), (8192, 10240, 18), (14336, 4096, 20), (6144, 6144, 20)]:
         w2 = _weight(pkg, K, N, 128)
         assert lib.q4_select_path(ctypes.byref(w2), last_gemv, 0) == L.PATH_GEMV, (K, N)
         assert lib.q4_select_path(ctypes.byref(w2), last_gemv + 1, 0) == L.PATH_GEMM, (K, N)
