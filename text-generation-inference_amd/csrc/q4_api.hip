@@ -121,7 +121,12 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
     // 15.1 / 17.2, but 6144 x 6144 23.5 / 17.0, 8192 x 7168 31.0 / 19.5, 8192 x 8192 22.5 / 20.3, 5120 x 5120
     // 21.3 / 15.2), beyond that on the smallest matrices only (5120 x 3072 12.1 / 13.6).
     const bool blocks2 = M <= 32 && weights <= (w->K <= 4096 ? (1L << 26) : (1L << 24));
-    const bool small = M <= 16 || gemv_rows32_supported(w, M) || blocks2 || blocks34;
+    bool small = M <= 16 || gemv_rows32_supported(w, M) || blocks2 || blocks34;
+    // bf16: past 16 rows the decode kernel converts every unpacked pair and the prefill kernel does
+    // not; it keeps 17 to 32 rows on the smallest matrices only (us at M = 24, decode / prefill:
+    // 4096 x 4096 12.7 / 13.8, but 4096 x 14336 23.4 / 19.0, 2048 x 8192 13.4 / 11.7, 8192 x 8192 at
+    // M = 17 20.9 / 18.8, 14336 x 4096 at M = 20 20.4 / 19.0)
+    if (dtype == Q4_DTYPE_BF16 && M > 16) small = M <= 32 && weights <= (1L << 24) && w->K >= 3072;
     if (small && gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
     if (gemm_supported(w, M, dtype)) return Q4_PATH_GEMM;
     if (gemv_supported(w, M, dtype)) return Q4_PATH_GEMV;
