@@ -417,6 +417,13 @@ def act_mul(gate_up: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor
     return y
 
 
+def _plain_decode_is_lean(w: PackedWeight) -> bool:
+    """Whether q4_linear runs the instruction-lean decode kernel on this weight at up to 16 rows:
+    GPTQ layout, contiguous groups of whole 128-row chunks, 32 M weights or more."""
+    return (w.layout == LAYOUT_GPTQ and w.g_idx is None and w.groupsize >= 128 and w.groupsize % 128 == 0
+            and w.K % 128 == 0 and w.K >= 1024 and w.N % 64 == 0 and w.K * w.N >= (1 << 25))
+
+
 def linear_gate_up(
     w: PackedWeight,
     x: torch.Tensor,
@@ -449,6 +456,12 @@ def linear_gate_up(
     if M == 0 or inter == 0:
         return y
     fusable_bias = bias is None or (bias.dtype == x.dtype and bias.is_cuda and bias.numel() == w.N)
+    if fused is None and M <= 2 and _plain_decode_is_lean(w):
+        # one or two rows on a large layer: the instruction-lean decode kernel followed by the
+        # elementwise kernel beats the decode kernel with the gated epilogue (us on MI355X, fused / two
+        # launches: 4096 x 28672 17.7 / 16.6 at M = 1, 3072 x 16384 17.1 / 11.3 at M = 2, 8192 x 57344
+        # 53.7 / 47.5 at M = 2; 4096 x 22016 at M = 1, 16.1 / 17.0, is the one shape measured that loses)
+        fused = False
     if fused is not False and fusable_bias:
         lib = _lib.load()
         with _on_device(x.device):
