@@ -312,9 +312,12 @@ static GemvConfig pick_config_search(const q4_weight* w, int M, bool gate_up, bo
   // M = 16; 4096 x 6144 9.8 / 10.7 at M = 9, 10.5 / 11.9 at M = 16; 8192 x 1024 7.5 / 9.1,
   // 7.8 / 10.1, 8.3 / 9.5 at M = 4, 8, 16; 2048 x 8192 6.4 / 8.2, 7.1 / 8.2, 7.9 / 9.7.
   if (allow_lean && !gate_up && w->layout == Q4_LAYOUT_GPTQ && w->g_idx == nullptr && w->groupsize >= 128 &&
-      w->groupsize % 128 == 0 && M >= 4 && M <= 16 && chunks % 8 == 0 && chunks >= 16 && w->N % 64 == 0 &&
+      w->groupsize % 128 == 0 && M >= 4 && M <= 16 && chunks % 8 == 0 && chunks >= 8 && w->N % 64 == 0 &&
       // (4096 x 6144 up to 8 rows: no better than the rule below)
-      (M >= 9 || w->N <= 4096 || w->N / 32 >= 256)) {
+      (M >= 9 || w->N <= 4096 || w->N / 32 >= 256) &&
+      // K = 1024: the eight-wave tiles only, up to two rounds of them (1024 x 8192 6.8 / 7.2 / 8.3 ->
+      // 4.9 / 5.2 / 5.8 us at M = 4 / 8 / 16, 1024 x 2048 6.5 -> 4.7 us; 1024 x 28672, 896 tiles: 8.3 -> 10.6 us)
+      (chunks >= 16 || ((w->N / 32 >= 256 || w->N <= 2048) && w->N / 32 <= 512))) {
     const bool narrow = w->N / 32 >= 256 || w->N <= 2048;  // one 32-column tile per workgroup, eight waves along K
     GemvConfig t = c;
     t.words = 2;
