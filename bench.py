@@ -23,6 +23,7 @@ Prints exactly one JSON line on stdout.
 from __future__ import annotations
 
 import argparse
+import ctypes
 import importlib
 import json
 import os
@@ -41,13 +42,43 @@ MFMA_PEAK_TFLOPS = 2500.0    # MI355X dense fp16/bf16 MFMA peak
 TRAFFIC_FILE = ROOT / "profiles" / "hbm_traffic.json"
 
 
-def measured_traffic(key):
-    """Bytes per launch from the tracked counter summary, or None when there is none."""
+def measured_traffic(key, field="bytes_per_launch"):
+    """Bytes per launch from the tracked counter summary (or the commit it was measured at), or
+    None when there is none."""
     try:
         entry = json.loads(TRAFFIC_FILE.read_text())[key]
-        return int(entry["bytes_per_launch"])
+        return int(entry[field]) if field == "bytes_per_launch" else entry[field]
     except (OSError, KeyError, ValueError, TypeError):
         return None
+
+
+PACKAGE_DIR = ROOT / "text-generation-inference_amd"
+_probe_lib = None
+
+
+def load_probe_lib():
+    """The benchmark's own probe kernels (libq4probe.so, csrc/bench/q4_probe.hip): read-only and
+    LDS-read launches.  Not part of the product library."""
+    global _probe_lib
+    if _probe_lib is None:
+        path = PACKAGE_DIR / "libq4probe.so"
+        if not path.exists():
+            raise ImportError(f"{path} is missing: build it with `python {PACKAGE_DIR / 'build.py'}`")
+        lib = ctypes.CDLL(str(path))
+        vp, ci = ctypes.c_void_p, ctypes.c_int
+        lib.q4_probe_read.restype = ci
+        lib.q4_probe_read.argtypes = [vp, ctypes.c_size_t, ci, ci, ci, ci, ci, ci, vp, vp]
+        lib.q4_probe_lds.restype = ci
+        lib.q4_probe_lds.argtypes = [vp, ci, ci, vp, vp]
+        lib.q4_probe_last_error.restype = ctypes.c_char_p
+        lib.q4_probe_last_error.argtypes = []
+        _probe_lib = lib
+    return _probe_lib
+
+
+def probe_check(rc):
+    if rc < 0:
+        raise RuntimeError(f"libq4probe error {rc}: {load_probe_lib().q4_probe_last_error().decode()}")
 
 SHAPES = [  # name, K, N
     ("qkv_proj", 4096, 6144),
@@ -90,6 +121,12 @@ def parse_args():
                     help="a few launches of the act-order kernels that read the checkpoint through g_idx: decode at "
                          "M = 1 and 16 on 28672 x 8192, prefill (M = --gemm-m) on 8192 x 10240, for counter runs "
                          "under rocprofv3")
+    ap.add_argument("--probe-trace", action="store_true",
+                    help="eager launches of the empty and the read-only probe kernels on the decode kernels' own "
+                         "grids, then of the decode kernels, for a rocprofv3 --kernel-trace run; prints no JSON line")
+    ap.add_argument("--phase-breakdown", action="store_true",
+                    help="run the four decode projections (M = --m) on the phase-stamp build of the library "
+                         "(libq4linear_stamps.so) and print where a launch's time goes, wave by wave")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="eager launches only (a 256 MiB copy kernel, then each decode shape and one GEMM), "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs; prints no JSON line")
@@ -108,14 +145,21 @@ def make_weights(pkg, torch, device, K, N, seed):
     return pkg.ops.make_packed(qweight, qzeros, scales, None, GROUPSIZE, 0)
 
 
-def make_weights_variant(pkg, torch, device, K, N, seed, kind):
-    """The same synthetic tensors in the AWQ layout ("awq": qweight [K, N/8]) or as GPTQ with a
-    shuffled g_idx ("act_order")."""
+def make_weights_variant(pkg, torch, device, K, N, seed, kind, zeros=None):
+    """The same synthetic tensors in the AWQ layout ("awq": qweight [K, N/8], per-group zero
+    points uniform 0..15 as BASELINE.json configs[4] states) or as GPTQ with a shuffled g_idx
+    ("act_order": symmetric, one zero point, as configs[3] states; zeros="per_column" draws them
+    uniformly instead)."""
     g = torch.Generator(device=device)
     g.manual_seed(seed)
     G = K // GROUPSIZE
     scales = (torch.rand((G, N), device=device, generator=g) * (2e-2 - 1e-3) + 1e-3).to(torch.float16)
-    qzeros = torch.full((G, N // 8), 0x77777777, dtype=torch.int32, device=device)
+    if zeros is None:
+        zeros = "per_column" if kind == "awq" else "one"
+    if zeros == "per_column":
+        qzeros = torch.randint(-(2**31), 2**31 - 1, (G, N // 8), dtype=torch.int64, device=device, generator=g).to(torch.int32)
+    else:
+        qzeros = torch.full((G, N // 8), 0x77777777, dtype=torch.int32, device=device)
     if kind == "awq":
         qweight = torch.randint(-(2**31), 2**31 - 1, (K, N // 8), dtype=torch.int64, device=device, generator=g).to(torch.int32)
         return pkg.ops.make_packed(qweight, qzeros, scales, None, GROUPSIZE, 1)
@@ -233,46 +277,53 @@ def cpu_baseline(M):
 
 def read_floor_configs(K, N):
     """Grids of the read-only tile kernel for a [K/8, N] matrix of packed words: (workgroups,
-    threads, unroll) with the row steps dividing evenly, around the decode kernels' own grids."""
-    ntiles = N // 64
+    threads, unroll, column waves per workgroup) with the row steps dividing evenly, around the
+    decode kernels' own grids (two column waves x four K waves x unsplit K is the gate_up launch:
+    224 workgroups of 512 threads)."""
     steps_total = K // 32  # four packed rows per wave load
     out = []
-    for wk in (4, 8, 16):
-        for splits in (1, 2, 4, 7, 8, 14, 16):
-            slots = wk * splits
-            if steps_total % slots:
+    for wcol in (1, 2):
+        if N % (64 * wcol):
+            continue
+        ntiles = N // (64 * wcol)
+        for wk in (4, 8, 16):
+            if wcol * wk > 16:
                 continue
-            per = steps_total // slots
-            wgs = ntiles * splits
-            if wgs < 192 or wgs > 4096:
-                continue
-            for unroll in (2, 4, 8):
-                if per % unroll == 0:
-                    out.append((wgs, 64 * wk, unroll))
+            for splits in (1, 2, 4, 7, 8, 14, 16):
+                slots = wk * splits
+                if steps_total % slots:
+                    continue
+                per = steps_total // slots
+                wgs = ntiles * splits
+                if wgs < 192 or wgs > 4096:
+                    continue
+                for unroll in (2, 4, 8):
+                    if per % unroll == 0:
+                        out.append((wgs, 64 * wk * wcol, unroll, wcol))
     return out
 
 
-def time_read_floor(pkg, torch, lib, dev, pool, sink, nbytes, pattern, n_words, wgs, threads, unroll, hot, reps=24):
+def time_read_floor(torch, pool, sink, nbytes, pattern, n_words, wgs, threads, unroll, hot, reps=24, wcol=1):
     """Average us of one read-only launch over `nbytes`; the launches of a graph walk through
     `pool` (larger than the last-level cache) unless `hot`."""
+    lib = load_probe_lib()
     pieces = max(1, pool.numel() // nbytes)
-    stream = torch.cuda.Stream()
     fns = []
     for r in range(1 if hot else min(pieces, reps)):
         ptr = pool.data_ptr() + r * nbytes
 
         def fn(ptr=ptr):
-            rc = lib.q4_probe_read(ptr, nbytes, pattern, n_words, wgs, threads, unroll, sink.data_ptr(),
-                                   torch.cuda.current_stream().cuda_stream)
-            pkg._lib.check(rc)
+            probe_check(lib.q4_probe_read(ptr, nbytes, pattern, n_words, wgs, threads, unroll, wcol, sink.data_ptr(),
+                                          torch.cuda.current_stream().cuda_stream))
         fns.append(fn)
     avg, best = time_kernel_launches(torch, fns, reps)
     return avg * 1e6, best * 1e6
 
 
-def lds_probe(pkg, torch, lib, dev):
+def lds_probe(torch, dev):
     """ns per wave-level ds_read_b128 (16 waves per CU, all CUs) for lane -> 16-byte-unit maps.
     256 B per clock would be ~2.1 ns at the clock these launches run at."""
+    lib = load_probe_lib()
     sink = torch.zeros(4, dtype=torch.uint8, device=dev)
     blocks = lambda order: [u for b in order for u in range(8 * b, 8 * b + 8)]  # residues per 8-lane block
     maps = [
@@ -295,10 +346,10 @@ def lds_probe(pkg, torch, lib, dev):
         stream = torch.cuda.current_stream().cuda_stream
         best = None
         for rep in range(4):
-            pkg._lib.check(lib.q4_probe_lds(dm.data_ptr(), 10, 256, sink.data_ptr(), stream))
+            probe_check(lib.q4_probe_lds(dm.data_ptr(), 10, 256, sink.data_ptr(), stream))
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            pkg._lib.check(lib.q4_probe_lds(dm.data_ptr(), iters, 256, sink.data_ptr(), stream))
+            probe_check(lib.q4_probe_lds(dm.data_ptr(), iters, 256, sink.data_ptr(), stream))
             e1.record()
             e1.synchronize()
             ns = e0.elapsed_time(e1) * 1e6 / (16.0 * iters * 8)
@@ -308,7 +359,7 @@ def lds_probe(pkg, torch, lib, dev):
     return rows
 
 
-def floor_probe(pkg, torch, lib, dev):
+def floor_probe(torch, dev):
     """Table of read-only launches: empty grids, linear reads and the decode tile pattern at the
     four projections' sizes, HBM-rotating (1 GiB pool) and cache-hot."""
     pool = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
@@ -316,7 +367,7 @@ def floor_probe(pkg, torch, lib, dev):
     rows = []
     for wgs in (256, 1024, 4096):
         for threads in (256, 512):
-            us, _ = time_read_floor(pkg, torch, lib, dev, pool, sink, 4096, 2, 0, wgs, threads, 1, True)
+            us, _ = time_read_floor(torch, pool, sink, 4096, 2, 0, wgs, threads, 1, True)
             rows.append({"what": "empty", "workgroups": wgs, "threads": threads, "us": round(us, 2)})
             print(f"empty kernel           wgs {wgs:5d} x {threads:4d}                       {us:7.2f} us", flush=True)
     summary = {}
@@ -331,28 +382,141 @@ def floor_probe(pkg, torch, lib, dev):
                     if (nbytes // 16 // wgs // rnd * rnd) * 16 * wgs != nbytes:
                         continue
                     for hot in (False, True):
-                        us, _ = time_read_floor(pkg, torch, lib, dev, pool, sink, nbytes, 0, 0, wgs, threads, unroll, hot)
+                        us, _ = time_read_floor(torch, pool, sink, nbytes, 0, 0, wgs, threads, unroll, hot)
                         key = "linear_hot" if hot else "linear"
                         if key not in best or us < best[key]["us"]:
                             best[key] = {"workgroups": wgs, "threads": threads, "unroll": unroll, "us": round(us, 2)}
                         rows.append({"what": key, "shape": name, "workgroups": wgs, "threads": threads, "unroll": unroll,
                                      "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1)})
-        for wgs, threads, unroll in read_floor_configs(K, N):
+        for wgs, threads, unroll, wcol in read_floor_configs(K, N):
             for hot in (False, True):
-                us, _ = time_read_floor(pkg, torch, lib, dev, pool, sink, nbytes, 1, N, wgs, threads, unroll, hot)
+                us, _ = time_read_floor(torch, pool, sink, nbytes, 1, N, wgs, threads, unroll, hot, wcol=wcol)
                 key = "tile_hot" if hot else "tile"
                 if key not in best or us < best[key]["us"]:
-                    best[key] = {"workgroups": wgs, "threads": threads, "unroll": unroll, "us": round(us, 2)}
+                    best[key] = {"workgroups": wgs, "threads": threads, "unroll": unroll, "column_waves": wcol, "us": round(us, 2)}
                 rows.append({"what": key, "shape": name, "workgroups": wgs, "threads": threads, "unroll": unroll,
-                             "bytes_in_flight_per_wave": unroll * 1024, "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1)})
-                print(f"{name:13s} {key:9s} wgs {wgs:5d} x {threads:4d} unroll {unroll}  {nbytes / 1e6:6.1f} MB  {us:7.2f} us  "
-                      f"{nbytes / us / 1e3:7.1f} GB/s", flush=True)
+                             "column_waves": wcol, "bytes_in_flight_per_wave": unroll * 1024, "us": round(us, 2),
+                             "GBps": round(nbytes / us / 1e3, 1)})
+                print(f"{name:13s} {key:9s} wgs {wgs:5d} x {threads:4d} ({wcol} column waves) unroll {unroll}  "
+                      f"{nbytes / 1e6:6.1f} MB  {us:7.2f} us  {nbytes / us / 1e3:7.1f} GB/s", flush=True)
         for key, b in best.items():
             b["GBps"] = round(nbytes / b["us"] / 1e3, 1)
         summary[name] = {"bytes": nbytes, **best}
         print(f"== {name}: " + "  ".join(f"{k} {v['us']} us ({v['GBps']} GB/s, {v['workgroups']}x{v['threads']} u{v['unroll']})"
                                           for k, v in best.items()), flush=True)
     print(json.dumps({"read_floor": summary}))
+
+
+# the decode kernels' own launch geometry at M = 1 on the four projections: (workgroups, threads,
+# column waves per workgroup), for the probe launches that are to be compared with them
+DECODE_GRIDS = {"qkv_proj": (768, 256, 1), "o_proj": (512, 256, 1), "gate_up_proj": (224, 512, 2), "down_proj": (256, 512, 1)}
+
+
+def probe_trace(pkg, torch, dev, weights, xs, ys, copies, reps=40):
+    """Eager launches for a rocprofv3 --kernel-trace run: per projection an empty kernel and the
+    read-only tile kernel on the decode kernel's grid (weights-sized ranges of a 1 GiB pool, so
+    every launch reads from HBM), then the decode kernel itself on rotating weights.  The trace
+    gives all three in the same unit (begin -> end of a dispatch)."""
+    lib = load_probe_lib()
+    pool = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+    sink = torch.zeros(4, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    for i, (name, K, N) in enumerate(SHAPES):
+        wgs, threads, wcol = DECODE_GRIDS[name]
+        nbytes = K * N // 2
+        pieces = pool.numel() // nbytes
+        steps = (K // 32) // ((wgs // (N // (64 * wcol))) * (threads // 64 // wcol))
+        unroll = 8 if steps % 8 == 0 else (4 if steps % 4 == 0 else (2 if steps % 2 == 0 else 1))
+        for r in range(reps):
+            probe_check(lib.q4_probe_read(pool.data_ptr(), 4096, 2, 0, wgs, threads, 1, 1, sink.data_ptr(), stream))
+        torch.cuda.synchronize()
+        for r in range(reps):
+            probe_check(lib.q4_probe_read(pool.data_ptr() + (r % pieces) * nbytes, nbytes, 1, N, wgs, threads, unroll, wcol,
+                                          sink.data_ptr(), stream))
+        torch.cuda.synchronize()
+        for r in range(reps):
+            pkg.ops.linear(weights[r % copies][i], xs[i], None, out=ys[i])
+        torch.cuda.synchronize()
+        print(f"probe trace: {name} {K}x{N}: {reps} empty launches ({wgs} x {threads}), {reps} read-only launches of "
+              f"{nbytes} B (unroll {unroll}, {wcol} column waves), {reps} decode launches", file=sys.stderr)
+
+
+PHASES = ["entry", "activations staged", "first chunk consumed", "K loop done",
+          "K waves combined (LDS)", "split-K combine returned", "first weight loads issued", "exit"]
+PHASE_ORDER = [0, 6, 1, 2, 3, 4, 5, 7]
+
+
+def phase_breakdown(pkg, torch, dev, M, copies, launches=24):
+    """Where a decode launch's time goes.  Runs the phase-stamp build of the library: every wave
+    reads the 100 MHz clock at its phase boundaries (PhaseStamps, csrc/q4_gemv_kernels.cuh) and
+    stores the readings when it ends.  Launches run as a HIP graph over rotating weights, like the
+    timed legs.  Per stamp: the earliest / median / latest wave, in us since the first wave of the
+    launch entered, averaged over the launches."""
+    import numpy as np
+
+    lib = pkg._lib.load()
+    lib.q4_phase_stamps_target.restype = None
+    lib.q4_phase_stamps_target.argtypes = [ctypes.c_void_p]
+    out = {}
+    slots = 8192  # waves per launch the buffer has room for
+    for i, (name, K, N) in enumerate(SHAPES):
+        ws = [make_weights(pkg, torch, dev, K, N, seed=17 * c + i) for c in range(copies)]
+        x = torch.randn((M, K), device=dev, dtype=torch.float16)
+        y = torch.empty((M, N), device=dev, dtype=torch.float16)
+        stamps = torch.zeros((launches, slots, 8), dtype=torch.int64, device=dev)
+        pkg.ops.reserve_workspace(dev, pkg.ops.workspace_bytes(M, K, N))
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            lib.q4_phase_stamps_target(None)
+            pkg.ops.linear(ws[0], x, None, out=y)
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for r in range(launches):
+                    lib.q4_phase_stamps_target(stamps[r].data_ptr())
+                    pkg.ops.linear(ws[r % copies], x, None, out=y)
+            lib.q4_phase_stamps_target(None)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            stamps.zero_()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(side)
+            graph.replay()
+            e1.record(side)
+            torch.cuda.synchronize()
+            us_per_launch = e0.elapsed_time(e1) * 1e3 / launches
+        t = stamps.cpu().numpy().astype(np.int64)
+        rows = {ph: [] for ph in range(8)}
+        spans, waves = [], 0
+        for r in range(launches):
+            live = t[r][t[r][:, 0] != 0]
+            if live.shape[0] == 0:
+                continue
+            waves = live.shape[0]
+            t0 = live[:, 0].min()
+            spans.append((live[:, 7].max() - t0) * 0.01)
+            for ph in range(8):
+                v = live[:, ph]
+                v = v[v != 0]
+                if v.size:
+                    rel = (v - t0) * 0.01  # 100 MHz counter -> us
+                    rows[ph].append((rel.min(), np.median(rel), rel.max(), v.size))
+        entry = {"K": K, "N": N, "waves": int(waves), "us_per_launch_with_stamps": round(us_per_launch, 2),
+                 "first_entry_to_last_exit_us": round(float(np.mean(spans)), 2) if spans else None, "phases": {}}
+        print(f"== {name} {K}x{N} M={M}: {waves} waves, {us_per_launch:.2f} us per launch (graph replay, stamps on), "
+              f"first wave in -> last wave out {entry['first_entry_to_last_exit_us']} us", flush=True)
+        for ph in PHASE_ORDER:
+            if rows[ph]:
+                a = np.array([r[:3] for r in rows[ph]], dtype=np.float64).mean(axis=0)
+                n = int(np.mean([r[3] for r in rows[ph]]))
+                entry["phases"][PHASES[ph]] = {"first_wave_us": round(a[0], 2), "median_wave_us": round(a[1], 2),
+                                               "last_wave_us": round(a[2], 2), "waves": n}
+                print(f"   {PHASES[ph]:42s} first {a[0]:6.2f}  median {a[1]:6.2f}  last {a[2]:6.2f}  ({n} waves)", flush=True)
+        out[name] = entry
+        del ws, stamps, graph
+        torch.cuda.empty_cache()
+    print(json.dumps({"phase_breakdown": out}))
 
 
 def main():
@@ -364,7 +528,10 @@ def main():
     import torch
 
     pkg = importlib.import_module("text-generation-inference_amd")
-    lib = pkg._lib.load()
+    if args.phase_breakdown:
+        # this process runs the measurement build of the library (same sources, -DQ4_PHASE_STAMPS)
+        pkg._lib.LIB_PATH = PACKAGE_DIR / "libq4linear_stamps.so"
+    pkg._lib.load()
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
@@ -375,6 +542,9 @@ def main():
     step_bytes = sum(gemv_bytes(M, K, N) for _, K, N in SHAPES)
     copies = args.copies or max(2, -(-512 * 1024 * 1024 // step_weight_bytes) + 1)
 
+    if args.phase_breakdown:
+        phase_breakdown(pkg, torch, dev, M, copies)
+        return
     weights = [[make_weights(pkg, torch, dev, K, N, seed=17 * c + i) for i, (_, K, N) in enumerate(SHAPES)]
                for c in range(copies)]
     xs = [torch.randn((M, K), device=dev, dtype=torch.float16) for _, K, N in SHAPES]
@@ -387,7 +557,7 @@ def main():
             pkg.ops.linear(weights[c % copies][i], xs[i], None, out=ys[i])
 
     if args.lds_probe:
-        print(json.dumps({"lds_probe": lds_probe(pkg, torch, lib, dev)}))
+        print(json.dumps({"lds_probe": lds_probe(torch, dev)}))
         return
     if args.awq_probe:
         K, N, Mg = 4096, 14336, args.gemm_m
@@ -425,7 +595,10 @@ def main():
               % (Kd, Nd, Mg, Kp, Np), file=sys.stderr)
         return
     if args.floor_probe:
-        floor_probe(pkg, torch, lib, dev)
+        floor_probe(torch, dev)
+        return
+    if args.probe_trace:
+        probe_trace(pkg, torch, dev, weights, xs, ys, copies)
         return
 
     if args.traffic_probe:
@@ -503,8 +676,8 @@ def main():
         pool = torch.empty(1 << 29, dtype=torch.uint8, device=dev).random_(0, 255)
         sink = torch.zeros(4, dtype=torch.uint8, device=dev)
         for name, K, N in SHAPES:
-            floor = min(time_read_floor(pkg, torch, lib, dev, pool, sink, K * N // 2, 1, N, wgs, threads, unroll, False)[0]
-                        for wgs, threads, unroll in read_floor_configs(K, N) if unroll == 4)
+            floor = min(time_read_floor(torch, pool, sink, K * N // 2, 1, N, wgs, threads, unroll, False, wcol=wcol)[0]
+                        for wgs, threads, unroll, wcol in read_floor_configs(K, N) if unroll == 4)
             per_shape[name]["read_only_floor_us"] = round(floor, 2)
         del pool
     # the same call outside a graph: Python + ctypes + launch per call (o_proj, M rows)
@@ -529,6 +702,7 @@ def main():
         # workload (mean over the four projections, calibrated with a 256 MiB copy kernel);
         # only valid for the default M=1 workload, null otherwise
         "traffic": measured_traffic("decode_m1") if M == 1 else None,
+        "traffic_measured_at_commit": measured_traffic("decode_m1", "measured_at_commit") if M == 1 else None,
         "bytes_per_launch": all_bytes // len(SHAPES),
         "us_per_launch": round(sum(all_durs) / len(SHAPES) * 1e6, 2),
     }
@@ -642,7 +816,8 @@ def main():
                 "roofline": {"bound": "mfma", "kernel": "q4::gemm_gptq_kernel", "achieved": round(tot_f / tot_t / 1e12, 1),
                              "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                              "frac": round(tot_f / tot_t / 1e12 / MFMA_PEAK_TFLOPS, 4),
-                             "traffic": measured_traffic(f"gemm_m{Mg}")},
+                             "traffic": measured_traffic(f"gemm_m{Mg}"),
+                             "traffic_measured_at_commit": measured_traffic(f"gemm_m{Mg}", "measured_at_commit")},
                 "power_probe": power,
                 "gated_mlp": gated,
             }
@@ -668,6 +843,30 @@ def main():
 
         for Mb in (4, 16, 18, 32, 64):
             batch[f"gptq_m{Mb}"] = step_us(weights, Mb)
+
+        # ---- BASELINE.json configs[1] beyond one row, projection by projection, and configs[0]
+        # (K = N = 4096, M = 16: the o_proj shape at 16 rows)
+        rows_leg = {}
+        for Mb in (2, 4, 8, 16):
+            entry = {}
+            tot_t = 0.0
+            tot_b = 0
+            for i, (name, K, N) in enumerate(SHAPES):
+                xb = torch.randn((Mb, K), device=dev, dtype=torch.float16)
+                yb = torch.empty((Mb, N), device=dev, dtype=torch.float16)
+                fns = [(lambda c=c, i=i: pkg.ops.linear(weights[c][i], xb, None, out=yb)) for c in range(copies)]
+                avg, _ = time_kernel_launches(torch, fns, 96)
+                b = gemv_bytes(Mb, K, N)
+                entry[name] = {"us": round(avg * 1e6, 2), "GBps": round(b / avg / 1e9, 1),
+                               "frac_of_hbm_peak": round(b / avg / 1e9 / HBM_PEAK_GBS, 4)}
+                tot_t += avg
+                tot_b += b
+                del xb, yb
+            entry["all_four"] = {"us": round(tot_t * 1e6, 2), "GBps": round(tot_b / tot_t / 1e9, 1),
+                                 "frac_of_hbm_peak": round(tot_b / tot_t / 1e9 / HBM_PEAK_GBS, 4)}
+            rows_leg[f"m{Mb}"] = entry
+        out["cfg2_decode_rows"] = rows_leg
+        out["cfg1_4096x4096_m16"] = dict(rows_leg["m16"]["o_proj"], path=pkg.ops.select_path(weights[0][1], 16))
         # awq / act_order: the kernels that read the checkpoint layout (what the layers run);
         # *_converted / *_repacked: the opt-in load-time conversions (AWQ -> GPTQ layout, rows
         # into group order with x read through the permutation)
@@ -720,9 +919,13 @@ def main():
             nc = max(2, -(-600 * 1024 * 1024 // (K * N // 2)))
             for Mb in (1, 16, 1024):
                 entry = {}
-                for label, seq in (("g_idx_kernels", False), ("rows_in_group_order", True)):
-                    def make(c, seq=seq):
-                        w = make_weights_variant(pkg, torch, dev, K, N, 71 * c + Mb, "act_order")
+                # symmetric weights (one zero point: what configs[3] states) and, for the kernels that
+                # look zero points up per weight, the same with a zero point per group and column
+                variants = [("g_idx_kernels", False, "one"), ("g_idx_kernels_per_column_zeros", False, "per_column"),
+                            ("rows_in_group_order", True, "one")]
+                for label, seq, zeros in variants:
+                    def make(c, seq=seq, zeros=zeros):
+                        w = make_weights_variant(pkg, torch, dev, K, N, 71 * c + Mb, "act_order", zeros=zeros)
                         return pkg.ops.make_sequential(w) if seq else w
                     avg, path = shape_us(make, K, N, Mb, nc)
                     entry[label] = {"us": round(avg * 1e6, 1), "path": path}

@@ -233,30 +233,6 @@ int q4_noalloc_init(void);
 int q4_linear_noalloc(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype, void* stream);
 
 /*
- * Measurement aid, no counterpart in the reference: launches a kernel that only reads `bytes`
- * from buf (device memory) and keeps nothing.  Timed next to q4_linear it gives the floor of
- * a launch that pulls the same bytes out of HBM and does nothing else.
- *   pattern 0  linear: `workgroups` contiguous ranges, 1 KB per wave instruction
- *   pattern 1  the decode kernels' pattern on a [bytes / (4 n_words), n_words] matrix of
- *              packed words: a wave reads 4 rows x 256 B per instruction and walks down the
- *              rows; workgroups = (n_words / 64) * K splits, threads = 64 * K waves
- *   pattern 2  an empty kernel of the same grid (launch cost alone)
- * unroll (1, 2, 4, 8) is the number of 16-byte loads a lane keeps in flight.  sink: 4 bytes
- * of device memory, never written in practice.  Shapes that do not divide are rejected.
- */
-int q4_probe_read(const void* buf, size_t bytes, int pattern, int n_words, int workgroups, int threads, int unroll,
-                  void* sink, void* stream);
-
-/*
- * Measurement aid, no counterpart in the reference: every wave of `workgroups` workgroups of
- * 1024 threads issues `iters` rounds of eight 128-bit LDS reads, lane l at the 16-byte unit
- * lane_unit[l] (64 device ints, each 0..2887).  Timed with different maps it shows which
- * lanes the LDS serves in the same pass, which is what the activation tiles' layouts of the
- * prefill kernels are built on.  Synchronizes the stream once to validate the map.
- */
-int q4_probe_lds(const int32_t* lane_unit, int iters, int workgroups, void* sink, void* stream);
-
-/*
  * ---- Mixture of experts: the same linear layer, grouped over experts -----------------
  *
  * Replaces, for GPTQ and AWQ checkpoints, what the reference's sparse MoE layer

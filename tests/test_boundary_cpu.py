@@ -205,34 +205,6 @@ def test_noalloc_entry_point_validation_without_gpu(pkg):
     assert lib.q4_linear_noalloc(ctypes.byref(w), None, None, None, 0, 0, None) == 0  # no rows: nothing to do
 
 
-def test_probe_read_rejects_shapes_that_do_not_divide(pkg):
-    """The read-only probe checks its grid against the buffer on the host (nothing is launched here)."""
-    lib = pkg._lib.load()
-    L = pkg._lib
-    buf, sink = 0x1000, 0x2000
-    nbytes = 4096 * 4096 // 2
-    assert lib.q4_probe_read(buf, nbytes, 0, 0, 256, 256, 4, None, None) == L.ERR_INVALID_ARGUMENT      # no sink
-    assert lib.q4_probe_read(buf, nbytes, 0, 0, 256, 100, 4, sink, None) == L.ERR_INVALID_ARGUMENT      # not whole waves
-    assert lib.q4_probe_read(buf, nbytes, 0, 0, 256, 256, 3, sink, None) == L.ERR_INVALID_ARGUMENT      # unroll
-    assert lib.q4_probe_read(buf, 4096, 0, 0, 256, 256, 4, sink, None) == L.ERR_INVALID_ARGUMENT        # less than a round
-    assert lib.q4_probe_read(buf, nbytes, 1, 4096, 100, 256, 4, sink, None) == L.ERR_INVALID_ARGUMENT   # grid vs column tiles
-    assert lib.q4_probe_read(buf, nbytes, 1, 4096, 64 * 3, 256, 4, sink, None) == L.ERR_INVALID_ARGUMENT  # steps do not divide
-    assert lib.q4_probe_read(buf, nbytes, 1, 1000, 64, 256, 4, sink, None) == L.ERR_INVALID_ARGUMENT    # n_words % 64
-    assert lib.q4_probe_read(buf, nbytes, 7, 0, 256, 256, 4, sink, None) == L.ERR_INVALID_ARGUMENT      # pattern
-    assert b"q4_probe_read" in lib.q4_last_error()
-
-
-def test_probe_lds_rejects_missing_arguments(pkg):
-    """The LDS probe validates its arguments before it touches the device."""
-    lib = pkg._lib.load()
-    L = pkg._lib
-    assert lib.q4_probe_lds(None, 10, 256, 0x2000, None) == L.ERR_INVALID_ARGUMENT    # no lane map
-    assert lib.q4_probe_lds(0x1000, 10, 256, None, None) == L.ERR_INVALID_ARGUMENT    # no sink
-    assert lib.q4_probe_lds(0x1000, 0, 256, 0x2000, None) == L.ERR_INVALID_ARGUMENT   # no iterations
-    assert lib.q4_probe_lds(0x1000, 10, 0, 0x2000, None) == L.ERR_INVALID_ARGUMENT    # no workgroups
-    assert b"q4_probe_lds" in lib.q4_last_error()
-
-
 def test_path_selection_and_workspace(pkg):
     lib = pkg._lib.load()
     L = pkg._lib

@@ -101,8 +101,6 @@ SIGNATURES = {
     "q4_linear_plan": (c_int, [POINTER(Q4Weight), c_int, c_int, POINTER(c_int), POINTER(c_size_t)]),
     "q4_noalloc_init": (c_int, []),
     "q4_linear_noalloc": (c_int, [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
-    "q4_probe_read": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
-    "q4_probe_lds": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "q4_moe_route": (
         c_int,
         [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],

@@ -1,12 +1,31 @@
-// Measurement aid: kernels that only read.  They give the time a launch of the decode
-// kernel's shape needs when it does nothing but pull its weight bytes out of HBM, which is
-// the floor the decode kernels are compared with.  Nothing in the product path calls them.
+// Measurement aid of the benchmark, built into its own library (libq4probe.so): kernels that
+// only read.  They give the time a launch of the decode kernel's shape needs when it does
+// nothing but pull its weight bytes out of HBM, which is the floor the decode kernels are
+// compared with.  Not part of libq4linear.so or of its header; nothing in the product calls them.
+//
+//   q4_probe_read(buf, bytes, pattern, n_words, workgroups, threads, unroll, wcol, sink, stream)
+//     pattern 0  linear: `workgroups` contiguous ranges, 1 KB per wave instruction
+//     pattern 1  the decode kernels' pattern on a [bytes / (4 n_words), n_words] matrix of packed
+//                words: a wave reads 4 rows x 256 B per instruction and walks down the rows;
+//                a workgroup holds wcol column waves x (threads / 64 / wcol) K waves,
+//                workgroups = n_words / (64 wcol) * K splits
+//     pattern 2  an empty kernel of the same grid (launch cost alone)
+//     unroll (1, 2, 4, 8): 16-byte loads a lane keeps in flight.  sink: 4 bytes of device memory,
+//     never written in practice.  Shapes that do not divide are rejected (-1).
+//   q4_probe_lds(lane_unit, iters, workgroups, sink, stream)
+//     every wave of `workgroups` workgroups of 1024 threads issues `iters` rounds of eight 128-bit
+//     LDS reads, lane l at the 16-byte unit lane_unit[l] (64 device ints, each 0..2887): timed with
+//     different maps it shows which lanes the LDS serves in the same pass.  Synchronizes the
+//     stream once to validate the map.
+//   q4_probe_last_error()  message of the last refused call on this thread
 #include <hip/hip_runtime.h>
-
-#include "q4_common.cuh"
-#include "q4_linear.h"
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
 
 namespace q4 {
+
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 // One workgroup per contiguous range; every wave instruction reads 1 KB of consecutive bytes.
 template <int U>
@@ -25,14 +44,15 @@ __global__ __launch_bounds__(1024) void probe_read_linear_kernel(const uint4_t* 
 }
 
 // The decode kernels' pattern on a [rows, n_words] matrix of packed words: a wave load covers
-// four rows x 64 words (256 B per row); wave (tile, K slot) walks `steps` such loads down the
-// rows.  grid = ntiles * splits, block = 64 * wk.
+// four rows x 64 words (256 B per row); wave (tile, column wave, K slot) walks `steps` such loads
+// down the rows.  grid = ntiles * splits, block = 64 * wcol * wk.
 template <int U>
-__global__ __launch_bounds__(1024) void probe_read_tile_kernel(const uint32_t* __restrict__ p, int n_words, int wk, int steps,
-                                                               int ntiles, uint32_t* sink) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+__global__ __launch_bounds__(1024) void probe_read_tile_kernel(const uint32_t* __restrict__ p, int n_words, int wcol, int wk,
+                                                               int steps, int ntiles, uint32_t* sink) {
+  const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wc = w % wcol, wave = w / wcol;
   const int tile = blockIdx.x % ntiles, split = blockIdx.x / ntiles;
-  const int col = tile * 64 + (lane & 15) * 4;
+  const int col = (tile * wcol + wc) * 64 + (lane & 15) * 4;
   const size_t row0 = ((size_t)split * wk + wave) * steps * 4 + (lane >> 4);
   const uint4_t* q = (const uint4_t*)(p + row0 * n_words + col);
   const size_t stride = (size_t)n_words;  // uint4 units between loads: 4 rows * n_words / 4
@@ -75,10 +95,22 @@ __global__ __launch_bounds__(1024) void probe_lds_read_kernel(const int* __restr
 }  // namespace q4
 
 using namespace q4;
-using q4host::set_error;
+
+namespace {
+constexpr int Q4_OK = 0, Q4_ERR_INVALID_ARGUMENT = -1, Q4_ERR_LAUNCH = -4;
+thread_local char g_probe_error[256] = "";
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_probe_error, sizeof(g_probe_error), fmt, ap);
+  va_end(ap);
+}
+}  // namespace
+
+extern "C" const char* q4_probe_last_error(void) { return g_probe_error; }
 
 extern "C" int q4_probe_read(const void* buf, size_t bytes, int pattern, int n_words, int workgroups, int threads, int unroll,
-                             void* sink, void* stream) {
+                             int wcol, void* sink, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   if (sink == nullptr || workgroups <= 0 || threads <= 0 || threads > 1024 || threads % 64 != 0) {
     set_error("q4_probe_read: needs a sink, a positive grid and a block of whole waves (<= 1024 threads)");
@@ -106,12 +138,13 @@ extern "C" int q4_probe_read(const void* buf, size_t bytes, int pattern, int n_w
     else if (unroll == 4) launch(probe_read_linear_kernel<4>);
     else launch(probe_read_linear_kernel<8>);
   } else if (pattern == 1) {
-    const int wk = threads / 64;
-    if (n_words <= 0 || n_words % 64 != 0 || bytes % ((size_t)n_words * 16) != 0) {
-      set_error("q4_probe_read: tile pattern needs n_words %% 64 == 0 and a whole number of four-row steps");
+    if (wcol < 1 || (threads / 64) % wcol != 0 || n_words <= 0 || n_words % (64 * wcol) != 0 ||
+        bytes % ((size_t)n_words * 16) != 0) {
+      set_error("q4_probe_read: tile pattern needs n_words %% (64 wcol) == 0, whole K waves and a whole number of four-row steps");
       return Q4_ERR_INVALID_ARGUMENT;
     }
-    const int ntiles = n_words / 64;
+    const int wk = threads / 64 / wcol;
+    const int ntiles = n_words / (64 * wcol);
     const size_t steps_total = bytes / ((size_t)n_words * 16);
     if (workgroups % ntiles != 0) {
       set_error("q4_probe_read: %d workgroups are not a multiple of the %d column tiles", workgroups, ntiles);
@@ -123,7 +156,7 @@ extern "C" int q4_probe_read(const void* buf, size_t bytes, int pattern, int n_w
       return Q4_ERR_INVALID_ARGUMENT;
     }
     const int steps = (int)(steps_total / slots);
-    auto launch = [&](auto k) { hipLaunchKernelGGL(k, dim3(workgroups), dim3(threads), 0, st, (const uint32_t*)buf, n_words, wk, steps, ntiles, (uint32_t*)sink); };
+    auto launch = [&](auto k) { hipLaunchKernelGGL(k, dim3(workgroups), dim3(threads), 0, st, (const uint32_t*)buf, n_words, wcol, wk, steps, ntiles, (uint32_t*)sink); };
     if (unroll == 1) launch(probe_read_tile_kernel<1>);
     else if (unroll == 2) launch(probe_read_tile_kernel<2>);
     else if (unroll == 4) launch(probe_read_tile_kernel<4>);

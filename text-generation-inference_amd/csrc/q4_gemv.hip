@@ -6,6 +6,13 @@
 
 #include "q4_gemv_kernels.cuh"
 
+#ifdef Q4_PHASE_STAMPS
+// Measurement builds only: where the decode kernels of the following launches leave their clock
+// readings ([workgroups][waves][8] 64-bit values; nullptr switches the stamps off).
+static unsigned long long* g_phase_stamps = nullptr;
+extern "C" void q4_phase_stamps_target(void* device_buffer) { g_phase_stamps = (unsigned long long*)device_buffer; }
+#endif
+
 namespace q4host {
 
 using q4::GemvParams;
@@ -735,6 +742,9 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.ntiles = ntiles;
   gp.rows_per_block_alloc = rows;
   gp.wave_slab = wave_slab ? 1 : 0;
+#ifdef Q4_PHASE_STAMPS
+  gp.stamps = g_phase_stamps;
+#endif
   dim3 grid((unsigned)(ntiles * cfg.splits), (unsigned)mchunks);
   dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
   if (diag) {

@@ -62,6 +62,9 @@ struct GemvParams {
   int ntiles, kd_Q, kd_R, kd_q0, kd_r0, kd_q1, kd_r1;
   int rows_per_block_alloc;  // lean kernel: activation rows every wave's piece of LDS has room for
   int wave_slab;             // lean kernel: 1 = every wave stages its own K range, 0 = one slab per workgroup
+#ifdef Q4_PHASE_STAMPS
+  unsigned long long* __restrict__ stamps;  // [workgroups][waves][8] clock readings, or nullptr
+#endif
 };
 
 // Fills the K partition of gp for `chunks` chunks over `splits` workgroups of `wk` waves
@@ -173,6 +176,46 @@ __device__ __forceinline__ Decomp make_decomp(const GemvParams& gp, int wave_col
   d.mloc = min(gp.rows_per_block, gp.p.M - d.mb);
   return d;
 }
+
+// Clock readings of a wave at the phase boundaries of a decode launch.  Measurement builds only
+// (-DQ4_PHASE_STAMPS, a second library next to the product one): the readings stay in scalar
+// registers and go to memory with one store per wave right before it ends, so nothing is added
+// to the path being timed except the reads of the constant 100 MHz counter themselves.  In the
+// product build every member is empty and the calls compile to nothing.
+//   0 entry   1 activations staged (behind the workgroup barrier, where there is one)
+//   2 first chunk consumed   3 last chunk consumed (K loop done)   4 K waves of the workgroup
+//   combined through LDS   5 split-K combine returned (atomic / ticket)   6 first weight loads
+//   issued   7 exit
+struct PhaseStamps {
+#ifdef Q4_PHASE_STAMPS
+  unsigned long long t[8];
+  __device__ __forceinline__ PhaseStamps() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t[i] = 0ull;
+    t[0] = __builtin_amdgcn_s_memrealtime();
+  }
+  __device__ __forceinline__ void mark(int i) { t[i] = __builtin_amdgcn_s_memrealtime(); }
+  // reading taken once `v` has been computed (pins the stamp behind the work that makes v)
+  __device__ __forceinline__ void mark_after(int i, float v) {
+    asm volatile("" ::"v"(v));
+    mark(i);
+  }
+  __device__ __forceinline__ void flush(const GemvParams& gp, const Decomp& d) {
+    if (gp.stamps == nullptr) return;
+    mark(7);
+    if (d.lane == 0) {
+      unsigned long long* dst =
+          gp.stamps + (((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + d.wave) * 8;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dst[i] = t[i];
+    }
+  }
+#else
+  __device__ __forceinline__ void mark(int) {}
+  __device__ __forceinline__ void mark_after(int, float) {}
+  __device__ __forceinline__ void flush(const GemvParams&, const Decomp&) {}
+#endif
+};
 
 // Entry of a grouped (MOE) decode launch: narrows gp to the expert blockIdx.z.  Returns false
 // when this workgroup's row block lies beyond the expert's rows (the whole workgroup leaves).
@@ -299,9 +342,9 @@ __device__ __forceinline__ float cell_value(unsigned long long now) {
 // FUSE (NT = 8): gated-MLP epilogue.  out[0..3] are four gate columns col0 .. col0 + 3 and
 // out[4..7] the matching up columns N/2 + col0 ..; the output is act(gate) * up, [M, N/2].
 template <int DTYPE, int NT, int RMAX, bool FUSE = false, bool KQROWS = false>
-__device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& d,
-                                            float (&out)[NT][RMAX], int col0,
-                                            unsigned char* smem) {
+__device__ __forceinline__ void gemv_finish_impl(const GemvParams& gp, const Decomp& d,
+                                                 float (&out)[NT][RMAX], int col0,
+                                                 unsigned char* smem, PhaseStamps& ps) {
   const Problem& p = gp.p;
   const int N = p.N;
   // ---- combine the wk waves of the workgroup through LDS (fixed order)
@@ -326,6 +369,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
       }
     }
   }
+  ps.mark_after(4, out[0][0]);
 
   uint16_t* y = (uint16_t*)p.y;
   const int half_n = N >> 1;
@@ -422,6 +466,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
               inc[u] = cell_increment(tile[m * TW + d.lane + 64 * u]);
               before[u] = __hip_atomic_fetch_add(cell + 64 * u, inc[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
+            ps.mark_after(5, __builtin_bit_cast(float, (uint32_t)before[0]));
 #pragma unroll
             for (int u = 0; u < PER_LANE; ++u) {
               const unsigned long long now = before[u] + inc[u];
@@ -490,6 +535,7 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
     ticket_s = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
+  ps.mark(5);
   if (ticket_s != (uint32_t)(gp.splits - 1)) return;
   {
     const size_t sstride = (size_t)gp.partial_rows * N;
@@ -579,6 +625,19 @@ __device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& 
   }
 }
 
+template <int DTYPE, int NT, int RMAX, bool FUSE = false, bool KQROWS = false>
+__device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& d, float (&out)[NT][RMAX], int col0,
+                                            unsigned char* smem, PhaseStamps& ps) {
+  gemv_finish_impl<DTYPE, NT, RMAX, FUSE, KQROWS>(gp, d, out, col0, smem, ps);
+  ps.flush(gp, d);
+}
+template <int DTYPE, int NT, int RMAX, bool FUSE = false, bool KQROWS = false>
+__device__ __forceinline__ void gemv_finish(const GemvParams& gp, const Decomp& d, float (&out)[NT][RMAX], int col0,
+                                            unsigned char* smem) {
+  PhaseStamps ps;
+  gemv_finish_impl<DTYPE, NT, RMAX, FUSE, KQROWS>(gp, d, out, col0, smem, ps);
+}
+
 // ---------------------------------------------------------------------------------------
 // GPTQ, contiguous groups.
 // GSTEPS: MFMA steps (32 rows) per quantisation group inside a chunk: 1, 2 or 4.
@@ -596,6 +655,7 @@ template <int DTYPE, int RMAX, int GSTEPS, bool STATIC128, int WORDS, bool FUSE 
 __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
   static_assert(FUSE == (WORDS == 8), "eight words per lane = four gate + four up columns (fused only)");
   extern __shared__ __align__(16) unsigned char smem[];
+  PhaseStamps ps;
   const int32_t* moe_rows = nullptr;
   if constexpr (MOE) {
     if (!moe_enter_decode(gp, moe_rows, FUSE)) return;
@@ -675,9 +735,11 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
 #pragma unroll
   for (int b = 0; b < PF; ++b)
     if (b < nchunks) load_chunk(b, wq[b], sc[b], zw[b]);
+  ps.mark(6);
 
   slab.store(gp, d, smem);
   __syncthreads();
+  ps.mark(1);
 
   const bool row_live = d.j < d.mloc;  // A-operand row of this lane
   // RMAX = 8: a second block of 16 activation rows takes the same unpacked weights
@@ -771,10 +833,12 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
       const int c = c0 + b;
       if (c < nchunks) {
         process_chunk(c, wq[b], sc[b], zw[b]);
+        if (c == 0) ps.mark_after(2, tot[0][0]);
         if (c + PF < nchunks) load_chunk(c + PF, wq[b], sc[b], zw[b]);
       }
     }
   }
+  ps.mark_after(3, tot[0][0]);
 
   float out[WORDS][RMAX];
 #pragma unroll
@@ -784,7 +848,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_kernel(GemvParams gp) {
       if constexpr (ROWS32) out[t][r] = r < 4 ? tot[t][r & 3] : tot2[t][r & 3];
       else out[t][r] = tot[t][r];
     }
-  gemv_finish<DTYPE, WORDS, RMAX, FUSE>(gp, d, out, nl, smem);
+  gemv_finish<DTYPE, WORDS, RMAX, FUSE>(gp, d, out, nl, smem, ps);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -87,6 +87,7 @@ __global__ __launch_bounds__(1024) void gemv_gptq_lean_kernel(GemvParams gp) {
   static_assert(MP == 1 || MP == 2 || MP == 4 || MP == 8 || MP == 16, "rows are padded to a power of two");
   static_assert(MP != 8 || PF % 2 == 0, "eight rows: the chunks of a ring round alternate between two accumulator rows");
   extern __shared__ __align__(16) unsigned char smem[];
+  PhaseStamps ps;
   const Problem& p = gp.p;
   const Decomp d = make_decomp(gp, 64);
   const int N = p.N;
@@ -160,6 +161,7 @@ __global__ __launch_bounds__(1024) void gemv_gptq_lean_kernel(GemvParams gp) {
     SlabStager<true> slab;
     slab.issue(gp, d);
     issue_first_chunks();
+    ps.mark(6);
     slab.store(gp, d, smem);
     wslab = smem + (size_t)d.kwo * 2;
   } else {
@@ -200,6 +202,7 @@ __global__ __launch_bounds__(1024) void gemv_gptq_lean_kernel(GemvParams gp) {
     for (int u = 0; u < XB; ++u)
       if (u < d.mloc && d.lane < kbw) x0[u] = fetch(u, d.lane);
     issue_first_chunks();
+    ps.mark(6);
 #pragma unroll
     for (int u = 0; u < XB; ++u)
       if (u < d.mloc && d.lane < kbw) put(u, d.lane, x0[u]);
@@ -219,6 +222,7 @@ __global__ __launch_bounds__(1024) void gemv_gptq_lean_kernel(GemvParams gp) {
   // Every wave writes it (same values) so that none depends on another.
   if (d.lane < 32) ((uint4_t*)(smem + gp.slab_bytes))[d.lane] = uint4_t{0u, 0u, 0u, 0u};
   if (!gp.wave_slab) __syncthreads();
+  ps.mark(1);
 
   // MFMA row j of this lane's A operand: activation row mj, chunk slot glj of the accumulators
   const int mj = d.j / GACC, glj = d.j % GACC;
@@ -310,6 +314,7 @@ __global__ __launch_bounds__(1024) void gemv_gptq_lean_kernel(GemvParams gp) {
       const int c = c0 + b;
       if (c < nchunks) {
         process_chunk(c, b, wq[b]);
+        if (c == 0) ps.mark_after(2, acc[0][0]);
         if (c + PF < nchunks) {
           load_chunk(c + PF, wq[b]);
           if constexpr (PER_CHUNK) ring[b] = load_params(c + PF);
@@ -319,6 +324,7 @@ __global__ __launch_bounds__(1024) void gemv_gptq_lean_kernel(GemvParams gp) {
     }
   }
 
+  ps.mark_after(3, tot[0][0]);
   // hand the sums to the common epilogue: slot r of lane (j, kq) is activation row 4 kq + r
   float out[4][RMAX];
 #pragma unroll
@@ -346,7 +352,7 @@ __global__ __launch_bounds__(1024) void gemv_gptq_lean_kernel(GemvParams gp) {
       for (int r = 0; r < 4; ++r) out[t][r] = tot[t][r];
     }
   }
-  gemv_finish<DTYPE, 4, RMAX>(gp, d, out, nl, smem);
+  gemv_finish<DTYPE, 4, RMAX>(gp, d, out, nl, smem, ps);
 }
 
 }  // namespace q4

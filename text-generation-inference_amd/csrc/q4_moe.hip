@@ -436,6 +436,9 @@ int launch_moe_linear(const q4_moe_weight* w, const void* x, const int32_t* x_ro
       partials = (float*)((char*)workspace + Q4_WORKSPACE_COUNTER_BYTES);
     }
     GemvParams gp;
+#ifdef Q4_PHASE_STAMPS
+    gp.stamps = nullptr;  // (measurement builds stamp the dense launches only)
+#endif
     gp.p = Problem{e0->qweight, e0->qzeros, (const half_t*)e0->scales, e0->g_idx, x, nullptr, y,
                    0,           e0->K,      e0->N,                     e0->groupsize, e0->num_groups};
     gp.p.gate_up_act = gate_up_act;
