@@ -108,6 +108,9 @@ def parse_args():
     ap.add_argument("--no-batch", action="store_true",
                     help="skip the batched-decode leg (GPTQ at 4..64 rows, AWQ and act-order at 1 and 16 rows)")
     ap.add_argument("--copies", type=int, default=0, help="weight copies to rotate over (0 = auto)")
+    ap.add_argument("--no-autotune", action="store_true",
+                    help="skip the load-time tuning pass (ops.autotune, what the layers run in their Warmup hook): "
+                         "every call then takes the library's own fitted decomposition")
     ap.add_argument("--no-dense-ref", action="store_true",
                     help="skip timing torch's dense fp16 matmul (hipBLASLt) on the GEMM shapes")
     ap.add_argument("--floor-probe", action="store_true",
@@ -127,6 +130,9 @@ def parse_args():
     ap.add_argument("--phase-breakdown", action="store_true",
                     help="run the four decode projections (M = --m) on the phase-stamp build of the library "
                          "(libq4linear_stamps.so) and print where a launch's time goes, wave by wave")
+    ap.add_argument("--phase-configs", default="",
+                    help="with --phase-breakdown: JSON object projection name -> explicit decode configuration "
+                         "[column waves, K waves, splits, words] (as q4_gemv_tuned takes it) instead of the library's choice")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="eager launches only (a 256 MiB copy kernel, then each decode shape and one GEMM), "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs; prints no JSON line")
@@ -412,7 +418,7 @@ def floor_probe(torch, dev):
 DECODE_GRIDS = {"qkv_proj": (768, 256, 1), "o_proj": (512, 256, 1), "gate_up_proj": (224, 512, 2), "down_proj": (256, 512, 1)}
 
 
-def probe_trace(pkg, torch, dev, weights, xs, ys, copies, reps=40):
+def probe_trace(pkg, torch, dev, weights, xs, ys, reps=40):
     """Eager launches for a rocprofv3 --kernel-trace run: per projection an empty kernel and the
     read-only tile kernel on the decode kernel's grid (weights-sized ranges of a 1 GiB pool, so
     every launch reads from HBM), then the decode kernel itself on rotating weights.  The trace
@@ -435,7 +441,7 @@ def probe_trace(pkg, torch, dev, weights, xs, ys, copies, reps=40):
                                           sink.data_ptr(), stream))
         torch.cuda.synchronize()
         for r in range(reps):
-            pkg.ops.linear(weights[r % copies][i], xs[i], None, out=ys[i])
+            pkg.ops.linear(weights[r % len(weights)][i], xs[i], None, out=ys[i])
         torch.cuda.synchronize()
         print(f"probe trace: {name} {K}x{N}: {reps} empty launches ({wgs} x {threads}), {reps} read-only launches of "
               f"{nbytes} B (unroll {unroll}, {wcol} column waves), {reps} decode launches", file=sys.stderr)
@@ -446,7 +452,7 @@ PHASES = ["entry", "activations staged", "first chunk consumed", "K loop done",
 PHASE_ORDER = [0, 6, 1, 2, 3, 4, 5, 7]
 
 
-def phase_breakdown(pkg, torch, dev, M, copies, launches=24):
+def phase_breakdown(pkg, torch, dev, M, copies, launches=24, configs=None):
     """Where a decode launch's time goes.  Runs the phase-stamp build of the library: every wave
     reads the 100 MHz clock at its phase boundaries (PhaseStamps, csrc/q4_gemv_kernels.cuh) and
     stores the readings when it ends.  Launches run as a HIP graph over rotating weights, like the
@@ -455,8 +461,16 @@ def phase_breakdown(pkg, torch, dev, M, copies, launches=24):
     import numpy as np
 
     lib = pkg._lib.load()
-    lib.q4_phase_stamps_target.restype = None
-    lib.q4_phase_stamps_target.argtypes = [ctypes.c_void_p]
+    targets = [lib.q4_phase_stamps_target, lib.q4_phase_stamps_target_direct]
+    for fn in targets:
+        fn.restype = None
+        fn.argtypes = [ctypes.c_void_p]
+
+    def set_target(ptr):
+        for fn in targets:
+            fn(ptr)
+
+    configs = configs or {}
     out = {}
     slots = 8192  # waves per launch the buffer has room for
     for i, (name, K, N) in enumerate(SHAPES):
@@ -468,14 +482,15 @@ def phase_breakdown(pkg, torch, dev, M, copies, launches=24):
         side = torch.cuda.Stream()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.stream(side):
-            lib.q4_phase_stamps_target(None)
-            pkg.ops.linear(ws[0], x, None, out=y)
+            cfg = tuple(configs[name]) if name in configs else None
+            set_target(None)
+            pkg.ops.linear(ws[0], x, None, out=y, gemv_config=cfg)
             torch.cuda.synchronize()
             with torch.cuda.graph(graph, stream=side):
                 for r in range(launches):
-                    lib.q4_phase_stamps_target(stamps[r].data_ptr())
-                    pkg.ops.linear(ws[r % copies], x, None, out=y)
-            lib.q4_phase_stamps_target(None)
+                    set_target(stamps[r].data_ptr())
+                    pkg.ops.linear(ws[r % copies], x, None, out=y, gemv_config=cfg)
+            set_target(None)
             torch.cuda.synchronize()
             graph.replay()
             torch.cuda.synchronize()
@@ -504,7 +519,7 @@ def phase_breakdown(pkg, torch, dev, M, copies, launches=24):
                     rows[ph].append((rel.min(), np.median(rel), rel.max(), v.size))
         entry = {"K": K, "N": N, "waves": int(waves), "us_per_launch_with_stamps": round(us_per_launch, 2),
                  "first_entry_to_last_exit_us": round(float(np.mean(spans)), 2) if spans else None, "phases": {}}
-        print(f"== {name} {K}x{N} M={M}: {waves} waves, {us_per_launch:.2f} us per launch (graph replay, stamps on), "
+        print(f"== {name} {K}x{N} M={M}{' config ' + str(cfg) if cfg else ''}: {waves} waves, {us_per_launch:.2f} us per launch (graph replay, stamps on), "
               f"first wave in -> last wave out {entry['first_entry_to_last_exit_us']} us", flush=True)
         for ph in PHASE_ORDER:
             if rows[ph]:
@@ -543,7 +558,7 @@ def main():
     copies = args.copies or max(2, -(-512 * 1024 * 1024 // step_weight_bytes) + 1)
 
     if args.phase_breakdown:
-        phase_breakdown(pkg, torch, dev, M, copies)
+        phase_breakdown(pkg, torch, dev, M, copies, configs=json.loads(args.phase_configs) if args.phase_configs else None)
         return
     weights = [[make_weights(pkg, torch, dev, K, N, seed=17 * c + i) for i, (_, K, N) in enumerate(SHAPES)]
                for c in range(copies)]
@@ -551,6 +566,27 @@ def main():
     ys = [torch.empty((M, N), device=dev, dtype=torch.float16) for _, K, N in SHAPES]
     for _, K, N in SHAPES:
         pkg.ops.reserve_workspace(dev, pkg.ops.workspace_bytes(M, K, N))
+
+    # Per-projection legs rotate over enough copies of that one shape to exceed the 256 MB
+    # last-level cache as well (the whole-step legs get there with `copies` of all four)
+    COLD_BYTES = 512 * 1024 * 1024
+    probe_mode = (args.lds_probe or args.awq_probe or args.act_probe or args.floor_probe)
+    shape_ws = []
+    for i, (_, K, N) in enumerate(SHAPES):
+        n = copies if probe_mode else max(copies, -(-COLD_BYTES // gemv_bytes(0, K, N)))
+        shape_ws.append([weights[c][i] for c in range(copies)] +
+                        [make_weights(pkg, torch, dev, K, N, seed=1000 + 17 * c + i) for c in range(copies, n)])
+
+    # Load-time step, as the layers do it in their Warmup hook: measured decode plans for the row
+    # counts this run times
+    tuning = None
+    if not args.no_autotune and not probe_mode:
+        t0 = time.perf_counter()
+        rows = sorted({M, 1, 2, 4, 8, 16} if M <= 16 else {1, 2, 4, 8, 16})
+        report = pkg.ops.autotune([w for ws in shape_ws for w in ws], rows=rows)
+        tuning = {"seconds": round(time.perf_counter() - t0, 2),
+                  "plans": {f"{K}x{N}_m{Mr}": {"config": list(cfg) if cfg else None, "library_choice_us": base, "chosen_us": best}
+                            for (K, N, _, Mr), (cfg, base, best) in report.items()}}
 
     def step(c):
         for i in range(len(SHAPES)):
@@ -598,7 +634,7 @@ def main():
         floor_probe(torch, dev)
         return
     if args.probe_trace:
-        probe_trace(pkg, torch, dev, weights, xs, ys, copies)
+        probe_trace(pkg, torch, dev, weights, xs, ys)
         return
 
     if args.traffic_probe:
@@ -657,8 +693,8 @@ def main():
     all_bytes = 0
     reps = max(200, copies * 8)
     for i, (name, K, N) in enumerate(SHAPES):
-        fns = [(lambda c=c, i=i: pkg.ops.linear(weights[c][i], xs[i], None, out=ys[i])) for c in range(copies)]
-        avg, best = time_kernel_launches(torch, fns, reps)
+        fns = [(lambda w=w, i=i: pkg.ops.linear(w, xs[i], None, out=ys[i])) for w in shape_ws[i]]
+        avg, best = time_kernel_launches(torch, fns, max(reps, 2 * len(fns)))
         b = gemv_bytes(M, K, N)
         hot_avg, _ = time_kernel_launches(torch, fns[:1], reps)
         per_shape[name] = {
@@ -667,6 +703,8 @@ def main():
             "GBps": round(b / avg / 1e9, 1), "frac_of_hbm_peak": round(b / avg / 1e9 / HBM_PEAK_GBS, 4),
             "cache_hot_us": round(hot_avg * 1e6, 2), "cache_hot_GBps": round(b / hot_avg / 1e9, 1),
             "path": pkg.ops.select_path(weights[0][i], M),
+            "tuned_config": pkg.ops.PackedWeight.plan(weights[0][i], M, 0)[2],
+            "weight_copies_rotated": len(shape_ws[i]),
         }
         all_durs.append(avg)
         all_bytes += b
@@ -724,11 +762,13 @@ def main():
             "workload": f"GPTQ int4 decode GEMV M={M}, Llama-3-8B projections (qkv/o/gate_up/down), fp16, "
                         f"groupsize 128, sym; one step = the four projections once",
             "weight_copies_rotated": copies,
+            "per_projection_legs": "rotate over enough copies of the one shape to exceed 512 MB",
             "bytes_per_step": step_bytes,
             "timing": "one HIP graph of all timed steps, bracketed by HIP events + synchronize",
         },
         "roofline": roofline,
         "per_shape": per_shape,
+        "load_time_tuning": tuning,
     }
 
     # ---- prefill GEMM leg (M=2048) when the kernel is available
@@ -827,14 +867,15 @@ def main():
     if not args.no_batch:
         batch = {}
 
-        def step_us(wlist, Mb):
+        def step_us(wlist, Mb, per_shape=None):
             tot = 0.0
             paths = []
             for i, (name, K, N) in enumerate(SHAPES):
                 xb = torch.randn((Mb, K), device=dev, dtype=torch.float16)
                 yb = torch.empty((Mb, N), device=dev, dtype=torch.float16)
-                fns = [(lambda c=c, i=i: pkg.ops.linear(wlist[c][i], xb, None, out=yb)) for c in range(len(wlist))]
-                avg, _ = time_kernel_launches(torch, fns, 48)
+                rot = per_shape[i] if per_shape is not None else [row[i] for row in wlist]
+                fns = [(lambda w=w: pkg.ops.linear(w, xb, None, out=yb)) for w in rot]
+                avg, _ = time_kernel_launches(torch, fns, max(48, 2 * len(fns)))
                 tot += avg
                 paths.append(pkg.ops.select_path(wlist[0][i], Mb))
                 del xb, yb
@@ -842,7 +883,7 @@ def main():
                     "paths": "/".join(paths)}
 
         for Mb in (4, 16, 18, 32, 64):
-            batch[f"gptq_m{Mb}"] = step_us(weights, Mb)
+            batch[f"gptq_m{Mb}"] = step_us(weights, Mb, per_shape=shape_ws)
 
         # ---- BASELINE.json configs[1] beyond one row, projection by projection, and configs[0]
         # (K = N = 4096, M = 16: the o_proj shape at 16 rows)
@@ -854,8 +895,8 @@ def main():
             for i, (name, K, N) in enumerate(SHAPES):
                 xb = torch.randn((Mb, K), device=dev, dtype=torch.float16)
                 yb = torch.empty((Mb, N), device=dev, dtype=torch.float16)
-                fns = [(lambda c=c, i=i: pkg.ops.linear(weights[c][i], xb, None, out=yb)) for c in range(copies)]
-                avg, _ = time_kernel_launches(torch, fns, 96)
+                fns = [(lambda w=w: pkg.ops.linear(w, xb, None, out=yb)) for w in shape_ws[i]]
+                avg, _ = time_kernel_launches(torch, fns, max(96, 2 * len(fns)))
                 b = gemv_bytes(Mb, K, N)
                 entry[name] = {"us": round(avg * 1e6, 2), "GBps": round(b / avg / 1e9, 1),
                                "frac_of_hbm_peak": round(b / avg / 1e9 / HBM_PEAK_GBS, 4)}

@@ -178,18 +178,33 @@ int q4_moe_gather_columns(const void* x, const int32_t* x_rows, const int32_t* e
 int q4_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, void* stream);
 
 /*
- * Decode kernel with an explicit work decomposition, for tuning sweeps: `wcol` waves
- * across columns and `wk` waves across K per workgroup (wcol * wk <= 8), `splits`
+ * Decode kernel with an explicit work decomposition, for tuning sweeps and measured plans:
+ * `wcol` waves across columns and `wk` waves across K per workgroup (wcol * wk <= 8), `splits`
  * workgroups across K, `words` packed words per lane (4, 2 or 1: column tiles of 64, 32 or
  * 16 per wave; GPTQ layout with contiguous groups of at least 128 rows, otherwise forced to
- * 4; the AWQ kernel's tile is 256 columns).  K must be a multiple of 128 * wk * splits and
- * N of tile * wcol.
+ * 4; the AWQ kernel's tile is 256 columns; 0: the instruction-lean kernel / the AWQ kernel that
+ * feeds the stored words to the matrix core; -1: the short-launch kernel for up to 16 rows of
+ * contiguous GPTQ groups, wcol unused).  N must be a multiple of tile * wcol.
  * Plays the role of exllama's `set_tuning_params`
  * (server/exllama_kernels/exllama_kernels/exllama_ext.cpp:78-100) without global state.
  */
 int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                   void* workspace, size_t workspace_bytes, int wcol, int wk, int splits, int words,
                   void* stream);
+
+/*
+ * Decode decompositions worth timing for this problem at load time, as (wcol, wk, splits, words)
+ * quadruples for q4_gemv_tuned, written to configs[4 * i ..]; returns how many (0 when q4_linear
+ * would not run a decode kernel here or no alternative to its own choice exists), at most
+ * max_configs.  A caller that wants measured instead of fitted plans times q4_linear and each
+ * candidate on its own weights once per layer shape and row count and keeps the winner (the
+ * Python layers do so in their Warmup hook).  Plays the role of the autotuner of the reference's
+ * Triton path (server/text_generation_server/layers/gptq/custom_autotune.py:1-80, the config
+ * list of layers/gptq/triton.py:14-103).  q4_gemv_tuned_workspace_bytes: workspace such a call
+ * needs (the zero-initialised head included).
+ */
+int q4_gemv_candidates(const q4_weight* w, int M, int dtype, int32_t* configs, int max_configs);
+size_t q4_gemv_tuned_workspace_bytes(const q4_weight* w, int M, int dtype, int wcol, int wk, int splits, int words);
 
 /*
  * Bytes of workspace q4_linear needs for an [M, K] x [K, N] problem (split-K partial

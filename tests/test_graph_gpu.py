@@ -140,3 +140,50 @@ def test_first_forward_of_a_fresh_layer_is_capturable(pkg, oracle, gpu, kind, M)
         assert torch.equal(y, want), (kind, M, i)
         _ = layer(x + 1.0)  # eager work between the replays
         torch.cuda.synchronize()
+
+
+def test_replay_after_the_workspace_grew_does_not_touch_freed_memory(pkg, oracle, gpu):
+    """A graph captured with a small workspace keeps its address.  When a larger layer makes the
+    shared workspace grow afterwards, the old buffer must stay allocated: replays write tickets,
+    cells and partial sums there, and tensors allocated in between must not change."""
+    ops = pkg.ops
+    saved = dict(ops._workspaces)
+    ops._workspaces.clear()  # this test starts from no workspace at all
+    try:
+        qw, qz, sc, _ = oracle.make_gptq(4096, 1024, 128, seed=31, sym=False)
+        small = ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
+        small.prepare(rows=(4,))
+        x = to_dev(oracle.make_x(4, 4096, seed=2), gpu)
+        eager = ops.linear(small, x)
+        out = torch.empty_like(eager)
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                ops.linear(small, x, None, out=out)
+        torch.cuda.synchronize()
+        used = ops._workspaces[(gpu.index, ops.SHARED)]
+        # a larger layer, planned for many rows: the shared workspace is replaced by a bigger one
+        g = torch.Generator(device=gpu).manual_seed(5)
+        big = ops.make_packed(
+            torch.randint(-(2**31), 2**31 - 1, (14336 // 8, 4096), dtype=torch.int64, device=gpu, generator=g).to(torch.int32),
+            torch.full((112, 512), 0x77777777, dtype=torch.int32, device=gpu),
+            (torch.rand((112, 4096), device=gpu, generator=g) * 0.019 + 0.001).half(), None, 128, 0)
+        big.prepare(max_rows=1024)
+        assert ops._workspaces[(gpu.index, ops.SHARED)] is not used, "the workspace did not grow: the test shows nothing"
+        assert any(t is used for t in ops._retired_workspaces)
+        # memory the allocator would hand out if the old buffer had been freed
+        del used
+        torch.cuda.empty_cache()
+        fillers = [torch.full((1 << 20,), 7, dtype=torch.int32, device=gpu) for _ in range(8)]
+        torch.cuda.synchronize()
+        for _ in range(3):
+            out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
+        for f in fillers:
+            assert bool((f == 7).all())
+    finally:
+        ops._workspaces.clear()
+        ops._workspaces.update(saved)

@@ -90,7 +90,12 @@ def check(pkg, oracle, gpu, layout, K, N, M, dtype, kind, cfg, seed, path=0):
     x = oracle.f32_to_bf16_bits(x32) if bf else x32.astype(np.float16)
     y32 = oracle.matmul_fp32(oracle.to_f32(x, dtype), w32)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0 if layout == "gptq" else 1)
-    got = pkg.ops.linear(pk, to_dev(x, gpu, bf16=bf), None, path=path, gemv_config=cfg)
+    try:
+        got = pkg.ops.linear(pk, to_dev(x, gpu, bf16=bf), None, path=path, gemv_config=cfg)
+    except pkg._lib.Q4Error as e:
+        if cfg is None or "LDS" not in str(e):
+            raise
+        pytest.skip("the activations of this many rows do not fit LDS in this decomposition")
     torch.cuda.synchronize()
     g = to_f32(got)
     assert np.isfinite(g).all()

@@ -85,7 +85,12 @@ def test_forced_paths_read_x_through_perm(pkg, oracle, gpu, path, M):
     got = pkg.ops.linear(seq, x, bias, path=path)
     plain = pkg.ops.PackedWeight(seq.qweight, seq.qzeros, seq.scales, None, K, N, gs, K // gs, 0)
     want = pkg.ops.linear(plain, x[:, seq.perm.long()].contiguous(), bias, path=path)
-    assert torch.equal(got, want)
+    if path == 1 and M <= 3:
+        # up to three rows the plain call runs the short-launch kernel, the call through perm the
+        # kernel that gathers while it stages: same sums, roundings of different arithmetic
+        assert float((got.float() - want.float()).abs().max() / want.float().abs().max()) <= 2e-3
+    else:
+        assert torch.equal(got, want)
     w = oracle.dequant_gptq(qw, qz, sc, gi, gs, "f16")
     y32, _ = oracle.linear_forward(x.cpu().numpy(), w, bias.cpu().numpy(), "f16")
     assert max_rel_err(got.float().cpu().numpy(), y32) <= TOL
@@ -274,8 +279,9 @@ def test_gated_mlp_first_half_on_rows_in_group_order(pkg, oracle, gpu, K, M):
 @pytest.mark.parametrize("gate_up_act_order", [False, True])
 def test_down_permutation_folded_into_gate_up_columns(pkg, oracle, gpu, gate_up_act_order, monkeypatch):
     """The gated MLP of an act-order model: applying the down projection's permutation to the
-    gate and up output columns at load time leaves every output bit for bit as it was with the
-    run-time gather, and the down projection becomes a plain contiguous-group layer."""
+    gate and up output columns at load time leaves every output as it was with the run-time gather
+    (bit for bit where both routes run the same kernel), and the down projection becomes a plain
+    contiguous-group layer."""
     _act_order_mode(monkeypatch, "repack")
     H, I, gs = 1024, 2048, 128
     gq = oracle.make_gptq(H, 2 * I, gs, seed=1, sym=False, act_order=gate_up_act_order)
@@ -299,7 +305,12 @@ def test_down_permutation_folded_into_gate_up_columns(pkg, oracle, gpu, gate_up_
         x = to_dev(oracle.make_x(M, H, seed=M), gpu)
         y0 = dn0(pkg.gate_up_act(gu0, x, "silu"))
         y1 = dn1(pkg.gate_up_act(gu1, x, "silu"))
-        assert torch.equal(y0, y1), M
+        if M <= 3:
+            # up to three rows the folded (plain) down projection runs the short-launch kernel, the
+            # one that still gathers the kernel that gathers while it stages: different roundings
+            assert float((y0.float() - y1.float()).abs().max() / y0.float().abs().max()) <= 2e-3, M
+        else:
+            assert torch.equal(y0, y1), M
     # against the oracle, once
     wg = oracle.dequant_gptq(gq[0], gq[1], gq[2], gq[3], gs, "f16")
     wd = oracle.dequant_gptq(dq[0], dq[1], dq[2], dq[3], gs, "f16")

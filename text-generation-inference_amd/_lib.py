@@ -81,6 +81,8 @@ SIGNATURES = {
         c_int,
         [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p],
     ),
+    "q4_gemv_candidates": (c_int, [POINTER(Q4Weight), c_int, c_int, POINTER(c_int32), c_int]),
+    "q4_gemv_tuned_workspace_bytes": (c_size_t, [POINTER(Q4Weight), c_int, c_int, c_int, c_int, c_int, c_int]),
     "q4_linear_gate_up": (
         c_int,
         [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],

@@ -21,9 +21,9 @@ CSRC = HERE / "csrc"
 LIB_NAME = "libq4linear.so"
 LIB_PATH = HERE / LIB_NAME
 
-SOURCES = ["q4_api.hip", "q4_dequant.hip", "q4_generic.hip", "q4_gemv.hip", "q4_gemv_lean.hip", "q4_gemv_awq.hip", "q4_gemv_gate_up.hip", "q4_gemm.hip", "q4_gemm_awq.hip", "q4_gemm_awq_direct.hip", "q4_act_mul.hip", "q4_moe.hip", "q4_sequential.hip", "q4_gptq_solve.hip"]
+SOURCES = ["q4_api.hip", "q4_dequant.hip", "q4_generic.hip", "q4_gemv.hip", "q4_gemv_lean.hip", "q4_gemv_direct.hip", "q4_gemv_awq.hip", "q4_gemv_gate_up.hip", "q4_gemm.hip", "q4_gemm_awq.hip", "q4_gemm_awq_direct.hip", "q4_act_mul.hip", "q4_moe.hip", "q4_sequential.hip", "q4_gptq_solve.hip"]
 # translation units that see the decode kernels' parameter block (recompiled for the stamps build)
-STAMP_SOURCES = ["q4_gemv.hip", "q4_gemv_lean.hip", "q4_gemv_awq.hip", "q4_gemv_gate_up.hip", "q4_moe.hip"]
+STAMP_SOURCES = ["q4_gemv.hip", "q4_gemv_lean.hip", "q4_gemv_direct.hip", "q4_gemv_direct.hip", "q4_gemv_awq.hip", "q4_gemv_gate_up.hip", "q4_moe.hip"]
 PROBE_LIB_PATH = HERE / "libq4probe.so"
 STAMPS_LIB_PATH = HERE / "libq4linear_stamps.so"
 

@@ -585,6 +585,50 @@ int q4_linear(const q4_weight* w, const void* x, const void* bias, void* y, int 
   return q4_linear_ex(w, x, bias, y, M, dtype, workspace, workspace_bytes, Q4_PATH_AUTO, stream);
 }
 
+int q4_gemv_candidates(const q4_weight* w, int M, int dtype, int32_t* configs, int max_configs) {
+  if (validate_weight(w, "q4_gemv_candidates") != Q4_OK || validate_dtype(dtype, "q4_gemv_candidates") != Q4_OK) return Q4_ERR_INVALID_ARGUMENT;
+  if (configs == nullptr || max_configs < 0) {
+    set_error("q4_gemv_candidates: null output");
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  if (M < 1 || w->K == 0 || w->N == 0 || q4_select_path(w, M, dtype) != Q4_PATH_GEMV) return 0;
+  // The short-launch kernel's decompositions: K waves per workgroup x workgroups along K.  Kept:
+  // even K deals where the chunk count has them, between one and sixty-four waves per CU in all.
+  const int chunks = w->K / 128;
+  const long tiles = w->N / 64;
+  static const int kWaves[] = {4, 8, 2, 1};
+  static const int kSplits[] = {1, 2, 4, 8, 7, 14, 3, 5, 6, 10, 12, 16};
+  int n = 0;
+  for (int pass = 0; pass < 2 && n == 0; ++pass) {  // second pass: ragged deals, for a K without even ones
+    for (int wk : kWaves) {
+      for (int sp : kSplits) {
+        if (n >= max_configs) return n;
+        if (!gemv_direct_supported(w, M, dtype, wk, sp)) continue;
+        if (pass == 0 && chunks % (wk * sp) != 0) continue;
+        const long waves = tiles * wk * sp;
+        if (waves < 256 || waves > 16384) continue;
+        configs[4 * n + 0] = 1;
+        configs[4 * n + 1] = wk;
+        configs[4 * n + 2] = sp;
+        configs[4 * n + 3] = -1;
+        ++n;
+      }
+    }
+  }
+  return n;
+}
+
+size_t q4_gemv_tuned_workspace_bytes(const q4_weight* w, int M, int dtype, int wcol, int wk, int splits, int words) {
+  (void)wcol;
+  (void)wk;
+  if (validate_weight(w, "q4_gemv_tuned_workspace_bytes") != Q4_OK || M < 1) return Q4_WORKSPACE_COUNTER_BYTES;
+  if (words == -1) {
+    const size_t need = gemv_direct_workspace_bytes(w, M, dtype, splits);
+    return need > (size_t)Q4_WORKSPACE_COUNTER_BYTES ? need : (size_t)Q4_WORKSPACE_COUNTER_BYTES;
+  }
+  return (size_t)Q4_WORKSPACE_COUNTER_BYTES + (splits > 1 ? (size_t)splits * M * w->N * sizeof(float) : 0);
+}
+
 int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                   void* workspace, size_t workspace_bytes, int wcol, int wk, int splits, int words,
                   void* stream) {
@@ -595,6 +639,8 @@ int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, 
     set_error("q4_gemv_tuned: bad M=%d or null x/y", M);
     return Q4_ERR_INVALID_ARGUMENT;
   }
+  if (words == -1)  // the short-launch kernel: wk K waves per workgroup, `splits` workgroups along K (wcol unused)
+    return launch_gemv_direct(w, x, bias, y, M, dtype, workspace, workspace_bytes, wk, splits, (hipStream_t)stream);
   GemvConfig cfg{wcol, wk, splits, words};
   if (words == 0) {  // the lean contiguous-group kernel / the AWQ kernel that feeds the words as stored
     cfg.words = 4;

@@ -223,6 +223,12 @@ GemvConfig gemv_pick_config(const q4_weight* w, int M, bool gate_up);
 int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype,
                 void* workspace, size_t workspace_bytes, const GemvConfig* cfg, hipStream_t stream,
                 int gate_up_act = 0, const int32_t* x_perm = nullptr);
+// the short-launch decode kernel (q4_gemv_direct.cuh): up to 16 rows, contiguous GPTQ groups
+bool gemv_direct_supported(const q4_weight* w, int M, int dtype, int wk, int splits);
+size_t gemv_direct_workspace_bytes(const q4_weight* w, int M, int dtype, int splits);
+bool gemv_direct_default(const q4_weight* w, int M, int dtype, int* wk, int* splits);
+int launch_gemv_direct(const q4_weight* w, const void* x, const void* bias, void* y, int M, int dtype, void* workspace,
+                       size_t workspace_bytes, int wk, int splits, hipStream_t stream);
 bool gemv_gate_up_supported(const q4_weight* w, int M, int dtype);
 int launch_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, hipStream_t stream);
 bool gemm_gate_up_supported(const q4_weight* w, int M, int dtype);

@@ -1,0 +1,324 @@
+// Decode kernel for the GPTQ layout with contiguous groups, up to 16 activation rows: the
+// short-launch variant.
+//
+// A decode launch over a small projection (4096 x 4096: 8.4 MB) lives for a few microseconds,
+// and what it does before its first weight load is out and after its last one has arrived is
+// most of what separates it from a kernel that only reads.  This kernel keeps both ends short:
+//   * The work decomposition is the grid itself (blockIdx.x = column tile of 64, blockIdx.y =
+//     K split); the 128-row chunks are dealt to the splits x waves slots in order, the first
+//     `rem` slots one more than the others, so a wave finds its range with a multiply and a
+//     minimum: no division, a parameter block of about 100 bytes.
+//   * No activation slab and no barrier before the first MFMA.  Only the lanes whose MFMA row
+//     is a live activation row (lane % 16 < M) fetch 16 bytes of x per 32-row step, straight
+//     from global memory (x stays in L2), issued ahead of the weight words they meet; one byte
+//     permute per register puts them in the K order of the nibble splice.
+//   * The arithmetic is that of gemv_gptq_lean_kernel: spliced nibbles enter the MFMA with
+//     their offsets (1024 + q / 64 + q; bf16: 128 + q), one more MFMA per step against a
+//     constant B operand gives P = sum x_k c_k and S = sum x_k, and a chunk contributes
+//     scale * (acc - P - z * S) in fp32.
+//   * One barrier at the end: every K wave leaves its 64 x M sums in LDS and they are added with
+//     lane l owning column l.  K split across workgroups: up to three fp16 rows take one 64-bit
+//     fixed-point atomic per output element (the workgroup that completes a cell writes y and
+//     clears it: cell_increment / cell_value in q4_gemv_kernels.cuh); more rows and bf16 write
+//     fp32 partial sums, draw a ticket per column tile, and the last workgroup adds the partials
+//     in split order (what that sequence relies on is described at gemv_finish).
+#pragma once
+#include "q4_gemv_lean.cuh"
+
+namespace q4 {
+
+struct DirectParams {
+  const uint32_t* __restrict__ qweight;
+  const uint32_t* __restrict__ qzeros;
+  const half_t* __restrict__ scales;
+  const void* __restrict__ x;
+  const void* __restrict__ bias;
+  void* __restrict__ y;
+  unsigned long long* __restrict__ cells;  // [M][N] accumulation cells, zero between launches, or nullptr
+  float* __restrict__ partials;            // [splits][M][N] partial sums (ticket combine), or nullptr
+  uint32_t* __restrict__ tickets;          // one per column tile, zero between launches
+  int N, K, M;
+  int cpw;         // 128-row chunks per (split, wave) slot ...
+  int rem;         // ... the first `rem` slots walk one more
+  int gshift;      // group of chunk c = min(c >> gshift, num_groups - 1)
+  int num_groups;
+  int splits;
+#ifdef Q4_PHASE_STAMPS
+  unsigned long long* __restrict__ stamps;
+#endif
+};
+
+typedef __amdgpu_buffer_rsrc_t direct_rsrc_t;
+__device__ __forceinline__ direct_rsrc_t direct_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// MR: activation rows padded to 1, 2, 4 or 16.  Up to four rows sit in the first register quad
+// of the MFMA result (lanes of K block 0); sixteen fill it (lane block kq holds rows 4 kq .. 4 kq + 3).
+template <int DTYPE, int MR>
+__global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) {
+  static_assert(MR == 1 || MR == 2 || MR == 4 || MR == 16, "rows are padded to 1, 2, 4 or 16");
+  extern __shared__ __align__(16) unsigned char smem[];
+  PhaseStamps ps;
+  constexpr int RL = MR < 4 ? MR : 4;  // live rows among a lane's four
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wk = blockDim.x >> 6;
+  const int j = lane & 15, kq = lane >> 4;
+  const int N = dp.N;
+  const int col = blockIdx.x * 64 + 4 * j;  // lane's first column
+  const int slot = blockIdx.y * wk + wave;
+  const int c0 = slot * dp.cpw + min(slot, dp.rem);
+  const int nchunks = dp.cpw + (slot < dp.rem ? 1 : 0);
+  constexpr int PF = 2;  // chunks of loads in flight per wave
+
+  // Buffer loads: a scalar descriptor, one constant 32-bit lane offset and a scalar offset that
+  // moves (no 64-bit vector address arithmetic).  Ranges are checked on the host.
+  const direct_rsrc_t wrsrc = direct_rsrc(dp.qweight, (uint32_t)(dp.K >> 3) * (uint32_t)N * 4u);
+  const direct_rsrc_t srsrc = direct_rsrc(dp.scales, (uint32_t)dp.num_groups * (uint32_t)N * 2u);
+  const direct_rsrc_t zrsrc = direct_rsrc(dp.qzeros, (uint32_t)dp.num_groups * (uint32_t)(N >> 3) * 4u);
+  const direct_rsrc_t xrsrc = direct_rsrc(dp.x, (uint32_t)dp.M * (uint32_t)dp.K * 2u);
+  const uint32_t w_lane = ((uint32_t)kq * (uint32_t)N + (uint32_t)col) * 4u;
+  const uint32_t s_lane = (uint32_t)col * 2u;
+  const uint32_t z_lane = (uint32_t)(col >> 3) * 4u;
+  const int zshift = (col & 7) * 4;
+  const bool row_live = j < dp.M;  // this lane's MFMA row carries an activation row
+  const uint32_t x_lane = ((uint32_t)(row_live ? j : 0) * (uint32_t)dp.K + (uint32_t)kq * 8u) * 2u;
+  const uint32_t step_bytes = (uint32_t)N * 16u;  // four packed rows
+
+  struct Chunk {
+    uint4_t x[kChunkSteps];
+    uint4_t w[kChunkSteps];
+    uint2_t s;
+    uint32_t z;
+  };
+  Chunk ring[PF];
+  auto load_chunk = [&](int c, Chunk& q) {
+    const uint32_t chunk = (uint32_t)(c0 + c);
+    // activations first: memory returns in issue order, and an L2 hit must not queue behind
+    // the weight stream of this wave
+#pragma unroll
+    for (int st = 0; st < kChunkSteps; ++st) {
+      q.x[st] = uint4_t{0u, 0u, 0u, 0u};
+      if (row_live)
+        q.x[st] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, x_lane, (chunk * kChunkRows + st * 32) * 2u, 0));
+    }
+    const uint32_t gi = (uint32_t)min((int)(chunk >> dp.gshift), dp.num_groups - 1);
+    q.s = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(srsrc, s_lane, gi * (uint32_t)N * 2u, 0));
+    q.z = __builtin_amdgcn_raw_buffer_load_b32(zrsrc, z_lane, gi * (uint32_t)(N >> 3) * 4u, 0);
+#pragma unroll
+    for (int st = 0; st < kChunkSteps; ++st)
+      q.w[st] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, w_lane, (chunk * kChunkSteps + st) * step_bytes, 2));
+  };
+#pragma unroll
+  for (int b = 0; b < PF; ++b)
+    if (b < nchunks) load_chunk(b, ring[b]);
+  ps.mark(6);
+  ps.mark(1);
+
+  // constant B operand: column 0 the splice offsets c_k, column 1 ones
+  uint4_t bconst = {0u, 0u, 0u, 0u};
+  if (j == 0) bconst = uint4_t{LeanSplice<DTYPE>::kOffLo, LeanSplice<DTYPE>::kOffHi, LeanSplice<DTYPE>::kOffLo, LeanSplice<DTYPE>::kOffHi};
+  if (j == 1) bconst = uint4_t{LeanSplice<DTYPE>::kOnes, LeanSplice<DTYPE>::kOnes, LeanSplice<DTYPE>::kOnes, LeanSplice<DTYPE>::kOnes};
+  const LeanConsts kc = lean_consts<DTYPE>();
+  const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  const int row_lane0 = lane & 48;  // first lane of this lane's row of 16
+  float tot[4][RL];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int i = 0; i < RL; ++i) tot[t][i] = 0.f;
+  bool poisoned = false;  // some chunk of this wave met an inf or NaN activation
+
+  auto process_chunk = [&](const Chunk& q) {
+    float4_t acc[4], accc;
+#pragma unroll
+    for (int st = 0; st < kChunkSteps; ++st) {
+      // K order [0,4,1,5,2,6,3,7] of the splice
+      uint4_t a;
+      a.x = __builtin_amdgcn_perm(q.x[st].z, q.x[st].x, 0x05040100u);
+      a.y = __builtin_amdgcn_perm(q.x[st].z, q.x[st].x, 0x07060302u);
+      a.z = __builtin_amdgcn_perm(q.x[st].w, q.x[st].y, 0x05040100u);
+      a.w = __builtin_amdgcn_perm(q.x[st].w, q.x[st].y, 0x07060302u);
+      const uint32_t words[4] = {q.w[st].x, q.w[st].y, q.w[st].z, q.w[st].w};
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc[t] = lean_mfma<DTYPE>(a, lean_unpack<DTYPE>(words[t], kc), st == 0 ? zero4 : acc[t]);
+      accc = lean_mfma<DTYPE>(a, bconst, st == 0 ? zero4 : accc);
+    }
+    // scale * (acc - P - z * S); P and S of a row sit in columns 0 and 1 of the constant product
+    const uint32_t z4 = gptq_zero_plus_one(q.z) >> zshift;
+    float sf[4], zf[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const half2_t sp = as_half2(t < 2 ? q.s.x : q.s.y);
+      sf[t] = (float)((t & 1) ? sp.y : sp.x);
+      zf[t] = (float)((z4 >> (4 * t)) & 0xFu);
+    }
+#pragma unroll
+    for (int i = 0; i < RL; ++i) {
+      // (a copy first: __builtin_bit_cast of a vector element reads element 0 whatever the index)
+      const float ci = accc[i];
+      float P, S;
+      if constexpr (MR <= 4) {  // the rows sit in lane block 0: wave-uniform values
+        P = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ci), 0));
+        S = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ci), 1));
+      } else {
+        P = row_lane(ci, row_lane0);
+        S = row_lane(ci, row_lane0 + 1);
+      }
+      poisoned |= !(fabsf(S) <= 3.0e38f);  // an inf or NaN activation in this row's chunk
+#pragma unroll
+      for (int t = 0; t < 4; ++t) tot[t][i] = fmaf(sf[t], acc[t][i] - fmaf(zf[t], S, P), tot[t][i]);
+    }
+  };
+
+  for (int cb = 0; cb < nchunks; cb += PF) {
+#pragma unroll
+    for (int b = 0; b < PF; ++b) {
+      const int c = cb + b;
+      if (c < nchunks) {
+        process_chunk(ring[b]);
+        if (c == 0) ps.mark_after(2, tot[0][0]);
+        if (c + PF < nchunks) load_chunk(c + PF, ring[b]);
+      }
+    }
+  }
+  ps.mark_after(3, tot[0][0]);
+
+  // A row with an infinite activation: acc, P and S are all infinite and their difference is NaN,
+  // where the dot product with the dequantized weights is +-inf.  A wave that met one (rare)
+  // walks its K range again, step by step, with the zero point taken out of the weights before
+  // the MFMA: the class of every output is then that of fp32 arithmetic on s * (q - z).
+  if (__builtin_amdgcn_ballot_w64(poisoned) != 0ull) {
+    const SpliceConsts splice = splice_consts();
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int i = 0; i < RL; ++i) tot[t][i] = 0.f;
+    for (int c = 0; c < nchunks; ++c) {
+      const uint32_t chunk = (uint32_t)(c0 + c);
+      const uint32_t gi = (uint32_t)min((int)(chunk >> dp.gshift), dp.num_groups - 1);
+      const uint2_t sv = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(srsrc, s_lane, gi * (uint32_t)N * 2u, 0));
+      const uint32_t z4 = gptq_zero_plus_one(__builtin_amdgcn_raw_buffer_load_b32(zrsrc, z_lane, gi * (uint32_t)(N >> 3) * 4u, 0)) >> zshift;
+      half2_t czlo[4], czhi[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const uint32_t zz = (z4 >> (4 * t)) & 0xFu;
+        czlo[t] = as_half2(0xE400E400u | zz | (zz << 16));         // -(1024 + z)
+        czhi[t] = as_half2(0xD400D400u | (zz << 4) | (zz << 20));  // -(64 + z)
+      }
+      float4_t ex[4] = {zero4, zero4, zero4, zero4};
+      for (int st = 0; st < kChunkSteps; ++st) {
+        uint4_t xv = {0u, 0u, 0u, 0u};
+        if (row_live)
+          xv = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, x_lane, (chunk * kChunkRows + st * 32) * 2u, 0));
+        const uint4_t wv = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, w_lane, (chunk * kChunkSteps + st) * step_bytes, 0));
+        uint4_t a;
+        a.x = __builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u);
+        a.y = __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u);
+        a.z = __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u);
+        a.w = __builtin_amdgcn_perm(xv.w, xv.y, 0x07060302u);
+        const uint32_t words[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          half2_t b[4];
+          unpack_word_f16(words[t], czlo[t], czhi[t], splice, b);
+          ex[t] = mfma16<DTYPE>(a, b, ex[t]);
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const half2_t sp = as_half2(t < 2 ? sv.x : sv.y);
+        const float sf = (float)((t & 1) ? sp.y : sp.x);
+#pragma unroll
+        for (int i = 0; i < RL; ++i) tot[t][i] = fmaf(sf, ex[t][i], tot[t][i]);
+      }
+    }
+  }
+
+  // ---- the K waves meet in LDS: wave w leaves row r at red[(w * MR + r) * 64 + column]
+  float* red = (float*)smem;
+  if (MR == 16 || kq == 0) {
+#pragma unroll
+    for (int i = 0; i < RL; ++i) {
+      const int r = (MR == 16 ? 4 * kq : 0) + i;
+      *(float4_t*)(red + (wave * MR + r) * 64 + 4 * j) = float4_t{tot[0][i], tot[1][i], tot[2][i], tot[3][i]};
+    }
+  }
+  if (wk > 1) __syncthreads();
+  uint16_t* y = (uint16_t*)dp.y;
+  const int n = blockIdx.x * 64 + lane;
+  auto row_sum = [&](int r) {
+    float v = red[r * 64 + lane];
+    for (int w = 1; w < wk; ++w) v += red[(w * MR + r) * 64 + lane];
+    return v;
+  };
+
+  if (dp.cells != nullptr) {
+    // one 64-bit fixed-point atomic per element; wave 0 takes the rows one at a time (with the
+    // adds of several rows in flight the splits of a row arrive together and the combine
+    // measured slower)
+    if (wave == 0) {
+#pragma unroll
+      for (int m = 0; m < RL; ++m) {
+        if (m < dp.M) {
+          const float v = row_sum(m);
+          if (m == 0) ps.mark_after(4, v);
+          unsigned long long* cell = dp.cells + (size_t)m * N + n;
+          const unsigned long long inc = cell_increment(v);
+          const unsigned long long before = __hip_atomic_fetch_add(cell, inc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          ps.mark_after(5, __builtin_bit_cast(float, (uint32_t)before));
+          const unsigned long long now = before + inc;
+          if (cell_complete(now, dp.splits)) {
+            y[(size_t)m * N + n] = finish_output<DTYPE>(cell_value(now), dp.bias, n);
+            __hip_atomic_store(cell, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+      }
+    }
+  } else if (dp.splits == 1) {
+    // the rows are dealt to the waves: wave w finishes rows w, w + wk, ..
+    for (int r = wave; r < dp.M; r += wk) {
+      const float v = row_sum(r);
+      if (r == wave) ps.mark_after(4, v);
+      y[(size_t)r * N + n] = finish_output<DTYPE>(v, dp.bias, n);
+    }
+  } else {
+    // fp32 partial sums, a ticket per column tile, the last workgroup adds in split order
+    for (int r = wave; r < dp.M; r += wk) {
+      const float v = row_sum(r);
+      if (r == wave) ps.mark_after(4, v);
+      __hip_atomic_store(dp.partials + ((size_t)blockIdx.y * dp.M + r) * N + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    uint32_t* ticket_s = (uint32_t*)(smem + (size_t)wk * MR * 64 * sizeof(float));
+    uint32_t* ticket = dp.tickets + blockIdx.x;
+    if (threadIdx.x == 0) *ticket_s = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    ps.mark(5);
+    if (*ticket_s == (uint32_t)(dp.splits - 1)) {
+      const size_t sstride = (size_t)dp.M * N;
+      for (int r = wave; r < dp.M; r += wk) {
+        const float* src = dp.partials + (size_t)r * N + n;
+        float sum = 0.f;
+        int sp = 0;
+        for (; sp + 8 <= dp.splits; sp += 8) {
+          float v[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) v[u] = __hip_atomic_load(src + (size_t)(sp + u) * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) sum += v[u];
+        }
+        for (; sp < dp.splits; ++sp) sum += __hip_atomic_load(src + (size_t)sp * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        y[(size_t)r * N + n] = finish_output<DTYPE>(sum, dp.bias, n);
+      }
+      if (threadIdx.x == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+#ifdef Q4_PHASE_STAMPS
+  ps.flush_to(dp.stamps, lane, wave);
+#endif
+}
+
+}  // namespace q4

@@ -200,16 +200,17 @@ struct PhaseStamps {
     asm volatile("" ::"v"(v));
     mark(i);
   }
-  __device__ __forceinline__ void flush(const GemvParams& gp, const Decomp& d) {
-    if (gp.stamps == nullptr) return;
+  // all eight readings of this wave -> base[workgroup][wave][8]
+  __device__ __forceinline__ void flush_to(unsigned long long* base, int lane, int wave) {
+    if (base == nullptr) return;
     mark(7);
-    if (d.lane == 0) {
-      unsigned long long* dst =
-          gp.stamps + (((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + d.wave) * 8;
+    if (lane == 0) {
+      unsigned long long* dst = base + (((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + wave) * 8;
 #pragma unroll
       for (int i = 0; i < 8; ++i) dst[i] = t[i];
     }
   }
+  __device__ __forceinline__ void flush(const GemvParams& gp, const Decomp& d) { flush_to(gp.stamps, d.lane, d.wave); }
 #else
   __device__ __forceinline__ void mark(int) {}
   __device__ __forceinline__ void mark_after(int, float) {}

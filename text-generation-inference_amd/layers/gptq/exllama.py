@@ -5,11 +5,16 @@ server/text_generation_server/layers/gptq/exllamav2.py:178-231 and
 gptq/exllama.py:66-134.  The reference needs a Warmup hook (`set_device`,
 `create_exllama_buffers`, server.py:103-116) to allocate a dequant scratch buffer and to
 repack qweight in place; nothing of that exists here (the kernels read the checkpoint
-layout and never materialise W), so both hooks are kept as no-ops for call
-compatibility.
+layout and never materialise W).  `set_device` is kept as a no-op for call compatibility;
+`create_exllama_buffers(max_total_tokens)`, which the server calls once after the model is
+loaded and before it captures its decode graphs, is where this package does its own one-time
+work over all layers: the shared workspace is sized for `max_total_tokens` rows and the decode
+launch plans are measured (`ops.autotune`; `Q4_AUTOTUNE=0` keeps the library's fitted choices).
 """
 
 from __future__ import annotations
+
+import os
 
 import torch
 import torch.nn as nn
@@ -28,8 +33,18 @@ def set_device(device):
     DEVICE = device
 
 
-def create_exllama_buffers(max_total_tokens: int):
-    """No scratch buffers to create: W is never materialised (exllamav2.py:159-175)."""
+def create_exllama_buffers(max_total_tokens: int = 4096):
+    """The reference's Warmup hook (exllamav2.py:159-175: scratch sized for max_total_tokens,
+    device matrices built).  Here: every layer built so far fetches its launch plans up to
+    `max_total_tokens` rows and the shared workspace grows to the largest need, then the decode
+    plans of all layers are measured on the GPU (one pass per distinct layer shape; the report is
+    kept in `ops.last_autotune_report`).  Returns None, like the reference's hook."""
+    weights = [r() for r in ops._prepared]
+    weights = [w for w in weights if w is not None and w.qweight.is_cuda]
+    for w in weights:
+        w.prepare(max_rows=int(max_total_tokens))
+    if weights and os.environ.get("Q4_AUTOTUNE", "1") != "0":
+        ops.autotune(weights)
     return None
 
 

@@ -7,6 +7,7 @@ kernels of libq4linear.so.  CPU tensors are rejected: there is no host fallback.
 from __future__ import annotations
 
 import ctypes
+import weakref
 from dataclasses import dataclass, field
 from typing import Optional
 
@@ -26,6 +27,20 @@ _DTYPES = {torch.float16: DTYPE_F16, torch.bfloat16: DTYPE_BF16}
 
 # (device index, stream handle) -> zero-initialised workspace tensor (uint8)
 _workspaces: dict[tuple[int, int], torch.Tensor] = {}
+# Workspaces that were replaced by larger ones.  A HIP graph captured earlier holds the raw
+# address of the buffer it was recorded with and writes tickets, cells and partial sums there on
+# every replay: handing that memory back to the allocator would let replays corrupt whatever
+# tensor gets it next.  Buffers grow geometrically, so everything retired stays below the size of
+# the live one.
+_retired_workspaces: list[torch.Tensor] = []
+# weights whose layers were built on the GPU (prepare()), for the load-time tuning pass
+_prepared: list = []
+# what the last autotune() call measured and chose
+last_autotune_report: dict = {}
+
+# row counts whose launch plans a layer fetches when it is built: every decode batch up to 16
+# rows and a ladder up to the prefill limit
+_PLAN_ROWS = tuple(range(1, 17)) + (17, 20, 24, 32, 33, 48, 64, 65, 96, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096)
 
 
 def _require_cuda(t: torch.Tensor, name: str) -> None:
@@ -79,7 +94,9 @@ class PackedWeight:
         return self._struct
 
     def plan(self, M: int, dtype_code: int) -> tuple:
-        """(Q4_PATH_* the library picks, workspace bytes the call needs) for M rows."""
+        """(Q4_PATH_* the library picks, workspace bytes the call needs, explicit decode
+        configuration or None) for M rows.  The configuration is None until a tuning pass
+        (autotune) has measured a faster one than the library's own choice."""
         key = (M, dtype_code)
         got = self._plans.get(key)
         if got is None:
@@ -91,21 +108,30 @@ class PackedWeight:
                 # weight in group order: x is gathered into the tail of the workspace (all but the
                 # shortest decode calls, which gather inside the kernel)
                 nbytes = max(nbytes, int(lib.q4_workspace_bytes_perm(M, self.K, self.N)))
-            got = (int(path.value), nbytes)
+            got = (int(path.value), nbytes, None)
             self._plans[key] = got
         return got
 
-    def prepare(self, rows=tuple(range(1, 17)) + (32, 64)) -> None:
-        """Load-time step of a layer: fetch the launch plans of the decode row counts and
-        reserve the device's shared workspace for them, so that the first forward neither asks
-        the library for a plan nor allocates (it can be captured into a HIP graph)."""
+    def prepare(self, rows=None, max_rows: int = 4096) -> None:
+        """Load-time step of a layer: fetch the launch plans of the decode row counts and of a
+        ladder of prefill row counts up to `max_rows` (the reference sizes its scratch for
+        max_total_tokens at Warmup, layers/gptq/exllamav2.py:159-175), and reserve the device's
+        shared workspace for the largest of them, so that a first forward at any of these row
+        counts neither asks the library for a plan nor allocates (it can be captured into a HIP
+        graph)."""
         if not self.qweight.is_cuda:
             return
+        if rows is None:
+            rows = tuple(M for M in _PLAN_ROWS if M <= max(max_rows, 16))
+            if max_rows > 16 and max_rows not in rows:
+                rows = rows + (max_rows,)
         need = max(self.plan(M, DTYPE_F16)[1] for M in rows)
         for M in rows:
-            self.plan(M, DTYPE_BF16)
+            need = max(need, self.plan(M, DTYPE_BF16)[1])
         with torch.cuda.device(self.qweight.device):
             reserve_workspace(self.qweight.device, need, SHARED)
+        if not any(r() is self for r in _prepared):
+            _prepared.append(weakref.ref(self))
 
     def _make_struct(self) -> Q4Weight:
         return Q4Weight(
@@ -264,7 +290,8 @@ def reserve_workspace(device: torch.device, nbytes: int, stream: Optional[int] =
     """Return this (device, stream)'s workspace, growing it to at least `nbytes`.
 
     The first bytes hold the split-K ticket counters: they must start at zero and the
-    kernels leave them at zero, so a grown buffer is freshly zeroed and the old one dropped.
+    kernels leave them at zero, so a grown buffer is freshly zeroed; the old one is kept (not
+    freed), because HIP graphs captured earlier hold its address.
     `stream=SHARED` names the device's shared workspace: the layers reserve it when they are
     built, and calls made while a stream is capturing (where nothing may be allocated or
     cleared) fall back to it.
@@ -274,6 +301,11 @@ def reserve_workspace(device: torch.device, nbytes: int, stream: Optional[int] =
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if ws is not None:
+            # a captured graph may still write into the old buffer on replay: it is kept alive,
+            # and the new one is at least twice its size so that the retired ones stay bounded
+            _retired_workspaces.append(ws)
+            nbytes = max(int(nbytes), 2 * ws.numel())
         ws = torch.zeros(int(nbytes), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
@@ -363,9 +395,11 @@ def linear(
         stream = _stream_handle(x.device)
         # decode: split-K partial sums, tickets, accumulation cells; prefill GEMM: split-K
         # partial tiles when the tile grid alone would leave CUs idle
-        planned_path, need = w.plan(M, _DTYPES[x.dtype])
+        planned_path, need, tuned = w.plan(M, _DTYPES[x.dtype])
         if path == PATH_AUTO and gemv_config is None:
             path = planned_path
+            if tuned is not None and w.perm is None:
+                gemv_config = tuned  # the decomposition a tuning pass measured fastest
         ws = _workspace_for_call(x.device, need, stream)
         st = w.struct()
         if gemv_config is not None:
@@ -373,7 +407,7 @@ def linear(
             words = gemv_config[3] if len(gemv_config) > 3 else 4
             need = _lib.WORKSPACE_COUNTER_BYTES + splits * M * w.N * 4
             if ws.numel() < need:
-                ws = reserve_workspace(x.device, need, stream)
+                ws = _workspace_for_call(x.device, need, stream)
             rc = lib.q4_gemv_tuned(
                 ctypes.byref(st), x.data_ptr(), bias_ptr, y.data_ptr(), M, _DTYPES[x.dtype],
                 ws.data_ptr(), ws.numel(), wcol, wk, splits, words, stream,
@@ -395,6 +429,99 @@ def linear(
         else:
             y = y + bias
     return y
+
+
+def _time_graph_launches(fns, reps: int) -> float:
+    """Seconds per launch: `reps` launches (rotating over fns) captured into one HIP graph on a
+    side stream, replayed and bracketed by events on that stream."""
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        fns[0]()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(reps):
+                fns[i % len(fns)]()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(side)
+            graph.replay()
+            e1.record(side)
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) * 1e-3 / reps
+            best = t if best is None or t < best else best
+    del graph
+    return best
+
+
+def decode_candidates(w: PackedWeight, M: int, dtype: torch.dtype = torch.float16) -> list:
+    """Explicit decode configurations the library offers for timing against its own choice."""
+    buf = (ctypes.c_int32 * (4 * 32))()
+    n = int(_lib.load().q4_gemv_candidates(ctypes.byref(w.struct()), int(M), _DTYPES[dtype], buf, 32))
+    _lib.check(n)
+    return [tuple(int(buf[4 * i + k]) for k in range(4)) for i in range(n)]
+
+
+def autotune(weights=None, rows=(1, 2, 3, 4, 8, 16), dtype: torch.dtype = torch.float16, reps: int = 24,
+             min_gain: float = 0.03) -> dict:
+    """Measured launch plans for the decode row counts, the load-time counterpart of the
+    autotuner of the reference's Triton path (layers/gptq/custom_autotune.py:1-80).
+
+    Weights of the same geometry (the layers of one model that share a shape) form a group.  For
+    every group and row count the library's own choice and each configuration it offers
+    (q4_gemv_candidates) are timed as HIP graphs of `reps` launches that rotate over the group's
+    weights (so that a group larger than the last-level cache streams from HBM, as in serving),
+    and the fastest one is kept in every weight's plan when it beats the library's choice by
+    `min_gain` or more.  `weights=None`: every weight whose layer was built on the GPU.
+    Synchronizes the device; call it once after the model is loaded and before any stream
+    capture (the layers do: `create_exllama_buffers`, the reference's Warmup hook).
+    Returns {(K, N, groupsize, M): (chosen configuration or None, us of the library's choice,
+    us of the chosen one)}."""
+    if weights is None:
+        weights = [r() for r in _prepared]
+        weights = [w for w in weights if w is not None]
+    groups: dict = {}
+    for w in weights:
+        if not w.qweight.is_cuda or w.perm is not None:
+            continue
+        key = (w.qweight.device, w.K, w.N, w.groupsize, w.num_groups, w.layout, w.g_idx is not None)
+        groups.setdefault(key, []).append(w)
+    code = _DTYPES[dtype]
+    report = {}
+    lib = _lib.load()
+    for (device, K, N, groupsize, _, _, _), ws in groups.items():
+        with torch.cuda.device(device):
+            rot = ws[:: max(1, len(ws) // 8)][:8]  # up to eight weights of the group, spread over it
+            for M in rows:
+                if ws[0].plan(M, code)[0] != _lib.PATH_GEMV:
+                    continue
+                cands = decode_candidates(ws[0], M, dtype)
+                if not cands:
+                    continue
+                x = torch.randn((M, K), device=device, dtype=dtype)
+                y = torch.empty((M, N), device=device, dtype=dtype)
+                need = max([ws[0].plan(M, code)[1]] + [
+                    int(lib.q4_gemv_tuned_workspace_bytes(ctypes.byref(ws[0].struct()), M, code, *cfg)) for cfg in cands])
+                reserve_workspace(device, need, SHARED)
+                base = _time_graph_launches([(lambda w=w: linear(w, x, None, path=_lib.PATH_GEMV, out=y)) for w in rot], reps)
+                best_t, best_cfg = base, None
+                for cfg in cands:
+                    t = _time_graph_launches([(lambda w=w, cfg=cfg: linear(w, x, None, gemv_config=cfg, out=y)) for w in rot], reps)
+                    if t < best_t:
+                        best_t, best_cfg = t, cfg
+                if best_cfg is not None and best_t > (1.0 - min_gain) * base:
+                    best_t, best_cfg = base, None
+                for w in ws:
+                    path, nbytes, _ = w.plan(M, code)
+                    w._plans[(M, code)] = (path, max(nbytes, need), best_cfg)
+                report[(K, N, groupsize, M)] = (best_cfg, round(base * 1e6, 2), round(best_t * 1e6, 2))
+    global last_autotune_report
+    last_autotune_report = report
+    return report
 
 
 def act_mul(gate_up: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor] = None) -> torch.Tensor:
