@@ -8,9 +8,11 @@
 //     K split); the 128-row chunks are dealt to the splits x waves slots in order, the first
 //     `rem` slots one more than the others, so a wave finds its range with a multiply and a
 //     minimum: no division, a parameter block of about 100 bytes.
-//   * No activation slab and no barrier before the first MFMA.  Only the lanes whose MFMA row
-//     is a live activation row (lane % 16 < M) fetch 16 bytes of x per 32-row step, straight
-//     from global memory (x stays in L2), issued ahead of the weight words they meet; one byte
+//   * No activation slab and no barrier before the first MFMA.  Up to four rows a wave fetches
+//     the 128-row chunk of all its rows with one 16-byte load per lane and passes it through 1 KB
+//     of LDS of its own into operand order; beyond, the lanes whose MFMA row is a live
+//     activation row fetch 16 bytes of x per 32-row step straight from global memory (x stays
+//     in L2).  Either way the loads are issued ahead of the weight words they meet, and one byte
 //     permute per register puts them in the K order of the nibble splice.
 //   * The arithmetic is that of gemv_gptq_lean_kernel: spliced nibbles enter the MFMA with
 //     their offsets (1024 + q / 64 + q; bf16: 128 + q), one more MFMA per step against a
@@ -86,8 +88,17 @@ __global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) 
   const uint32_t x_lane = ((uint32_t)(row_live ? j : 0) * (uint32_t)dp.K + (uint32_t)kq * 8u) * 2u;
   const uint32_t step_bytes = (uint32_t)N * 16u;  // four packed rows
 
+  // Up to four rows: the whole 128-row chunk of all of them is 4 x 256 bytes, one 16-byte load
+  // per lane (lane l: row l / 16, bytes 16 (l % 16) ..); the wave passes it through its own 1 KB
+  // of LDS into MFMA operand order.  Sixteen rows: every lane fetches the 16 bytes of its (row,
+  // K block) per 32-row step itself.
+  constexpr bool XLDS = MR <= 4;
+  constexpr int XREGS = XLDS ? 1 : kChunkSteps;
+  const bool xl_live = (lane >> 4) < dp.M;
+  const uint32_t xl_lane = ((uint32_t)(xl_live ? (lane >> 4) : 0) * (uint32_t)dp.K + (uint32_t)(lane & 15) * 8u) * 2u;
+  unsigned char* xbuf = smem + wave * 1024;  // this wave's activation chunk (XLDS)
   struct Chunk {
-    uint4_t x[kChunkSteps];
+    uint4_t x[XREGS];
     uint4_t w[kChunkSteps];
     uint2_t s;
     uint32_t z;
@@ -97,18 +108,25 @@ __global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) 
     const uint32_t chunk = (uint32_t)(c0 + c);
     // activations first: memory returns in issue order, and an L2 hit must not queue behind
     // the weight stream of this wave
+    if constexpr (XLDS) {
+      q.x[0] = uint4_t{0u, 0u, 0u, 0u};
+      if (xl_live) q.x[0] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xl_lane, chunk * (kChunkRows * 2u), 0));
+    } else {
 #pragma unroll
-    for (int st = 0; st < kChunkSteps; ++st) {
-      q.x[st] = uint4_t{0u, 0u, 0u, 0u};
-      if (row_live)
-        q.x[st] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, x_lane, (chunk * kChunkRows + st * 32) * 2u, 0));
+      for (int st = 0; st < kChunkSteps; ++st) {
+        q.x[st] = uint4_t{0u, 0u, 0u, 0u};
+        if (row_live)
+          q.x[st] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, x_lane, (chunk * kChunkRows + st * 32) * 2u, 0));
+      }
     }
-    const uint32_t gi = (uint32_t)min((int)(chunk >> dp.gshift), dp.num_groups - 1);
-    q.s = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(srsrc, s_lane, gi * (uint32_t)N * 2u, 0));
-    q.z = __builtin_amdgcn_raw_buffer_load_b32(zrsrc, z_lane, gi * (uint32_t)(N >> 3) * 4u, 0);
 #pragma unroll
     for (int st = 0; st < kChunkSteps; ++st)
       q.w[st] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, w_lane, (chunk * kChunkSteps + st) * step_bytes, 2));
+    // scale and zero point are needed when the chunk's last MFMA is done: asked for behind the
+    // weights, they arrive with them instead of holding their return back
+    const uint32_t gi = (uint32_t)min((int)(chunk >> dp.gshift), dp.num_groups - 1);
+    q.s = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(srsrc, s_lane, gi * (uint32_t)N * 2u, 0));
+    q.z = __builtin_amdgcn_raw_buffer_load_b32(zrsrc, z_lane, gi * (uint32_t)(N >> 3) * 4u, 0);
   };
 #pragma unroll
   for (int b = 0; b < PF; ++b)
@@ -130,16 +148,26 @@ __global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) 
     for (int i = 0; i < RL; ++i) tot[t][i] = 0.f;
   bool poisoned = false;  // some chunk of this wave met an inf or NaN activation
 
+  // 16 bytes of activations into the K order [0,4,1,5,2,6,3,7] of the splice
+  auto k_order = [](const uint4_t v) {
+    uint4_t a;
+    a.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+    a.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+    a.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+    a.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+    return a;
+  };
   auto process_chunk = [&](const Chunk& q) {
     float4_t acc[4], accc;
+    if constexpr (XLDS) *(uint4_t*)(xbuf + lane * 16) = k_order(q.x[0]);  // rows beyond M: zeros
 #pragma unroll
     for (int st = 0; st < kChunkSteps; ++st) {
-      // K order [0,4,1,5,2,6,3,7] of the splice
-      uint4_t a;
-      a.x = __builtin_amdgcn_perm(q.x[st].z, q.x[st].x, 0x05040100u);
-      a.y = __builtin_amdgcn_perm(q.x[st].z, q.x[st].x, 0x07060302u);
-      a.z = __builtin_amdgcn_perm(q.x[st].w, q.x[st].y, 0x05040100u);
-      a.w = __builtin_amdgcn_perm(q.x[st].w, q.x[st].y, 0x07060302u);
+      uint4_t a = {0u, 0u, 0u, 0u};
+      if constexpr (XLDS) {
+        if (j < 4) a = *(const uint4_t*)(xbuf + j * 256 + (st * 4 + kq) * 16);
+      } else {
+        a = k_order(q.x[st]);
+      }
       const uint32_t words[4] = {q.w[st].x, q.w[st].y, q.w[st].z, q.w[st].w};
 #pragma unroll
       for (int t = 0; t < 4; ++t) acc[t] = lean_mfma<DTYPE>(a, lean_unpack<DTYPE>(words[t], kc), st == 0 ? zero4 : acc[t]);
@@ -237,7 +265,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) 
   }
 
   // ---- the K waves meet in LDS: wave w leaves row r at red[(w * MR + r) * 64 + column]
-  float* red = (float*)smem;
+  float* red = (float*)(smem + (XLDS ? wk * 1024 : 0));
   if (MR == 16 || kq == 0) {
 #pragma unroll
     for (int i = 0; i < RL; ++i) {
@@ -292,7 +320,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) 
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    uint32_t* ticket_s = (uint32_t*)(smem + (size_t)wk * MR * 64 * sizeof(float));
+    uint32_t* ticket_s = (uint32_t*)(red + wk * MR * 64);
     uint32_t* ticket = dp.tickets + blockIdx.x;
     if (threadIdx.x == 0) *ticket_s = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
