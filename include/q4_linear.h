@@ -117,6 +117,13 @@ int q4_linear_gate_up(const q4_weight* w, const void* x, const void* bias, void*
                       int act, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Which route is faster for the gated first half of an MLP on this problem: *fused = 1 when a
+ * fused kernel exists (q4_linear_gate_up will run) and it measured faster than q4_linear into an
+ * [M, N] buffer followed by q4_act_mul, else 0.  A pure function of (w's geometry, M, dtype).
+ */
+int q4_linear_gate_up_plan(const q4_weight* w, int M, int dtype, int* fused);
+
+/*
  * Act-order by row order instead of per-weight lookups, as the reference's exllamav2 path does
  * (QMatrix::make_sequential and make_sequential_kernel,
  * server/exllamav2_kernels/exllamav2_kernels/cuda/q_matrix.cu:524-640; activations read

@@ -100,3 +100,59 @@ def test_packed_gate_up_forward(pkg, oracle, gpu, tmp_path):
         want = np.concatenate([y_full[:, rank * q:(rank + 1) * q],
                                y_full[:, 2 * q + rank * q: 2 * q + (rank + 1) * q]], axis=1)
         assert max_rel_err(got, want) <= TOL
+
+
+@pytest.mark.parametrize("act_order", [True, False])
+def test_solver_made_checkpoint_through_the_loader(pkg, oracle, gpu, tmp_path, act_order):
+    """The route a self-quantized model takes: GPTQ solve and pack one layer with act-order
+    (`quantize_linear`), write its tensors the way the reference's quantizer saves them
+    (server/text_generation_server/layers/gptq/quantize.py:957-1012: the module's state dict plus
+    the `gptq_bits` / `gptq_groupsize` / `gptq_sym` marker tensors, and a quantize config beside
+    it), read the directory back with `get_loader("gptq")` -> `Weights` -> `get_linear`, and run
+    it.  The g_idx here is the solver's (groups in order of the Hessian diagonal), not a random
+    permutation.  Bars: the loaded layer reproduces the in-memory packed layer bit for bit, and
+    it tracks the dense layer on held-out inputs better than round-to-nearest does."""
+    import json
+
+    rng = np.random.default_rng(12)
+    K2, N2, gs = 1024, 384, 128
+    # correlated calibration inputs (a few strong shared directions plus noise: what the solver's
+    # error feedback exploits) with very different column scales, so that act-order reorders
+    basis = rng.standard_normal((8, K2))
+    col_scale = np.exp(rng.standard_normal(K2))
+    X = ((rng.standard_normal((2048, 8)) @ basis * 1.5 + 0.3 * rng.standard_normal((2048, K2))) * col_scale).astype(np.float32)
+    W = (rng.standard_normal((N2, K2)) * 0.05).astype(np.float32)
+    lin = torch.nn.Linear(K2, N2, bias=True)
+    lin.weight.data = torch.from_numpy(W.copy())
+    bias = lin.bias.data.clone()
+    lin = lin.to(gpu)
+    layer, err = pkg.quantize_linear(lin, torch.from_numpy(X[:1536]).to(gpu), groupsize=gs, act_order=act_order, sym=True)
+    g_idx = layer.g_idx.cpu()
+    trivial = bool(torch.equal(g_idx, (torch.arange(K2) // gs).to(g_idx.dtype)))
+    assert trivial != act_order, "act-order must reorder the rows of this calibration set (and only act-order)"
+
+    model_dir = tmp_path / "quantized"
+    model_dir.mkdir()
+    tensors = {f"model.proj.{k}": v.detach().cpu().contiguous() for k, v in layer.state_dict().items()}
+    tensors.update({"gptq_bits": torch.tensor(4), "gptq_groupsize": torch.tensor(gs), "gptq_sym": torch.tensor(True)})
+    save_file(tensors, str(model_dir / "model.safetensors"))
+    (model_dir / "quantize_config.json").write_text(json.dumps(
+        {"bits": 4, "group_size": gs, "desc_act": act_order, "sym": True, "quant_method": "gptq"}))
+
+    loader = pkg.get_loader("gptq", str(model_dir))
+    weights = pkg.Weights([model_dir / "model.safetensors"], gpu, torch.float16, None, loader)
+    loaded = pkg.get_linear(weights.get_weights("model.proj"), weights.get_tensor("model.proj.bias"))
+
+    held = X[1536:1600]
+    xt = torch.from_numpy(held.astype(np.float16)).to(gpu)
+    for M in (1, 16, 64):
+        assert torch.equal(loaded(xt[:M]), layer(xt[:M])), f"loaded layer differs from the packed one at M={M}"
+    y = to_f32(loaded(xt))
+    want = held.astype(np.float16).astype(np.float64) @ W.T.astype(np.float64) + bias.numpy()
+    # round-to-nearest with the same grid, for the bar
+    Wg = W.reshape(N2, K2 // gs, gs)
+    absmax = np.abs(Wg).max(axis=2, keepdims=True)
+    scale = np.maximum(absmax, 1e-9) * 2 / 15
+    rtn = (np.clip(np.round(Wg / scale) + 8, 0, 15) - 8) * scale
+    out_rtn = np.linalg.norm(held.astype(np.float64) @ (W - rtn.reshape(N2, K2)).T)
+    assert np.linalg.norm(y - want) < out_rtn

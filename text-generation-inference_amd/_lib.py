@@ -87,6 +87,7 @@ SIGNATURES = {
         c_int,
         [POINTER(Q4Weight), c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),
+    "q4_linear_gate_up_plan": (c_int, [POINTER(Q4Weight), c_int, c_int, POINTER(c_int)]),
     "q4_act_mul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "q4_gptq_make_sequential": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "q4_gather_columns": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),

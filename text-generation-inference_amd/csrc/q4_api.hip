@@ -464,6 +464,32 @@ int q4_linear_gate_up(const q4_weight* w, const void* x, const void* bias, void*
   return Q4_ERR_UNSUPPORTED;
 }
 
+int q4_linear_gate_up_plan(const q4_weight* w, int M, int dtype, int* fused) {
+  int rc = validate_weight(w, "q4_linear_gate_up_plan");
+  if (rc == Q4_OK) rc = validate_dtype(dtype, "q4_linear_gate_up_plan");
+  if (rc != Q4_OK) return rc;
+  if (fused == nullptr || M < 0) {
+    set_error("q4_linear_gate_up_plan: null output or negative M=%d", M);
+    return Q4_ERR_INVALID_ARGUMENT;
+  }
+  *fused = 0;
+  if (M == 0 || w->K == 0 || w->N == 0 || (w->N & 1)) return Q4_OK;
+  const int path = q4_select_path(w, M, dtype);
+  if (path == Q4_PATH_GEMM) {
+    *fused = gemm_gate_up_supported(w, M, dtype) ? 1 : 0;
+    return Q4_OK;
+  }
+  if (path != Q4_PATH_GEMV || !gemv_gate_up_supported(w, M, dtype)) return Q4_OK;
+  // One or two rows on a large layer: the plain call runs the lean / short-launch kernels there,
+  // and that followed by the elementwise kernel beats the decode kernel with the gated epilogue
+  // (us on MI355X, fused / two launches: 4096 x 28672 17.7 / 16.6 at M = 1, 3072 x 16384 17.1 / 11.3 at
+  // M = 2, 8192 x 57344 53.7 / 47.5 at M = 2; 4096 x 22016 at M = 1, 16.1 / 17.0, is the one shape
+  // measured that loses).  Smaller layers keep the single launch.
+  const bool large = gemv_lean_supported(w, dtype) && (long)w->K * w->N >= (1L << 25) && w->K >= 1024;
+  *fused = large ? 0 : 1;
+  return Q4_OK;
+}
+
 int q4_act_mul(const void* gate_up, void* y, int M, int inter, int dtype, int act, void* stream) {
   int rc = validate_dtype(dtype, "q4_act_mul");
   if (rc != Q4_OK) return rc;

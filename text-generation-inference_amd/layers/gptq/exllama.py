@@ -69,6 +69,14 @@ class ExllamaQuantLinear(nn.Module):
             bool((g_idx == 0).all()) or is_trivial_g_idx(g_idx, weight.groupsize)
         ):
             g_idx = None
+        if g_idx is not None:
+            # The exllama kernels only look at the *order* of g_idx (rows are sorted by it and
+            # group i of the sorted rows is i // groupsize: exllamav2.py:106-130 -> make_sequential,
+            # q_matrix.cu:566-650), and the loader hands this module `g_idx - g_idx[0]`
+            # (gptq/__init__.py:163-164, 395-397), whose smallest entry is negative whenever row 0
+            # is not in the first group.  The kernels here index the scale / zero tables with
+            # g_idx itself, so it is rebased to start at 0: the same groups exllama would form.
+            g_idx = g_idx - g_idx.min()
         self.act_order = g_idx is not None
         groupsize = weight.groupsize
         if g_idx is None and weight.scales.shape[0] == 1:

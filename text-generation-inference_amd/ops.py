@@ -544,11 +544,17 @@ def act_mul(gate_up: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor
     return y
 
 
-def _plain_decode_is_lean(w: PackedWeight) -> bool:
-    """Whether q4_linear runs the instruction-lean decode kernel on this weight at up to 16 rows:
-    GPTQ layout, contiguous groups of whole 128-row chunks, 32 M weights or more."""
-    return (w.layout == LAYOUT_GPTQ and w.g_idx is None and w.groupsize >= 128 and w.groupsize % 128 == 0
-            and w.K % 128 == 0 and w.K >= 1024 and w.N % 64 == 0 and w.K * w.N >= (1 << 25))
+def _gate_up_fused_preferred(w: PackedWeight, M: int, dtype_code: int) -> bool:
+    """The library's own answer (q4_linear_gate_up_plan) to: one fused launch, or the linear
+    kernel followed by the elementwise kernel?  Kept with the weight's plans."""
+    key = ("gate_up", M, dtype_code)
+    got = w._plans.get(key)
+    if got is None:
+        fused = ctypes.c_int(0)
+        _lib.check(_lib.load().q4_linear_gate_up_plan(ctypes.byref(w.struct()), int(M), dtype_code, ctypes.byref(fused)))
+        got = bool(fused.value)
+        w._plans[key] = got
+    return got
 
 
 def linear_gate_up(
@@ -583,12 +589,8 @@ def linear_gate_up(
     if M == 0 or inter == 0:
         return y
     fusable_bias = bias is None or (bias.dtype == x.dtype and bias.is_cuda and bias.numel() == w.N)
-    if fused is None and M <= 2 and _plain_decode_is_lean(w):
-        # one or two rows on a large layer: the instruction-lean decode kernel followed by the
-        # elementwise kernel beats the decode kernel with the gated epilogue (us on MI355X, fused / two
-        # launches: 4096 x 28672 17.7 / 16.6 at M = 1, 3072 x 16384 17.1 / 11.3 at M = 2, 8192 x 57344
-        # 53.7 / 47.5 at M = 2; 4096 x 22016 at M = 1, 16.1 / 17.0, is the one shape measured that loses)
-        fused = False
+    if fused is None and not _gate_up_fused_preferred(w, M, _DTYPES[x.dtype]):
+        fused = False  # no fused kernel here, or the two launches measured faster (the library's rule)
     if fused is not False and fusable_bias:
         lib = _lib.load()
         with _on_device(x.device):
