@@ -2,13 +2,13 @@
 straight from global memory, the grid as the work decomposition) against the oracle, forced
 through explicit decompositions (`words = -1` in the tuned entry point selects it; the tuple is
 (unused, K waves per workgroup, workgroups along K, -1)): every row count, both dtypes, unsplit
-and split K (fixed-point cells up to three fp16 rows, tickets beyond), even and ragged K deals,
+and split K (fixed-point cells for fp16 rows, tickets for bf16), even and ragged K deals,
 group sizes, and one-hot rows that must read the dequantized weights back bit for bit."""
 import numpy as np
 import pytest
 import torch
 
-from tests.util import bits_of, to_dev
+from tests.util import bits_of, max_rel_err, to_dev, to_f32
 from tests.test_linear_gpu import _run
 
 pytestmark = pytest.mark.gpu
@@ -68,18 +68,26 @@ def test_direct_one_hot_reads_weights_back(pkg, oracle, gpu, dtype, rows):
         assert np.array_equal(bits_of(y), w[ks].view(np.uint16)), cfg
 
 
-@pytest.mark.parametrize("M", [3, 16])
-def test_direct_split_k_is_reproducible_and_leaves_the_counters_zero(pkg, oracle, gpu, M):
-    """Cells (3 rows) and tickets (16 rows): the same bits on every call, counters back at zero."""
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M", [3, 4, 7, 16])
+@pytest.mark.parametrize("cfg", [(1, 4, 8, -1), (1, 8, 4, -1), (1, 1, 14, -1), None])
+def test_direct_split_k_is_reproducible_and_leaves_the_counters_zero(pkg, oracle, gpu, M, cfg, dtype):
+    """Cells (fp16: wave 0 row by row up to three rows, the rows dealt to the waves beyond) and
+    tickets (bf16): the same bits on every call, the oracle's result, counters back at zero.
+    cfg None: the decomposition the plain call takes."""
+    bf = dtype == "bf16"
     qw, qz, sc, _ = oracle.make_gptq(4096, 4096, 128, seed=8, sym=False)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 0)
-    x = to_dev(oracle.make_x(M, 4096, seed=5), gpu)
-    a = pkg.ops.linear(pk, x, None, gemv_config=(1, 4, 8, -1))
-    b = pkg.ops.linear(pk, x, None, gemv_config=(1, 4, 8, -1))
+    x = oracle.make_x(M, 4096, seed=5, dtype=dtype)
+    xd = to_dev(x, gpu, bf16=bf)
+    a = pkg.ops.linear(pk, xd, None, gemv_config=cfg, path=1)
+    b = pkg.ops.linear(pk, xd, None, gemv_config=cfg, path=1)
     torch.cuda.synchronize()
     assert torch.equal(a, b)
     for ws in pkg.ops._workspaces.values():
         assert int(ws[: pkg._lib.WORKSPACE_COUNTER_BYTES].sum().item()) == 0
+    ref = oracle.matmul_fp32(oracle.to_f32(x, dtype), oracle.to_f32(oracle.dequant_gptq(qw, qz, sc, None, 128, dtype), dtype))
+    assert max_rel_err(to_f32(a), ref) <= (8e-3 if bf else 2e-3)
 
 
 @pytest.mark.parametrize("M,cfg", [(1, (1, 4, 8, -1)), (2, (1, 2, 1, -1)), (3, (1, 4, 4, -1)), (4, (1, 4, 2, -1)), (16, (1, 8, 1, -1)), (9, (1, 4, 4, -1))])

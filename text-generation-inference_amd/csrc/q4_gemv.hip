@@ -634,13 +634,13 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
               w->layout, (const void*)w->g_idx, M, w->K, w->N, w->groupsize, dtype);
     return Q4_ERR_UNSUPPORTED;
   }
-  // Up to three fp16 rows on contiguous GPTQ groups, plain call: the short-launch kernel.  Four
-  // K waves per workgroup; the K splits (at most 14: they meet in the fixed-point cells) are as
-  // many as it takes to leave every wave the fewest chunks, and no more.  Same-box A/B on
-  // MI355X against the kernels below (us at M = 1 / 2 / 3): 4096 x 4096 5.33 / 6.20 / 6.94 ->
-  // 4.33 / 4.99 / 5.75, 4096 x 6144 5.91 / 6.74 / 7.49 -> 5.00 / 5.74 / 6.36, 14336 x 4096
-  // 9.33 / 9.87 / 10.97 -> 8.12 / 8.85 / 9.96, 4096 x 28672 13.55 / 13.72 / 15.59 -> 12.65 / 13.77 / 15.9.
-  if (cfg_in == nullptr && gate_up_act == 0 && x_perm == nullptr && M <= 3 && dtype == Q4_DTYPE_F16) {
+  // Up to sixteen fp16 rows on contiguous GPTQ groups, plain call: the short-launch kernel in
+  // the decomposition of gemv_direct_default (which leaves the wide projections with more than
+  // four rows to the kernels below).  Same-box A/B on MI355X against the kernels below, us at
+  // M = 1 / 4 / 16: 4096 x 4096 5.33 / 7.90 / 8.81 -> 4.33 / 5.17 / 6.71, 4096 x 6144
+  // 5.91 / 8.62 / 10.38 -> 5.00 / 5.93 / 8.29, 14336 x 4096 9.33 / 12.41 / 13.67 -> 8.12 / 9.50 /
+  // 13.03, 4096 x 28672 13.55 / 16.71 -> 12.65 / 14.9 (16 rows: not taken).
+  if (cfg_in == nullptr && gate_up_act == 0 && x_perm == nullptr && M <= 16 && dtype == Q4_DTYPE_F16) {
     int wk = 0, splits = 0;
     if (gemv_direct_default(w, M, dtype, &wk, &splits))
       return launch_gemv_direct(w, x, bias, y, M, dtype, workspace, workspace_bytes, wk, splits, stream);

@@ -29,10 +29,11 @@ bool gemv_direct_supported(const q4_weight* w, int M, int dtype, int wk, int spl
   return true;
 }
 
-// K splits meet in the fixed-point cells (one atomic per element) for up to three fp16 rows and
-// 14 splits; otherwise through fp32 partial sums and a ticket per column tile.
+// K splits meet in the fixed-point cells (one atomic per output element) for fp16 rows and up to
+// 14 splits while the rows' cells fit their part of the workspace; otherwise through fp32 partial
+// sums and a ticket per column tile.
 static bool direct_uses_cells(const q4_weight* w, int M, int dtype, int splits) {
-  return splits > 1 && splits <= 14 && dtype == Q4_DTYPE_F16 && M <= 3 && (size_t)M * w->N * 8 <= Q4_WORKSPACE_CELL_BYTES;
+  return splits > 1 && splits <= 14 && dtype == Q4_DTYPE_F16 && M <= 16 && (size_t)M * w->N * 8 <= Q4_WORKSPACE_CELL_BYTES;
 }
 
 size_t gemv_direct_workspace_bytes(const q4_weight* w, int M, int dtype, int splits) {
@@ -41,25 +42,45 @@ size_t gemv_direct_workspace_bytes(const q4_weight* w, int M, int dtype, int spl
   return (size_t)Q4_WORKSPACE_COUNTER_BYTES + (size_t)splits * M * w->N * sizeof(float);
 }
 
-// The decomposition the plain call takes when it runs this kernel: four K waves per workgroup
-// (fewer on a K shorter than four chunks) and the fewest K splits, up to the 14 the cells count,
-// that leave every wave the fewest chunks.  False when the kernel does not take the problem
-// or the splits would not meet in the cells.
+// The decomposition the plain call takes when it runs this kernel; false when the kernel does
+// not take the problem, the splits would not meet in the cells, or the slab kernels are the
+// better choice.
+//   Up to three rows: four K waves per workgroup (fewer on a K shorter than four chunks) and the
+// fewest K splits, up to the 14 the cells count, that leave every wave the fewest chunks.
+//   Four to sixteen rows: about one workgroup per CU (splits = 256 / column tiles, rounded), eight
+// K waves beyond four rows.  With 256 column tiles or more (no split) and more than four rows
+// every wave would re-read its share of the activations from L2 next to a long weight stream;
+// the kernels that stage the activations once per workgroup are faster there (4096 x 28672, 16
+// rows: 19.5 against 17.7 us), so those shapes are not taken.
 bool gemv_direct_default(const q4_weight* w, int M, int dtype, int* wk_out, int* splits_out) {
   const int chunks = w->K / 128;
-  const int wk = chunks >= 4 ? 4 : (chunks >= 2 ? 2 : 1);
-  if (!gemv_direct_supported(w, M, dtype, wk, 1)) return false;
-  int best_s = 1, best = (chunks + wk - 1) / wk;
-  for (int s = 2; s <= 14 && wk * s <= chunks; ++s) {
-    const int per = (chunks + wk * s - 1) / (wk * s);
-    if (per < best) {
-      best = per;
-      best_s = s;
+  if (M <= 3) {
+    const int wk = chunks >= 4 ? 4 : (chunks >= 2 ? 2 : 1);
+    if (!gemv_direct_supported(w, M, dtype, wk, 1)) return false;
+    int best_s = 1, best = (chunks + wk - 1) / wk;
+    for (int s = 2; s <= 14 && wk * s <= chunks; ++s) {
+      const int per = (chunks + wk * s - 1) / (wk * s);
+      if (per < best) {
+        best = per;
+        best_s = s;
+      }
     }
+    if (best_s > 1 && !direct_uses_cells(w, M, dtype, best_s)) return false;
+    *wk_out = wk;
+    *splits_out = best_s;
+    return true;
   }
-  if (best_s > 1 && !direct_uses_cells(w, M, dtype, best_s)) return false;
+  const int tiles = w->N / 64;
+  if (tiles < 1 || (tiles >= 256 && M > 4)) return false;
+  int s = tiles >= 256 ? 1 : (256 + tiles / 2) / tiles;
+  s = s < 1 ? 1 : (s > 14 ? 14 : s);
+  int wk = M > 4 ? 8 : 4;
+  while (wk > 1 && wk * s > chunks) wk >>= 1;
+  while (s > 1 && wk * s > chunks) --s;
+  if (!gemv_direct_supported(w, M, dtype, wk, s)) return false;
+  if (s > 1 && !direct_uses_cells(w, M, dtype, s)) return false;
   *wk_out = wk;
-  *splits_out = best_s;
+  *splits_out = s;
   return true;
 }
 

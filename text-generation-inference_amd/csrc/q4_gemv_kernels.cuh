@@ -235,18 +235,29 @@ __device__ __forceinline__ bool moe_enter_decode(GemvParams& gp, const int32_t*&
 // (memory returns in issue order, so L2 hits must not queue behind the HBM stream they are
 // needed to consume) and stored after them.  PERMUTE stores every 8-block in the K order
 // [0,4,1,5,2,6,3,7] of the GPTQ nibble splice.
-template <bool PERMUTE>
+template <bool PERMUTE, int LOADS = 2>
 struct SlabStager {
-  static constexpr int kLoads = 2;  // 16-byte activation loads per thread kept in flight
+  static constexpr int kLoads = LOADS;  // 16-byte activation loads per thread in flight before the weight loads
+  static constexpr int kBatch = 4;      // ... and per round of what is left (many rows, a long K range)
   uint4_t xv[kLoads];
   const uint16_t* xs;
   const int32_t* rows;  // grouped launches: row of x behind every staged row, else nullptr
   const int32_t* cols;  // column of x behind every K row of the workgroup's range, else nullptr
-  int kb_per_row, items;
+  // Item i of a thread is 16-byte block tid + i * nthreads of the slab, counted row by row.  Its
+  // (row, block) is walked incrementally: one division per thread, none per item.
+  int kb_per_row, mloc;
+  int m0, kb0;   // the thread's first item
+  int dm, dkb;   // (row, block) step between a thread's items: nthreads = dm * kb_per_row + dkb
 
-  __device__ __forceinline__ uint4_t fetch(const GemvParams& gp, int idx) const {
-    const int m = idx / kb_per_row;
-    const int kb = idx - m * kb_per_row;
+  __device__ __forceinline__ void advance(int& m, int& kb) const {
+    m += dm;
+    kb += dkb;
+    if (kb >= kb_per_row) {
+      kb -= kb_per_row;
+      ++m;
+    }
+  }
+  __device__ __forceinline__ uint4_t fetch(const GemvParams& gp, int m, int kb) const {
     const int mr = rows != nullptr ? rows[m] : m;
     if (cols != nullptr) {
       // eight scattered columns of the row (it stays in L2); a bad index is clamped
@@ -269,17 +280,19 @@ struct SlabStager {
     cols = gp.p.x_perm != nullptr ? gp.p.x_perm + d.kwg0 : nullptr;
     xs = (const uint16_t*)gp.p.x + (row_map != nullptr ? 0 : (size_t)d.mb * gp.p.K) + (cols != nullptr ? 0 : d.kwg0);
     kb_per_row = d.KR >> 3;
-    items = d.mloc * kb_per_row;
+    mloc = d.mloc;
+    m0 = d.tid / kb_per_row;
+    kb0 = d.tid - m0 * kb_per_row;
+    dm = d.nthreads / kb_per_row;
+    dkb = d.nthreads - dm * kb_per_row;
+    int m = m0, kb = kb0;
 #pragma unroll
     for (int u = 0; u < kLoads; ++u) {
-      const int idx = d.tid + u * d.nthreads;
-      if (idx < items) xv[u] = fetch(gp, idx);
+      if (m < mloc) xv[u] = fetch(gp, m, kb);
+      advance(m, kb);
     }
   }
-  __device__ __forceinline__ void put(const GemvParams& gp, unsigned char* smem, int idx,
-                                      uint4_t v) const {
-    const int m = idx / kb_per_row;
-    const int kb = idx - m * kb_per_row;
+  __device__ __forceinline__ void put(const GemvParams& gp, unsigned char* smem, int m, int kb, uint4_t v) const {
     uint4_t o = v;
     if constexpr (PERMUTE) {
       o.x = (v.x & 0xFFFFu) | (v.z << 16);
@@ -289,15 +302,30 @@ struct SlabStager {
     }
     *(uint4_t*)(smem + (size_t)m * gp.slab_stride + kb * 16) = o;
   }
-  __device__ __forceinline__ void store(const GemvParams& gp, const Decomp& d,
-                                        unsigned char* smem) {
+  __device__ __forceinline__ void store(const GemvParams& gp, const Decomp& d, unsigned char* smem) {
+    (void)d;
+    int m = m0, kb = kb0;
 #pragma unroll
     for (int u = 0; u < kLoads; ++u) {
-      const int idx = d.tid + u * d.nthreads;
-      if (idx < items) put(gp, smem, idx, xv[u]);
+      if (m < mloc) put(gp, smem, m, kb, xv[u]);
+      advance(m, kb);
     }
-    for (int idx = d.tid + kLoads * d.nthreads; idx < items; idx += d.nthreads)
-      put(gp, smem, idx, fetch(gp, idx));
+    // the rest in rounds of kBatch loads per thread: one memory round trip per round, not per
+    // load (a row past the end is clamped for the load and not stored)
+    while (m < mloc) {
+      uint4_t t[kBatch];
+      int ms[kBatch], kbs[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        ms[u] = m;
+        kbs[u] = kb;
+        t[u] = fetch(gp, min(m, mloc - 1), kb);
+        advance(m, kb);
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u)
+        if (ms[u] < mloc) put(gp, smem, ms[u], kbs[u], t[u]);
+    }
   }
 };
 

@@ -158,7 +158,7 @@ __global__ __launch_bounds__(1024) void gemv_gptq_lean_kernel(GemvParams gp) {
   const int wstride = gp.slab_stride;  // bytes between activation rows of a wave's piece
   unsigned char* wslab = smem + (size_t)d.wave * gp.rows_per_block_alloc * wstride;
   if (!gp.wave_slab) {
-    SlabStager<true> slab;
+    SlabStager<true, (MP == 16 ? 8 : 4)> slab;
     slab.issue(gp, d);
     issue_first_chunks();
     ps.mark(6);
