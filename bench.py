@@ -413,9 +413,13 @@ def floor_probe(torch, dev):
     print(json.dumps({"read_floor": summary}))
 
 
-# the decode kernels' own launch geometry at M = 1 on the four projections: (workgroups, threads,
-# column waves per workgroup), for the probe launches that are to be compared with them
-DECODE_GRIDS = {"qkv_proj": (768, 256, 1), "o_proj": (512, 256, 1), "gate_up_proj": (224, 512, 2), "down_proj": (256, 512, 1)}
+# launch geometries at M = 1 on the four projections: (workgroups, threads, column waves per
+# workgroup) for the probe launches that are compared with the decode kernels.  First the
+# short-launch kernel's own grid (column tiles x K splits workgroups of four K waves), then, where
+# it differs, the grid of the kernels that stage an activation slab per workgroup (gate_up: 224
+# workgroups of two column waves x four K waves, unsplit).
+DECODE_GRIDS = {"qkv_proj": [(768, 256, 1)], "o_proj": [(512, 256, 1)],
+                "gate_up_proj": [(3584, 256, 1), (224, 512, 2)], "down_proj": [(896, 256, 1), (256, 512, 1)]}
 
 
 def probe_trace(pkg, torch, dev, weights, xs, ys, reps=40):
@@ -428,23 +432,24 @@ def probe_trace(pkg, torch, dev, weights, xs, ys, reps=40):
     sink = torch.zeros(4, dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     for i, (name, K, N) in enumerate(SHAPES):
-        wgs, threads, wcol = DECODE_GRIDS[name]
         nbytes = K * N // 2
         pieces = pool.numel() // nbytes
-        steps = (K // 32) // ((wgs // (N // (64 * wcol))) * (threads // 64 // wcol))
-        unroll = 8 if steps % 8 == 0 else (4 if steps % 4 == 0 else (2 if steps % 2 == 0 else 1))
-        for r in range(reps):
-            probe_check(lib.q4_probe_read(pool.data_ptr(), 4096, 2, 0, wgs, threads, 1, 1, sink.data_ptr(), stream))
-        torch.cuda.synchronize()
-        for r in range(reps):
-            probe_check(lib.q4_probe_read(pool.data_ptr() + (r % pieces) * nbytes, nbytes, 1, N, wgs, threads, unroll, wcol,
-                                          sink.data_ptr(), stream))
-        torch.cuda.synchronize()
+        for wgs, threads, wcol in DECODE_GRIDS[name]:
+            steps = (K // 32) // ((wgs // (N // (64 * wcol))) * (threads // 64 // wcol))
+            unroll = 8 if steps % 8 == 0 else (4 if steps % 4 == 0 else (2 if steps % 2 == 0 else 1))
+            for r in range(reps):
+                probe_check(lib.q4_probe_read(pool.data_ptr(), 4096, 2, 0, wgs, threads, 1, 1, sink.data_ptr(), stream))
+            torch.cuda.synchronize()
+            for r in range(reps):
+                probe_check(lib.q4_probe_read(pool.data_ptr() + (r % pieces) * nbytes, nbytes, 1, N, wgs, threads, unroll, wcol,
+                                              sink.data_ptr(), stream))
+            torch.cuda.synchronize()
+            print(f"probe trace: {name} {K}x{N}: {reps} empty launches ({wgs} x {threads}), {reps} read-only launches of "
+                  f"{nbytes} B (unroll {unroll}, {wcol} column waves)", file=sys.stderr)
         for r in range(reps):
             pkg.ops.linear(weights[r % len(weights)][i], xs[i], None, out=ys[i])
         torch.cuda.synchronize()
-        print(f"probe trace: {name} {K}x{N}: {reps} empty launches ({wgs} x {threads}), {reps} read-only launches of "
-              f"{nbytes} B (unroll {unroll}, {wcol} column waves), {reps} decode launches", file=sys.stderr)
+        print(f"probe trace: {name} {K}x{N}: {reps} decode launches", file=sys.stderr)
 
 
 PHASES = ["entry", "activations staged", "first chunk consumed", "K loop done",
@@ -472,7 +477,9 @@ def phase_breakdown(pkg, torch, dev, M, copies, launches=24, configs=None):
 
     configs = configs or {}
     out = {}
-    slots = 8192  # waves per launch the buffer has room for
+    lib.q4_phase_stamps_slots.restype = ctypes.c_int
+    lib.q4_phase_stamps_slots.argtypes = []
+    slots = int(lib.q4_phase_stamps_slots())  # waves per launch the library stamps at most (a larger launch leaves none)
     for i, (name, K, N) in enumerate(SHAPES):
         ws = [make_weights(pkg, torch, dev, K, N, seed=17 * c + i) for c in range(copies)]
         x = torch.randn((M, K), device=dev, dtype=torch.float16)
@@ -649,14 +656,16 @@ def main():
         torch.cuda.synchronize()
         Mg = args.gemm_m
         for i, (name, K, N) in enumerate(SHAPES):
+            if args.no_gemm:
+                break
             xg = torch.randn((Mg, K), device=dev, dtype=torch.float16)
             yg = torch.empty((Mg, N), device=dev, dtype=torch.float16)
             for c in range(copies):
                 pkg.ops.linear(weights[c][i], xg, None, out=yg)
             torch.cuda.synchronize()
             del xg, yg
-        print("traffic probe done: copy 268435456 B x5, decode steps x%d, gemm M=%d x%d per shape"
-              % (3 * copies, Mg, copies), file=sys.stderr)
+        print("traffic probe done: copy 268435456 B x5, decode steps (M=%d) x%d%s"
+              % (M, 3 * copies, "" if args.no_gemm else ", gemm M=%d x%d per shape" % (Mg, copies)), file=sys.stderr)
         return
 
     # ---- whole-job throughput: W warmup steps, then exactly K steps in one HIP graph

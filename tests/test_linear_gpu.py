@@ -234,6 +234,31 @@ def test_gemm_two_k_groups_small_groupsizes(pkg, oracle, gpu, gs, dtype, M):
     _run(pkg, oracle, gpu, 512, 4096, gs, M, dtype=dtype, sym=False, bias=True, path=2, seed=gs + M)
 
 
+@pytest.mark.parametrize("K,N,M,gs,dtype,bias", [(256, 6144, 2048, 128, "f16", False), (512, 6144, 1999, 64, "bf16", True),
+                                                  (256, 6144, 1536, 256, "f16", True), (192, 3072, 4096, 64, "f16", False),
+                                                  (320, 6144, 1290, -1, "bf16", False)])
+def test_gemm_wide_tile(pkg, oracle, gpu, K, N, M, gs, dtype, bias):
+    """N a multiple of 384 and a grid of 257 .. 511 tiles of 128 x 256: the launch takes the
+    128 x 384 tile of eight 48-column waves (gemm_gptq_wide_kernel).  Full and ragged last row
+    tiles, an odd number of K tiles, group sizes, asymmetric zero points, bias, both dtypes."""
+    _run(pkg, oracle, gpu, K, N, gs, M, dtype=dtype, sym=False, bias=bias, path=2, seed=K + M)
+
+
+def test_gemm_wide_tile_bit_exact_weights(pkg, oracle, gpu):
+    """One-hot activation rows through the 128 x 384 tile: row m of the output is row k(m) of the
+    dequantized matrix bit for bit (column order of the three fragments, the 96-bit word loads
+    and the paired stores of the epilogue included)."""
+    K, N, gs, M = 256, 6144, 128, 2048
+    qw, qz, sc, _ = oracle.make_gptq(K, N, gs, seed=12, sym=False)
+    w = oracle.dequant_gptq(qw, qz, sc, None, gs, "f16")
+    pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, gs, 0)
+    ks = np.arange(M) % K
+    x = torch.zeros((M, K), dtype=torch.float16, device=gpu)
+    x[torch.arange(M, device=gpu), torch.from_numpy(ks).to(gpu)] = 1.0
+    got = pkg.ops.linear(pk, x, None, path=2)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), w[ks].view(np.uint16))
+
+
 def test_gemm_bit_exact_weights_through_identity(pkg, oracle, gpu):
     """x = identity rows: y[m, :] must be W[m, :] exactly (fp16 W is what the MFMA sees, and
     a one-hot fp32 accumulation adds nothing), so the in-register unpack of the GEMM kernel is

@@ -7,6 +7,10 @@
 // The pairing (j, j+4) is kept all the way into the MFMA operand; the activation tile
 // is permuted to the same order instead of repacking the weights.
 #pragma once
+#ifdef Q4_PHASE_STAMPS
+// measurement build: waves per launch the phase-stamp buffer has room for
+#define Q4_PHASE_STAMP_SLOTS 16384
+#endif
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>

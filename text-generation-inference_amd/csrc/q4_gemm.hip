@@ -1,6 +1,7 @@
 // Prefill path, host side: tile and split-K plan, launch of the GPTQ MFMA kernel and of the
 // split-K reduction.  The device code is in q4_gemm_kernels.cuh.
 #include "q4_gemm_kernels.cuh"
+#include "q4_gemm_wide.cuh"
 
 namespace q4host {
 
@@ -102,6 +103,26 @@ static GemmPlan gemm_plan(int M, int K, int N) {
   // four-wave kernel, two to a CU, is the faster one (4096 x 6144: 115 against 127 us).
   if (g.bm == 128 && g.nw == 2 && g.tiles * g.splits <= 256 && (K / q4::kBK) % (2 * g.splits) == 0) g.kg = 2;
   return g;
+}
+
+// The 128 x 384 tile (gemm_gptq_wide_kernel, one workgroup of eight waves per CU) against the
+// 128 x 256 tile (two workgroups of four waves per CU): taken when the narrower tile runs unsplit
+// in a single, partly filled round of its 512 workgroup slots and the wide one fills its round of
+// 256 clearly better.  4096 x 6144: M = 2048, 384 tiles of 128 x 256 (half of the CUs with a
+// single workgroup) against 256 of 128 x 384, 110.4 -> 106.4 us; M = 1536, 288 against 192 tiles,
+// 96.3 -> 84.1 us.
+static bool gemm_wide_plan(const q4_weight* w, int M, const GemmPlan& g) {
+  if (w->N % q4::kWideBN != 0 || w->groupsize < 64 || w->groupsize % 64 != 0) return false;
+  if (g.bm != 128 || g.nw != 2 || g.splits != 1 || g.kg != 1) return false;
+  if ((long)(w->K >> 3) * w->N * 4 >= (1L << 32)) return false;
+  const long wide = (long)((M + 127) / 128) * (w->N / q4::kWideBN);
+  if (g.tiles <= 256 || g.tiles >= 512 || wide > 256) return false;  // one round of either (two: 191 against 182 us at M = 4096)
+  return (double)wide / 256.0 >= (double)g.tiles / 512.0 + 0.15;
+}
+
+template <int DTYPE>
+static void launch_wide(const GemmParams& gp, dim3 grid, hipStream_t stream) {
+  hipLaunchKernelGGL(q4::gemm_gptq_wide_kernel<DTYPE>, grid, dim3(512), 2 * q4::kWideBM * q4::kDirectRowBytes, stream, gp);
 }
 
 // per_cu: workgroups of this kernel that fit on a CU together (1 or 2)
@@ -234,6 +255,17 @@ int launch_gemm(const q4_weight* w, const void* x, const void* bias, void* y, in
     g.splits = 1;
   gp.splits = g.splits;
   gp.partials = g.splits > 1 ? (float*)((char*)workspace + Q4_WORKSPACE_COUNTER_BYTES) : nullptr;
+  if (gemm_wide_plan(w, M, g)) {
+    const long wide = (long)((M + 127) / 128) * (w->N / kWideBN);
+    if (dtype == Q4_DTYPE_F16) launch_wide<Q4_DTYPE_F16>(gp, dim3((unsigned)wide), stream);
+    else launch_wide<Q4_DTYPE_BF16>(gp, dim3((unsigned)wide), stream);
+    const hipError_t werr = hipGetLastError();
+    if (werr != hipSuccess) {
+      set_error("q4_linear(gemm): launch failed: %s", hipGetErrorString(werr));
+      return Q4_ERR_LAUNCH;
+    }
+    return Q4_OK;
+  }
   const int bm = g.bm, nw = g.nw;
   const long total = g.tiles * g.splits;
   if (total > 0x7fffffffL) {

@@ -11,6 +11,9 @@
 // readings ([workgroups][waves][8] 64-bit values; nullptr switches the stamps off).
 static unsigned long long* g_phase_stamps = nullptr;
 extern "C" void q4_phase_stamps_target(void* device_buffer) { g_phase_stamps = (unsigned long long*)device_buffer; }
+// waves per launch the target buffer has room for (8 readings of 8 bytes each); a launch with more
+// waves leaves no stamps
+extern "C" int q4_phase_stamps_slots(void) { return Q4_PHASE_STAMP_SLOTS; }
 #endif
 
 namespace q4host {
@@ -753,11 +756,11 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.ntiles = ntiles;
   gp.rows_per_block_alloc = rows;
   gp.wave_slab = wave_slab ? 1 : 0;
-#ifdef Q4_PHASE_STAMPS
-  gp.stamps = g_phase_stamps;
-#endif
   dim3 grid((unsigned)(ntiles * cfg.splits), (unsigned)mchunks);
   dim3 block((unsigned)(64 * cfg.wcol * cfg.wk));
+#ifdef Q4_PHASE_STAMPS
+  gp.stamps = (long)grid.x * grid.y * (block.x >> 6) <= Q4_PHASE_STAMP_SLOTS ? g_phase_stamps : nullptr;
+#endif
   if (diag) {
     launch_gemv_awq_diag(gp, dtype, rmax, grid, block, smem, stream);
   } else if (lean) {

@@ -140,12 +140,12 @@ int launch_gemv_direct(const q4_weight* w, const void* x, const void* bias, void
   }
   dp.num_groups = w->num_groups;
   dp.splits = splits;
-#ifdef Q4_PHASE_STAMPS
-  dp.stamps = g_direct_stamps;
-#endif
   const int mr = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 16));
   const dim3 grid((unsigned)(w->N / 64), (unsigned)splits);
   const dim3 block((unsigned)(64 * wk));
+#ifdef Q4_PHASE_STAMPS
+  dp.stamps = (long)grid.x * grid.y * wk <= Q4_PHASE_STAMP_SLOTS ? g_direct_stamps : nullptr;
+#endif
   // every wave's activation chunk (up to four rows), the K waves' sums, then the ticket drawn
   const size_t smem = (mr <= 4 ? (size_t)wk * 1024 : 0) + (size_t)wk * mr * 64 * sizeof(float) + 16;
   if (dtype == Q4_DTYPE_F16) launch_dtype<Q4_DTYPE_F16>(dp, mr, grid, block, smem, stream);
