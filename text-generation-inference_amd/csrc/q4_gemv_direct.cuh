@@ -59,7 +59,9 @@ __device__ __forceinline__ direct_rsrc_t direct_rsrc(const void* base, uint32_t 
 
 // MR: activation rows padded to 1, 2, 4 or 16.  Up to four rows sit in the first register quad
 // of the MFMA result (lanes of K block 0); sixteen fill it (lane block kq holds rows 4 kq .. 4 kq + 3).
-template <int DTYPE, int MR>
+// LOOP: some wave walks four chunks or more (the K loop proper); without it a wave has one to
+// three chunks and the kernel is straight-line code with fewer registers.
+template <int DTYPE, int MR, bool LOOP>
 __global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) {
   static_assert(MR == 1 || MR == 2 || MR == 4 || MR == 16, "rows are padded to 1, 2, 4 or 16");
   extern __shared__ __align__(16) unsigned char smem[];
@@ -87,7 +89,8 @@ __global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) 
   const uint32_t z_lane = (uint32_t)(col >> 3) * 4u;
   const int zshift = (col & 7) * 4;
   const bool row_live = j < dp.M;  // this lane's MFMA row carries an activation row
-  const uint32_t x_lane = ((uint32_t)(row_live ? j : 0) * (uint32_t)dp.K + (uint32_t)kq * 8u) * 2u;
+  // (a row beyond M is beyond the end of x: the buffer load returns zeros without a memory access)
+  const uint32_t x_lane = ((uint32_t)j * (uint32_t)dp.K + (uint32_t)kq * 8u) * 2u;
   const uint32_t step_bytes = (uint32_t)N * 16u;  // four packed rows
 
   // Up to four rows: the whole 128-row chunk of all of them is 4 x 256 bytes, one 16-byte load
@@ -96,8 +99,7 @@ __global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) 
   // K block) per 32-row step itself.
   constexpr bool XLDS = MR <= 4;
   constexpr int XREGS = XLDS ? 1 : kChunkSteps;
-  const bool xl_live = (lane >> 4) < dp.M;
-  const uint32_t xl_lane = ((uint32_t)(xl_live ? (lane >> 4) : 0) * (uint32_t)dp.K + (uint32_t)(lane & 15) * 8u) * 2u;
+  const uint32_t xl_lane = ((uint32_t)(lane >> 4) * (uint32_t)dp.K + (uint32_t)(lane & 15) * 8u) * 2u;
   unsigned char* xbuf = smem + wave * 1024;  // this wave's activation chunk (XLDS)
   struct Chunk {
     uint4_t x[XREGS];
@@ -105,36 +107,36 @@ __global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) 
     uint2_t s;
     uint32_t z;
   };
-  Chunk ring[PF];
+  Chunk qa, qb;  // the ring: two chunks of loads in flight
+  // No load of the K loop sits behind a branch: an activation row past M lies past the end of x
+  // (such a buffer load returns zeros and touches no memory), one to three chunks per wave are
+  // straight-line code, and the loop variant issues its refills unconditionally, the ones past
+  // the wave's range out of bounds.  With a branch around a load the compiler cannot count the
+  // loads in flight and waits for all of them, the newest chunk included, before it touches
+  // the oldest (measured: one memory round trip per chunk, 1.25 us, whatever the ring holds).
   auto load_chunk = [&](int c, Chunk& q) {
     const uint32_t chunk = (uint32_t)(c0 + c);
+    // loop variant: a chunk past the wave's range gets bit 31 into its lane offsets, which puts
+    // it past the end of every tensor (the host keeps them below 2 GB there): zeros, no access
+    const uint32_t past = LOOP && c >= nchunks ? 0x80000000u : 0u;
     // activations first: memory returns in issue order, and an L2 hit must not queue behind
     // the weight stream of this wave
     if constexpr (XLDS) {
-      q.x[0] = uint4_t{0u, 0u, 0u, 0u};
-      if (xl_live) q.x[0] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xl_lane, chunk * (kChunkRows * 2u), 0));
+      q.x[0] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xl_lane | past, chunk * (kChunkRows * 2u), 0));
     } else {
 #pragma unroll
-      for (int st = 0; st < kChunkSteps; ++st) {
-        q.x[st] = uint4_t{0u, 0u, 0u, 0u};
-        if (row_live)
-          q.x[st] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, x_lane, (chunk * kChunkRows + st * 32) * 2u, 0));
-      }
+      for (int st = 0; st < kChunkSteps; ++st)
+        q.x[st] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, x_lane | past, (chunk * kChunkRows + st * 32) * 2u, 0));
     }
 #pragma unroll
     for (int st = 0; st < kChunkSteps; ++st)
-      q.w[st] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, w_lane, (chunk * kChunkSteps + st) * step_bytes, 2));
+      q.w[st] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, w_lane | past, (chunk * kChunkSteps + st) * step_bytes, 2));
     // scale and zero point are needed when the chunk's last MFMA is done: asked for behind the
     // weights, they arrive with them instead of holding their return back
     const uint32_t gi = (uint32_t)min((int)(chunk >> dp.gshift), dp.num_groups - 1);
-    q.s = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(srsrc, s_lane, gi * (uint32_t)N * 2u, 0));
-    q.z = __builtin_amdgcn_raw_buffer_load_b32(zrsrc, z_lane, gi * (uint32_t)(N >> 3) * 4u, 0);
+    q.s = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(srsrc, s_lane | past, gi * (uint32_t)N * 2u, 0));
+    q.z = __builtin_amdgcn_raw_buffer_load_b32(zrsrc, z_lane | past, gi * (uint32_t)(N >> 3) * 4u, 0);
   };
-#pragma unroll
-  for (int b = 0; b < PF; ++b)
-    if (b < nchunks) load_chunk(b, ring[b]);
-  ps.mark(6);
-  ps.mark(1);
 
   // constant B operand: column 0 the splice offsets c_k, column 1 ones
   uint4_t bconst = {0u, 0u, 0u, 0u};
@@ -160,6 +162,9 @@ __global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) 
     return a;
   };
   auto process_chunk = [&](const Chunk& q) {
+    // (scheduling fences around a chunk: without them the copies of this block in the schedule
+    // below are interleaved with each other and the register count doubles)
+    __builtin_amdgcn_sched_barrier(0);
     float4_t acc[4], accc;
     if constexpr (XLDS) *(uint4_t*)(xbuf + lane * 16) = k_order(q.x[0]);  // rows beyond M: zeros
 #pragma unroll
@@ -200,17 +205,48 @@ __global__ __launch_bounds__(512) void gemv_gptq_direct_kernel(DirectParams dp) 
 #pragma unroll
       for (int t = 0; t < 4; ++t) tot[t][i] = fmaf(sf[t], acc[t][i] - fmaf(zf[t], S, P), tot[t][i]);
     }
+    __builtin_amdgcn_sched_barrier(0);
   };
 
-  for (int cb = 0; cb < nchunks; cb += PF) {
-#pragma unroll
-    for (int b = 0; b < PF; ++b) {
-      const int c = cb + b;
-      if (c < nchunks) {
-        process_chunk(ring[b]);
-        if (c == 0) ps.mark_after(2, tot[0][0]);
-        if (c + PF < nchunks) load_chunk(c + PF, ring[b]);
-      }
+  // The wave's chunks, two in flight.  One, two and three chunks are straight-line code (a
+  // kernel variant of its own: 88-120 registers); from four on a loop whose refills are
+  // unconditional.  Either way every wait can be counted at compile time.
+  static_assert(PF == 2, "the schedule below is written for two chunks in flight");
+  // chunks c (in qa), c + 1 (in qb) and, with three left, c + 2
+  auto end_piece = [&](int c, bool three, bool first) {
+    process_chunk(qa);
+    if (first) ps.mark_after(2, tot[0][0]);
+    if (three) {
+      load_chunk(c + 2, qa);
+      process_chunk(qb);
+      process_chunk(qa);
+    } else {
+      process_chunk(qb);
+    }
+  };
+  if (nchunks == 1) {
+    load_chunk(0, qa);
+    ps.mark(6);
+    ps.mark(1);
+    process_chunk(qa);
+    ps.mark_after(2, tot[0][0]);
+  } else if (nchunks <= 3) {
+    load_chunk(0, qa);
+    load_chunk(1, qb);
+    ps.mark(6);
+    ps.mark(1);
+    end_piece(0, nchunks == 3, true);
+  } else if constexpr (LOOP) {
+    load_chunk(0, qa);
+    load_chunk(1, qb);
+    ps.mark(6);
+    ps.mark(1);
+    for (int c = 0; c < nchunks; c += 2) {
+      process_chunk(qa);
+      if (c == 0) ps.mark_after(2, tot[0][0]);
+      load_chunk(c + 2, qa);
+      if (c + 1 < nchunks) process_chunk(qb);
+      load_chunk(c + 3, qb);
     }
   }
   ps.mark_after(3, tot[0][0]);

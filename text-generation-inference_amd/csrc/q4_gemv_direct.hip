@@ -22,9 +22,15 @@ bool gemv_direct_supported(const q4_weight* w, int M, int dtype, int wk, int spl
     if (w->groupsize % 128 != 0 || per < 1 || (per & (per - 1)) != 0) return false;
   }
   if ((long)w->num_groups * w->groupsize < w->K) return false;
-  if ((long)(w->K / 8) * w->N * 4 >= (1L << 32) || (long)w->num_groups * w->N * 2 >= (1L << 32) || (long)M * w->K * 2 >= (1L << 32))
+  // 32-bit byte offsets; the lane offset of an activation row past M must not wrap either
+  if ((long)(w->K / 8) * w->N * 4 >= (1L << 32) || (long)w->num_groups * w->N * 2 >= (1L << 32) || (long)16 * w->K * 2 >= (1L << 32))
     return false;
   if (wk < 1 || wk > 8 || splits < 1 || splits > 65535 || (long)wk * splits > w->K / 128) return false;
+  // four chunks or more per wave: the loop variant marks refills past a wave's range with bit 31 of
+  // the lane offset, so every tensor must end below 2 GB
+  if ((w->K / 128 + wk * splits - 1) / (wk * splits) > 3 &&
+      ((long)(w->K / 8) * w->N * 4 >= (1L << 31) || (long)w->num_groups * w->N * 2 >= (1L << 31) || (long)16 * w->K * 2 >= (1L << 31)))
+    return false;
   if (splits > 1 && w->N / 64 > Q4_WORKSPACE_TICKET_BYTES / 4) return false;
   return true;
 }
@@ -47,11 +53,13 @@ size_t gemv_direct_workspace_bytes(const q4_weight* w, int M, int dtype, int spl
 // better choice.
 //   Up to three rows: four K waves per workgroup (fewer on a K shorter than four chunks) and the
 // fewest K splits, up to the 14 the cells count, that leave every wave the fewest chunks.
-//   Four to sixteen rows: about one workgroup per CU (splits = 256 / column tiles, rounded), eight
-// K waves beyond four rows.  With 256 column tiles or more (no split) and more than four rows
-// every wave would re-read its share of the activations from L2 next to a long weight stream;
-// the kernels that stage the activations once per workgroup are faster there (4096 x 28672, 16
-// rows: 19.5 against 17.7 us), so those shapes are not taken.
+//   Four rows: about one workgroup per CU (splits = 256 / column tiles, rounded), four K waves.
+// Five to sixteen rows: eight K waves and the fewest splits that deal K evenly, leave a wave at
+// most two chunks and make 192 workgroups or more (else the four-row rule).  With 256 column
+// tiles or more (no split) and more than four rows every wave would re-read its share of the
+// activations from L2 next to a long weight stream; the kernels that stage the activations once
+// per workgroup are faster there (4096 x 28672, 16 rows: 19.8 against 17.5 us), so those shapes
+// are not taken.
 bool gemv_direct_default(const q4_weight* w, int M, int dtype, int* wk_out, int* splits_out) {
   const int chunks = w->K / 128;
   if (M <= 3) {
@@ -75,6 +83,16 @@ bool gemv_direct_default(const q4_weight* w, int M, int dtype, int* wk_out, int*
   int s = tiles >= 256 ? 1 : (256 + tiles / 2) / tiles;
   s = s < 1 ? 1 : (s > 14 ? 14 : s);
   int wk = M > 4 ? 8 : 4;
+  if (M > 4) {
+    // the fewest splits that deal K evenly, leave a wave at most two chunks and make 192
+    // workgroups or more (4096 x 6144: 8 x 2, 4096 x 4096: 8 x 4, 14336 x 4096: 8 x 7)
+    for (int t = 1; t <= 14; ++t) {
+      if (chunks % (8 * t) == 0 && chunks / (8 * t) <= 2 && (long)tiles * t >= 192) {
+        s = t;
+        break;
+      }
+    }
+  }
   while (wk > 1 && wk * s > chunks) wk >>= 1;
   while (s > 1 && wk * s > chunks) --s;
   if (!gemv_direct_supported(w, M, dtype, wk, s)) return false;
@@ -86,7 +104,9 @@ bool gemv_direct_default(const q4_weight* w, int M, int dtype, int* wk_out, int*
 
 template <int DTYPE, int MR>
 static void launch_one(const DirectParams& dp, dim3 grid, dim3 block, size_t smem, hipStream_t stream) {
-  hipLaunchKernelGGL((q4::gemv_gptq_direct_kernel<DTYPE, MR>), grid, block, smem, stream, dp);
+  // the straight-line variant when no wave walks more than three chunks
+  if (dp.cpw + (dp.rem > 0 ? 1 : 0) <= 3) hipLaunchKernelGGL((q4::gemv_gptq_direct_kernel<DTYPE, MR, false>), grid, block, smem, stream, dp);
+  else hipLaunchKernelGGL((q4::gemv_gptq_direct_kernel<DTYPE, MR, true>), grid, block, smem, stream, dp);
 }
 
 template <int DTYPE>

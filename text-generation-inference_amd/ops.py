@@ -460,8 +460,8 @@ def _time_graph_launches(fns, reps: int) -> float:
 
 def decode_candidates(w: PackedWeight, M: int, dtype: torch.dtype = torch.float16) -> list:
     """Explicit decode configurations the library offers for timing against its own choice."""
-    buf = (ctypes.c_int32 * (4 * 32))()
-    n = int(_lib.load().q4_gemv_candidates(ctypes.byref(w.struct()), int(M), _DTYPES[dtype], buf, 32))
+    buf = (ctypes.c_int32 * (4 * 64))()
+    n = int(_lib.load().q4_gemv_candidates(ctypes.byref(w.struct()), int(M), _DTYPES[dtype], buf, 64))
     _lib.check(n)
     return [tuple(int(buf[4 * i + k]) for k in range(4)) for i in range(n)]
 
