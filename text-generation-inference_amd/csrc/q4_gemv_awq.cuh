@@ -68,7 +68,13 @@ __global__ __launch_bounds__(512) void gemv_awq_diag_kernel(GemvParams gp) {
   const int cw = (d.tile * d.tile_cols + d.wc * 256) / 8 + 2 * d.j;  // first of this lane's 2 words
   const int col0 = cw * 8;
   const int nsteps = d.KW / 32;
-  constexpr int PF = 3;  // 32-row steps (8 x 64-bit loads each) in flight per wave
+  // 32-row steps (8 x 64-bit loads each) in flight per wave: one 128-row chunk.  A wave's K
+  // range is whole chunks, so the first four steps are loaded unconditionally and the loop
+  // refills a step's registers with the same step of the next chunk without a test; the last
+  // chunk is processed outside the loop.  (With a branch around a load the compiler cannot count
+  // the loads in flight: the activation staging below then waits for the whole weight prefetch
+  // and every step for the newest refill.)
+  constexpr int PF = 4;
 
   SlabStager<false> slab;
   slab.issue(gp, d, nullptr);
@@ -83,8 +89,7 @@ __global__ __launch_bounds__(512) void gemv_awq_diag_kernel(GemvParams gp) {
       w[r] = __builtin_nontemporal_load((const uint2_t*)(wbase + (size_t)(st * 32 + r) * row_bytes + w_lane));
   };
 #pragma unroll
-  for (int b = 0; b < PF; ++b)
-    if (b < nsteps) load_step(b, wq[b]);
+  for (int b = 0; b < PF; ++b) load_step(b, wq[b]);
 
   // scales (16 halves) and zero points (2 words) of the lane's columns for one group: asked
   // for when the group starts, used when it ends
@@ -209,16 +214,16 @@ __global__ __launch_bounds__(512) void gemv_awq_diag_kernel(GemvParams gp) {
     }
   };
 
-  for (int s0 = 0; s0 < nsteps; s0 += PF) {
+  int s0 = 0;
+  for (; s0 + PF < nsteps; s0 += PF) {
 #pragma unroll
     for (int b = 0; b < PF; ++b) {
-      const int st = s0 + b;
-      if (st < nsteps) {
-        process_step(st, wq[b]);
-        if (st + PF < nsteps) load_step(st + PF, wq[b]);
-      }
+      process_step(s0 + b, wq[b]);
+      load_step(s0 + PF + b, wq[b]);
     }
   }
+#pragma unroll
+  for (int b = 0; b < PF; ++b) process_step(s0 + b, wq[b]);
 
   gemv_finish<DTYPE, 16, G, false, true>(gp, d, tot, col0, smem);
 }

@@ -52,11 +52,6 @@ struct DirectParams {
 #endif
 };
 
-typedef __amdgpu_buffer_rsrc_t direct_rsrc_t;
-__device__ __forceinline__ direct_rsrc_t direct_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
-
 // MR: activation rows padded to 1, 2, 4 or 16.  Up to four rows sit in the first register quad
 // of the MFMA result (lanes of K block 0); sixteen fill it (lane block kq holds rows 4 kq .. 4 kq + 3).
 // LOOP: some wave walks four chunks or more (the K loop proper); without it a wave has one to

@@ -84,6 +84,16 @@ inline int max_wave_rows(const GemvParams& gp) {
   return (a > b ? a : b) * 128;
 }
 
+// Buffer loads: a scalar descriptor (base, byte count), one 32-bit lane offset and a scalar offset
+// that moves.  A lane offset at or past the byte count makes the load return zeros without a
+// memory access, which is how the decode loops keep their refill loads free of branches: with a
+// branch around a load the compiler cannot count the loads in flight and waits for all of them.
+typedef __amdgpu_buffer_rsrc_t direct_rsrc_t;
+__device__ __forceinline__ direct_rsrc_t direct_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint32_t scalar_u32(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+
 // Constants of the nibble splice, hidden from constant folding (empty asm, no instruction
 // is emitted): as literals the compiler must split (w & mask) | magic into v_and + v_or
 // because a three-operand VALU instruction cannot carry a literal; as register operands it
