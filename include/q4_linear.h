@@ -207,8 +207,11 @@ int q4_gemv_tuned(const q4_weight* w, const void* x, const void* bias, void* y, 
  * candidate on its own weights once per layer shape and row count and keeps the winner (the
  * Python layers do so in their Warmup hook).  Plays the role of the autotuner of the reference's
  * Triton path (server/text_generation_server/layers/gptq/custom_autotune.py:1-80, the config
- * list of layers/gptq/triton.py:14-103).  q4_gemv_tuned_workspace_bytes: workspace such a call
- * needs (the zero-initialised head included).
+ * list of layers/gptq/triton.py:14-103).  GPTQ weights with contiguous groups: decompositions
+ * of the short-launch kernel (words = -1); AWQ weights up to 8 rows: of the words-as-stored kernel
+ * (words = 0).  A candidate whose activations do not fit LDS makes q4_gemv_tuned return
+ * Q4_ERR_UNSUPPORTED; skip it.  q4_gemv_tuned_workspace_bytes: workspace such a call needs (the
+ * zero-initialised head included).
  */
 int q4_gemv_candidates(const q4_weight* w, int M, int dtype, int32_t* configs, int max_configs);
 size_t q4_gemv_tuned_workspace_bytes(const q4_weight* w, int M, int dtype, int wcol, int wk, int splits, int words);

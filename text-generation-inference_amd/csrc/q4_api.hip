@@ -618,6 +618,30 @@ int q4_gemv_candidates(const q4_weight* w, int M, int dtype, int32_t* configs, i
     return Q4_ERR_INVALID_ARGUMENT;
   }
   if (M < 1 || w->K == 0 || w->N == 0 || q4_select_path(w, M, dtype) != Q4_PATH_GEMV) return 0;
+  if (w->layout == Q4_LAYOUT_AWQ) {
+    // the words-as-stored kernel (up to 8 rows, 256-column wave tiles): K waves x K splits that
+    // deal K evenly, between one and thirty-two waves per CU
+    if (M > 8 || w->N % 256 != 0 || w->K % 128 != 0) return 0;
+    const int achunks = w->K / 128;
+    const long atiles = w->N / 256;
+    static const int kAwqWaves[] = {8, 4, 2};
+    static const int kAwqSplits[] = {1, 2, 4, 8, 7, 14, 3, 5, 6, 10, 12, 16};
+    int na = 0;
+    for (int wk : kAwqWaves) {
+      for (int sp : kAwqSplits) {
+        if (na >= max_configs) return na;
+        if (wk * sp > achunks || achunks % (wk * sp) != 0) continue;
+        const long waves = atiles * wk * sp;
+        if (waves < 256 || waves > 8192) continue;
+        configs[4 * na + 0] = 1;
+        configs[4 * na + 1] = wk;
+        configs[4 * na + 2] = sp;
+        configs[4 * na + 3] = 0;
+        ++na;
+      }
+    }
+    return na;
+  }
   // The short-launch kernel's decompositions: K waves per workgroup x workgroups along K.  Kept:
   // even K deals where the chunk count has them, between one and sixty-four waves per CU in all.
   const int chunks = w->K / 128;

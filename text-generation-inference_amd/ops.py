@@ -510,6 +510,10 @@ def autotune(weights=None, rows=(1, 2, 3, 4, 8, 16), dtype: torch.dtype = torch.
                 base = _time_graph_launches([(lambda w=w: linear(w, x, None, path=_lib.PATH_GEMV, out=y)) for w in rot], reps)
                 best_t, best_cfg = base, None
                 for cfg in cands:
+                    try:
+                        linear(rot[0], x, None, gemv_config=cfg, out=y)  # a decomposition that does not fit (LDS) is skipped
+                    except _lib.Q4Error:
+                        continue
                     t = _time_graph_launches([(lambda w=w, cfg=cfg: linear(w, x, None, gemv_config=cfg, out=y)) for w in rot], reps)
                     if t < best_t:
                         best_t, best_cfg = t, cfg
