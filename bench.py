@@ -740,7 +740,7 @@ def main():
     achieved = all_bytes / sum(all_durs) / 1e9
     roofline = {
         "bound": "hbm",
-        "kernel": "q4::gemv_gptq_kernel / q4::gemv_gptq_lean_kernel",
+        "kernel": "q4::gemv_gptq_direct_kernel",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
@@ -862,7 +862,7 @@ def main():
         if gm:
             out["gemm"] = {
                 "M": Mg, "per_shape": gm,
-                "roofline": {"bound": "mfma", "kernel": "q4::gemm_gptq_kernel", "achieved": round(tot_f / tot_t / 1e12, 1),
+                "roofline": {"bound": "mfma", "kernel": "q4::gemm_gptq_kernel / q4::gemm_gptq_wide_kernel (qkv)", "achieved": round(tot_f / tot_t / 1e12, 1),
                              "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                              "frac": round(tot_f / tot_t / 1e12 / MFMA_PEAK_TFLOPS, 4),
                              "traffic": measured_traffic(f"gemm_m{Mg}"),
