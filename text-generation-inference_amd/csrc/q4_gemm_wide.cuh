@@ -170,57 +170,100 @@ __global__ __launch_bounds__(512, 1) void gemm_gptq_wide_kernel(GemmParams gp) {
   afrag[0] = read_a(0, 0);
   afrag[1] = read_a(0, 1);
 
-  // One K tile.  A step unpacks its words, asks for the same step two tiles on into the freed
-  // registers and runs its MFMAs with the A fragments read two ahead; the second step moves tile
-  // kt + 1 from registers to the other LDS buffer and asks for tile kt + 2.  Tile indices past
-  // the end are clamped (fetched again, ignored): no branches.  (Unpacking a step ahead, spread
-  // between the MFMAs of the step before, measured slower: 110 against 106 us on 4096 x 6144 at
-  // M = 2048; with two waves per SIMD the other wave's MFMAs cover this one's unpacking.)
-  auto tile_step = [&](int kt, auto cur_c) {
+  // The pieces of a K tile.  A step = unpack (vector ALU: three words to 24 halves, then the
+  // refill of the freed registers two tiles on) + 24 MFMAs with the A fragments read two ahead.
+  // Tile indices past the end are clamped (fetched again, ignored): no branches.
+  auto unpack = [&](auto par_c, auto s_c, int kt_refill) {
+    constexpr int par = decltype(par_c)::value, s = decltype(s_c)::value;
+#pragma unroll
+    for (int f = 0; f < NF; ++f) bfrag[f] = dequant_word<DTYPE>(bq[par][s].v[f], cc[f], splice);
+    __builtin_amdgcn_sched_barrier(0);  // the unpacking stays in front of the MFMAs that follow
+    load_b(kt_refill, s, bq[par][s]);
+  };
+  // tail_barrier: the last two reads of step 1 cross into the next tile's buffer behind the
+  // tile's barrier; otherwise step 1 ends without them (the caller reads them after its barrier)
+  auto mfma_step = [&](auto cur_c, auto s_c, auto tail_c) {
+    constexpr int cur = decltype(cur_c)::value, s = decltype(s_c)::value;
+    constexpr bool tail_barrier = decltype(tail_c)::value;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int g = s * MT + mt;
+      const int gn = g + 2;
+      if (gn < FR) {
+        afrag[gn & 3] = read_a(cur, gn);
+      } else if constexpr (tail_barrier) {
+        // One barrier per tile: every wave has issued its last reads of this tile's buffer
+        // and written its share of the next tile into the other one.
+        if (gn == FR) __syncthreads();
+        afrag[gn & 3] = read_a(cur ^ 1, gn - FR);
+      }
+#pragma unroll
+      for (int f = 0; f < NF; ++f) acc[mt][f] = mfma16<DTYPE>(afrag[g & 3], bfrag[f], acc[mt][f]);
+      // per row fragment: its LDS read, three MFMAs, a share of the step's global loads
+      __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  // Odd and even waves walk a tile in opposite phase.  The tile barrier keeps the eight waves in
+  // step: left alone they all unpack together (vector ALU, the activation tile's LDS writes) and
+  // all multiply together (every MFMA group behind a 1 KB fragment read: 85 bytes per clock of
+  // the LDS's 128 when all four SIMDs multiply).  Even waves run unpack 0, MFMAs 0, unpack 1,
+  // MFMAs 1; odd waves run MFMAs 0, unpack 1, MFMAs 1, unpack 0 of the next tile, and both reach
+  // the tile's barrier at the same time.  Measured on 4096 x 6144, same box: M = 1536 86.1 ->
+  // 81.4 us, 2000 105.6 -> 102.8, 2048 106.4 -> 105.7; bf16 93.0 -> 87.8, 99.1 -> 95.9, 100.1 ->
+  // 97.2.  Splitting the two waves of one SIMD instead (by hardware SIMD id, or w and w + 4)
+  // gained nothing.  (Unpacking a step ahead inside one wave, spread between the MFMAs of the
+  // step before, measured slower: 110 against 106 us at M = 2048.)
+  auto tile_early = [&](int kt, auto cur_c) {
     constexpr int cur = decltype(cur_c)::value;
+    using Cur = std::integral_constant<int, cur>;
     const int kt1 = min(kt + 1, last_tile), kt2 = min(kt + 2, last_tile);
     make_group();
     load_group_raw(kt1);
-#pragma unroll
-    for (int s = 0; s < kDirectSteps; ++s) {
-#pragma unroll
-      for (int f = 0; f < NF; ++f) bfrag[f] = dequant_word<DTYPE>(bq[cur][s].v[f], cc[f], splice);
-      __builtin_amdgcn_sched_barrier(0);  // the unpacking stays in front of the step's MFMAs
-      load_b(kt2, s, bq[cur][s]);
-      if (s == 1) {
-        store_a(cur ^ 1);
-        load_a(kt2);
-      }
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const int g = s * MT + mt;
-        const int gn = g + 2;
-        if (gn < FR) {
-          afrag[gn & 3] = read_a(cur, gn);
-        } else {
-          // One barrier per tile: every wave has issued its last reads of this tile's buffer
-          // and written its share of the next tile into the other one.
-          if (gn == FR) __syncthreads();
-          afrag[gn & 3] = read_a(cur ^ 1, gn - FR);
-        }
-#pragma unroll
-        for (int f = 0; f < NF; ++f) acc[mt][f] = mfma16<DTYPE>(afrag[g & 3], bfrag[f], acc[mt][f]);
-        // per row fragment: its LDS read, three MFMAs, a share of the step's global loads
-        __builtin_amdgcn_sched_group_barrier(0x080, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      }
-    }
+    unpack(Cur{}, I0{}, kt2);
+    mfma_step(Cur{}, I0{}, std::true_type{});
+    unpack(Cur{}, I1{}, kt2);
+    store_a(cur ^ 1);
+    load_a(kt2);
+    mfma_step(Cur{}, I1{}, std::true_type{});
   };
-  {
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
+  auto tile_late = [&](int kt, auto cur_c) {
+    constexpr int cur = decltype(cur_c)::value;
+    using Cur = std::integral_constant<int, cur>;
+    using Nxt = std::integral_constant<int, cur ^ 1>;
+    const int kt2 = min(kt + 2, last_tile), kt3 = min(kt + 3, last_tile);
+    mfma_step(Cur{}, I0{}, std::true_type{});
+    unpack(Cur{}, I1{}, kt2);
+    store_a(cur ^ 1);
+    load_a(kt2);
+    mfma_step(Cur{}, I1{}, std::false_type{});
+    make_group();  // the next tile's group (its raw values were asked for a tile ago)
+    load_group_raw(kt2);
+    unpack(Nxt{}, I0{}, kt3);
+    __syncthreads();
+    afrag[0] = read_a(cur ^ 1, 0);
+    afrag[1] = read_a(cur ^ 1, 1);
+  };
+  if ((wave & 1) == 0) {
     int kt = 0;
     for (; kt + 1 < KT; kt += 2) {
-      tile_step(kt, I0{});
-      tile_step(kt + 1, I1{});
+      tile_early(kt, I0{});
+      tile_early(kt + 1, I1{});
     }
-    if (kt < KT) tile_step(kt, I0{});
+    if (kt < KT) tile_early(kt, I0{});
+  } else {
+    make_group();
+    load_group_raw(min(1, last_tile));
+    unpack(I0{}, I0{}, min(2, last_tile));
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+      tile_late(kt, I0{});
+      tile_late(kt + 1, I1{});
+    }
+    if (kt < KT) tile_late(kt, I0{});
   }
 
   // ---- epilogue.  C layout of the 16x16 MFMA: register r of lane (c16, kb) is row 4 kb + r,
