@@ -51,9 +51,10 @@ size_t gemv_direct_workspace_bytes(const q4_weight* w, int M, int dtype, int spl
 // The decomposition the plain call takes when it runs this kernel; false when the kernel does
 // not take the problem, the splits would not meet in the cells, or the slab kernels are the
 // better choice.
-//   Up to three rows: four K waves per workgroup (fewer on a K shorter than four chunks) and the
-// fewest K splits, up to the 14 the cells count, that leave every wave the fewest chunks.
-//   Four rows: about one workgroup per CU (splits = 256 / column tiles, rounded), four K waves.
+//   Up to two rows, and three or four rows on fewer than 256 column tiles: four K waves per
+// workgroup (fewer on a K shorter than four chunks) and the fewest K splits, up to the 14 the
+// cells count, that leave every wave the fewest chunks.
+//   Three and four rows on 256 column tiles or more: four K waves, K whole (no atomics).
 // Five to sixteen rows: eight K waves and the fewest splits that deal K evenly, leave a wave at
 // most two chunks and make 192 workgroups or more (else the four-row rule).  With 256 column
 // tiles or more (no split) and more than four rows every wave would re-read its share of the
@@ -62,7 +63,11 @@ size_t gemv_direct_workspace_bytes(const q4_weight* w, int M, int dtype, int spl
 // are not taken.
 bool gemv_direct_default(const q4_weight* w, int M, int dtype, int* wk_out, int* splits_out) {
   const int chunks = w->K / 128;
-  if (M <= 3) {
+  const int tiles = w->N / 64;
+  // (sweep of the four Llama-3-8B projections at three and four rows, us, this rule against the
+  // one-workgroup-per-CU rule it replaces there: 4096 x 6144 M = 4 5.92 / 7.05, 4096 x 4096 5.13 /
+  // 5.52, 14336 x 4096 9.75 / 10.00; 4096 x 28672 M = 3 with K whole 14.35 against 16.19 in 8 splits)
+  if (M <= 2 || (M <= 4 && tiles < 256)) {
     const int wk = chunks >= 4 ? 4 : (chunks >= 2 ? 2 : 1);
     if (!gemv_direct_supported(w, M, dtype, wk, 1)) return false;
     int best_s = 1, best = (chunks + wk - 1) / wk;
@@ -78,7 +83,6 @@ bool gemv_direct_default(const q4_weight* w, int M, int dtype, int* wk_out, int*
     *splits_out = best_s;
     return true;
   }
-  const int tiles = w->N / 64;
   if (tiles < 1 || (tiles >= 256 && M > 4)) return false;
   int s = tiles >= 256 ? 1 : (256 + tiles / 2) / tiles;
   s = s < 1 ? 1 : (s > 14 ? 14 : s);
