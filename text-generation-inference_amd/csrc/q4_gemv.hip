@@ -725,17 +725,16 @@ int launch_gemv(const q4_weight* w, const void* x, const void* bias, void* y, in
   gp.wcol = cfg.wcol;
   gp.wk = cfg.wk;
   gp.splits = cfg.splits;
-  // fp16, few rows, plain epilogue, at least four columns per lane: one atomic per element beats
-  // the ticket.  The kernel first transposes a wave's sums through LDS (behind the K-wave
-  // partials) so that an atomic instruction covers 64 consecutive cells of one row: issued
-  // straight from the 16 lanes that hold a row, the four instructions of a GPTQ row cost 1 us
-  // more than the one (4096 x 4096, M = 1: 7.05 against 5.97 us; tickets 7.8 us).  The adds
-  // execute at the memory side, about 0.8 us per row of 4096 cells x 8 splits: up to three rows
-  // they beat the tickets (GPTQ 4096 x 4096, M = 2: 6.8 against 8.1 us, M = 3: 7.5 / 8.3; AWQ
-  // 14336 x 4096, M = 3: 18.1 / 22.4), from four rows on they do not.
-  constexpr int kCellRowsMax = 3;
+  // fp16, plain epilogue, at least four columns per lane: one atomic per element beats the
+  // ticket.  The kernel first transposes a wave's sums through LDS (behind the K-wave partials)
+  // so that an atomic instruction covers 64 consecutive cells of one row: issued straight from
+  // the 16 lanes that hold a row, the four instructions of a GPTQ row cost 1 us more than the
+  // one (4096 x 4096, M = 1: 7.05 against 5.97 us; tickets 7.8 us).  With several K waves the rows
+  // are dealt to them (one round trip for all rows); a single K wave takes up to three rows in
+  // turn, beyond that the tickets win.
+  const int cell_rows_max = cfg.wk > 1 ? 16 : 3;
   gp.fixed_point_split = cfg.splits > 1 && cfg.splits <= 14 && dtype == Q4_DTYPE_F16 && gate_up_act == 0 &&
-                         (nt >= 4 ? M <= kCellRowsMax : M == 1) && (size_t)M * w->N * 8 <= Q4_WORKSPACE_CELL_BYTES;
+                         (nt >= 4 ? M <= cell_rows_max : M == 1) && (size_t)M * w->N * 8 <= Q4_WORKSPACE_CELL_BYTES;
   if (gp.fixed_point_split && nt >= 4) {
     const int tile_rows = diag ? (4 * rmax < kRowsPerBlock ? 4 * rmax : kRowsPerBlock) : (rmax < 4 ? rmax : kRowsPerBlock);
     const size_t tile = red + (size_t)cfg.wcol * tile_rows * 16 * nt * sizeof(float);

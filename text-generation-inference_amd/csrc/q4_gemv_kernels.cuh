@@ -484,8 +484,8 @@ __device__ __forceinline__ void gemv_finish_impl(const GemvParams& gp, const Dec
         constexpr int TW = 16 * NT;
         constexpr int TILE_ROWS = KQROWS ? (4 * RMAX < kRowsPerBlock ? 4 * RMAX : kRowsPerBlock) : (RMAX < 4 ? RMAX : kRowsPerBlock);
         if (gp.wk == 1 && gp.wcol > 1) __syncthreads();  // other column waves may still read the slab
+        float* tile = (float*)smem + (size_t)(gp.wk - 1) * gp.wcol * NT * RMAX * 64 + (size_t)d.wc * TILE_ROWS * TW;
         if (d.wkk == 0) {
-          float* tile = (float*)smem + (size_t)(gp.wk - 1) * gp.wcol * NT * RMAX * 64 + (size_t)d.wc * TILE_ROWS * TW;
 #pragma unroll
           for (int r = 0; r < RMAX; ++r) {
             const int m = out_row<KQROWS>(d, r);
@@ -494,25 +494,53 @@ __device__ __forceinline__ void gemv_finish_impl(const GemvParams& gp, const Dec
               for (int t = 0; t < NT; ++t) tile[m * TW + d.j * NT + t] = out[t][r];
             }
           }
+        }
+        // Several rows: they are dealt to the K waves of the column wave, every wave with the adds
+        // of two rows in flight.  (One wave taking the rows in turn pays a memory round trip per
+        // row; the adds of several rows issued by one wave made the splits of a row arrive together
+        // and measured 5-20 % slower than that.)
+        const bool deal = d.mloc > 1 && gp.wk > 1;
+        if (deal) __syncthreads();  // the tile is visible to the other K waves
+        if (deal || d.wkk == 0) {
           const int nbase = col0 - d.j * NT;  // first column of this wave
-          // One row at a time: with the adds of several rows in flight at once the cells of a
-          // row see their splits arrive together and the whole combine measured 5-20 % slower.
-          for (int m = 0; m < d.mloc; ++m) {
-            unsigned long long* cell = gp.cells + (size_t)(d.mb + m) * N + nbase + d.lane;
-            unsigned long long before[PER_LANE], inc[PER_LANE];
+          const int step = deal ? gp.wk : 1;
+          for (int m0 = deal ? d.wkk : 0; m0 < d.mloc; m0 += 2 * step) {
+            const int m1 = m0 + step;
+            const bool two = deal && m1 < d.mloc;
+            unsigned long long* cell0 = gp.cells + (size_t)(d.mb + m0) * N + nbase + d.lane;
+            unsigned long long* cell1 = gp.cells + (size_t)(d.mb + (two ? m1 : m0)) * N + nbase + d.lane;
+            unsigned long long before0[PER_LANE], inc0[PER_LANE], before1[PER_LANE], inc1[PER_LANE];
 #pragma unroll
             for (int u = 0; u < PER_LANE; ++u) {
-              inc[u] = cell_increment(tile[m * TW + d.lane + 64 * u]);
-              before[u] = __hip_atomic_fetch_add(cell + 64 * u, inc[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              inc0[u] = cell_increment(tile[m0 * TW + d.lane + 64 * u]);
+              before0[u] = __hip_atomic_fetch_add(cell0 + 64 * u, inc0[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            ps.mark_after(5, __builtin_bit_cast(float, (uint32_t)before[0]));
+            if (two) {
+#pragma unroll
+              for (int u = 0; u < PER_LANE; ++u) {
+                inc1[u] = cell_increment(tile[m1 * TW + d.lane + 64 * u]);
+                before1[u] = __hip_atomic_fetch_add(cell1 + 64 * u, inc1[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              }
+            }
+            ps.mark_after(5, __builtin_bit_cast(float, (uint32_t)before0[0]));
 #pragma unroll
             for (int u = 0; u < PER_LANE; ++u) {
-              const unsigned long long now = before[u] + inc[u];
+              const unsigned long long now = before0[u] + inc0[u];
               if (cell_complete(now, gp.splits)) {
                 const int n = nbase + d.lane + 64 * u;
-                y[(size_t)(d.mb + m) * N + n] = finish_output<DTYPE>(cell_value(now), p.bias, n);
-                __hip_atomic_store(cell + 64 * u, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                y[(size_t)(d.mb + m0) * N + n] = finish_output<DTYPE>(cell_value(now), p.bias, n);
+                __hip_atomic_store(cell0 + 64 * u, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              }
+            }
+            if (two) {
+#pragma unroll
+              for (int u = 0; u < PER_LANE; ++u) {
+                const unsigned long long now = before1[u] + inc1[u];
+                if (cell_complete(now, gp.splits)) {
+                  const int n = nbase + d.lane + 64 * u;
+                  y[(size_t)(d.mb + m1) * N + n] = finish_output<DTYPE>(cell_value(now), p.bias, n);
+                  __hip_atomic_store(cell1 + 64 * u, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
               }
             }
           }
