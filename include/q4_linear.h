@@ -223,8 +223,8 @@ size_t q4_gemv_tuned_workspace_bytes(const q4_weight* w, int M, int dtype, int w
  * (temp_dq_size / temp_fwd_size / scratch_space_fixed).
  */
 #define Q4_WORKSPACE_TICKET_BYTES 16384   /* split-K arrival tickets, one per column tile */
-#define Q4_WORKSPACE_CELL_BYTES 1048576   /* 64-bit fixed-point accumulation cells (fp16 decode, few rows) */
-#define Q4_WORKSPACE_COUNTER_BYTES 1064960 /* = tickets + cells: the part that must start zero */
+#define Q4_WORKSPACE_CELL_BYTES 4194304   /* 64-bit fixed-point accumulation cells (fp16 decode: 16 rows x 32768 columns) */
+#define Q4_WORKSPACE_COUNTER_BYTES 4210688 /* = tickets + cells: the part that must start zero */
 size_t q4_workspace_bytes(int M, int K, int N);
 /*
  * The same for one weight: exactly what q4_linear / q4_linear_gate_up need for `w` at M rows

@@ -23,7 +23,7 @@ PATH_GEMV = 1
 PATH_GEMM = 2
 PATH_GENERIC = 3
 PATH_NAMES = {PATH_GEMV: "gemv", PATH_GEMM: "gemm", PATH_GENERIC: "generic"}
-WORKSPACE_COUNTER_BYTES = 1064960
+WORKSPACE_COUNTER_BYTES = 4210688
 
 ERR_INVALID_ARGUMENT = -1
 ERR_UNSUPPORTED = -2
