@@ -357,9 +357,9 @@ def test_awq_decompositions(pkg, oracle, gpu, cfg):
 def test_awq_auto_path_is_native(pkg, oracle, gpu):
     qw, qz, sc = oracle.make_awq(1024, 512, 128, seed=0)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 1)
-    for M in (1, 4):
+    for M in (1, 4, 6):
         assert pkg.ops.select_path(pk, M) == "gemv"
-    for M in (5, 9, 17, 100, 256):
+    for M in (7, 9, 17, 100, 256):
         assert pkg.ops.select_path(pk, M) == "gemm"  # the register-unpack MFMA kernel, split-K on small grids
     qw, qz, sc, gi = oracle.make_gptq(1024, 512, 128, seed=0, act_order=True)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), to_dev(gi, gpu), 128, 0)
@@ -467,15 +467,15 @@ def test_awq_gemm_bit_exact_weights_through_identity(pkg, oracle, gpu):
 def test_awq_dispatch_large_m(pkg, oracle, gpu):
     qw, qz, sc = oracle.make_awq(1024, 14336, 128, seed=0)
     pk = pkg.ops.make_packed(to_dev(qw, gpu), to_dev(qz, gpu), to_dev(sc, gpu), None, 128, 1)
-    assert pkg.ops.select_path(pk, 4) == "gemv"
-    assert pkg.ops.select_path(pk, 5) == "gemm"
+    assert pkg.ops.select_path(pk, 6) == "gemv"
+    assert pkg.ops.select_path(pk, 7) == "gemm"
     assert pkg.ops.select_path(pk, 64) == "gemm"
     # the kernel that unpacks the words in registers (groups of 64 rows or more, N a multiple of
-    # 256) takes over from 5 rows on whatever the shape
+    # 256) takes over from 7 rows on whatever the shape
     for K, N in [(4096, 4096), (4096, 6144), (14336, 4096), (4096, 14336), (8192, 28672), (28672, 8192)]:
         w = pkg.ops.PackedWeight(pk.qweight, pk.qzeros, pk.scales, None, K, N, 128, K // 128, 1)  # geometry only
-        assert pkg.ops.select_path(w, 4) == "gemv", (K, N)
-        assert pkg.ops.select_path(w, 5) == "gemm", (K, N)
+        assert pkg.ops.select_path(w, 6) == "gemv", (K, N)
+        assert pkg.ops.select_path(w, 7) == "gemm", (K, N)
     # groups of 32 rows go through the kernel that unpacks through LDS: the first row count that
     # goes to it moves with the shape (measured crossovers)
     for K, N, first in [(4096, 4096, 9), (4096, 6144, 14), (11008, 4096, 10), (14336, 4096, 17), (4096, 14336, 17),

@@ -141,7 +141,7 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
   // 41.6 / 56.4, 28672 x 8192 92.7 / 153; at M = 48 the three blocks win on some shapes, 18.5 /
   // 21.3 and 45.8 / 55.5, and lose on others, 46.6 / 42.7 and 182 / 155), from about M = 48 on
   // when it has to gather scales and zero points from global memory (~2x slower per tile).
-  // AWQ: up to 4 rows the decode kernel that feeds the words to the MFMA as stored; from 5 rows on
+  // AWQ: up to 6 rows the decode kernel that feeds the words to the MFMA as stored; from 7 rows on
   // the MFMA kernel that unpacks them in registers wherever it applies (split-K on small tile
   // grids, flat in M up to 32 rows: 17.4 against 28.3 us for 4096 x 14336 at M = 16, 17.9 against
   // 31.4 us for 14336 x 4096, 12.5 against 12.7 us for 4096 x 4096).  Other AWQ weights (N not a
@@ -156,10 +156,12 @@ int q4_select_path(const q4_weight* w, int M, int dtype) {
     else if (weights <= (1L << 24)) first_gemm_m = 9;
     else if (weights <= (1L << 25)) first_gemm_m = 14;
     else if ((w->K / 128) % 8 != 0 && weights <= (1L << 26)) first_gemm_m = 10;
-    // (the words-as-stored decode kernel takes a second accumulator set from five rows on: at
-    // M = 5 .. 8 it measured 13.2-25.9 us on 14 layer shapes where this kernel, flat in M, takes
-    // 11.2-22.7 us; 28672 x 8192 and 8192 x 28672 tie)
-    if (gemm_awq_direct_supported(w, M, dtype)) first_gemm_m = 5;
+    // (the words-as-stored decode kernel takes a second accumulator set from five rows on; since
+    // its K splits meet in the fixed-point cells at any row count it holds five and six rows --
+    // decode / this kernel in us at M = 6: 14336 x 4096 16.8 / 19.8, 4096 x 4096 11.3 / 13.5,
+    // 4096 x 6144 11.6 / 13.7, 4096 x 28672 23.2 / 23.5, 4096 x 14336 16.4 / 15.6 -- and loses from
+    // eight on: 14.9 / 13.5, 15.0 / 13.8, 17.0 / 16.0, except 14336 x 4096 17.4 / 20.0)
+    if (gemm_awq_direct_supported(w, M, dtype)) first_gemm_m = 7;
     small = M < first_gemm_m;
   }
   if (!small && gemm_awq_supported(w, M, dtype)) return Q4_PATH_GEMM;
